@@ -1,0 +1,334 @@
+/*
+ * rai_hip.h — C ABI of librai_hip.so, the gfx950 (MI355X) execution device for
+ * the rai lazy-tensor framework.
+ *
+ * Every entry point below is what a `Hip` device in rai-core would bind through
+ * `extern "C"`: one launcher per primitive that rai's evaluator dispatches
+ * (`trait Eval<D, P>::eval`, rai-core/src/backend/mod.rs:48-54), plus the storage
+ * calls behind `TensorLike` (rai-core/src/tensor.rs:19-26).  The comment above
+ * each declaration cites the reference implementation it replaces
+ * (paths relative to the rai source tree, v0.11.0).
+ *
+ * Conventions
+ *   - Plain C: pointers, sizes, PODs.  No C++/torch types.
+ *   - Every function returns 0 on success or a negative rai_hip_status;
+ *     rai_hip_last_error() returns a thread-local message for the last failure.
+ *     The reference backend `unwrap()`s every backend error (panic); a binding
+ *     should panic/raise on any non-zero status.
+ *   - All device work is enqueued on one HIP stream per device and is
+ *     asynchronous; only rai_hip_sync / rai_hip_d2h / rai_hip_timer_elapsed_ms block.
+ *   - A tensor is a strided view: element (i0..ir) lives at
+ *     data + (offset + sum(i_k * stride[k])) * sizeof(dtype).  Strides are in
+ *     elements, may be 0 (broadcast) and are never negative.
+ *   - Outputs never alias inputs (functional semantics, like the reference).
+ */
+#ifndef RAI_HIP_H
+#define RAI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RAI_HIP_MAX_RANK 8
+
+/* rai-core/src/dtype.rs: U8, U32, I64, F16, BF16, F32, F64 */
+typedef enum rai_hip_dtype {
+  RAI_U8 = 0,
+  RAI_U32 = 1,
+  RAI_I64 = 2,
+  RAI_F16 = 3,
+  RAI_BF16 = 4,
+  RAI_F32 = 5,
+  RAI_F64 = 6
+} rai_hip_dtype;
+
+typedef enum rai_hip_status {
+  RAI_OK = 0,
+  RAI_ERR_BAD_DTYPE = -1,
+  RAI_ERR_BAD_SHAPE = -2,
+  RAI_ERR_BAD_STRIDE = -3,
+  RAI_ERR_OOM = -4,
+  RAI_ERR_HIP = -5,
+  RAI_ERR_BAD_ARG = -6,
+  RAI_ERR_UNSUPPORTED = -7, /* rai-core/src/error.rs:10-14 Error::Unimplemented */
+  RAI_ERR_INDEX = -8        /* gather index out of range: never silent */
+} rai_hip_status;
+
+/* Strided tensor view over device memory (the storage half of
+ * rai-core/src/tensor.rs:19-37; candle's Layout{shape,stride,start_offset}). */
+typedef struct rai_hip_tensor {
+  void *data;     /* device pointer to the start of the underlying buffer */
+  int32_t dtype;  /* rai_hip_dtype */
+  int32_t rank;   /* 0..RAI_HIP_MAX_RANK */
+  int64_t shape[RAI_HIP_MAX_RANK];
+  int64_t stride[RAI_HIP_MAX_RANK]; /* elements */
+  int64_t offset;                   /* elements */
+} rai_hip_tensor;
+
+/* Unary primitives of rai-core/src/ops/ evaluated at
+ * rai-core/src/backend/candle.rs:445-473,525-553,608-656,947-978 */
+typedef enum rai_hip_unary_op {
+  RAI_UN_SIN = 0,
+  RAI_UN_COS = 1,
+  RAI_UN_NEG = 2,
+  RAI_UN_SQUARE = 3,
+  RAI_UN_SQRT = 4,
+  RAI_UN_RSQRT = 5, /* sqrt then reciprocal, candle.rs:545-553 */
+  RAI_UN_ABS = 6,
+  RAI_UN_EXP = 7,
+  RAI_UN_LOG = 8,
+  RAI_UN_LOG2 = 9,  /* ln(x)/ln(2), candle.rs:628-636 */
+  RAI_UN_LOG10 = 10,
+  RAI_UN_ERF = 11,
+  RAI_UN_TANH = 12,
+  RAI_UN_POWF = 13, /* param = exponent */
+  RAI_UN_SIGN = 14, /* (x>=0) - (x<=0), candle.rs:595-606 */
+  /* fused activations (rai-core/src/hlops/activations.rs:5-32) */
+  RAI_UN_GELU = 15,     /* x*0.5*(1+erf(x/sqrt(2))) */
+  RAI_UN_NEW_GELU = 16, /* tanh approximation */
+  RAI_UN_SILU = 17,     /* x/(exp(-x)+1) */
+  RAI_UN_RELU = 18,
+  RAI_UN_COUNT_
+} rai_hip_unary_op;
+
+/* rai-core/src/backend/candle.rs:275-325 (arith), :658-760 (compare, max/min) */
+typedef enum rai_hip_binary_op {
+  RAI_BIN_ADD = 0,
+  RAI_BIN_SUB = 1,
+  RAI_BIN_MUL = 2,
+  RAI_BIN_DIV = 3,
+  RAI_BIN_MAXIMUM = 4,
+  RAI_BIN_MINIMUM = 5,
+  RAI_BIN_EQ = 6, /* comparisons write U8 0/1 */
+  RAI_BIN_NE = 7,
+  RAI_BIN_GT = 8,
+  RAI_BIN_GE = 9,
+  RAI_BIN_LT = 10,
+  RAI_BIN_LE = 11,
+  RAI_BIN_COUNT_
+} rai_hip_binary_op;
+
+typedef enum rai_hip_reduce_op { RAI_RED_SUM = 0, RAI_RED_MAX = 1, RAI_RED_MIN = 2 } rai_hip_reduce_op;
+
+/* ------------------------------------------------------------------ runtime */
+
+/* Thread-local text of the last failure on the calling thread ("" if none). */
+const char *rai_hip_last_error(void);
+
+/* Number of visible HIP devices (rai-core/src/device.rs:198-204 cuda_if_available). */
+int rai_hip_device_count(int *count);
+
+/* Lazily create the per-device context: one stream, allocator pools.  Idempotent.
+ * Replaces the device cache at rai-core/src/backend/candle.rs:139-195. */
+int rai_hip_init(int dev);
+
+/* Block until everything enqueued on the device's stream has finished. */
+int rai_hip_sync(int dev);
+
+/* Ref-counted device allocation (refcount starts at 1).  Freed blocks go back to
+ * a per-device size-class pool, so steady-state evaluation calls no hipMalloc.
+ * Replaces candle's Arc<Storage> behind rai-core/src/tensor.rs:151-165 set_data. */
+int rai_hip_alloc(int dev, size_t bytes, void **out);
+int rai_hip_retain(void *ptr);
+int rai_hip_release(void *ptr);
+/* bytes currently handed out / bytes held in the pool / number of real hipMalloc calls */
+int rai_hip_mem_stats(int dev, uint64_t *in_use, uint64_t *pooled, uint64_t *n_device_mallocs);
+/* Return pooled blocks to the driver. */
+int rai_hip_trim(int dev);
+
+/* Host<->device copies of raw bytes.  h2d is stream-ordered and returns after the
+ * host buffer is consumed; d2h synchronises (TensorLike::as_vec / as_bytes,
+ * rai-core/src/backend/candle.rs:41-67; FromArray, candle.rs:258-273). */
+int rai_hip_h2d(int dev, void *dst_dev, const void *src_host, size_t bytes);
+int rai_hip_d2h(int dev, void *dst_host, const void *src_dev, size_t bytes);
+int rai_hip_d2d(int dev, void *dst_dev, const void *src_dev, size_t bytes);
+
+/* hipEvent timers on the device's stream (measurement only). */
+int rai_hip_timer_create(int dev, void **timer);
+int rai_hip_timer_start(void *timer);
+int rai_hip_timer_stop(void *timer);
+int rai_hip_timer_elapsed_ms(void *timer, float *ms); /* blocks on the stop event */
+int rai_hip_timer_destroy(void *timer);
+
+/* ----------------------------------------------------- creation primitives */
+
+/* Full<T>: rai-core/src/backend/candle.rs:197-209, ops/full.rs:63-72.
+ * `out` must be contiguous. */
+int rai_hip_fill(int dev, const rai_hip_tensor *out, double value);
+
+/* Arange<T>: candle.rs:241-256, ops/arange.rs:102-117.  out[i] = start + i*step. */
+int rai_hip_arange(int dev, const rai_hip_tensor *out, double start, double step);
+
+/* ------------------------------------------------- elementwise primitives */
+
+/* ToDType<T>: candle.rs:762-774.  Float->bf16/f16 rounds to nearest even;
+ * float->integer truncates toward zero (Rust `as`), saturating. */
+int rai_hip_cast(int dev, const rai_hip_tensor *in, const rai_hip_tensor *out);
+
+/* Strided copy, same dtype, same shape; `out` may itself be a strided view
+ * (used for ToContiguous candle.rs:980-988, Reshape of a non-contiguous view
+ * :565-573, Concatenate :880-889 — one call per piece into a narrowed output). */
+int rai_hip_copy(int dev, const rai_hip_tensor *in, const rai_hip_tensor *out);
+
+/* Unary primitives and fused activations; `in` may be strided, `out` contiguous. */
+int rai_hip_unary(int dev, int op, const rai_hip_tensor *in, const rai_hip_tensor *out, double param);
+
+/* Broadcast binary: operands already expanded to the output shape by stride-0
+ * views (rai-core/src/ops/mod.rs:298-340 wraps them in Broadcast nodes).
+ * Arithmetic output dtype = operand dtype; comparisons write U8. */
+int rai_hip_binary(int dev, int op, const rai_hip_tensor *lhs, const rai_hip_tensor *rhs,
+                   const rai_hip_tensor *out);
+
+/* Where: candle.rs:901-915 — out = cond ? on_true : on_false, cond is U8/U32/I64
+ * (non-zero = true). */
+int rai_hip_where(int dev, const rai_hip_tensor *cond, const rai_hip_tensor *on_true,
+                  const rai_hip_tensor *on_false, const rai_hip_tensor *out);
+
+/* ------------------------------------------------------------- reductions */
+
+/* ReduceSum/Max/Min over `ndims` axes of `in` (candle.rs:475-523).  `out` is
+ * contiguous with the reduced axes removed (keep_dim=0) or kept as size 1. */
+int rai_hip_reduce(int dev, int op, const rai_hip_tensor *in, const int32_t *dims, int32_t ndims,
+                   int32_t keep_dim, const rai_hip_tensor *out);
+
+/* Softmax along `dim`: candle.rs:793-826 (max, sub, exp, sum, div) in one pass.
+ * Arithmetic in f32 (f64 for F64), result rounded once to the tensor dtype. */
+int rai_hip_softmax(int dev, const rai_hip_tensor *in, int32_t dim, const rai_hip_tensor *out);
+int rai_hip_log_softmax(int dev, const rai_hip_tensor *in, int32_t dim, const rai_hip_tensor *out);
+
+/* ArgMax/ArgMin along `dim`: candle.rs:917-944, ops/argmax.rs:48-61.  Output U32,
+ * first index wins ties; NaN never wins.  `out` has `dim` removed or kept as 1. */
+int rai_hip_argmax(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
+                   const rai_hip_tensor *out);
+int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
+                   const rai_hip_tensor *out);
+
+/* ---------------------------------------------------------------- indexing */
+
+/* IndexSelect: candle.rs:867-878, ops/index_select.rs:52-61.  index is a rank-1
+ * U8/U32/I64 tensor; out.shape[dim] == index length.  An index >= in.shape[dim]
+ * makes the call fail with RAI_ERR_INDEX at the next synchronising call and the
+ * offending row is zero-filled. */
+int rai_hip_index_select(int dev, const rai_hip_tensor *in, const rai_hip_tensor *index, int32_t dim,
+                         const rai_hip_tensor *out);
+/* Number of out-of-range indices seen by gathers since the last call (syncs). */
+int rai_hip_index_errors(int dev, uint64_t *count);
+
+/* ------------------------------------------------------------ contraction */
+
+/* MatMul: candle.rs:327-443, ops/matmul.rs:34-70, shape.rs:130-160.
+ * a[..., M, K] x b[..., K, N] -> out[..., M, N]; leading dims already broadcast
+ * to out's (stride 0 allowed); any strides accepted for the last two dims.
+ * bf16/f16 accumulate in f32 and round once; f32 accumulates in f32. */
+int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, const rai_hip_tensor *out);
+
+/* ------------------------------------------- fused compositions (rai-nn) */
+
+/* Linear::fwd rai-nn/src/linear.rs:59-69: out[.., n] = act(sum_k x[.., k] w[n, k] + bias[n]) (+ residual).
+ * w is [N, K] row-major; bias (nullable) is [N]; act is a rai_hip_unary_op
+ * activation or -1; residual (nullable) has out's shape.  x rows must be
+ * K-contiguous. */
+int rai_hip_linear(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, const rai_hip_tensor *bias,
+                   int32_t act, const rai_hip_tensor *residual, const rai_hip_tensor *out);
+
+/* LayerNorm::fwd rai-nn/src/layer_norm.rs:32-42 over the last dim (population
+ * variance, eps inside the square root); w, b nullable together. */
+int rai_hip_layer_norm(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, const rai_hip_tensor *b,
+                       double eps, const rai_hip_tensor *out);
+
+/* RmsNorm::fwd rai-nn/src/rms_norm.rs:18-22 (add_one=0) and Gemma's
+ * rai-models/src/llm/gemma.rs:42-54 (add_one=1: x/sqrt(mean(x^2)+eps) * (1+w)). */
+int rai_hip_rms_norm(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, double eps, int32_t add_one,
+                     const rai_hip_tensor *out);
+
+/* Rotary embedding, NeoX rotate-half over the first rot_dim of the last dim of
+ * x[B, H, S, D] (any strides): rai-models/src/llm/phi2.rs:44-78, qwen2.rs:33-72,
+ * gemma.rs:64-103.  cos/sin tables are [max_pos, rot_dim] in x's dtype or F32;
+ * rows offset..offset+S are used. */
+int rai_hip_rope(int dev, const rai_hip_tensor *x, const rai_hip_tensor *cos, const rai_hip_tensor *sin,
+                 int32_t rot_dim, int64_t offset, const rai_hip_tensor *out);
+/* Build the tables on device: inv_freq[i] = theta^(-2i/rot_dim) (f32 powf as
+ * phi2.rs:48-51 when f64_powf=0; f64 powf then cast as qwen2.rs:45-48 when 1),
+ * angle = pos * inv_freq in f32, table[pos][i] = table[pos][i+rot_dim/2]. */
+int rai_hip_rope_tables(int dev, double theta, int32_t rot_dim, int32_t f64_powf, const rai_hip_tensor *cos,
+                        const rai_hip_tensor *sin);
+
+/* Scaled-dot-product attention over q[B, Hq, S, D], k/v[B, Hkv, T, D] with
+ * Hq % Hkv == 0 (repeat_kv gemma.rs:191-201 is implied, never materialised).
+ * causal!=0 masks key j > (T - S) + i as phi2.rs:104-117 / gemma.rs:341-362.
+ * f32_scores!=0 follows phi2.rs:244-260 (f32 logits and softmax); otherwise
+ * scores are rounded to the tensor dtype before softmax as qwen2.rs:205-216.
+ * out is [B, S, Hq*D] contiguous (the transpose(1,2)+reshape of phi2.rs:261-262). */
+int rai_hip_attention(int dev, const rai_hip_tensor *q, const rai_hip_tensor *k, const rai_hip_tensor *v,
+                      double scale, int32_t causal, int32_t f32_scores, const rai_hip_tensor *out);
+
+/* ------------------------------------------- decoder-only model drivers */
+
+typedef enum rai_hip_arch {
+  RAI_ARCH_PHI2 = 0,  /* rai-models/src/llm/phi2.rs */
+  RAI_ARCH_QWEN2 = 1, /* rai-models/src/llm/qwen2.rs */
+  RAI_ARCH_GEMMA = 2  /* rai-models/src/llm/gemma.rs */
+} rai_hip_arch;
+
+/* Union of the serde Config structs phi2.rs:9-24, qwen2.rs:8-24, gemma.rs:12-27. */
+typedef struct rai_hip_decoder_config {
+  int32_t arch;
+  int32_t dtype; /* RAI_BF16 or RAI_F32 */
+  int32_t vocab_size;
+  int32_t hidden_size;
+  int32_t intermediate_size;
+  int32_t num_hidden_layers;
+  int32_t num_attention_heads;
+  int32_t num_key_value_heads;
+  int32_t head_dim;
+  int32_t rotary_dim; /* phi2: partial_rotary_factor*head_dim; others: head_dim */
+  int32_t max_position_embeddings;
+  int32_t hidden_act; /* RAI_UN_NEW_GELU / RAI_UN_GELU / RAI_UN_SILU */
+  int32_t tie_word_embeddings;
+  int32_t max_batch;   /* KV cache is preallocated for max_batch x max_context */
+  int32_t max_context;
+  /* 0: rotary tables computed in the model dtype exactly as the reference does
+   * (phi2.rs:53-57: positions and pos*inv_freq rounded to bf16 for a bf16
+   * model); 1: angles computed in f32 and rounded once. */
+  int32_t rope_tables_f32;
+  double rope_theta;
+  double norm_eps;
+} rai_hip_decoder_config;
+
+typedef struct rai_hip_decoder rai_hip_decoder;
+
+/* Model::new (phi2.rs:316-332): allocates weights (uninitialised), KV cache and
+ * activation arena once; no allocation happens in forward afterwards. */
+int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_decoder **out);
+int rai_hip_decoder_destroy(rai_hip_decoder *dec);
+/* Module::update_by_safetensors naming (rai-core/src/nn.rs:183-205, renames
+ * phi2.rs:307-313): copy one named parameter from host memory, e.g.
+ * "model.layers.3.self_attn.q_proj.weight".  `data` is row-major in the model dtype. */
+int rai_hip_decoder_load_param(rai_hip_decoder *dec, const char *name, const void *host_data, size_t bytes);
+/* Number of parameter names the architecture expects / i-th name (for loaders). */
+int rai_hip_decoder_param_count(rai_hip_decoder *dec, int32_t *count);
+int rai_hip_decoder_param_name(rai_hip_decoder *dec, int32_t i, char *buf, size_t buflen, int64_t *numel);
+/* Model::fwd (phi2.rs:334-347): ids_host[batch*seq] u32 are appended after the
+ * cached context; returns last-position logits [batch, vocab] as f32 in
+ * logits_host (nullable) and greedy tokens (device argmax, first-max) in
+ * tokens_host (nullable).  Synchronises only if an output pointer is given. */
+int rai_hip_decoder_forward(rai_hip_decoder *dec, const uint32_t *ids_host, int32_t batch, int32_t seq,
+                            float *logits_host, uint32_t *tokens_host);
+/* Greedy loop of examples/phi2/src/main.rs:75-95 without repeat penalty: prefill
+ * prompt[batch*prompt_len], then n_new single-token steps feeding the device
+ * argmax back without host round trips.  tokens_host[batch*n_new]. prefill_ms /
+ * decode_ms (nullable) are hipEvent times of the two phases. */
+int rai_hip_decoder_generate(rai_hip_decoder *dec, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                             int32_t n_new, uint32_t *tokens_host, float *prefill_ms, float *decode_ms);
+/* Model::clear_kv_cache (phi2.rs:349-353). */
+int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *dec);
+/* Current cached context length. */
+int rai_hip_decoder_context_len(rai_hip_decoder *dec, int32_t *len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAI_HIP_H */

@@ -1,0 +1,30 @@
+// Internal launcher of the attention kernels (shared by the C ABI and the
+// decoder drivers).
+#pragma once
+#include "common.h"
+
+namespace rai {
+
+// q[B, Hq, S, D], k/v[B, Hkv, T, D] with unit stride on D; out[B, S, Hq*D].
+// Query row s of a length-S block sits at absolute position T - S + s, so with
+// causal != 0 it sees keys 0 .. T - S + s.
+struct AttnArgs {
+  const void *q, *k, *v;
+  void *out;
+  int64_t qs[3], ks[3], vs[3];  // element strides of dims B, H, S/T
+  int64_t out_row_stride;       // elements between consecutive (b, s) rows of out
+  int B, Hq, Hkv, S, T, D;
+  float scale;
+  int causal;
+  int f32_scores;  // 1: phi2.rs:244-260 numerics; 0: qwen2.rs:205-216 / gemma.rs:238-254
+  int dtype;       // RAI_BF16 / RAI_F16 / RAI_F32
+  // When t_dev is non-null the key count is read on the device (*t_dev + t_add)
+  // instead of T, so one captured launch serves every decode step; T is then
+  // the capacity bound.
+  const int *t_dev;
+  int t_add;
+};
+
+int launch_attention(hipStream_t st, const AttnArgs &a);
+
+}  // namespace rai

@@ -1,0 +1,206 @@
+// Scaled-dot-product attention.
+//   k_attn_row: one 256-thread block per (query row, head, batch).  K and V of the
+//   head are streamed once per block with 16-byte loads; scores live in LDS as
+//   f32.  This is the decode kernel (S == 1: HBM-bound on the KV cache) and the
+//   dtype-generic fallback for short prefills.
+//
+// Reference semantics: rai-models/src/llm/phi2.rs:244-262 (f32 scores, -inf mask,
+// f32 softmax, P cast to V's dtype), qwen2.rs:205-221 and gemma.rs:238-254
+// (scores, scale and softmax rounded to the model dtype), repeat_kv
+// gemma.rs:191-201 (query head h reads kv head h / (Hq/Hkv)).
+#include "attention.h"
+
+namespace rai {
+
+template <typename T> struct AttnVec;
+template <> struct AttnVec<float> { static constexpr int V = 4; };
+template <> struct AttnVec<bf16_raw> { static constexpr int V = 8; };
+template <> struct AttnVec<f16_raw> { static constexpr int V = 8; };
+template <typename T, int V> struct alignas(sizeof(T) * V) APack { T v[V]; };
+
+template <typename T> __device__ __forceinline__ float round_to(float x) {
+  T t;
+  Scalar<T>::store(&t, x);
+  return (float)Scalar<T>::load(&t);
+}
+template <> __device__ __forceinline__ float round_to<float>(float x) { return x; }
+
+template <typename T>
+__global__ void __launch_bounds__(256) k_attn_row(AttnArgs a) {
+  constexpr int V = AttnVec<T>::V;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  // layout: q[D] | red[groups*D] | scores[T]
+  const int D = a.D, ncol = D / V;
+  const int groups = 256 / ncol;
+  float *qf = smem;
+  float *red = qf + D;
+  float *scores = red + groups * D;
+  __shared__ float sh[8];
+
+  const int s = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int hk = h / (a.Hq / a.Hkv);
+  int n_keys = a.T;
+  if (a.t_dev) {
+    n_keys = *a.t_dev + a.t_add;
+    if (n_keys > a.T) n_keys = a.T;
+  }
+  int t_end = a.causal ? (n_keys - a.S + s + 1) : n_keys;
+  if (t_end > n_keys) t_end = n_keys;
+  if (t_end < 0) t_end = 0;
+
+  const T *q = (const T *)a.q + b * a.qs[0] + h * a.qs[1] + s * a.qs[2];
+  const T *K = (const T *)a.k + b * a.ks[0] + hk * a.ks[1];
+  const T *Vp = (const T *)a.v + b * a.vs[0] + hk * a.vs[1];
+  for (int d = tid; d < D; d += 256) qf[d] = (float)Scalar<T>::load(q + d);
+  __syncthreads();
+
+  // ---- scores: 16 lanes cooperate on one key row
+  {
+    const int g = tid >> 4, gl = tid & 15;
+    for (int t = g; t < t_end; t += 16) {
+      const T *kr = K + (int64_t)t * a.ks[2];
+      float acc = 0.f;
+      for (int c = gl; c < ncol; c += 16) {
+        APack<T, V> pk = *reinterpret_cast<const APack<T, V> *>(kr + c * V);
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&pk.v[j]), acc);
+      }
+      acc += __shfl_xor(acc, 8, 64);
+      acc += __shfl_xor(acc, 4, 64);
+      acc += __shfl_xor(acc, 2, 64);
+      acc += __shfl_xor(acc, 1, 64);
+      if (gl == 0) {
+        float sc;
+        if (a.f32_scores) sc = acc * a.scale;
+        else sc = round_to<T>(round_to<T>(acc) * round_to<T>(a.scale));
+        scores[t] = sc;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- softmax over scores[0..t_end)
+  float m = -INFINITY;
+  for (int t = tid; t < t_end; t += 256) m = fmaxf(m, scores[t]);
+  m = wave_max(m);
+  if (lane == 0) sh[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  float sum = 0.f;
+  for (int t = tid; t < t_end; t += 256) {
+    float e = expf(scores[t] - m);
+    if (!a.f32_scores) e = round_to<T>(e);
+    scores[t] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) sh[4 + wave] = sum;
+  __syncthreads();
+  sum = sh[4] + sh[5] + sh[6] + sh[7];
+  if (!a.f32_scores) sum = round_to<T>(sum);
+  const float inv = 1.0f / sum;
+
+  // ---- P.V: thread (grp, col) accumulates keys grp, grp+groups, ... for V
+  //      consecutive output features
+  {
+    const int col = tid % ncol, grp = tid / ncol;
+    float acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = 0.f;
+    if (grp < groups) {
+      for (int t = grp; t < t_end; t += groups) {
+        // the reference rounds the normalised probabilities to V's dtype
+        const float p = a.f32_scores ? round_to<T>(scores[t] * inv) : round_to<T>(scores[t] / sum);
+        APack<T, V> pk = *reinterpret_cast<const APack<T, V> *>(Vp + (int64_t)t * a.vs[2] + col * V);
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&pk.v[j]), acc[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) red[grp * D + col * V + j] = acc[j];
+    }
+  }
+  __syncthreads();
+  T *o = (T *)a.out + ((int64_t)b * a.S + s) * a.out_row_stride + (int64_t)h * D;
+  for (int d = tid; d < D; d += 256) {
+    float r = 0.f;
+    for (int g = 0; g < groups; ++g) r += red[g * D + d];
+    Scalar<T>::store(o + d, (typename Scalar<T>::compute)r);
+  }
+}
+
+template <typename T> static int launch_row(hipStream_t st, const AttnArgs &a) {
+  constexpr int V = AttnVec<T>::V;
+  RAI_REQUIRE(a.D % V == 0 && a.D / V <= 256, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
+  const int ncol = a.D / V, groups = 256 / ncol;
+  const size_t lds = sizeof(float) * ((size_t)a.D + (size_t)groups * a.D + (size_t)a.T);
+  RAI_REQUIRE(lds <= 150 * 1024, RAI_ERR_UNSUPPORTED, "attention: context %d too long for the row kernel", a.T);
+  static size_t attr_bytes = 0;
+  if (lds > 64 * 1024 && lds > attr_bytes) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_row<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    150 * 1024));
+    attr_bytes = 150 * 1024;
+  }
+  RAI_REQUIRE(a.Hq <= 65535 && a.B <= 65535, RAI_ERR_UNSUPPORTED, "attention: grid too large");
+  hipLaunchKernelGGL((k_attn_row<T>), dim3(a.S, a.Hq, a.B), dim3(256), lds, st, a);
+  return launch_check("attention_row");
+}
+
+int launch_attention(hipStream_t st, const AttnArgs &a) {
+  RAI_REQUIRE(a.B > 0 && a.Hq > 0 && a.Hkv > 0 && a.S > 0 && a.T > 0 && a.D > 0, RAI_ERR_BAD_SHAPE,
+              "attention: empty problem");
+  RAI_REQUIRE(a.Hq % a.Hkv == 0, RAI_ERR_BAD_SHAPE, "attention: %d query heads not divisible by %d kv heads", a.Hq,
+              a.Hkv);
+  switch (a.dtype) {
+    case RAI_F32: return launch_row<float>(st, a);
+    case RAI_BF16: return launch_row<bf16_raw>(st, a);
+    case RAI_F16: return launch_row<f16_raw>(st, a);
+    default: return fail(RAI_ERR_BAD_DTYPE, "attention: dtype %s unsupported", dtype_name(a.dtype));
+  }
+}
+
+}  // namespace rai
+
+using namespace rai;
+
+extern "C" int rai_hip_attention(int dev, const rai_hip_tensor *q, const rai_hip_tensor *k, const rai_hip_tensor *v,
+                                 double scale, int32_t causal, int32_t f32_scores, const rai_hip_tensor *out) {
+  RAI_TRY(validate(q, "q"));
+  RAI_TRY(validate(k, "k"));
+  RAI_TRY(validate(v, "v"));
+  RAI_TRY(validate(out, "out"));
+  RAI_REQUIRE(q->rank == 4 && k->rank == 4 && v->rank == 4 && out->rank == 3, RAI_ERR_BAD_SHAPE,
+              "attention: q/k/v must be rank 4 and out rank 3");
+  RAI_REQUIRE(q->dtype == k->dtype && q->dtype == v->dtype && q->dtype == out->dtype, RAI_ERR_BAD_DTYPE,
+              "attention: dtype mismatch");
+  const int64_t B = q->shape[0], Hq = q->shape[1], S = q->shape[2], D = q->shape[3];
+  const int64_t Hkv = k->shape[1], T = k->shape[2];
+  RAI_REQUIRE(k->shape[0] == B && v->shape[0] == B && k->shape[3] == D && v->shape[3] == D && v->shape[1] == Hkv &&
+                  v->shape[2] == T,
+              RAI_ERR_BAD_SHAPE, "attention: k/v shapes do not match q");
+  RAI_REQUIRE(out->shape[0] == B && out->shape[1] == S && out->shape[2] == Hq * D && is_contiguous(out),
+              RAI_ERR_BAD_SHAPE, "attention: out must be contiguous [B, S, Hq*D]");
+  RAI_REQUIRE((q->stride[3] == 1 && k->stride[3] == 1 && v->stride[3] == 1) || D == 1, RAI_ERR_BAD_STRIDE,
+              "attention: head_dim must have unit stride");
+  RAI_REQUIRE(!causal || S <= T, RAI_ERR_BAD_SHAPE, "attention: causal needs S <= T");
+  hipStream_t st = stream_of(dev);
+  if (!st) return RAI_ERR_HIP;
+  if (numel(out) == 0) return RAI_OK;
+  const size_t es = dtype_size(q->dtype);
+  const int vec = (int)(16 / es);
+  auto ok = [&](const rai_hip_tensor *t) {
+    if ((uintptr_t)base_ptr(t) % 16) return false;
+    for (int i = 0; i < 3; ++i)
+      if (t->shape[i] > 1 && t->stride[i] % vec) return false;
+    return true;
+  };
+  RAI_REQUIRE(ok(k) && ok(v) && D % vec == 0, RAI_ERR_BAD_STRIDE, "attention: k/v rows must be 16-byte aligned");
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.q = base_ptr(q); a.k = base_ptr(k); a.v = base_ptr(v); a.out = base_ptr(out);
+  for (int i = 0; i < 3; ++i) { a.qs[i] = q->stride[i]; a.ks[i] = k->stride[i]; a.vs[i] = v->stride[i]; }
+  a.out_row_stride = Hq * D;
+  a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.S = (int)S; a.T = (int)T; a.D = (int)D;
+  a.scale = (float)scale; a.causal = causal; a.f32_scores = f32_scores; a.dtype = q->dtype;
+  return launch_attention(st, a);
+}

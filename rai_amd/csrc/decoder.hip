@@ -1,0 +1,666 @@
+// Decoder-only model drivers: the fused, allocation-free evaluation of
+// rai-models/src/llm/phi2.rs (Model::fwd :334-347, DecoderLayer::fwd :293-299,
+// Attention::fwd :202-264, MLP::fwd :99-101) and the greedy loop of
+// examples/phi2/src/main.rs:75-95.
+//
+// Layout in HBM (per layer, built once at load time so decode streams each
+// weight byte exactly once with unit stride):
+//   Wa [QD + 2*KD + I, H]  rows = q_proj | k_proj | v_proj | fc1   (all read the same LayerNorm output)
+//   Wb [H, QD + I]         row n = dense[n, :] | fc2[n, :]         (attn output and MLP activation are
+//                                                                   adjacent columns of one buffer)
+//   KV cache K, V [L][B][Hkv][Tmax][D], preallocated; appending a token writes one row.
+// Per layer a prefill runs LayerNorm, one GEMM over Wa (bias + gelu on the fc1
+// columns), rotary + cache append, attention, one GEMM over Wb (both biases +
+// residual).  A decode step fuses the LayerNorm into the weight-streaming
+// kernel: 3 launches per layer.  Context length and the current tokens live in
+// device memory, so consecutive greedy steps need no host round trip.
+#include <map>
+#include <string>
+#include <vector>
+
+#include "attention.h"
+#include "gemm.h"
+
+namespace rai {
+
+struct ParamSlot {
+  std::string name;
+  int64_t rows, cols;       // logical [rows, cols] (1-D params: rows = 1)
+  char *dst;                // device address of element [0, 0]
+  int64_t pitch;            // elements between consecutive rows at dst
+  bool loaded;
+};
+
+struct Layer {
+  char *Wa, *ba, *Wb, *bd, *bf, *ln_w, *ln_b;
+};
+
+struct DevState {
+  int pos;   // tokens already in the KV cache
+  int step;  // greedy steps taken by the current generate call
+};
+
+}  // namespace rai
+
+using namespace rai;
+
+struct rai_hip_decoder {
+  int dev;
+  rai_hip_decoder_config cfg;
+  size_t es;
+  int H, I, QD, KD, D, Hq, Hkv, V, L, NA, KB;
+  std::vector<ParamSlot> slots;
+  std::map<std::string, int> slot_by_name;
+  std::vector<Layer> layers;
+  char *embed, *lnf_w, *lnf_b, *head_w, *head_b;
+  char *cos_t, *sin_t;  // [max_pos, rot] in the model dtype
+  char *kcache, *vcache;
+  // activations (sized for max_batch * max_context rows)
+  char *x, *x2, *ln, *qkv, *cat, *last, *logits;
+  uint32_t *ids, *tokens, *history;
+  DevState *state;
+  std::vector<void *> allocs;
+  int ctx_len;
+  int64_t max_rows;
+  int history_cap;
+};
+
+namespace rai {
+
+// ------------------------------------------------------------------ small kernels
+template <typename T>
+__global__ void __launch_bounds__(256)
+k_embed(T *out, const T *table, const uint32_t *ids, int64_t rows, int H, int vocab, unsigned long long *errors) {
+  for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < rows * H; e += (int64_t)gridDim.x * blockDim.x) {
+    int64_t r = e / H;
+    int c = (int)(e - r * H);
+    uint32_t id = ids[r];
+    if (id >= (uint32_t)vocab) {
+      if (c == 0) atomicAdd(errors, 1ull);
+      memset(&out[e], 0, sizeof(T));
+    } else {
+      out[e] = table[(int64_t)id * H + c];
+    }
+  }
+}
+
+// Rotary embedding (NeoX rotate-half over the first `rot` features) applied in
+// place to q, and to k while it is appended to the cache together with v.
+// qkv rows are [q (QD) | k (KD) | v (KD)] per token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+k_rope_append(T *qkv, T *kcache, T *vcache, const T *cos_t, const T *sin_t, const DevState *state, int B, int S, int Hq,
+              int Hkv, int D, int rot, int Tmax) {
+  const int pos0 = state->pos;
+  const int QD = Hq * D, KD = Hkv * D, ld = QD + 2 * KD;
+  const int half = rot / 2;
+  const int heads = Hq + 2 * Hkv;
+  const int64_t total = (int64_t)B * S * heads * D;
+  for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
+    int d = (int)(e % D);
+    int64_t r = e / D;
+    int hh = (int)(r % heads);
+    r /= heads;
+    int s = (int)(r % S);
+    int b = (int)(r / S);
+    T *row = qkv + ((int64_t)b * S + s) * ld;
+    const int pos = pos0 + s;
+    if (hh < Hq + Hkv) {  // q or k head: rotate
+      T *hp = row + (hh < Hq ? hh * D : QD + (hh - Hq) * D);
+      float v = (float)Scalar<T>::load(hp + d);
+      // pair (d, d+half): the lane with d < half computes both to keep the update in place
+      if (d < half) {
+        float v2 = (float)Scalar<T>::load(hp + d + half);
+        float c1 = (float)Scalar<T>::load(cos_t + (int64_t)pos * rot + d);
+        float s1 = (float)Scalar<T>::load(sin_t + (int64_t)pos * rot + d);
+        float c2 = (float)Scalar<T>::load(cos_t + (int64_t)pos * rot + d + half);
+        float s2 = (float)Scalar<T>::load(sin_t + (int64_t)pos * rot + d + half);
+        // reference rounds x*cos, rot*sin and their sum separately (phi2.rs:75)
+        T a, bb, o1, o2;
+        Scalar<T>::store(&a, v * c1);
+        Scalar<T>::store(&bb, -v2 * s1);
+        Scalar<T>::store(&o1, (float)Scalar<T>::load(&a) + (float)Scalar<T>::load(&bb));
+        Scalar<T>::store(&a, v2 * c2);
+        Scalar<T>::store(&bb, v * s2);
+        Scalar<T>::store(&o2, (float)Scalar<T>::load(&a) + (float)Scalar<T>::load(&bb));
+        if (hh < Hq) {
+          hp[d] = o1;
+          hp[d + half] = o2;
+        } else {
+          T *kc = kcache + (((int64_t)b * Hkv + (hh - Hq)) * Tmax + pos) * D;
+          kc[d] = o1;
+          kc[d + half] = o2;
+        }
+      } else if (d >= rot && hh >= Hq) {
+        kcache[(((int64_t)b * Hkv + (hh - Hq)) * Tmax + pos) * D + d] = hp[d];
+      }
+    } else {
+      int hv = hh - Hq - Hkv;
+      vcache[(((int64_t)b * Hkv + hv) * Tmax + pos) * D + d] = row[QD + KD + hv * D + d];
+    }
+  }
+}
+
+__global__ void k_set_state(DevState *st, int pos, int step) {
+  st->pos = pos;
+  st->step = step;
+}
+__global__ void k_advance(DevState *st, int dpos, int dstep) {
+  st->pos += dpos;
+  st->step += dstep;
+}
+
+// argmax over bf16/f32 logits rows; first maximum wins, NaN never wins except at
+// index 0.  One block per row (vocab-sized rows, a handful of rows).
+template <typename T>
+__global__ void __launch_bounds__(1024)
+k_argmax_rows(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, const DevState *state, int B) {
+  __shared__ float sv[16];
+  __shared__ uint32_t si[16];
+  const int b = blockIdx.x;
+  const T *x = logits + (int64_t)b * n;
+  float bv = -INFINITY;
+  uint32_t bi = 0xffffffffu;
+  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = (float)Scalar<T>::load(x + i);
+    if (v > bv || (bi == 0xffffffffu && v == v)) { bv = v; bi = (uint32_t)i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(bv, o, 64);
+    uint32_t oi = (uint32_t)__shfl_xor((int)bi, o, 64);
+    if (oi != 0xffffffffu && (bi == 0xffffffffu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+  }
+  if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
+      float ov = sv[w];
+      uint32_t oi = si[w];
+      if (oi != 0xffffffffu && (bi == 0xffffffffu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+    }
+    float first = (float)Scalar<T>::load(x);
+    if (bi == 0xffffffffu || first != first) bi = 0;
+    tokens[b] = bi;
+    if (history) history[(int64_t)state->step * B + b] = bi;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) k_to_f32(float *out, const T *in, int64_t n) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = (float)Scalar<T>::load(in + i);
+}
+
+static int grid1d(int64_t n) {
+  int64_t b = (n + 255) / 256;
+  return (int)(b < kNumCU * 16 ? (b < 1 ? 1 : b) : kNumCU * 16);
+}
+
+// ------------------------------------------------------------------ host-side construction
+static int dalloc(rai_hip_decoder *d, size_t bytes, char **out) {
+  void *p = nullptr;
+  RAI_HIP_TRY(hipSetDevice(d->dev));
+  hipError_t e = hipMalloc(&p, bytes ? bytes : 16);
+  if (e != hipSuccess) return fail(RAI_ERR_OOM, "decoder: hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  d->allocs.push_back(p);
+  *out = (char *)p;
+  return RAI_OK;
+}
+
+static void add_slot(rai_hip_decoder *d, const std::string &name, int64_t rows, int64_t cols, char *dst, int64_t pitch) {
+  d->slot_by_name[name] = (int)d->slots.size();
+  d->slots.push_back(ParamSlot{name, rows, cols, dst, pitch, false});
+}
+
+// Rotary tables.  Reference chain (phi2.rs:44-64): inv_freq computed with f32
+// powf, cast to the model dtype; positions cast to the model dtype; their
+// product (a K=1 matmul) rounded to the model dtype; sin/cos rounded again.
+static float round_dt(float v, int dtype) {
+  if (dtype != RAI_BF16) return v;
+  uint32_t u;
+  memcpy(&u, &v, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return v;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  u &= 0xffff0000u;
+  memcpy(&v, &u, 4);
+  return v;
+}
+
+static int build_rope_tables(rai_hip_decoder *d) {
+  const auto &c = d->cfg;
+  const int rot = c.rotary_dim, half = rot / 2, P = c.max_position_embeddings;
+  std::vector<float> cs((size_t)P * rot), sn((size_t)P * rot);
+  for (int i = 0; i < half; ++i) {
+    float inv;
+    if (c.arch == RAI_ARCH_PHI2) inv = 1.0f / powf((float)c.rope_theta, (float)(2 * i) / (float)rot);
+    else inv = 1.0f / (float)pow(c.rope_theta, (double)(2 * i) / (double)rot);
+    for (int p = 0; p < P; ++p) {
+      float ang;
+      if (c.rope_tables_f32) ang = (float)p * inv;
+      else ang = round_dt(round_dt((float)p, c.dtype) * round_dt(inv, c.dtype), c.dtype);
+      float cv = round_dt(cosf(ang), c.dtype), sv = round_dt(sinf(ang), c.dtype);
+      cs[(size_t)p * rot + i] = cs[(size_t)p * rot + i + half] = cv;
+      sn[(size_t)p * rot + i] = sn[(size_t)p * rot + i + half] = sv;
+    }
+  }
+  const size_t n = (size_t)P * rot;
+  if (c.dtype == RAI_F32) {
+    RAI_HIP_TRY(hipMemcpy(d->cos_t, cs.data(), n * 4, hipMemcpyHostToDevice));
+    RAI_HIP_TRY(hipMemcpy(d->sin_t, sn.data(), n * 4, hipMemcpyHostToDevice));
+  } else {
+    std::vector<uint16_t> cb(n), sb(n);
+    for (size_t i = 0; i < n; ++i) {
+      uint32_t u;
+      memcpy(&u, &cs[i], 4);
+      cb[i] = (uint16_t)(u >> 16);
+      memcpy(&u, &sn[i], 4);
+      sb[i] = (uint16_t)(u >> 16);
+    }
+    RAI_HIP_TRY(hipMemcpy(d->cos_t, cb.data(), n * 2, hipMemcpyHostToDevice));
+    RAI_HIP_TRY(hipMemcpy(d->sin_t, sb.data(), n * 2, hipMemcpyHostToDevice));
+  }
+  return RAI_OK;
+}
+
+static int create_phi2(rai_hip_decoder *d) {
+  const size_t es = d->es;
+  const int H = d->H, I = d->I, QD = d->QD, KD = d->KD, V = d->V;
+  RAI_TRY(dalloc(d, (size_t)V * H * es, &d->embed));
+  add_slot(d, "model.embed_tokens.weight", V, H, d->embed, H);
+  d->layers.resize(d->L);
+  for (int l = 0; l < d->L; ++l) {
+    Layer &ly = d->layers[l];
+    RAI_TRY(dalloc(d, (size_t)d->NA * H * es, &ly.Wa));
+    RAI_TRY(dalloc(d, (size_t)d->NA * es, &ly.ba));
+    RAI_TRY(dalloc(d, (size_t)H * d->KB * es, &ly.Wb));
+    RAI_TRY(dalloc(d, (size_t)H * es, &ly.bd));
+    RAI_TRY(dalloc(d, (size_t)H * es, &ly.bf));
+    RAI_TRY(dalloc(d, (size_t)H * es, &ly.ln_w));
+    RAI_TRY(dalloc(d, (size_t)H * es, &ly.ln_b));
+    const std::string p = "model.layers." + std::to_string(l) + ".";
+    add_slot(d, p + "self_attn.q_proj.weight", QD, H, ly.Wa, H);
+    add_slot(d, p + "self_attn.q_proj.bias", 1, QD, ly.ba, QD);
+    add_slot(d, p + "self_attn.k_proj.weight", KD, H, ly.Wa + (size_t)QD * H * es, H);
+    add_slot(d, p + "self_attn.k_proj.bias", 1, KD, ly.ba + (size_t)QD * es, KD);
+    add_slot(d, p + "self_attn.v_proj.weight", KD, H, ly.Wa + (size_t)(QD + KD) * H * es, H);
+    add_slot(d, p + "self_attn.v_proj.bias", 1, KD, ly.ba + (size_t)(QD + KD) * es, KD);
+    add_slot(d, p + "self_attn.dense.weight", H, QD, ly.Wb, d->KB);
+    add_slot(d, p + "self_attn.dense.bias", 1, H, ly.bd, H);
+    add_slot(d, p + "mlp.fc1.weight", I, H, ly.Wa + (size_t)(QD + 2 * KD) * H * es, H);
+    add_slot(d, p + "mlp.fc1.bias", 1, I, ly.ba + (size_t)(QD + 2 * KD) * es, I);
+    add_slot(d, p + "mlp.fc2.weight", H, I, ly.Wb + (size_t)QD * es, d->KB);
+    add_slot(d, p + "mlp.fc2.bias", 1, H, ly.bf, H);
+    add_slot(d, p + "input_layernorm.weight", 1, H, ly.ln_w, H);
+    add_slot(d, p + "input_layernorm.bias", 1, H, ly.ln_b, H);
+  }
+  RAI_TRY(dalloc(d, (size_t)H * es, &d->lnf_w));
+  RAI_TRY(dalloc(d, (size_t)H * es, &d->lnf_b));
+  add_slot(d, "model.final_layernorm.weight", 1, H, d->lnf_w, H);
+  add_slot(d, "model.final_layernorm.bias", 1, H, d->lnf_b, H);
+  if (d->cfg.tie_word_embeddings) {
+    d->head_w = d->embed;
+    d->head_b = nullptr;
+  } else {
+    RAI_TRY(dalloc(d, (size_t)V * H * es, &d->head_w));
+    RAI_TRY(dalloc(d, (size_t)V * es, &d->head_b));
+    add_slot(d, "lm_head.weight", V, H, d->head_w, H);
+    add_slot(d, "lm_head.bias", 1, V, d->head_b, V);
+  }
+  return RAI_OK;
+}
+
+// ------------------------------------------------------------------ forward
+template <typename T> static void launch_embed(rai_hip_decoder *d, hipStream_t st, int64_t rows) {
+  hipLaunchKernelGGL((k_embed<T>), dim3(grid1d(rows * d->H)), dim3(256), 0, st, (T *)d->x, (const T *)d->embed, d->ids,
+                     rows, d->H, d->V, index_error_counter(d->dev));
+}
+template <typename T> static void launch_rope_append(rai_hip_decoder *d, hipStream_t st, int l, int B, int S) {
+  const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
+  int64_t total = (int64_t)B * S * (d->Hq + 2 * d->Hkv) * d->D;
+  hipLaunchKernelGGL((k_rope_append<T>), dim3(grid1d(total)), dim3(256), 0, st, (T *)d->qkv,
+                     (T *)d->kcache + per_layer * l, (T *)d->vcache + per_layer * l, (const T *)d->cos_t,
+                     (const T *)d->sin_t, d->state, B, S, d->Hq, d->Hkv, d->D, d->cfg.rotary_dim, d->cfg.max_context);
+}
+
+static rai_hip_tensor desc2(void *p, int dtype, int64_t rows, int64_t cols, int64_t row_stride) {
+  rai_hip_tensor t;
+  memset(&t, 0, sizeof(t));
+  t.data = p;
+  t.dtype = dtype;
+  t.rank = 2;
+  t.shape[0] = rows;
+  t.shape[1] = cols;
+  t.stride[0] = row_stride;
+  t.stride[1] = 1;
+  return t;
+}
+static rai_hip_tensor desc1(void *p, int dtype, int64_t n) {
+  rai_hip_tensor t;
+  memset(&t, 0, sizeof(t));
+  t.data = p;
+  t.dtype = dtype;
+  t.rank = 1;
+  t.shape[0] = n;
+  t.stride[0] = 1;
+  return t;
+}
+
+static int linear(rai_hip_decoder *d, hipStream_t st, const LinearArgs &a) {
+  return d->cfg.dtype == RAI_BF16 ? launch_linear_bf16(st, a) : launch_linear_f32(st, a);
+}
+
+// ids (B*S u32) are already in d->ids; device state holds the context length.
+static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step) {
+  hipStream_t st = stream_of(d->dev);
+  if (!st) return RAI_ERR_HIP;
+  const int dt = d->cfg.dtype;
+  const int H = d->H, QD = d->QD, KD = d->KD, I = d->I;
+  const int64_t M = (int64_t)B * S;
+  const int ldq = QD + 2 * KD;
+  const bool fuse_ln = dt == RAI_BF16 && M <= 8;
+  const int T_after = d->ctx_len + S;
+
+  if (dt == RAI_BF16) launch_embed<bf16_raw>(d, st, M); else launch_embed<float>(d, st, M);
+  RAI_TRY(launch_check("embed"));
+
+  char *x = d->x, *xn = d->x2;
+  for (int l = 0; l < d->L; ++l) {
+    const Layer &ly = d->layers[l];
+    LinearArgs a = linear_args_default();
+    if (fuse_ln) {
+      a.A = x; a.lda = H;
+      a.ln_kind = 0; a.ln_w = ly.ln_w; a.ln_b = ly.ln_b; a.ln_eps = (float)d->cfg.norm_eps;
+    } else {
+      rai_hip_tensor tx = desc2(x, dt, M, H, H), tw = desc1(ly.ln_w, dt, H), tb = desc1(ly.ln_b, dt, H),
+                     to = desc2(d->ln, dt, M, H, H);
+      RAI_TRY(rai_hip_layer_norm(d->dev, &tx, &tw, &tb, d->cfg.norm_eps, &to));
+      a.A = d->ln; a.lda = H;
+    }
+    a.W = ly.Wa; a.ldw = H; a.bias = ly.ba;
+    a.out1 = d->qkv; a.ld1 = ldq;
+    a.out2 = d->cat + (size_t)QD * d->es; a.ld2 = d->KB;
+    a.M = (int)M; a.N = d->NA; a.K = H; a.n_split = ldq;
+    a.act = d->cfg.hidden_act; a.act_from = ldq;
+    RAI_TRY(linear(d, st, a));
+
+    if (dt == RAI_BF16) launch_rope_append<bf16_raw>(d, st, l, B, S); else launch_rope_append<float>(d, st, l, B, S);
+    RAI_TRY(launch_check("rope_append"));
+
+    AttnArgs t;
+    memset(&t, 0, sizeof(t));
+    const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
+    t.q = d->qkv;
+    t.k = d->kcache + per_layer * l * d->es;
+    t.v = d->vcache + per_layer * l * d->es;
+    t.out = d->cat;
+    t.qs[0] = (int64_t)S * ldq; t.qs[1] = d->D; t.qs[2] = ldq;
+    t.ks[0] = t.vs[0] = (int64_t)d->Hkv * d->cfg.max_context * d->D;
+    t.ks[1] = t.vs[1] = (int64_t)d->cfg.max_context * d->D;
+    t.ks[2] = t.vs[2] = d->D;
+    t.out_row_stride = d->KB;
+    t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.S = S; t.D = d->D;
+    t.scale = (float)(1.0 / sqrt((double)d->D));
+    t.causal = 1; t.f32_scores = 1; t.dtype = dt;
+    if (S == 1) {  // decode: key count comes from device state, capacity bounds LDS
+      t.T = d->cfg.max_context;
+      t.t_dev = &d->state->pos;
+      t.t_add = 1;
+    } else {
+      t.T = T_after;
+    }
+    RAI_TRY(launch_attention(st, t));
+
+    LinearArgs b = linear_args_default();
+    b.A = d->cat; b.lda = d->KB;
+    b.W = ly.Wb; b.ldw = d->KB;
+    b.bias = ly.bd; b.bias2 = ly.bf;
+    b.residual = x; b.ldr = H;
+    b.out1 = xn; b.ld1 = H;
+    b.M = (int)M; b.N = H; b.K = d->KB; b.n_split = H;
+    RAI_TRY(linear(d, st, b));
+    char *tmp = x; x = xn; xn = tmp;
+  }
+
+  // final LayerNorm on the last position of every sequence, then the head
+  // (phi2.rs:345-346: narrow(1, S-1, 1) before lm_head).
+  LinearArgs h = linear_args_default();
+  char *last_rows = x + (size_t)(S - 1) * H * d->es;  // row b*S + S-1, stride S*H
+  if (dt == RAI_BF16 && B <= 8) {
+    h.A = last_rows; h.lda = (int64_t)S * H;
+    h.ln_kind = 0; h.ln_w = d->lnf_w; h.ln_b = d->lnf_b; h.ln_eps = (float)d->cfg.norm_eps;
+  } else {
+    rai_hip_tensor tx = desc2(last_rows, dt, B, H, (int64_t)S * H), tw = desc1(d->lnf_w, dt, H),
+                   tb = desc1(d->lnf_b, dt, H), to = desc2(d->last, dt, B, H, H);
+    RAI_TRY(rai_hip_layer_norm(d->dev, &tx, &tw, &tb, d->cfg.norm_eps, &to));
+    h.A = d->last; h.lda = H;
+  }
+  h.W = d->head_w; h.ldw = H; h.bias = d->head_b;
+  h.out1 = d->logits; h.ld1 = d->V;
+  h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
+  RAI_TRY(linear(d, st, h));
+
+  uint32_t *hist = advance_step ? d->history : nullptr;
+  if (dt == RAI_BF16)
+    hipLaunchKernelGGL((k_argmax_rows<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits, (int64_t)d->V,
+                       d->tokens, hist, d->state, B);
+  else
+    hipLaunchKernelGGL((k_argmax_rows<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
+                       d->tokens, hist, d->state, B);
+  RAI_TRY(launch_check("argmax_rows"));
+  hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, st, d->state, S, advance_step ? 1 : 0);
+  RAI_TRY(launch_check("advance"));
+  d->ctx_len = T_after;
+  return RAI_OK;
+}
+
+static int check_call(rai_hip_decoder *d, int B, int S) {
+  RAI_REQUIRE(d, RAI_ERR_BAD_ARG, "decoder is null");
+  RAI_REQUIRE(B >= 1 && B <= d->cfg.max_batch, RAI_ERR_BAD_SHAPE, "decoder: batch %d outside 1..%d", B, d->cfg.max_batch);
+  RAI_REQUIRE(S >= 1, RAI_ERR_BAD_SHAPE, "decoder: empty sequence");
+  RAI_REQUIRE(d->ctx_len + S <= d->cfg.max_context, RAI_ERR_BAD_SHAPE, "decoder: context %d + %d exceeds max_context %d",
+              d->ctx_len, S, d->cfg.max_context);
+  RAI_REQUIRE(d->ctx_len + S <= d->cfg.max_position_embeddings, RAI_ERR_BAD_SHAPE,
+              "decoder: position exceeds max_position_embeddings");
+  for (const ParamSlot &s : d->slots)
+    RAI_REQUIRE(s.loaded, RAI_ERR_BAD_ARG, "decoder: parameter %s was never loaded", s.name.c_str());
+  return RAI_OK;
+}
+
+}  // namespace rai
+
+extern "C" {
+
+int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_decoder **out) {
+  RAI_REQUIRE(cfg && out, RAI_ERR_BAD_ARG, "decoder_create: null argument");
+  RAI_REQUIRE(cfg->arch == RAI_ARCH_PHI2, RAI_ERR_UNSUPPORTED, "decoder_create: architecture %d not available", cfg->arch);
+  RAI_REQUIRE(cfg->dtype == RAI_BF16 || cfg->dtype == RAI_F32, RAI_ERR_BAD_DTYPE, "decoder_create: bf16 or f32");
+  RAI_REQUIRE(cfg->hidden_size > 0 && cfg->num_attention_heads > 0 && cfg->num_key_value_heads > 0 &&
+                  cfg->num_attention_heads % cfg->num_key_value_heads == 0 && cfg->head_dim > 0 &&
+                  cfg->vocab_size > 0 && cfg->intermediate_size > 0 && cfg->num_hidden_layers > 0 &&
+                  cfg->max_batch > 0 && cfg->max_context > 0 && cfg->max_position_embeddings > 0,
+              RAI_ERR_BAD_ARG, "decoder_create: bad config");
+  RAI_REQUIRE(cfg->rotary_dim > 0 && cfg->rotary_dim % 2 == 0 && cfg->rotary_dim <= cfg->head_dim, RAI_ERR_BAD_ARG,
+              "decoder_create: rotary_dim %d", cfg->rotary_dim);
+  RAI_REQUIRE(cfg->hidden_act == RAI_UN_NEW_GELU || cfg->hidden_act == RAI_UN_GELU || cfg->hidden_act == RAI_UN_SILU ||
+                  cfg->hidden_act == RAI_UN_RELU,
+              RAI_ERR_BAD_ARG, "decoder_create: hidden_act %d", cfg->hidden_act);
+  if (!ctx(dev)) return RAI_ERR_HIP;
+  rai_hip_decoder *d = new rai_hip_decoder();
+  d->dev = dev;
+  d->cfg = *cfg;
+  d->es = dtype_size(cfg->dtype);
+  d->H = cfg->hidden_size; d->I = cfg->intermediate_size; d->D = cfg->head_dim;
+  d->Hq = cfg->num_attention_heads; d->Hkv = cfg->num_key_value_heads;
+  d->QD = d->Hq * d->D; d->KD = d->Hkv * d->D; d->V = cfg->vocab_size; d->L = cfg->num_hidden_layers;
+  d->NA = d->QD + 2 * d->KD + d->I;
+  d->KB = d->QD + d->I;
+  d->ctx_len = 0;
+  const int vec = (int)(16 / d->es);
+  int st = RAI_OK;
+  auto bail = [&](int code) {
+    rai_hip_decoder_destroy(d);
+    return code;
+  };
+  if (d->H % vec || d->QD % vec || d->KD % vec || d->I % vec || d->D % vec)
+    return bail(fail(RAI_ERR_BAD_SHAPE, "decoder_create: sizes must be multiples of %d elements", vec));
+  if ((st = create_phi2(d)) != RAI_OK) return bail(st);
+  const size_t es = d->es;
+  d->max_rows = (int64_t)cfg->max_batch * cfg->max_context;
+  const size_t kv = (size_t)d->L * cfg->max_batch * d->Hkv * cfg->max_context * d->D * es;
+  const size_t rope = (size_t)cfg->max_position_embeddings * cfg->rotary_dim * es;
+  d->history_cap = cfg->max_context;
+  char *tmp = nullptr;
+  if ((st = dalloc(d, kv, &d->kcache)) || (st = dalloc(d, kv, &d->vcache)) || (st = dalloc(d, rope, &d->cos_t)) ||
+      (st = dalloc(d, rope, &d->sin_t)) || (st = dalloc(d, d->max_rows * d->H * es, &d->x)) ||
+      (st = dalloc(d, d->max_rows * d->H * es, &d->x2)) || (st = dalloc(d, d->max_rows * d->H * es, &d->ln)) ||
+      (st = dalloc(d, d->max_rows * (d->QD + 2 * d->KD) * es, &d->qkv)) ||
+      (st = dalloc(d, d->max_rows * d->KB * es, &d->cat)) || (st = dalloc(d, (size_t)cfg->max_batch * d->H * es, &d->last)) ||
+      (st = dalloc(d, (size_t)cfg->max_batch * d->V * es, &d->logits)))
+    return bail(st);
+  if ((st = dalloc(d, d->max_rows * sizeof(uint32_t), &tmp))) return bail(st);
+  d->ids = (uint32_t *)tmp;
+  if ((st = dalloc(d, (size_t)cfg->max_batch * sizeof(uint32_t), &tmp))) return bail(st);
+  d->tokens = (uint32_t *)tmp;
+  if ((st = dalloc(d, (size_t)d->history_cap * cfg->max_batch * sizeof(uint32_t), &tmp))) return bail(st);
+  d->history = (uint32_t *)tmp;
+  if ((st = dalloc(d, sizeof(DevState), &tmp))) return bail(st);
+  d->state = (DevState *)tmp;
+  if (hipMemset(d->state, 0, sizeof(DevState)) != hipSuccess || hipMemset(d->kcache, 0, kv) != hipSuccess ||
+      hipMemset(d->vcache, 0, kv) != hipSuccess)
+    return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
+  if ((st = build_rope_tables(d)) != RAI_OK) return bail(st);
+  *out = d;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_destroy(rai_hip_decoder *d) {
+  if (!d) return RAI_OK;
+  (void)hipSetDevice(d->dev);
+  (void)hipStreamSynchronize(stream_of(d->dev));
+  for (void *p : d->allocs) (void)hipFree(p);
+  delete d;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_param_count(rai_hip_decoder *d, int32_t *count) {
+  RAI_REQUIRE(d && count, RAI_ERR_BAD_ARG, "null argument");
+  *count = (int32_t)d->slots.size();
+  return RAI_OK;
+}
+
+int rai_hip_decoder_param_name(rai_hip_decoder *d, int32_t i, char *buf, size_t buflen, int64_t *numel) {
+  RAI_REQUIRE(d && buf && buflen > 0, RAI_ERR_BAD_ARG, "null argument");
+  RAI_REQUIRE(i >= 0 && i < (int32_t)d->slots.size(), RAI_ERR_BAD_ARG, "parameter index %d out of range", i);
+  snprintf(buf, buflen, "%s", d->slots[i].name.c_str());
+  if (numel) *numel = d->slots[i].rows * d->slots[i].cols;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_load_param(rai_hip_decoder *d, const char *name, const void *host_data, size_t bytes) {
+  RAI_REQUIRE(d && name && host_data, RAI_ERR_BAD_ARG, "null argument");
+  auto it = d->slot_by_name.find(name);
+  RAI_REQUIRE(it != d->slot_by_name.end(), RAI_ERR_BAD_ARG, "decoder: unknown parameter '%s'", name);
+  ParamSlot &s = d->slots[it->second];
+  const size_t want = (size_t)s.rows * s.cols * d->es;
+  RAI_REQUIRE(bytes == want, RAI_ERR_BAD_SHAPE, "decoder: parameter '%s' needs %zu bytes, got %zu", name, want, bytes);
+  RAI_HIP_TRY(hipSetDevice(d->dev));
+  RAI_HIP_TRY(hipStreamSynchronize(stream_of(d->dev)));
+  RAI_HIP_TRY(hipMemcpy2D(s.dst, (size_t)s.pitch * d->es, host_data, (size_t)s.cols * d->es, (size_t)s.cols * d->es,
+                          (size_t)s.rows, hipMemcpyHostToDevice));
+  s.loaded = true;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *d) {
+  RAI_REQUIRE(d, RAI_ERR_BAD_ARG, "decoder is null");
+  hipStream_t st = stream_of(d->dev);
+  hipLaunchKernelGGL(k_set_state, dim3(1), dim3(1), 0, st, d->state, 0, 0);
+  RAI_TRY(launch_check("set_state"));
+  d->ctx_len = 0;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_context_len(rai_hip_decoder *d, int32_t *len) {
+  RAI_REQUIRE(d && len, RAI_ERR_BAD_ARG, "null argument");
+  *len = d->ctx_len;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_forward(rai_hip_decoder *d, const uint32_t *ids_host, int32_t batch, int32_t seq, float *logits_host,
+                            uint32_t *tokens_host) {
+  RAI_REQUIRE(ids_host, RAI_ERR_BAD_ARG, "ids is null");
+  RAI_TRY(check_call(d, batch, seq));
+  hipStream_t st = stream_of(d->dev);
+  RAI_HIP_TRY(hipMemcpyAsync(d->ids, ids_host, (size_t)batch * seq * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+  RAI_TRY(forward_phi2(d, batch, seq, false));
+  if (logits_host) {
+    // widen on device, then one synchronous copy
+    void *ws = nullptr;
+    const int64_t n = (int64_t)batch * d->V;
+    RAI_TRY(workspace(d->dev, (size_t)n * sizeof(float), &ws));
+    if (d->cfg.dtype == RAI_BF16)
+      hipLaunchKernelGGL((k_to_f32<bf16_raw>), dim3(grid1d(n)), dim3(256), 0, st, (float *)ws, (const bf16_raw *)d->logits, n);
+    else
+      hipLaunchKernelGGL((k_to_f32<float>), dim3(grid1d(n)), dim3(256), 0, st, (float *)ws, (const float *)d->logits, n);
+    RAI_TRY(launch_check("to_f32"));
+    RAI_TRY(rai_hip_d2h(d->dev, logits_host, ws, (size_t)n * sizeof(float)));
+  }
+  if (tokens_host) RAI_TRY(rai_hip_d2h(d->dev, tokens_host, d->tokens, (size_t)batch * sizeof(uint32_t)));
+  if (logits_host || tokens_host) {
+    uint64_t bad = 0;
+    RAI_TRY(rai_hip_index_errors(d->dev, &bad));
+    RAI_REQUIRE(bad == 0, RAI_ERR_INDEX, "decoder: %llu token ids outside the vocabulary", (unsigned long long)bad);
+  }
+  return RAI_OK;
+}
+
+int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                             int32_t n_new, uint32_t *tokens_host, float *prefill_ms, float *decode_ms) {
+  RAI_REQUIRE(prompt_host && tokens_host, RAI_ERR_BAD_ARG, "null argument");
+  RAI_REQUIRE(n_new >= 1, RAI_ERR_BAD_ARG, "generate: n_new must be >= 1");
+  RAI_TRY(rai_hip_decoder_clear_kv_cache(d));
+  RAI_TRY(check_call(d, batch, prompt_len));
+  RAI_REQUIRE(prompt_len + n_new - 1 <= d->cfg.max_context && n_new <= d->history_cap, RAI_ERR_BAD_SHAPE,
+              "generate: %d + %d tokens exceed max_context %d", prompt_len, n_new, d->cfg.max_context);
+  hipStream_t st = stream_of(d->dev);
+  hipEvent_t e0, e1, e2;
+  RAI_HIP_TRY(hipEventCreate(&e0));
+  RAI_HIP_TRY(hipEventCreate(&e1));
+  RAI_HIP_TRY(hipEventCreate(&e2));
+  RAI_HIP_TRY(hipMemcpyAsync(d->ids, prompt_host, (size_t)batch * prompt_len * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+  RAI_HIP_TRY(hipStreamSynchronize(st));
+  RAI_HIP_TRY(hipEventRecord(e0, st));
+  int rc = forward_phi2(d, batch, prompt_len, true);
+  if (rc == RAI_OK) rc = hipEventRecord(e1, st) == hipSuccess ? RAI_OK : fail(RAI_ERR_HIP, "event record");
+  for (int step = 1; rc == RAI_OK && step < n_new; ++step) {
+    // next input = the tokens the previous step left on the device
+    if (hipMemcpyAsync(d->ids, d->tokens, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToDevice, st) != hipSuccess)
+      rc = fail(RAI_ERR_HIP, "generate: token feedback copy failed");
+    else
+      rc = forward_phi2(d, batch, 1, true);
+  }
+  if (rc == RAI_OK && hipEventRecord(e2, st) != hipSuccess) rc = fail(RAI_ERR_HIP, "event record");
+  if (rc == RAI_OK && hipStreamSynchronize(st) != hipSuccess) rc = fail(RAI_ERR_HIP, "generate: stream sync failed");
+  if (rc == RAI_OK) {
+    float ms = 0.f;
+    if (prefill_ms) { (void)hipEventElapsedTime(&ms, e0, e1); *prefill_ms = ms; }
+    if (decode_ms) { (void)hipEventElapsedTime(&ms, e1, e2); *decode_ms = ms; }
+    // history is [step][batch]; hand back [batch][step]
+    std::vector<uint32_t> h((size_t)n_new * batch);
+    rc = rai_hip_d2h(d->dev, h.data(), d->history, h.size() * sizeof(uint32_t));
+    for (int s = 0; rc == RAI_OK && s < n_new; ++s)
+      for (int b = 0; b < batch; ++b) tokens_host[(size_t)b * n_new + s] = h[(size_t)s * batch + b];
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  (void)hipEventDestroy(e2);
+  if (rc == RAI_OK) {
+    uint64_t bad = 0;
+    RAI_TRY(rai_hip_index_errors(d->dev, &bad));
+    RAI_REQUIRE(bad == 0, RAI_ERR_INDEX, "decoder: %llu token ids outside the vocabulary", (unsigned long long)bad);
+  }
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,67 @@
+// Internal launchers of the contraction kernels, shared by the C-ABI matmul /
+// linear entry points and by the decoder drivers.
+#pragma once
+#include "common.h"
+
+namespace rai {
+
+// out[m, n] = epilogue( sum_k A[m, k] * W[n, k] )     (the layout Linear produces,
+// rai-nn/src/linear.rs:59-69: x @ W^T with W stored [out_features, in_features])
+//
+// Epilogue per column n:  v = acc + bias[n] + bias2[n];  v = act(v) for n >= act_from;
+// v += residual[m, n];  round to bf16.  Columns [0, n_split) go to out1, columns
+// [n_split, N) go to out2 at column n - n_split (n_split == N: single output).
+struct LinearArgs {
+  const void *A;       // [M, K], K-contiguous rows
+  int64_t lda;
+  const void *W;       // [N, K]
+  int64_t ldw;
+  const void *bias;    // [N] or null
+  const void *bias2;   // second [N] bias added in f32 (sum of two Linear biases), or null
+  const void *residual;  // [M, N] or null
+  int64_t ldr;
+  void *out1;
+  int64_t ld1;
+  void *out2;
+  int64_t ld2;
+  int M, N, K;
+  int n_split;   // first column written to out2
+  int act;       // rai_hip_unary_op activation or -1
+  int act_from;  // activation applies to columns >= act_from
+  // Optional fused LayerNorm / RMSNorm of the rows of A before the product
+  // (skinny path only): A is normalised with ln_w / ln_b over K.
+  const void *ln_w;
+  const void *ln_b;
+  float ln_eps;
+  int ln_kind;  // -1 none, 0 layernorm, 1 rmsnorm, 2 rmsnorm(1+w)
+};
+inline LinearArgs linear_args_default() {
+  LinearArgs a;
+  memset(&a, 0, sizeof(a));
+  a.act = -1;
+  a.ln_kind = -1;
+  return a;
+}
+
+// bf16 MFMA tile kernel (M >= 1; efficient for M >= 64).
+int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a);
+// bf16 weight-streaming kernel for M <= 8 (decode): HBM-bound.
+int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a);
+// Picks between the two.
+int launch_linear_bf16(hipStream_t st, const LinearArgs &a);
+
+// f32 tile kernel for the same NT contraction, FMA in f32.
+int launch_linear_f32(hipStream_t st, const LinearArgs &a);
+
+__device__ __forceinline__ float act_eval(int act, float x) {
+  switch (act) {
+    case RAI_UN_GELU: return x * 0.5f * (1.0f + erff(x / 1.4142135623730951f));
+    case RAI_UN_NEW_GELU: return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+    case RAI_UN_SILU: return x / (expf(-x) + 1.0f);
+    case RAI_UN_RELU: return x > 0.f ? x : 0.f;
+    case RAI_UN_TANH: return tanhf(x);
+    default: return x;
+  }
+}
+
+}  // namespace rai

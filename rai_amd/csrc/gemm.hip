@@ -1,0 +1,640 @@
+// Dense contractions.
+//   k_linear_bf16_mfma   bf16 x bf16 -> f32 MFMA (v_mfma_f32_32x32x16_bf16), NT layout,
+//                        LDS-staged double-buffered tiles, fused bias/act/residual epilogue.
+//   k_linear_bf16_skinny weight-streaming kernel for M <= 8 rows (decode): each wave
+//                        streams whole weight rows with 16-byte loads; HBM-bound.
+//   k_linear_f32         f32 NT tile kernel (FMA) with the same epilogue.
+//   k_matmul_generic     any strides / batch broadcast, f32 or f64 accumulate.
+//
+// Reference semantics: rai-core/src/backend/candle.rs:327-443 (MatMul, stride rule),
+// rai-core/src/shape.rs:130-160 (batch broadcast), rai-nn/src/linear.rs:59-69.
+#include "gemm.h"
+
+namespace rai {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+struct alignas(16) U128 { uint32_t w[4]; };
+
+// ============================================================ bf16 MFMA tile kernel
+// Block tile BM x BN, K step BK; 4 waves in a 2x2 grid, each wave owns a
+// (BM/2) x (BN/2) sub-tile made of 32x32 MFMA tiles.
+template <int BM, int BN, int BK>
+__global__ void __launch_bounds__(256) k_linear_bf16_mfma(LinearArgs a) {
+  constexpr int PITCH = BK + 8;  // +16 bytes: conflict-free ds_read_b128 across 16 lanes
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int MT = WM / 32, NT = WN / 32;
+  constexpr int CPR = BK / 8;                  // 16-byte chunks per tile row
+  constexpr int A_CHUNKS = BM * CPR / 256;     // per thread
+  constexpr int B_CHUNKS = BN * CPR / 256;
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  uint16_t *As = lds;                          // [2][BM][PITCH]
+  uint16_t *Bs = lds + 2 * BM * PITCH;         // [2][BN][PITCH]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // Tiles that share a weight column block are adjacent in launch order so the
+  // (few) M tiles of one N block hit the same L2.
+  const int tiles_m = (a.M + BM - 1) / BM;
+  const int tile_n = blockIdx.x / tiles_m, tile_m = blockIdx.x % tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const uint16_t *A = (const uint16_t *)a.A;
+  const uint16_t *W = (const uint16_t *)a.W;
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  U128 ra[A_CHUNKS], rb[B_CHUNKS];
+  const int KT = (a.K + BK - 1) / BK;
+
+  auto g_load = [&](int kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      int c = tid + i * 256;
+      int row = c / CPR, kc = (c % CPR) * 8;
+      int m = m0 + row, k = k0 + kc;
+      U128 v = {{0u, 0u, 0u, 0u}};
+      if (m < a.M && k < a.K) v = *reinterpret_cast<const U128 *>(A + (int64_t)m * a.lda + k);
+      ra[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+      int c = tid + i * 256;
+      int row = c / CPR, kc = (c % CPR) * 8;
+      int n = n0 + row, k = k0 + kc;
+      U128 v = {{0u, 0u, 0u, 0u}};
+      if (n < a.N && k < a.K) v = *reinterpret_cast<const U128 *>(W + (int64_t)n * a.ldw + k);
+      rb[i] = v;
+    }
+  };
+  auto s_store = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      int c = tid + i * 256;
+      int row = c / CPR, kc = (c % CPR) * 8;
+      *reinterpret_cast<U128 *>(As + (buf * BM + row) * PITCH + kc) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+      int c = tid + i * 256;
+      int row = c / CPR, kc = (c % CPR) * 8;
+      *reinterpret_cast<U128 *>(Bs + (buf * BN + row) * PITCH + kc) = rb[i];
+    }
+  };
+
+  g_load(0);
+  s_store(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) g_load(kt + 1);
+    const uint16_t *as = As + (buf * BM + wm * WM + (lane & 31)) * PITCH + (lane >> 5) * 8;
+    const uint16_t *bs = Bs + (buf * BN + wn * WN + (lane & 31)) * PITCH + (lane >> 5) * 8;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 fa[MT], fb[NT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + ks * 16);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + ks * 16);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) s_store(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + wn * WN + j * 32 + (lane & 31);
+    if (n >= a.N) continue;
+    const float bv = (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
+    const bool do_act = a.act >= 0 && n >= a.act_from;
+    uint16_t *dst;
+    int64_t ld;
+    int col;
+    if (n < a.n_split) { dst = (uint16_t *)a.out1; ld = a.ld1; col = n; }
+    else { dst = (uint16_t *)a.out2; ld = a.ld2; col = n - a.n_split; }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m >= a.M) continue;
+        float v = acc[i][j][r] + bv;
+        if (do_act) v = act_eval(a.act, v);
+        if (res) v += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
+        dst[(int64_t)m * ld + col] = f32_to_bf16_bits(v);
+      }
+    }
+  }
+}
+
+// ============================================================ bf16 skinny (decode) kernel
+// M <= MROWS rows of A.  Each wave owns R consecutive weight rows at a time and
+// streams them with one 16-byte non-temporal load per lane per 512-element K
+// chunk; the (optionally normalised) activations live in LDS as bf16 and the
+// products are formed with v_dot2_f32_bf16 (two bf16 products per lane-op,
+// accumulated in f32).
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+// acc + dot(a[0..8), b[0..8)) over eight bf16 pairs packed in two 16-byte words.
+// The vector elements are named explicitly: indexing an ext_vector with a loop
+// variable inside __builtin_bit_cast made hipcc read element 0 four times.
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  bf16x2 p, q;
+  __builtin_memcpy(&p, &a, 4);
+  __builtin_memcpy(&q, &b, 4);
+  return __builtin_amdgcn_fdot2_f32_bf16(p, q, c, false);
+}
+__device__ __forceinline__ float dot8_bf16(u32x4 a, u32x4 b, float c) {
+  c = dot2_bf16(a.x, b.x, c);
+  c = dot2_bf16(a.y, b.y, c);
+  c = dot2_bf16(a.z, b.z, c);
+  return dot2_bf16(a.w, b.w, c);
+}
+
+template <int MROWS, int R>
+__global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [MROWS][K]
+  __shared__ float red[8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint16_t *A = (const uint16_t *)a.A;
+  const uint16_t *W = (const uint16_t *)a.W;
+  const int K = a.K;
+
+  // ---- stage activations, optionally normalising each row over K
+  for (int m = 0; m < MROWS; ++m) {
+    if (m >= a.M) break;
+    const uint16_t *xr = A + (int64_t)m * a.lda;
+    uint16_t *xd = xs + m * K;
+    for (int k = tid * 8; k < K; k += 256 * 8)
+      *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(xr + k);
+    if (a.ln_kind >= 0) {
+      __syncthreads();
+      float s = 0.f;
+      for (int k = tid; k < K; k += 256) {
+        float v = bf16_bits_to_f32(xd[k]);
+        s += a.ln_kind == 0 ? v : v * v;
+      }
+      s = wave_sum(s);
+      if (lane == 0) red[wave] = s;
+      __syncthreads();
+      s = red[0] + red[1] + red[2] + red[3];
+      float mean = 0.f, scale;
+      if (a.ln_kind == 0) {
+        mean = s / (float)K;
+        float q = 0.f;
+        for (int k = tid; k < K; k += 256) { float d = bf16_bits_to_f32(xd[k]) - mean; q += d * d; }
+        q = wave_sum(q);
+        if (lane == 0) red[4 + wave] = q;
+        __syncthreads();
+        q = red[4] + red[5] + red[6] + red[7];
+        scale = 1.0f / sqrtf(q / (float)K + a.ln_eps);
+      } else {
+        scale = 1.0f / sqrtf(s / (float)K + a.ln_eps);
+      }
+      const uint16_t *lw = (const uint16_t *)a.ln_w, *lb = (const uint16_t *)a.ln_b;
+      for (int k = tid; k < K; k += 256) {
+        float y = (bf16_bits_to_f32(xd[k]) - mean) * scale;
+        float wv = bf16_bits_to_f32(lw[k]);
+        y *= a.ln_kind == 2 ? 1.0f + wv : wv;
+        if (lb) y += bf16_bits_to_f32(lb[k]);
+        // the reference materialises the normalised activations in bf16 too
+        xd[k] = f32_to_bf16_bits(y);
+      }
+      __syncthreads();
+    }
+  }
+  __syncthreads();
+
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+  const int n_groups = (a.N + R - 1) / R;
+  for (int g = blockIdx.x * 4 + wave; g < n_groups; g += gridDim.x * 4) {
+    const int n_base = g * R;
+    float acc[R][MROWS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) acc[r][m] = 0.f;
+    const uint16_t *wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int n = n_base + r < a.N ? n_base + r : a.N - 1;
+      wrow[r] = W + (int64_t)n * a.ldw;
+    }
+#pragma unroll 2
+    for (int k = lane * 8; k < K; k += 64 * 8) {
+      u32x4 wv[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) wv[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[r] + k));
+      u32x4 xv[MROWS];
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) xv[m] = *reinterpret_cast<const u32x4 *>(xs + m * K + k);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) acc[r][m] = dot8_bf16(wv[r], xv[m], acc[r][m]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) acc[r][m] = wave_sum(acc[r][m]);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = n_base + r;
+        if (n >= a.N) break;
+        const float bv = (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
+        const bool do_act = a.act >= 0 && n >= a.act_from;
+        uint16_t *dst;
+        int64_t ld;
+        int col;
+        if (n < a.n_split) { dst = (uint16_t *)a.out1; ld = a.ld1; col = n; }
+        else { dst = (uint16_t *)a.out2; ld = a.ld2; col = n - a.n_split; }
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) {
+          if (m >= a.M) break;
+          float v = acc[r][m] + bv;
+          if (do_act) v = act_eval(a.act, v);
+          if (res) v += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
+          dst[(int64_t)m * ld + col] = f32_to_bf16_bits(v);
+        }
+      }
+    }
+  }
+}
+
+// ============================================================ f32 NT tile kernel
+// 64x64 tile, BK=16, 256 threads each computing a 4x4 micro-tile with FMA.
+__global__ void __launch_bounds__(256) k_linear_f32(LinearArgs a) {
+  constexpr int BM = 64, BN = 64, BK = 16;
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Bs[BK][BN + 4];
+  const int tid = threadIdx.x;
+  const int tiles_m = (a.M + BM - 1) / BM;
+  const int tile_n = blockIdx.x / tiles_m, tile_m = blockIdx.x % tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const float *A = (const float *)a.A;
+  const float *W = (const float *)a.W;
+  const int tx = tid & 15, ty = tid >> 4;  // 16 x 16 threads
+  float acc[4][4] = {};
+  const int lrow = tid >> 2, lk = (tid & 3) * 4;  // each thread loads 4 consecutive k of one row
+  const bool vec_ok = (a.lda % 4 == 0) && (a.ldw % 4 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    float va[4] = {0.f, 0.f, 0.f, 0.f}, vb[4] = {0.f, 0.f, 0.f, 0.f};
+    {
+      int m = m0 + lrow, k = k0 + lk;
+      if (m < a.M) {
+        const float *p = A + (int64_t)m * a.lda + k;
+        if (vec_ok && k + 3 < a.K) { float4 t = *reinterpret_cast<const float4 *>(p); va[0] = t.x; va[1] = t.y; va[2] = t.z; va[3] = t.w; }
+        else { for (int j = 0; j < 4; ++j) if (k + j < a.K) va[j] = p[j]; }
+      }
+      int n = n0 + lrow;
+      if (n < a.N) {
+        const float *p = W + (int64_t)n * a.ldw + k;
+        if (vec_ok && k + 3 < a.K) { float4 t = *reinterpret_cast<const float4 *>(p); vb[0] = t.x; vb[1] = t.y; vb[2] = t.z; vb[3] = t.w; }
+        else { for (int j = 0; j < 4; ++j) if (k + j < a.K) vb[j] = p[j]; }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { As[lk + j][lrow] = va[j]; Bs[lk + j][lrow] = vb[j]; }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      float4 av = *reinterpret_cast<const float4 *>(&As[k][ty * 4]);
+      float4 bv = *reinterpret_cast<const float4 *>(&Bs[k][tx * 4]);
+      float af[4] = {av.x, av.y, av.z, av.w}, bf[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(af[i], bf[j], acc[i][j]);
+    }
+  }
+  const float *bias = (const float *)a.bias;
+  const float *bias2 = (const float *)a.bias2;
+  const float *res = (const float *)a.residual;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int m = m0 + ty * 4 + i;
+    if (m >= a.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int n = n0 + tx * 4 + j;
+      if (n >= a.N) continue;
+      float v = acc[i][j] + (bias ? bias[n] : 0.f) + (bias2 ? bias2[n] : 0.f);
+      if (a.act >= 0 && n >= a.act_from) v = act_eval(a.act, v);
+      if (res) v += res[(int64_t)m * a.ldr + n];
+      if (n < a.n_split) ((float *)a.out1)[(int64_t)m * a.ld1 + n] = v;
+      else ((float *)a.out2)[(int64_t)m * a.ld2 + (n - a.n_split)] = v;
+    }
+  }
+}
+
+// ============================================================ generic strided batched matmul
+struct MatmulArgs {
+  int64_t M, N, K;
+  int64_t a_rs, a_cs, b_rs, b_cs;  // element strides of the last two dims
+  int batch_rank;
+  int64_t batch_shape[RAI_HIP_MAX_RANK];
+  int64_t a_bs[RAI_HIP_MAX_RANK], b_bs[RAI_HIP_MAX_RANK];
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) k_matmul_generic(T *out, const T *A, const T *B, MatmulArgs g) {
+  typedef typename Scalar<T>::compute C;
+  constexpr int BM = 64, BN = 64, BK = 16;
+  __shared__ C As[BK][BM + 1];
+  __shared__ C Bs[BK][BN + 1];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  int64_t rem = blockIdx.z, aoff = 0, boff = 0;
+  for (int d = g.batch_rank - 1; d >= 0; --d) {
+    int64_t q = rem / g.batch_shape[d], i = rem - q * g.batch_shape[d];
+    rem = q;
+    aoff += i * g.a_bs[d];
+    boff += i * g.b_bs[d];
+  }
+  A += aoff;
+  B += boff;
+  out += (int64_t)blockIdx.z * g.M * g.N;
+  const int64_t m0 = (int64_t)blockIdx.y * BM, n0 = (int64_t)blockIdx.x * BN;
+  C acc[4][4] = {};
+  for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
+    // 64x16 elements of A and of B: 4 per thread each
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int e = tid + i * 256;
+      int kk, mm;
+      // pick the traversal that makes consecutive threads touch consecutive memory
+      if (g.a_cs == 1) { kk = e & 15; mm = e >> 4; } else { mm = e & 63; kk = e >> 6; }
+      int64_t m = m0 + mm, k = k0 + kk;
+      As[kk][mm] = (m < g.M && k < g.K) ? Scalar<T>::load(A + m * g.a_rs + k * g.a_cs) : C(0);
+      int nn;
+      if (g.b_cs == 1) { nn = e & 63; kk = e >> 6; } else { kk = e & 15; nn = e >> 4; }
+      int64_t n = n0 + nn;
+      k = k0 + kk;
+      Bs[kk][nn] = (n < g.N && k < g.K) ? Scalar<T>::load(B + k * g.b_rs + n * g.b_cs) : C(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      C af[4], bf[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { af[i] = As[k][ty * 4 + i]; bf[i] = Bs[k][tx * 4 + i]; }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += af[i] * bf[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int64_t m = m0 + ty * 4 + i;
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int64_t n = n0 + tx * 4 + j;
+      if (n < g.N) Scalar<T>::store(out + m * g.N + n, acc[i][j]);
+    }
+  }
+}
+
+// ============================================================ launchers
+template <int BM, int BN, int BK> static int launch_mfma_cfg(hipStream_t st, const LinearArgs &a) {
+  constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(uint16_t);
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma<BM, BN, BK>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  hipLaunchKernelGGL((k_linear_bf16_mfma<BM, BN, BK>), dim3(tiles), dim3(256), lds, st, a);
+  return launch_check("linear_bf16_mfma");
+}
+
+static int check_linear_args(const LinearArgs &a, size_t es) {
+  RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
+  RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
+  RAI_REQUIRE(a.n_split >= 0 && a.n_split <= a.N && (a.n_split == a.N || a.out2), RAI_ERR_BAD_ARG,
+              "linear: bad output split");
+  const int v = (int)(16 / es);
+  RAI_REQUIRE(a.K % v == 0 && a.lda % v == 0 && a.ldw % v == 0, RAI_ERR_BAD_STRIDE,
+              "linear: K and row strides must be multiples of %d elements", v);
+  RAI_REQUIRE((uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0, RAI_ERR_BAD_STRIDE,
+              "linear: operands must be 16-byte aligned");
+  return RAI_OK;
+}
+
+int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
+  RAI_TRY(check_linear_args(a, 2));
+  RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear: fused norm only on the skinny path");
+  if (a.M <= 64) return launch_mfma_cfg<64, 128, 64>(st, a);
+  return launch_mfma_cfg<128, 128, 64>(st, a);
+}
+
+template <int MROWS, int R> static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a) {
+  const size_t lds = (size_t)MROWS * a.K * sizeof(uint16_t);
+  static size_t attr_bytes = 0;
+  if (lds > 64 * 1024 && lds > attr_bytes) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_skinny<MROWS, R>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_bytes = lds;
+  }
+  const int n_groups = (a.N + R - 1) / R;
+  int blocks = (n_groups + 3) / 4;
+  // keep whole multiples of the CU count in flight when there is enough work
+  const int cap = kNumCU * 8;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL((k_linear_bf16_skinny<MROWS, R>), dim3(blocks), dim3(256), lds, st, a);
+  return launch_check("linear_bf16_skinny");
+}
+
+int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
+  RAI_TRY(check_linear_args(a, 2));
+  RAI_REQUIRE(a.M <= 8, RAI_ERR_BAD_SHAPE, "linear skinny: M=%d > 8", a.M);
+  RAI_REQUIRE((size_t)a.M * a.K * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
+  if (a.M == 1) return launch_skinny_cfg<1, 4>(st, a);
+  if (a.M == 2) return launch_skinny_cfg<2, 4>(st, a);
+  if (a.M <= 4) return launch_skinny_cfg<4, 2>(st, a);
+  return launch_skinny_cfg<8, 2>(st, a);
+}
+
+int launch_linear_bf16(hipStream_t st, const LinearArgs &a) {
+  if (a.M <= 8 && (size_t)a.M * a.K * 2 <= 150 * 1024) return launch_linear_bf16_skinny(st, a);
+  return launch_linear_bf16_mfma(st, a);
+}
+
+int launch_linear_f32(hipStream_t st, const LinearArgs &a) {
+  RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem");
+  RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear f32: no fused norm");
+  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  hipLaunchKernelGGL(k_linear_f32, dim3(tiles), dim3(256), 0, st, a);
+  return launch_check("linear_f32");
+}
+
+}  // namespace rai
+
+using namespace rai;
+
+extern "C" {
+
+int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, const rai_hip_tensor *out) {
+  RAI_TRY(validate(a, "a"));
+  RAI_TRY(validate(b, "b"));
+  RAI_TRY(validate(out, "out"));
+  RAI_REQUIRE(a->dtype == b->dtype && a->dtype == out->dtype, RAI_ERR_BAD_DTYPE, "matmul: dtypes differ (%s, %s, %s)",
+              dtype_name(a->dtype), dtype_name(b->dtype), dtype_name(out->dtype));
+  RAI_REQUIRE(is_float(a->dtype), RAI_ERR_BAD_DTYPE, "matmul: float dtype required");
+  RAI_REQUIRE(a->rank >= 2 && b->rank == a->rank && out->rank == a->rank, RAI_ERR_BAD_SHAPE,
+              "matmul: operands must have equal rank >= 2 (got %d, %d, %d)", a->rank, b->rank, out->rank);
+  const int r = a->rank;
+  const int64_t M = a->shape[r - 2], K = a->shape[r - 1], N = b->shape[r - 1];
+  RAI_REQUIRE(b->shape[r - 2] == K, RAI_ERR_BAD_SHAPE, "matmul: inner dims %lld vs %lld", (long long)K,
+              (long long)b->shape[r - 2]);
+  RAI_REQUIRE(out->shape[r - 2] == M && out->shape[r - 1] == N, RAI_ERR_BAD_SHAPE, "matmul: output is not [%lld,%lld]",
+              (long long)M, (long long)N);
+  int64_t batch = 1;
+  for (int i = 0; i < r - 2; ++i) {
+    RAI_REQUIRE(a->shape[i] == out->shape[i] && b->shape[i] == out->shape[i], RAI_ERR_BAD_SHAPE,
+                "matmul: batch dims must be broadcast to the output's");
+    batch *= out->shape[i];
+  }
+  RAI_REQUIRE(is_contiguous(out), RAI_ERR_BAD_STRIDE, "matmul: output must be contiguous");
+  hipStream_t st = stream_of(dev);
+  if (!st) return RAI_ERR_HIP;
+  if (numel(out) == 0) return RAI_OK;
+  if (K == 0) return rai_hip_fill(dev, out, 0.0);
+
+  // Fast path: one weight matrix shared by every batch (stride-0 batch dims) in
+  // NT layout with K-contiguous activations whose rows share one stride -> the
+  // batch folds into M.
+  if ((a->dtype == RAI_BF16 || a->dtype == RAI_F32) && b->stride[r - 2] == 1 && (a->stride[r - 1] == 1 || K == 1)) {
+    bool b_shared = true;
+    for (int i = 0; i < r - 2; ++i)
+      if (b->shape[i] != 1 && b->stride[i] != 0) b_shared = false;
+    rai_hip_tensor rows = *a;
+    rows.rank = r - 1;
+    const rai_hip_tensor *ts[1] = {&rows};
+    StridedArgs ca;
+    coalesce(1, ts, &ca);
+    const size_t es = dtype_size(a->dtype);
+    const int v = (int)(16 / es);
+    int64_t lda = (batch * M == 1) ? K : ca.stride[0][0];
+    int64_t ldw = N == 1 ? K : b->stride[r - 1];
+    bool aligned = K % v == 0 && lda % v == 0 && ldw % v == 0 && (uintptr_t)base_ptr(a) % 16 == 0 &&
+                   (uintptr_t)base_ptr(b) % 16 == 0;
+    if (b_shared && ca.rank == 1 && batch * M < (1LL << 31) && (a->dtype == RAI_F32 || aligned) && ldw >= K) {
+      LinearArgs la = linear_args_default();
+      la.A = base_ptr(a);
+      la.lda = lda;
+      la.W = base_ptr(b);
+      la.ldw = ldw;
+      la.out1 = base_ptr(out);
+      la.ld1 = N;
+      la.M = (int)(batch * M);
+      la.N = (int)N;
+      la.K = (int)K;
+      la.n_split = (int)N;
+      return a->dtype == RAI_BF16 ? launch_linear_bf16(st, la) : launch_linear_f32(st, la);
+    }
+  }
+
+  MatmulArgs g;
+  g.M = M; g.N = N; g.K = K;
+  g.a_rs = a->stride[r - 2]; g.a_cs = a->stride[r - 1];
+  g.b_rs = b->stride[r - 2]; g.b_cs = b->stride[r - 1];
+  g.batch_rank = r - 2;
+  for (int i = 0; i < RAI_HIP_MAX_RANK; ++i) {
+    bool in = i < r - 2;
+    g.batch_shape[i] = in ? out->shape[i] : 1;
+    g.a_bs[i] = in ? a->stride[i] : 0;
+    g.b_bs[i] = in ? b->stride[i] : 0;
+  }
+  RAI_REQUIRE(batch <= 65535, RAI_ERR_UNSUPPORTED, "matmul: batch %lld exceeds grid limit", (long long)batch);
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch);
+  RAI_DISPATCH_FLOAT(a->dtype, T,
+                     hipLaunchKernelGGL((k_matmul_generic<T>), grid, dim3(256), 0, st, (T *)base_ptr(out),
+                                        (const T *)base_ptr(a), (const T *)base_ptr(b), g));
+  return launch_check("matmul_generic");
+}
+
+int rai_hip_linear(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, const rai_hip_tensor *bias, int32_t act,
+                   const rai_hip_tensor *residual, const rai_hip_tensor *out) {
+  RAI_TRY(validate(x, "x"));
+  RAI_TRY(validate(w, "w"));
+  RAI_TRY(validate(out, "out"));
+  RAI_REQUIRE(x->dtype == RAI_BF16 || x->dtype == RAI_F32, RAI_ERR_BAD_DTYPE, "linear: bf16 or f32 required");
+  RAI_REQUIRE(w->dtype == x->dtype && out->dtype == x->dtype, RAI_ERR_BAD_DTYPE, "linear: dtype mismatch");
+  RAI_REQUIRE(w->rank == 2 && x->rank >= 1 && out->rank == x->rank, RAI_ERR_BAD_SHAPE, "linear: bad ranks");
+  const int64_t N = w->shape[0], K = w->shape[1];
+  RAI_REQUIRE(x->shape[x->rank - 1] == K && out->shape[out->rank - 1] == N, RAI_ERR_BAD_SHAPE,
+              "linear: x[..,%lld] w[%lld,%lld] out[..,%lld]", (long long)x->shape[x->rank - 1], (long long)N,
+              (long long)K, (long long)out->shape[out->rank - 1]);
+  for (int i = 0; i < x->rank - 1; ++i)
+    RAI_REQUIRE(x->shape[i] == out->shape[i], RAI_ERR_BAD_SHAPE, "linear: leading dims differ");
+  RAI_REQUIRE(is_contiguous(out), RAI_ERR_BAD_STRIDE, "linear: output must be contiguous");
+  RAI_REQUIRE((w->stride[1] == 1 || K == 1) && (x->stride[x->rank - 1] == 1 || K == 1), RAI_ERR_BAD_STRIDE,
+              "linear: x and w must be K-contiguous");
+  RAI_REQUIRE(act == -1 || act == RAI_UN_GELU || act == RAI_UN_NEW_GELU || act == RAI_UN_SILU || act == RAI_UN_RELU ||
+                  act == RAI_UN_TANH,
+              RAI_ERR_BAD_ARG, "linear: unsupported activation %d", act);
+  const int64_t M = K ? numel(x) / K : 0;
+  if (numel(out) == 0) return RAI_OK;
+  RAI_REQUIRE(M < (1LL << 31) && K > 0, RAI_ERR_BAD_SHAPE, "linear: bad problem size");
+  rai_hip_tensor rows = *x;
+  rows.rank = x->rank - 1;
+  const rai_hip_tensor *ts[1] = {&rows};
+  StridedArgs ca;
+  coalesce(1, ts, &ca);
+  RAI_REQUIRE(ca.rank == 1, RAI_ERR_BAD_STRIDE, "linear: rows of x must share one stride");
+  LinearArgs la = linear_args_default();
+  la.A = base_ptr(x);
+  la.lda = M == 1 ? K : ca.stride[0][0];
+  la.W = base_ptr(w);
+  la.ldw = N == 1 ? K : w->stride[0];
+  if (bias) {
+    RAI_TRY(validate(bias, "bias"));
+    RAI_REQUIRE(bias->dtype == x->dtype && bias->rank == 1 && bias->shape[0] == N && (bias->stride[0] == 1 || N == 1),
+                RAI_ERR_BAD_SHAPE, "linear: bias must be a contiguous [%lld] vector of x's dtype", (long long)N);
+    la.bias = base_ptr(bias);
+  }
+  if (residual) {
+    RAI_TRY(validate(residual, "residual"));
+    RAI_REQUIRE(residual->dtype == x->dtype && same_shape(residual, out) && is_contiguous(residual), RAI_ERR_BAD_SHAPE,
+                "linear: residual must be contiguous with the output's shape");
+    la.residual = base_ptr(residual);
+    la.ldr = N;
+  }
+  la.out1 = base_ptr(out);
+  la.ld1 = N;
+  la.M = (int)M;
+  la.N = (int)N;
+  la.K = (int)K;
+  la.n_split = (int)N;
+  la.act = act;
+  la.act_from = 0;
+  hipStream_t st = stream_of(dev);
+  if (!st) return RAI_ERR_HIP;
+  return x->dtype == RAI_BF16 ? launch_linear_bf16(st, la) : launch_linear_f32(st, la);
+}
+
+}  // extern "C"
