@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Phi-2-architecture bf16 greedy decode / prefill on one MI355X.
+
+Workload (one "step"): the full 32-layer Phi-2-architecture model, random-init
+N(0, 0.02) bf16 weights, batch 1, KV cache, a 512-token uniform-random prompt
+(prefill) followed by 128 greedy tokens (decode), all on the device through the
+C ABI of librai_hip.so.  Weights, prompt and KV cache are resident in HBM when
+the timed region starts.
+
+Prints ONE JSON line.  `value` is decode tokens/s; prefill tokens/s, the
+roofline of the dominant kernel (the weight-streaming decode kernel, HBM-bound)
+and a CPU baseline (the NumPy oracle restating rai's Cpu path, timed on this
+host on a bounded sample) ride along in the same object.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PHI2 = dict(vocab_size=51200, hidden_size=2560, intermediate_size=10240, num_hidden_layers=32,
+            num_attention_heads=32, rotary_dim=32, max_position_embeddings=2048, hidden_act="gelu_new",
+            rope_theta=10000.0, norm_eps=1e-5)
+PROMPT, NEW = 512, 128
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def decode_bytes_per_token(cfg, ctx):
+    """Algorithmic HBM bytes of one decode token at context length ctx (bf16):
+    every layer's weights and biases once, the lm_head, one embedding row and the
+    K/V rows of the cached context."""
+    h, i, v, l = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    layer = 4 * h * h + 4 * h + 2 * h * i + i + h + 2 * h      # q,k,v,dense + biases, fc1, fc2 + biases, LayerNorm
+    head = v * h + v + 2 * h
+    kv = l * 2 * h * ctx
+    return 2.0 * (l * layer + head + h + kv)
+
+
+def prefill_flops(cfg, s):
+    h, i, v, l = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    nh = cfg["num_attention_heads"]
+    hd = h // nh
+    lin = 2.0 * (4 * h * h + 2 * h * i) * l * s
+    attn = l * 4.0 * nh * s * s * hd
+    return lin + attn + 2.0 * v * h
+
+
+def cpu_baseline(steps_decode=2, layers=2):
+    """The oracle (a NumPy port of rai's Cpu evaluation, bf16 storage with f32
+    math) timed on this host on a bounded sample: the first `layers` decoder
+    layers plus embedding and lm_head, 512-token prefill, then `steps_decode`
+    decode tokens; the per-layer times are scaled to 32 layers."""
+    from oracle import phi2
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    cfg = phi2.Config(num_hidden_layers=layers)
+    params = phi2.random_params(cfg, "bf16", seed=0)
+    model = phi2.Model(cfg, params, "bf16")
+    ids = np.random.Generator(np.random.PCG64(1)).integers(0, cfg.vocab_size, (1, PROMPT)).astype(np.uint32)
+
+    def timed_layers(x, mask):
+        t0 = time.perf_counter()
+        for l in range(layers):
+            x = model.layer(l, x, mask)
+        return x, time.perf_counter() - t0
+
+    from oracle import nn as onn, ops as oo
+    t0 = time.perf_counter()
+    x = onn.embedding(ids, params["model.embed_tokens.weight"])
+    t_embed = time.perf_counter() - t0
+    x, t_pre_layers = timed_layers(x, phi2.get_mask(PROMPT))
+
+    def head(x):
+        t0 = time.perf_counter()
+        y = onn.layer_norm(x, params["model.final_layernorm.weight"], params["model.final_layernorm.bias"], 1e-5, "bf16")
+        y = oo.narrow(y, 1, y.shape[1] - 1, 1)
+        logits = onn.linear(y, params["lm_head.weight"], params["lm_head.bias"], "bf16")
+        tok = oo.argmax(logits[:, 0, :], -1)
+        return tok, time.perf_counter() - t0
+
+    tok, t_head = head(x)
+    prefill_s = t_embed + t_pre_layers * (32.0 / layers) + t_head
+    dec_layers, dec_head = 0.0, 0.0
+    for _ in range(steps_decode):
+        x = onn.embedding(tok.reshape(1, 1), params["model.embed_tokens.weight"])
+        x, tl = timed_layers(x, None)
+        tok, th = head(x)
+        dec_layers += tl
+        dec_head += th
+    decode_s_per_tok = (dec_layers * (32.0 / layers) + dec_head) / steps_decode
+    return {
+        "value": round(1.0 / decode_s_per_tok, 4),
+        "unit": "tokens/s (decode)",
+        "prefill_tokens_per_s": round(PROMPT / prefill_s, 2),
+        "cores": threads,
+        "kind": "port",
+        "sample": f"NumPy oracle of rai's Cpu path (bf16 storage, f32 math): {layers} of 32 layers + embedding + "
+                  f"lm_head timed, 512-token prefill then {steps_decode} decode tokens, layer time scaled x{32 // layers}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layers", type=int, default=PHI2["num_hidden_layers"],
+                    help="debug only: fewer layers (the JSON line then says so and is not the headline workload)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (multi-GPU sharding is a design note only)")
+
+    from rai_amd import synthetic
+    from rai_amd.hip import sync
+    from rai_amd.models import Decoder
+
+    cfg = dict(PHI2)
+    cfg["num_hidden_layers"] = args.layers
+    t0 = time.perf_counter()
+    dec = Decoder("phi2", "bf16", max_batch=1, max_context=PROMPT + NEW, **cfg)
+    synthetic.load_random_params(dec, seed=0)
+    sync()
+    load_s = time.perf_counter() - t0
+    prompt = synthetic.prompt(cfg["vocab_size"], 1, PROMPT, seed=1)
+
+    for _ in range(args.warmup):
+        dec.generate(prompt, NEW)
+    sync()
+    wall0 = time.perf_counter()
+    pre_ms, dec_ms, toks = [], [], None
+    for _ in range(args.steps):
+        toks, p, d = dec.generate(prompt, NEW)
+        pre_ms.append(p)
+        dec_ms.append(d)
+    sync()
+    wall = time.perf_counter() - wall0
+    pre = float(np.mean(pre_ms))
+    dcd = float(np.mean(dec_ms))
+    decode_tok_s = (NEW - 1) / (dcd / 1e3)     # the prefill produces token 0; NEW-1 single-token steps follow
+    prefill_tok_s = PROMPT / (pre / 1e3)
+
+    # dominant kernel: the M=1 weight-streaming kernel, timed live with hipEvents on the library's stream
+    us, bytes_per_launch = dec.time_decode_linear(sweeps=20)
+    achieved = bytes_per_launch / (us * 1e-6) / 1e9
+    mean_ctx = PROMPT + (NEW - 1) / 2.0 + 1
+    step_bytes = decode_bytes_per_token(cfg, mean_ctx)
+    out = {
+        "metric": "Phi-2 bf16 decode tok/s on 1 MI355X",
+        "value": round(decode_tok_s, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"Phi-2 architecture {args.layers}L bf16, batch 1, KV cache, {PROMPT}-token prompt + "
+                               f"{NEW} greedy tokens (random-init N(0,0.02), uniform-random prompt)",
+                   "prompt_len": PROMPT, "new_tokens": NEW, "batch": 1},
+        "decode_ms_per_token": round(dcd / (NEW - 1), 4),
+        "decode_frac_of_hbm_roofline": round(step_bytes / (dcd / 1e3 / (NEW - 1)) / 1e9 / HBM_PEAK_GBS, 4),
+        "prefill_tokens_per_s": round(prefill_tok_s, 1),
+        "prefill_ms": round(pre, 3),
+        "prefill_frac_of_bf16_mfma_peak": round(prefill_flops(cfg, PROMPT) / (pre / 1e3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "weights_load_s": round(load_s, 1),
+        "first_tokens": [int(t) for t in toks[0, :8]],
+        "roofline": {
+            "kernel": "k_linear_bf16_skinny<1,4> (decode: fused LayerNorm + q|k|v|fc1 GEMV, dense|fc2 GEMV)",
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "us_per_launch": round(us, 3),
+            "bytes_per_launch": int(bytes_per_launch),
+        },
+    }
+    dec.close()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

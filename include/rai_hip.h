@@ -328,6 +328,15 @@ int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *dec);
 /* Current cached context length. */
 int rai_hip_decoder_context_len(rai_hip_decoder *dec, int32_t *len);
 
+/* Measurement only (no counterpart in the reference): launches the decode-step
+ * weight-streaming kernel back to back over every layer's two packed matrices
+ * (q|k|v|fc1 with the fused LayerNorm, then dense|fc2 with the residual; 2*L
+ * launches per sweep) between two hipEvents on the device's stream.  Reports the
+ * mean time of one launch in microseconds and the algorithmic bytes one launch
+ * moves on average (weights + biases + activation vectors in and out). */
+int rai_hip_decoder_time_decode_linear(rai_hip_decoder *dec, int32_t sweeps, float *us_per_launch,
+                                       double *bytes_per_launch);
+
 #ifdef __cplusplus
 }
 #endif

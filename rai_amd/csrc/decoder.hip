@@ -663,4 +663,53 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   return rc;
 }
 
+int rai_hip_decoder_time_decode_linear(rai_hip_decoder *d, int32_t sweeps, float *us_per_launch,
+                                       double *bytes_per_launch) {
+  RAI_REQUIRE(d && us_per_launch && bytes_per_launch && sweeps > 0, RAI_ERR_BAD_ARG, "bad argument");
+  RAI_REQUIRE(d->cfg.dtype == RAI_BF16, RAI_ERR_UNSUPPORTED, "time_decode_linear: bf16 models only");
+  hipStream_t st = stream_of(d->dev);
+  hipEvent_t e0, e1;
+  RAI_HIP_TRY(hipEventCreate(&e0));
+  RAI_HIP_TRY(hipEventCreate(&e1));
+  const int H = d->H, ldq = d->QD + 2 * d->KD;
+  auto sweep = [&]() -> int {
+    for (int l = 0; l < d->L; ++l) {
+      const Layer &ly = d->layers[l];
+      LinearArgs a = linear_args_default();
+      a.A = d->x; a.lda = H;
+      a.ln_kind = 0; a.ln_w = ly.ln_w; a.ln_b = ly.ln_b; a.ln_eps = (float)d->cfg.norm_eps;
+      a.W = ly.Wa; a.ldw = H; a.bias = ly.ba;
+      a.out1 = d->qkv; a.ld1 = ldq;
+      a.out2 = d->cat + (size_t)d->QD * d->es; a.ld2 = d->KB;
+      a.M = 1; a.N = d->NA; a.K = H; a.n_split = ldq;
+      a.act = d->cfg.hidden_act; a.act_from = ldq;
+      RAI_TRY(launch_linear_bf16(st, a));
+      LinearArgs b = linear_args_default();
+      b.A = d->cat; b.lda = d->KB;
+      b.W = ly.Wb; b.ldw = d->KB;
+      b.bias = ly.bd; b.bias2 = ly.bf;
+      b.residual = d->x; b.ldr = H;
+      b.out1 = d->x2; b.ld1 = H;
+      b.M = 1; b.N = H; b.K = d->KB; b.n_split = H;
+      RAI_TRY(launch_linear_bf16(st, b));
+    }
+    return RAI_OK;
+  };
+  RAI_TRY(sweep());  // warm-up
+  RAI_HIP_TRY(hipEventRecord(e0, st));
+  for (int s = 0; s < sweeps; ++s) RAI_TRY(sweep());
+  RAI_HIP_TRY(hipEventRecord(e1, st));
+  RAI_HIP_TRY(hipEventSynchronize(e1));
+  float ms = 0.f;
+  RAI_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  *us_per_launch = ms * 1000.0f / (float)(2 * d->L * sweeps);
+  const double es = (double)d->es;
+  const double bytes_a = ((double)d->NA * H + d->NA + 3.0 * H + d->NA) * es;          // W, bias, x + ln w/b, out
+  const double bytes_b = ((double)H * d->KB + 2.0 * H + d->KB + H + H) * es;          // W, 2 biases, in, residual, out
+  *bytes_per_launch = 0.5 * (bytes_a + bytes_b);
+  return RAI_OK;
+}
+
 }  // extern "C"
