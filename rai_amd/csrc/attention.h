@@ -27,4 +27,22 @@ struct AttnArgs {
 
 int launch_attention(hipStream_t st, const AttnArgs &a);
 
+// One new token per sequence (decode): rotary embedding of q and of the new k,
+// append of k/v to the cache, and attention over the cache plus the new token,
+// in one launch.  qkv rows are [q (Hq*D) | k (Hkv*D) | v (Hkv*D)], not yet rotated.
+struct AttnDecodeArgs {
+  const void *qkv;
+  void *kcache, *vcache;  // this layer's [B][Hkv][Tmax][D]
+  void *out;
+  int64_t out_row_stride;
+  const void *cos_t, *sin_t;  // [max_pos, rot] in the model dtype
+  const int *pos_dev;         // tokens already in the cache (device memory)
+  int rot;
+  int B, Hq, Hkv, D, Tmax;
+  float scale;
+  int f32_scores;
+  int dtype;
+};
+int launch_attention_decode(hipStream_t st, const AttnDecodeArgs &a);
+
 }  // namespace rai

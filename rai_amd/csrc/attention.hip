@@ -129,6 +129,164 @@ __global__ void __launch_bounds__(256) k_attn_row(AttnArgs a) {
   }
 }
 
+// Rotary embedding of feature d of one head for position pos, with the
+// reference's three roundings (x*cos, rotate_half(x)*sin, their sum:
+// rai-models/src/llm/phi2.rs:75).
+template <typename T>
+__device__ __forceinline__ float rope_feature(const T *head, int d, int rot, const T *cos_t, const T *sin_t, int pos) {
+  float v = (float)Scalar<T>::load(head + d);
+  if (d >= rot) return v;
+  const int half = rot >> 1;
+  float other = d < half ? -(float)Scalar<T>::load(head + d + half) : (float)Scalar<T>::load(head + d - half);
+  float c = (float)Scalar<T>::load(cos_t + (int64_t)pos * rot + d);
+  float s = (float)Scalar<T>::load(sin_t + (int64_t)pos * rot + d);
+  return round_to<T>(round_to<T>(v * c) + round_to<T>(other * s));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) k_attn_decode(AttnDecodeArgs a) {
+  constexpr int V = AttnVec<T>::V;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  // layout: q[D] | knew[D] | vnew[D] | red[groups*D] | scores[Tmax+1]
+  const int D = a.D, ncol = D / V;
+  const int groups = 256 / ncol;
+  float *qf = smem;
+  float *knew = qf + D;
+  float *vnew = knew + D;
+  float *red = vnew + D;
+  float *scores = red + groups * D;
+  __shared__ float sh[8];
+
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n_rep = a.Hq / a.Hkv, hk = h / n_rep;
+  int pos = *a.pos_dev;
+  if (pos > a.Tmax - 1) pos = a.Tmax - 1;  // capacity is checked on the host; never write past the cache
+  const int QD = a.Hq * D, KD = a.Hkv * D;
+  const T *row = (const T *)a.qkv + (int64_t)b * (QD + 2 * KD);
+  T *Kc = (T *)a.kcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
+  T *Vc = (T *)a.vcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
+  const T *cos_t = (const T *)a.cos_t, *sin_t = (const T *)a.sin_t;
+
+  for (int d = tid; d < D; d += 256) {
+    qf[d] = rope_feature<T>(row + h * D, d, a.rot, cos_t, sin_t, pos);
+    float kn = rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos);
+    float vn = (float)Scalar<T>::load(row + QD + KD + hk * D + d);
+    knew[d] = kn;
+    vnew[d] = vn;
+    if (h % n_rep == 0) {
+      Scalar<T>::store(Kc + (int64_t)pos * D + d, (typename Scalar<T>::compute)kn);
+      Scalar<T>::store(Vc + (int64_t)pos * D + d, (typename Scalar<T>::compute)vn);
+    }
+  }
+  __syncthreads();
+
+  auto finish_score = [&](float acc) -> float {
+    if (a.f32_scores) return acc * a.scale;
+    return round_to<T>(round_to<T>(acc) * round_to<T>(a.scale));
+  };
+  // ---- scores against the cached keys: 16 lanes per key row
+  {
+    const int g = tid >> 4, gl = tid & 15;
+    for (int t = g; t < pos; t += 16) {
+      const T *kr = Kc + (int64_t)t * D;
+      float acc = 0.f;
+      for (int c = gl; c < ncol; c += 16) {
+        APack<T, V> pk = *reinterpret_cast<const APack<T, V> *>(kr + c * V);
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&pk.v[j]), acc);
+      }
+      acc += __shfl_xor(acc, 8, 64);
+      acc += __shfl_xor(acc, 4, 64);
+      acc += __shfl_xor(acc, 2, 64);
+      acc += __shfl_xor(acc, 1, 64);
+      if (gl == 0) scores[t] = finish_score(acc);
+    }
+    // the new token's own key, still in LDS
+    if (wave == 3) {
+      float acc = 0.f;
+      for (int d = lane; d < D; d += 64) acc = fmaf(qf[d], knew[d], acc);
+      acc = wave_sum(acc);
+      if (lane == 0) scores[pos] = finish_score(acc);
+    }
+  }
+  __syncthreads();
+  const int t_end = pos + 1;
+  float m = -INFINITY;
+  for (int t = tid; t < t_end; t += 256) m = fmaxf(m, scores[t]);
+  m = wave_max(m);
+  if (lane == 0) sh[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  float sum = 0.f;
+  for (int t = tid; t < t_end; t += 256) {
+    float e = expf(scores[t] - m);
+    if (!a.f32_scores) e = round_to<T>(e);
+    scores[t] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) sh[4 + wave] = sum;
+  __syncthreads();
+  sum = sh[4] + sh[5] + sh[6] + sh[7];
+  if (!a.f32_scores) sum = round_to<T>(sum);
+  const float inv = 1.0f / sum;
+  auto prob = [&](int t) -> float {
+    return a.f32_scores ? round_to<T>(scores[t] * inv) : round_to<T>(scores[t] / sum);
+  };
+  {
+    const int col = tid % ncol, grp = tid / ncol;
+    float acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = 0.f;
+    if (grp < groups) {
+      for (int t = grp; t < pos; t += groups) {
+        const float p = prob(t);
+        APack<T, V> pk = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&pk.v[j]), acc[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) red[grp * D + col * V + j] = acc[j];
+    }
+  }
+  __syncthreads();
+  T *o = (T *)a.out + (int64_t)b * a.out_row_stride + (int64_t)h * D;
+  const float p_new = prob(pos);
+  for (int d = tid; d < D; d += 256) {
+    float r = p_new * vnew[d];
+    for (int g = 0; g < groups; ++g) r += red[g * D + d];
+    Scalar<T>::store(o + d, (typename Scalar<T>::compute)r);
+  }
+}
+
+template <typename T> static int launch_decode(hipStream_t st, const AttnDecodeArgs &a) {
+  constexpr int V = AttnVec<T>::V;
+  RAI_REQUIRE(a.D % V == 0 && a.D / V <= 256, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
+  const int ncol = a.D / V, groups = 256 / ncol;
+  const size_t lds = sizeof(float) * (3 * (size_t)a.D + (size_t)groups * a.D + (size_t)a.Tmax + 1);
+  RAI_REQUIRE(lds <= 150 * 1024, RAI_ERR_UNSUPPORTED, "attention: context %d too long for the decode kernel", a.Tmax);
+  static size_t attr_bytes = 0;
+  if (lds > 64 * 1024 && lds > attr_bytes) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_decode<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    150 * 1024));
+    attr_bytes = 150 * 1024;
+  }
+  hipLaunchKernelGGL((k_attn_decode<T>), dim3(a.Hq, a.B), dim3(256), lds, st, a);
+  return launch_check("attention_decode");
+}
+
+int launch_attention_decode(hipStream_t st, const AttnDecodeArgs &a) {
+  RAI_REQUIRE(a.B > 0 && a.Hq > 0 && a.Hkv > 0 && a.D > 0 && a.Tmax > 0 && a.Hq % a.Hkv == 0, RAI_ERR_BAD_SHAPE,
+              "attention decode: bad problem");
+  RAI_REQUIRE(a.rot > 0 && a.rot % 2 == 0 && a.rot <= a.D, RAI_ERR_BAD_ARG, "attention decode: rot %d", a.rot);
+  switch (a.dtype) {
+    case RAI_F32: return launch_decode<float>(st, a);
+    case RAI_BF16: return launch_decode<bf16_raw>(st, a);
+    default: return fail(RAI_ERR_BAD_DTYPE, "attention decode: dtype %s unsupported", dtype_name(a.dtype));
+  }
+}
+
 template <typename T> static int launch_row(hipStream_t st, const AttnArgs &a) {
   constexpr int V = AttnVec<T>::V;
   RAI_REQUIRE(a.D % V == 0 && a.D / V <= 256, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);

@@ -14,6 +14,7 @@
 // residual).  A decode step fuses the LayerNorm into the weight-streaming
 // kernel: 3 launches per layer.  Context length and the current tokens live in
 // device memory, so consecutive greedy steps need no host round trip.
+#include <cstdlib>
 #include <map>
 #include <string>
 #include <vector>
@@ -36,8 +37,10 @@ struct Layer {
 };
 
 struct DevState {
-  int pos;   // tokens already in the KV cache
-  int step;  // greedy steps taken by the current generate call
+  int pos;    // tokens already in the KV cache
+  int step;   // greedy steps taken by the current generate call
+  int done;   // blocks of the token-selection kernel that have finished (reset by the last one)
+  int pad;
 };
 
 }  // namespace rai
@@ -63,6 +66,9 @@ struct rai_hip_decoder {
   int ctx_len;
   int64_t max_rows;
   int history_cap;
+  hipGraphExec_t step_graph;  // one captured single-token step (batch step_graph_batch)
+  int step_graph_batch;
+  bool x_holds_next;          // d->x already holds the embedding of d->tokens
 };
 
 namespace rai {
@@ -144,20 +150,24 @@ k_rope_append(T *qkv, T *kcache, T *vcache, const T *cos_t, const T *sin_t, cons
 __global__ void k_set_state(DevState *st, int pos, int step) {
   st->pos = pos;
   st->step = step;
-}
-__global__ void k_advance(DevState *st, int dpos, int dstep) {
-  st->pos += dpos;
-  st->step += dstep;
+  st->done = 0;
 }
 
-// argmax over bf16/f32 logits rows; first maximum wins, NaN never wins except at
-// index 0.  One block per row (vocab-sized rows, a handful of rows).
+// Greedy token selection for every sequence, one 1024-thread block per row of
+// logits: argmax (first maximum wins; NaN never wins except at index 0), the
+// token goes to tokens[b] and to history[step][b], the token's embedding row
+// becomes the next step's input x[b], and the last block to finish advances the
+// device-side context length / step counters.  Everything the next
+// single-token step needs is then on the device.
 template <typename T>
 __global__ void __launch_bounds__(1024)
-k_argmax_rows(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, const DevState *state, int B) {
+k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
+               int dstep, const T *embed, T *x_next, int H) {
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
+  __shared__ uint32_t chosen;
   const int b = blockIdx.x;
+  const int step = state->step;
   const T *x = logits + (int64_t)b * n;
   float bv = -INFINITY;
   uint32_t bi = 0xffffffffu;
@@ -182,7 +192,23 @@ k_argmax_rows(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, c
     float first = (float)Scalar<T>::load(x);
     if (bi == 0xffffffffu || first != first) bi = 0;
     tokens[b] = bi;
-    if (history) history[(int64_t)state->step * B + b] = bi;
+    if (history) history[(int64_t)step * B + b] = bi;
+    chosen = bi;
+  }
+  __syncthreads();
+  if (x_next) {
+    const T *row = embed + (int64_t)chosen * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) x_next[(int64_t)b * H + c] = row[c];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    int prev = atomicAdd(&state->done, 1);
+    if (prev == B - 1) {  // every block has read `step` and written its outputs
+      state->done = 0;
+      state->pos += dpos;
+      state->step += dstep;
+    }
   }
 }
 
@@ -351,7 +377,9 @@ static int linear(rai_hip_decoder *d, hipStream_t st, const LinearArgs &a) {
 }
 
 // ids (B*S u32) are already in d->ids; device state holds the context length.
-static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step) {
+// With from_tokens the input embeddings were already written to d->x by the
+// previous step's token selection (single-token steps only).
+static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, bool from_tokens = false) {
   hipStream_t st = stream_of(d->dev);
   if (!st) return RAI_ERR_HIP;
   const int dt = d->cfg.dtype;
@@ -361,8 +389,10 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step) {
   const bool fuse_ln = dt == RAI_BF16 && M <= 8;
   const int T_after = d->ctx_len + S;
 
-  if (dt == RAI_BF16) launch_embed<bf16_raw>(d, st, M); else launch_embed<float>(d, st, M);
-  RAI_TRY(launch_check("embed"));
+  if (!from_tokens) {
+    if (dt == RAI_BF16) launch_embed<bf16_raw>(d, st, M); else launch_embed<float>(d, st, M);
+    RAI_TRY(launch_check("embed"));
+  }
 
   char *x = d->x, *xn = d->x2;
   for (int l = 0; l < d->L; ++l) {
@@ -384,32 +414,42 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step) {
     a.act = d->cfg.hidden_act; a.act_from = ldq;
     RAI_TRY(linear(d, st, a));
 
-    if (dt == RAI_BF16) launch_rope_append<bf16_raw>(d, st, l, B, S); else launch_rope_append<float>(d, st, l, B, S);
-    RAI_TRY(launch_check("rope_append"));
-
-    AttnArgs t;
-    memset(&t, 0, sizeof(t));
     const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
-    t.q = d->qkv;
-    t.k = d->kcache + per_layer * l * d->es;
-    t.v = d->vcache + per_layer * l * d->es;
-    t.out = d->cat;
-    t.qs[0] = (int64_t)S * ldq; t.qs[1] = d->D; t.qs[2] = ldq;
-    t.ks[0] = t.vs[0] = (int64_t)d->Hkv * d->cfg.max_context * d->D;
-    t.ks[1] = t.vs[1] = (int64_t)d->cfg.max_context * d->D;
-    t.ks[2] = t.vs[2] = d->D;
-    t.out_row_stride = d->KB;
-    t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.S = S; t.D = d->D;
-    t.scale = (float)(1.0 / sqrt((double)d->D));
-    t.causal = 1; t.f32_scores = 1; t.dtype = dt;
-    if (S == 1) {  // decode: key count comes from device state, capacity bounds LDS
-      t.T = d->cfg.max_context;
-      t.t_dev = &d->state->pos;
-      t.t_add = 1;
+    if (S == 1) {
+      // decode: rotary + cache append + attention in one launch, context length read on the device
+      AttnDecodeArgs t;
+      memset(&t, 0, sizeof(t));
+      t.qkv = d->qkv;
+      t.kcache = d->kcache + per_layer * l * d->es;
+      t.vcache = d->vcache + per_layer * l * d->es;
+      t.out = d->cat;
+      t.out_row_stride = d->KB;
+      t.cos_t = d->cos_t; t.sin_t = d->sin_t; t.rot = d->cfg.rotary_dim;
+      t.pos_dev = &d->state->pos;
+      t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.D = d->D; t.Tmax = d->cfg.max_context;
+      t.scale = (float)(1.0 / sqrt((double)d->D));
+      t.f32_scores = 1; t.dtype = dt;
+      RAI_TRY(launch_attention_decode(st, t));
     } else {
+      if (dt == RAI_BF16) launch_rope_append<bf16_raw>(d, st, l, B, S); else launch_rope_append<float>(d, st, l, B, S);
+      RAI_TRY(launch_check("rope_append"));
+      AttnArgs t;
+      memset(&t, 0, sizeof(t));
+      t.q = d->qkv;
+      t.k = d->kcache + per_layer * l * d->es;
+      t.v = d->vcache + per_layer * l * d->es;
+      t.out = d->cat;
+      t.qs[0] = (int64_t)S * ldq; t.qs[1] = d->D; t.qs[2] = ldq;
+      t.ks[0] = t.vs[0] = (int64_t)d->Hkv * d->cfg.max_context * d->D;
+      t.ks[1] = t.vs[1] = (int64_t)d->cfg.max_context * d->D;
+      t.ks[2] = t.vs[2] = d->D;
+      t.out_row_stride = d->KB;
+      t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.S = S; t.D = d->D;
+      t.scale = (float)(1.0 / sqrt((double)d->D));
+      t.causal = 1; t.f32_scores = 1; t.dtype = dt;
       t.T = T_after;
+      RAI_TRY(launch_attention(st, t));
     }
-    RAI_TRY(launch_attention(st, t));
 
     LinearArgs b = linear_args_default();
     b.A = d->cat; b.lda = d->KB;
@@ -442,14 +482,13 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step) {
 
   uint32_t *hist = advance_step ? d->history : nullptr;
   if (dt == RAI_BF16)
-    hipLaunchKernelGGL((k_argmax_rows<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits, (int64_t)d->V,
-                       d->tokens, hist, d->state, B);
+    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
+                       (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
+                       (bf16_raw *)d->x, H);
   else
-    hipLaunchKernelGGL((k_argmax_rows<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
-                       d->tokens, hist, d->state, B);
-  RAI_TRY(launch_check("argmax_rows"));
-  hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, st, d->state, S, advance_step ? 1 : 0);
-  RAI_TRY(launch_check("advance"));
+    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
+                       d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H);
+  RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
 }
@@ -496,6 +535,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->NA = d->QD + 2 * d->KD + d->I;
   d->KB = d->QD + d->I;
   d->ctx_len = 0;
+  d->step_graph = nullptr;
+  d->step_graph_batch = 0;
+  d->x_holds_next = false;
   const int vec = (int)(16 / d->es);
   int st = RAI_OK;
   auto bail = [&](int code) {
@@ -538,6 +580,7 @@ int rai_hip_decoder_destroy(rai_hip_decoder *d) {
   if (!d) return RAI_OK;
   (void)hipSetDevice(d->dev);
   (void)hipStreamSynchronize(stream_of(d->dev));
+  if (d->step_graph) (void)hipGraphExecDestroy(d->step_graph);
   for (void *p : d->allocs) (void)hipFree(p);
   delete d;
   return RAI_OK;
@@ -633,12 +676,38 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   RAI_HIP_TRY(hipEventRecord(e0, st));
   int rc = forward_phi2(d, batch, prompt_len, true);
   if (rc == RAI_OK) rc = hipEventRecord(e1, st) == hipSuccess ? RAI_OK : fail(RAI_ERR_HIP, "event record");
+  // Single-token steps: the previous step left the next input embedding, the
+  // token and the advanced context length on the device, so every step is the
+  // same sequence of launches.  The first step runs eagerly (it also performs
+  // any one-time kernel attribute set-up), the second is captured into a
+  // hipGraph, the rest replay it.
+  const bool use_graph = d->cfg.dtype == RAI_BF16 && getenv("RAI_HIP_NO_GRAPH") == nullptr;
   for (int step = 1; rc == RAI_OK && step < n_new; ++step) {
-    // next input = the tokens the previous step left on the device
-    if (hipMemcpyAsync(d->ids, d->tokens, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToDevice, st) != hipSuccess)
-      rc = fail(RAI_ERR_HIP, "generate: token feedback copy failed");
-    else
-      rc = forward_phi2(d, batch, 1, true);
+    if (use_graph && d->step_graph && d->step_graph_batch == batch) {
+      if (hipGraphLaunch(d->step_graph, st) != hipSuccess) rc = fail(RAI_ERR_HIP, "generate: graph launch failed");
+      else d->ctx_len += 1;
+      continue;
+    }
+    if (use_graph && step >= 2) {
+      if (d->step_graph) { (void)hipGraphExecDestroy(d->step_graph); d->step_graph = nullptr; }
+      hipGraph_t g = nullptr;
+      if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        rc = fail(RAI_ERR_HIP, "generate: begin capture failed");
+        break;
+      }
+      int frc = forward_phi2(d, batch, 1, true, true);
+      hipError_t ce = hipStreamEndCapture(st, &g);
+      if (frc != RAI_OK) { rc = frc; if (g) (void)hipGraphDestroy(g); break; }
+      if (ce != hipSuccess || !g) { rc = fail(RAI_ERR_HIP, "generate: end capture failed: %s", hipGetErrorString(ce)); break; }
+      d->ctx_len -= 1;  // capture only recorded the step; it has not run yet
+      hipError_t ie = hipGraphInstantiate(&d->step_graph, g, nullptr, nullptr, 0);
+      (void)hipGraphDestroy(g);
+      if (ie != hipSuccess) { d->step_graph = nullptr; rc = fail(RAI_ERR_HIP, "generate: graph instantiate: %s", hipGetErrorString(ie)); break; }
+      d->step_graph_batch = batch;
+      --step;  // run this step through the graph
+      continue;
+    }
+    rc = forward_phi2(d, batch, 1, true, true);
   }
   if (rc == RAI_OK && hipEventRecord(e2, st) != hipSuccess) rc = fail(RAI_ERR_HIP, "event record");
   if (rc == RAI_OK && hipStreamSynchronize(st) != hipSuccess) rc = fail(RAI_ERR_HIP, "generate: stream sync failed");

@@ -168,8 +168,11 @@ __device__ __forceinline__ float dot8_bf16(u32x4 a, u32x4 b, float c) {
   return dot2_bf16(a.w, b.w, c);
 }
 
-template <int MROWS, int R>
-__global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a) {
+// Every wave owns `rows_per_wave` consecutive weight rows (so all waves stream
+// the same number of bytes and are co-resident: no tail), R rows at a time, with
+// U 16-byte loads per row in flight per lane.
+template <int MROWS, int R, int U>
+__global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a, int rows_per_wave) {
   extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [MROWS][K]
   __shared__ float red[8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -225,9 +228,9 @@ __global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a) {
   const uint16_t *bias = (const uint16_t *)a.bias;
   const uint16_t *bias2 = (const uint16_t *)a.bias2;
   const uint16_t *res = (const uint16_t *)a.residual;
-  const int n_groups = (a.N + R - 1) / R;
-  for (int g = blockIdx.x * 4 + wave; g < n_groups; g += gridDim.x * 4) {
-    const int n_base = g * R;
+  const int n_begin = (blockIdx.x * 4 + wave) * rows_per_wave;
+  const int n_end = n_begin + rows_per_wave < a.N ? n_begin + rows_per_wave : a.N;
+  for (int n_base = n_begin; n_base < n_end; n_base += R) {
     float acc[R][MROWS];
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -236,21 +239,32 @@ __global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a) {
     const uint16_t *wrow[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      int n = n_base + r < a.N ? n_base + r : a.N - 1;
+      int n = n_base + r < n_end ? n_base + r : n_end - 1;  // tail rows re-read the last row; never stored
       wrow[r] = W + (int64_t)n * a.ldw;
     }
-#pragma unroll 2
-    for (int k = lane * 8; k < K; k += 64 * 8) {
-      u32x4 wv[R];
+    for (int k0 = lane * 8; k0 < K; k0 += 64 * 8 * U) {
+      u32x4 wv[U][R];
 #pragma unroll
-      for (int r = 0; r < R; ++r) wv[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[r] + k));
-      u32x4 xv[MROWS];
+      for (int u = 0; u < U; ++u) {
+        const int k = k0 + u * 512;
 #pragma unroll
-      for (int m = 0; m < MROWS; ++m) xv[m] = *reinterpret_cast<const u32x4 *>(xs + m * K + k);
+        for (int r = 0; r < R; ++r) {
+          if (k < K) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[r] + k));
+          else wv[u][r] = u32x4{0u, 0u, 0u, 0u};
+        }
+      }
 #pragma unroll
-      for (int r = 0; r < R; ++r)
+      for (int u = 0; u < U; ++u) {
+        const int k = k0 + u * 512;
+        if (k < K) {
 #pragma unroll
-        for (int m = 0; m < MROWS; ++m) acc[r][m] = dot8_bf16(wv[r], xv[m], acc[r][m]);
+          for (int m = 0; m < MROWS; ++m) {
+            const u32x4 xv = *reinterpret_cast<const u32x4 *>(xs + m * K + k);
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][m] = dot8_bf16(wv[u][r], xv, acc[r][m]);
+          }
+        }
+      }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -260,7 +274,7 @@ __global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int n = n_base + r;
-        if (n >= a.N) break;
+        if (n >= n_end) break;
         const float bv = (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
         const bool do_act = a.act >= 0 && n >= a.act_from;
         uint16_t *dst;
@@ -451,20 +465,17 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   return launch_mfma_cfg<128, 128, 64>(st, a);
 }
 
-template <int MROWS, int R> static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a) {
+template <int MROWS, int R, int U> static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a, int rows_per_wave) {
   const size_t lds = (size_t)MROWS * a.K * sizeof(uint16_t);
   static size_t attr_bytes = 0;
   if (lds > 64 * 1024 && lds > attr_bytes) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_skinny<MROWS, R>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_skinny<MROWS, R, U>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_bytes = lds;
   }
-  const int n_groups = (a.N + R - 1) / R;
-  int blocks = (n_groups + 3) / 4;
-  // keep whole multiples of the CU count in flight when there is enough work
-  const int cap = kNumCU * 8;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL((k_linear_bf16_skinny<MROWS, R>), dim3(blocks), dim3(256), lds, st, a);
+  const int waves = (a.N + rows_per_wave - 1) / rows_per_wave;
+  const int blocks = (waves + 3) / 4;
+  hipLaunchKernelGGL((k_linear_bf16_skinny<MROWS, R, U>), dim3(blocks), dim3(256), lds, st, a, rows_per_wave);
   return launch_check("linear_bf16_skinny");
 }
 
@@ -472,10 +483,25 @@ int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   RAI_TRY(check_linear_args(a, 2));
   RAI_REQUIRE(a.M <= 8, RAI_ERR_BAD_SHAPE, "linear skinny: M=%d > 8", a.M);
   RAI_REQUIRE((size_t)a.M * a.K * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
-  if (a.M == 1) return launch_skinny_cfg<1, 4>(st, a);
-  if (a.M == 2) return launch_skinny_cfg<2, 4>(st, a);
-  if (a.M <= 4) return launch_skinny_cfg<4, 2>(st, a);
-  return launch_skinny_cfg<8, 2>(st, a);
+  // About 8 waves per CU, all co-resident, each with the same number of rows.
+  const int target_waves = kNumCU * 8;
+  int rpw = (a.N + target_waves - 1) / target_waves;
+  if (a.M == 1) {
+    if (rpw >= 4) { rpw = (rpw / 4) * 4; return launch_skinny_cfg<1, 4, 5>(st, a, rpw); }
+    if (rpw >= 2) { rpw = 2; return launch_skinny_cfg<1, 2, 8>(st, a, rpw); }
+    return launch_skinny_cfg<1, 1, 8>(st, a, 1);
+  }
+  if (a.M == 2) {
+    if (rpw >= 4) { rpw = (rpw / 4) * 4; return launch_skinny_cfg<2, 4, 4>(st, a, rpw); }
+    if (rpw >= 2) return launch_skinny_cfg<2, 2, 8>(st, a, 2);
+    return launch_skinny_cfg<2, 1, 8>(st, a, 1);
+  }
+  if (a.M <= 4) {
+    if (rpw >= 2) { rpw = (rpw / 2) * 2; return launch_skinny_cfg<4, 2, 4>(st, a, rpw); }
+    return launch_skinny_cfg<4, 1, 8>(st, a, 1);
+  }
+  if (rpw >= 2) { rpw = (rpw / 2) * 2; return launch_skinny_cfg<8, 2, 4>(st, a, rpw); }
+  return launch_skinny_cfg<8, 1, 4>(st, a, 1);
 }
 
 int launch_linear_bf16(hipStream_t st, const LinearArgs &a) {

@@ -108,6 +108,25 @@ def test_greedy_generate_matches_oracle(hip, dt):
     dec.close()
 
 
+def test_graph_replay_equals_eager_steps(hip, monkeypatch):
+    # the captured single-token step must reproduce the eager launches on every replay,
+    # also when eager work and synchronisations happen between replays
+    cfg = small_cfg(num_hidden_layers=2)
+    dec, _ = make(cfg, "bf16", hip)
+    prompt = np.random.Generator(np.random.PCG64(5)).integers(0, cfg.vocab_size, (2, 11)).astype(np.uint32)
+    monkeypatch.setenv("RAI_HIP_NO_GRAPH", "1")
+    eager, _, _ = dec.generate(prompt, 20)
+    monkeypatch.delenv("RAI_HIP_NO_GRAPH")
+    for n in (20, 7, 20):
+        graph, _, _ = dec.generate(prompt, n)
+        assert np.array_equal(graph, eager[:, :n]), f"graph replay differs from eager at n={n}"
+        # eager forward + sync between graph uses
+        dec.clear_kv_cache()
+        _, tok = dec.forward(prompt)
+        assert np.array_equal(tok, eager[:, 0])
+    dec.close()
+
+
 def test_gqa_and_tied_head(hip):
     # num_key_value_heads < heads (repeat_kv phi2.rs:190-200) and tie_word_embeddings
     cfg = small_cfg(num_key_value_heads=2, tie_word_embeddings=True)
