@@ -143,19 +143,28 @@ __device__ __forceinline__ float rope_feature(const T *head, int d, int rot, con
   return round_to<T>(round_to<T>(v * c) + round_to<T>(other * s));
 }
 
+// Decode attention: one 1024-thread block per (head, batch) streams the head's
+// cached K and V once.  Sixty-four 16-lane groups each keep 4 key rows (16-byte
+// loads) in flight, so a 640-token context is covered in three rounds of loads.
+// The new token's rotated key and value are appended to the cache by the block
+// and used from LDS.  Probabilities stay in f32 until the product with V (the
+// reference rounds them to V's dtype first).
+constexpr int kDecodeThreads = 1024;
 template <typename T>
-__global__ void __launch_bounds__(256) k_attn_decode(AttnDecodeArgs a) {
+__global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a) {
   constexpr int V = AttnVec<T>::V;
+  constexpr int CC = 4;  // 16-byte chunks of one key row handled by one lane of a 16-lane group
+  constexpr int NW = kDecodeThreads / 64, NG = kDecodeThreads / 16;
   extern __shared__ __attribute__((aligned(16))) float smem[];
   // layout: q[D] | knew[D] | vnew[D] | red[groups*D] | scores[Tmax+1]
   const int D = a.D, ncol = D / V;
-  const int groups = 256 / ncol;
+  const int groups = kDecodeThreads / ncol;
   float *qf = smem;
   float *knew = qf + D;
   float *vnew = knew + D;
   float *red = vnew + D;
   float *scores = red + groups * D;
-  __shared__ float sh[8];
+  __shared__ float sh[2 * NW];
 
   const int h = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -168,7 +177,7 @@ __global__ void __launch_bounds__(256) k_attn_decode(AttnDecodeArgs a) {
   T *Vc = (T *)a.vcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   const T *cos_t = (const T *)a.cos_t, *sin_t = (const T *)a.sin_t;
 
-  for (int d = tid; d < D; d += 256) {
+  for (int d = tid; d < D; d += kDecodeThreads) {
     qf[d] = rope_feature<T>(row + h * D, d, a.rot, cos_t, sin_t, pos);
     float kn = rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos);
     float vn = (float)Scalar<T>::load(row + QD + KD + hk * D + d);
@@ -185,25 +194,40 @@ __global__ void __launch_bounds__(256) k_attn_decode(AttnDecodeArgs a) {
     if (a.f32_scores) return acc * a.scale;
     return round_to<T>(round_to<T>(acc) * round_to<T>(a.scale));
   };
-  // ---- scores against the cached keys: 16 lanes per key row
+  // ---- scores against the cached keys [0, pos)
   {
     const int g = tid >> 4, gl = tid & 15;
-    for (int t = g; t < pos; t += 16) {
-      const T *kr = Kc + (int64_t)t * D;
-      float acc = 0.f;
-      for (int c = gl; c < ncol; c += 16) {
-        APack<T, V> pk = *reinterpret_cast<const APack<T, V> *>(kr + c * V);
+    for (int tb = g; tb < pos; tb += 4 * NG) {
+      APack<T, V> pk[4][CC];
 #pragma unroll
-        for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&pk.v[j]), acc);
+      for (int u = 0; u < 4; ++u) {
+        const int t = tb + NG * u;
+#pragma unroll
+        for (int cc = 0; cc < CC; ++cc) {
+          const int c = gl + 16 * cc;
+          if (t < pos && c < ncol) pk[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
+        }
       }
-      acc += __shfl_xor(acc, 8, 64);
-      acc += __shfl_xor(acc, 4, 64);
-      acc += __shfl_xor(acc, 2, 64);
-      acc += __shfl_xor(acc, 1, 64);
-      if (gl == 0) scores[t] = finish_score(acc);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int t = tb + NG * u;
+        float acc = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < CC; ++cc) {
+          const int c = gl + 16 * cc;
+          if (t < pos && c < ncol) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&pk[u][cc].v[j]), acc);
+          }
+        }
+        acc += __shfl_xor(acc, 8, 64);
+        acc += __shfl_xor(acc, 4, 64);
+        acc += __shfl_xor(acc, 2, 64);
+        acc += __shfl_xor(acc, 1, 64);
+        if (gl == 0 && t < pos) scores[t] = finish_score(acc);
+      }
     }
-    // the new token's own key, still in LDS
-    if (wave == 3) {
+    if (wave == NW - 1) {  // the new token's own key, still in LDS
       float acc = 0.f;
       for (int d = lane; d < D; d += 64) acc = fmaf(qf[d], knew[d], acc);
       acc = wave_sum(acc);
@@ -211,40 +235,48 @@ __global__ void __launch_bounds__(256) k_attn_decode(AttnDecodeArgs a) {
     }
   }
   __syncthreads();
-  const int t_end = pos + 1;
+  const int cnt = pos + 1;
   float m = -INFINITY;
-  for (int t = tid; t < t_end; t += 256) m = fmaxf(m, scores[t]);
+  for (int t = tid; t < cnt; t += kDecodeThreads) m = fmaxf(m, scores[t]);
   m = wave_max(m);
   if (lane == 0) sh[wave] = m;
   __syncthreads();
-  m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  m = sh[0];
+  for (int w = 1; w < NW; ++w) m = fmaxf(m, sh[w]);
   float sum = 0.f;
-  for (int t = tid; t < t_end; t += 256) {
+  for (int t = tid; t < cnt; t += kDecodeThreads) {
     float e = expf(scores[t] - m);
-    if (!a.f32_scores) e = round_to<T>(e);
     scores[t] = e;
     sum += e;
   }
   sum = wave_sum(sum);
-  if (lane == 0) sh[4 + wave] = sum;
+  if (lane == 0) sh[NW + wave] = sum;
   __syncthreads();
-  sum = sh[4] + sh[5] + sh[6] + sh[7];
-  if (!a.f32_scores) sum = round_to<T>(sum);
-  const float inv = 1.0f / sum;
-  auto prob = [&](int t) -> float {
-    return a.f32_scores ? round_to<T>(scores[t] * inv) : round_to<T>(scores[t] / sum);
-  };
+  sum = 0.f;
+  for (int w = 0; w < NW; ++w) sum += sh[NW + w];
+  // ---- unnormalised P.V over the cached values, 4 rows in flight per thread
   {
     const int col = tid % ncol, grp = tid / ncol;
     float acc[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) acc[j] = 0.f;
     if (grp < groups) {
-      for (int t = grp; t < pos; t += groups) {
-        const float p = prob(t);
-        APack<T, V> pk = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+      for (int tb = grp; tb < pos; tb += 4 * groups) {
+        APack<T, V> pk[4];
 #pragma unroll
-        for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&pk.v[j]), acc[j]);
+        for (int u = 0; u < 4; ++u) {
+          const int t = tb + u * groups;
+          if (t < pos) pk[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int t = tb + u * groups;
+          if (t < pos) {
+            const float p = scores[t];
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&pk[u].v[j]), acc[j]);
+          }
+        }
       }
 #pragma unroll
       for (int j = 0; j < V; ++j) red[grp * D + col * V + j] = acc[j];
@@ -252,18 +284,18 @@ __global__ void __launch_bounds__(256) k_attn_decode(AttnDecodeArgs a) {
   }
   __syncthreads();
   T *o = (T *)a.out + (int64_t)b * a.out_row_stride + (int64_t)h * D;
-  const float p_new = prob(pos);
-  for (int d = tid; d < D; d += 256) {
+  const float p_new = scores[pos], inv = 1.0f / sum;
+  for (int d = tid; d < D; d += kDecodeThreads) {
     float r = p_new * vnew[d];
     for (int g = 0; g < groups; ++g) r += red[g * D + d];
-    Scalar<T>::store(o + d, (typename Scalar<T>::compute)r);
+    Scalar<T>::store(o + d, (typename Scalar<T>::compute)(r * inv));
   }
 }
 
 template <typename T> static int launch_decode(hipStream_t st, const AttnDecodeArgs &a) {
   constexpr int V = AttnVec<T>::V;
-  RAI_REQUIRE(a.D % V == 0 && a.D / V <= 256, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
-  const int ncol = a.D / V, groups = 256 / ncol;
+  RAI_REQUIRE(a.D % V == 0 && a.D / V <= 64, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
+  const int ncol = a.D / V, groups = kDecodeThreads / ncol;
   const size_t lds = sizeof(float) * (3 * (size_t)a.D + (size_t)groups * a.D + (size_t)a.Tmax + 1);
   RAI_REQUIRE(lds <= 150 * 1024, RAI_ERR_UNSUPPORTED, "attention: context %d too long for the decode kernel", a.Tmax);
   static size_t attr_bytes = 0;
@@ -272,7 +304,7 @@ template <typename T> static int launch_decode(hipStream_t st, const AttnDecodeA
                                     150 * 1024));
     attr_bytes = 150 * 1024;
   }
-  hipLaunchKernelGGL((k_attn_decode<T>), dim3(a.Hq, a.B), dim3(256), lds, st, a);
+  hipLaunchKernelGGL((k_attn_decode<T>), dim3(a.Hq, a.B), dim3(kDecodeThreads), lds, st, a);
   return launch_check("attention_decode");
 }
 

@@ -568,6 +568,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->history = (uint32_t *)tmp;
   if ((st = dalloc(d, sizeof(DevState), &tmp))) return bail(st);
   d->state = (DevState *)tmp;
+
   if (hipMemset(d->state, 0, sizeof(DevState)) != hipSuccess || hipMemset(d->kcache, 0, kv) != hipSuccess ||
       hipMemset(d->vcache, 0, kv) != hipSuccess)
     return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));

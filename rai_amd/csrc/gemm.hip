@@ -295,6 +295,130 @@ __global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a, int ro
   }
 }
 
+// ============================================================ bf16 GEMV with the activation vector in registers (M == 1)
+// One wave streams R weight rows at a time.  Lane l owns the K positions
+// l*8 + 512*u (u < KC), the same positions of the activation vector, which it
+// keeps in registers as packed bf16 pairs: no LDS, no block barriers, waves are
+// independent.  The weight loads of the first row group are issued before the
+// activation vector is fetched and normalised, so the fused LayerNorm/RMSNorm
+// prologue overlaps the first HBM round trip.
+template <int KC, int R>
+__global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_per_wave) {
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int K = a.K;
+  const uint16_t *W = (const uint16_t *)a.W;
+  const int n_begin = gw * rows_per_wave;
+  if (n_begin >= a.N) return;
+  const int n_end = n_begin + rows_per_wave < a.N ? n_begin + rows_per_wave : a.N;
+
+  u32x4 wv[R][KC];
+  auto load_group = [&](int n_base) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = n_base + r < n_end ? n_base + r : n_end - 1;
+      const uint16_t *wr = W + (int64_t)n * a.ldw + lane * 8;
+#pragma unroll
+      for (int u = 0; u < KC; ++u) {
+        if (lane * 8 + u * 512 < K) wv[r][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wr + u * 512));
+        else wv[r][u] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  };
+  load_group(n_begin);
+
+  // ---- activation vector (optionally normalised over K), packed bf16 in registers
+  u32x4 xv[KC];
+  {
+    const uint16_t *xr = (const uint16_t *)a.A + lane * 8;
+#pragma unroll
+    for (int u = 0; u < KC; ++u)
+      xv[u] = (lane * 8 + u * 512 < K) ? *reinterpret_cast<const u32x4 *>(xr + u * 512) : u32x4{0u, 0u, 0u, 0u};
+    if (a.ln_kind >= 0) {
+      float xf[KC][8];
+      float s = 0.f;
+#pragma unroll
+      for (int u = 0; u < KC; ++u) {
+        const uint32_t w4[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          xf[u][2 * j] = __uint_as_float(w4[j] << 16);
+          xf[u][2 * j + 1] = __uint_as_float(w4[j] & 0xffff0000u);
+          s += a.ln_kind == 0 ? xf[u][2 * j] + xf[u][2 * j + 1]
+                              : xf[u][2 * j] * xf[u][2 * j] + xf[u][2 * j + 1] * xf[u][2 * j + 1];
+        }
+      }
+      s = wave_sum(s);
+      float mean = 0.f, scale;
+      if (a.ln_kind == 0) {
+        mean = s / (float)K;
+        float q = 0.f;
+#pragma unroll
+        for (int u = 0; u < KC; ++u)
+          if (lane * 8 + u * 512 < K) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { float d = xf[u][j] - mean; q += d * d; }
+          }
+        q = wave_sum(q);
+        scale = 1.0f / sqrtf(q / (float)K + a.ln_eps);
+      } else {
+        scale = 1.0f / sqrtf(s / (float)K + a.ln_eps);
+      }
+      const uint16_t *lw = (const uint16_t *)a.ln_w + lane * 8;
+      const uint16_t *lb = a.ln_b ? (const uint16_t *)a.ln_b + lane * 8 : nullptr;
+#pragma unroll
+      for (int u = 0; u < KC; ++u) {
+        if (lane * 8 + u * 512 < K) {
+          const u32x4 wq = *reinterpret_cast<const u32x4 *>(lw + u * 512);
+          const u32x4 bq = lb ? *reinterpret_cast<const u32x4 *>(lb + u * 512) : u32x4{0u, 0u, 0u, 0u};
+          const uint32_t ww[4] = {wq.x, wq.y, wq.z, wq.w}, bb[4] = {bq.x, bq.y, bq.z, bq.w};
+          uint32_t o[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float y0 = (xf[u][2 * j] - mean) * scale, y1 = (xf[u][2 * j + 1] - mean) * scale;
+            float w0 = __uint_as_float(ww[j] << 16), w1 = __uint_as_float(ww[j] & 0xffff0000u);
+            y0 *= a.ln_kind == 2 ? 1.0f + w0 : w0;
+            y1 *= a.ln_kind == 2 ? 1.0f + w1 : w1;
+            y0 += __uint_as_float(bb[j] << 16);
+            y1 += __uint_as_float(bb[j] & 0xffff0000u);
+            // the reference materialises the normalised activations in bf16 too
+            o[j] = (uint32_t)f32_to_bf16_bits(y0) | ((uint32_t)f32_to_bf16_bits(y1) << 16);
+          }
+          xv[u] = u32x4{o[0], o[1], o[2], o[3]};
+        }
+      }
+    }
+  }
+
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+  for (int n_base = n_begin; n_base < n_end; n_base += R) {
+    if (n_base != n_begin) load_group(n_base);
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      acc[r] = 0.f;
+#pragma unroll
+      for (int u = 0; u < KC; ++u) acc[r] = dot8_bf16(wv[r][u], xv[u], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = n_base + r;
+        if (n >= n_end) break;
+        float v = acc[r] + (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
+        if (a.act >= 0 && n >= a.act_from) v = act_eval(a.act, v);
+        if (res) v += bf16_bits_to_f32(res[n]);
+        if (n < a.n_split) ((uint16_t *)a.out1)[n] = f32_to_bf16_bits(v);
+        else ((uint16_t *)a.out2)[n - a.n_split] = f32_to_bf16_bits(v);
+      }
+    }
+  }
+}
+
 // ============================================================ f32 NT tile kernel
 // 64x64 tile, BK=16, 256 threads each computing a 4x4 micro-tile with FMA.
 __global__ void __launch_bounds__(256) k_linear_f32(LinearArgs a) {
@@ -479,12 +603,29 @@ template <int MROWS, int R, int U> static int launch_skinny_cfg(hipStream_t st, 
   return launch_check("linear_bf16_skinny");
 }
 
+template <int KC, int R> static int launch_gemv_reg(hipStream_t st, const LinearArgs &a) {
+  // about 10 waves per CU (the register budget allows 12), all co-resident, each
+  // with a whole number of R-row groups
+  const int target_waves = kNumCU * 10;
+  int rpw = (a.N + target_waves - 1) / target_waves;
+  rpw = ((rpw + R - 1) / R) * R;
+  const int waves = (a.N + rpw - 1) / rpw;
+  hipLaunchKernelGGL((k_gemv_bf16_reg<KC, R>), dim3((waves + 3) / 4), dim3(256), 0, st, a, rpw);
+  return launch_check("gemv_bf16_reg");
+}
+
 int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   RAI_TRY(check_linear_args(a, 2));
   RAI_REQUIRE(a.M <= 8, RAI_ERR_BAD_SHAPE, "linear skinny: M=%d > 8", a.M);
   RAI_REQUIRE((size_t)a.M * a.K * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
-  // About 8 waves per CU, all co-resident, each with the same number of rows.
-  const int target_waves = kNumCU * 8;
+  if (a.M == 1 && a.K <= 4096 && a.N >= 1024) {
+    // activation vector in registers (at most 8 chunks of 16 bytes per lane)
+    if (a.K <= 2048) return launch_gemv_reg<4, 4>(st, a);
+    if (a.K <= 2560) return launch_gemv_reg<5, 4>(st, a);
+    return launch_gemv_reg<8, 2>(st, a);
+  }
+  // About 10 waves per CU, all co-resident, each with the same number of rows.
+  const int target_waves = kNumCU * 10;
   int rpw = (a.N + target_waves - 1) / target_waves;
   if (a.M == 1) {
     if (rpw >= 4) { rpw = (rpw / 4) * 4; return launch_skinny_cfg<1, 4, 5>(st, a, rpw); }
