@@ -61,6 +61,8 @@ struct rai_hip_decoder {
   // activations (sized for max_batch * max_context rows)
   char *x, *x2, *ln, *qkv, *cat, *last, *logits;
   uint32_t *ids, *tokens, *history;
+  char *splitk_ws;        // f32 scratch for prefill GEMMs that split K
+  size_t splitk_ws_bytes;
   DevState *state;
   std::vector<void *> allocs;
   int ctx_len;
@@ -458,6 +460,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
     b.residual = x; b.ldr = H;
     b.out1 = xn; b.ld1 = H;
     b.M = (int)M; b.N = H; b.K = d->KB; b.n_split = H;
+    b.splitk_ws = d->splitk_ws; b.splitk_ws_bytes = d->splitk_ws_bytes;
     RAI_TRY(linear(d, st, b));
     char *tmp = x; x = xn; xn = tmp;
   }
@@ -568,6 +571,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->history = (uint32_t *)tmp;
   if ((st = dalloc(d, sizeof(DevState), &tmp))) return bail(st);
   d->state = (DevState *)tmp;
+  d->splitk_ws_bytes = (size_t)8 * d->max_rows * d->H * sizeof(float);
+  if (d->splitk_ws_bytes > ((size_t)256 << 20)) d->splitk_ws_bytes = (size_t)256 << 20;
+  if ((st = dalloc(d, d->splitk_ws_bytes, &d->splitk_ws))) return bail(st);
 
   if (hipMemset(d->state, 0, sizeof(DevState)) != hipSuccess || hipMemset(d->kcache, 0, kv) != hipSuccess ||
       hipMemset(d->vcache, 0, kv) != hipSuccess)

@@ -34,6 +34,10 @@ struct LinearArgs {
   const void *ln_b;
   float ln_eps;
   int ln_kind;  // -1 none, 0 layernorm, 1 rmsnorm, 2 rmsnorm(1+w)
+  // Optional f32 scratch for splitting K over several blocks when M x N alone
+  // yields too few tiles to fill the GPU (tile kernel only).
+  void *splitk_ws;
+  size_t splitk_ws_bytes;
 };
 inline LinearArgs linear_args_default() {
   LinearArgs a;

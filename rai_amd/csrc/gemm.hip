@@ -1,6 +1,5 @@
 // Dense contractions.
-//   k_linear_bf16_mfma   bf16 x bf16 -> f32 MFMA (v_mfma_f32_32x32x16_bf16), NT layout,
-//                        LDS-staged double-buffered tiles, fused bias/act/residual epilogue.
+//   (the bf16 MFMA tile kernel lives in gemm_mfma.hip)
 //   k_linear_bf16_skinny weight-streaming kernel for M <= 8 rows (decode): each wave
 //                        streams whole weight rows with 16-byte loads; HBM-bound.
 //   k_linear_f32         f32 NT tile kernel (FMA) with the same epilogue.
@@ -12,136 +11,6 @@
 
 namespace rai {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-struct alignas(16) U128 { uint32_t w[4]; };
-
-// ============================================================ bf16 MFMA tile kernel
-// Block tile BM x BN, K step BK; 4 waves in a 2x2 grid, each wave owns a
-// (BM/2) x (BN/2) sub-tile made of 32x32 MFMA tiles.
-template <int BM, int BN, int BK>
-__global__ void __launch_bounds__(256) k_linear_bf16_mfma(LinearArgs a) {
-  constexpr int PITCH = BK + 8;  // +16 bytes: conflict-free ds_read_b128 across 16 lanes
-  constexpr int WM = BM / 2, WN = BN / 2;
-  constexpr int MT = WM / 32, NT = WN / 32;
-  constexpr int CPR = BK / 8;                  // 16-byte chunks per tile row
-  constexpr int A_CHUNKS = BM * CPR / 256;     // per thread
-  constexpr int B_CHUNKS = BN * CPR / 256;
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  uint16_t *As = lds;                          // [2][BM][PITCH]
-  uint16_t *Bs = lds + 2 * BM * PITCH;         // [2][BN][PITCH]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  // Tiles that share a weight column block are adjacent in launch order so the
-  // (few) M tiles of one N block hit the same L2.
-  const int tiles_m = (a.M + BM - 1) / BM;
-  const int tile_n = blockIdx.x / tiles_m, tile_m = blockIdx.x % tiles_m;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const uint16_t *A = (const uint16_t *)a.A;
-  const uint16_t *W = (const uint16_t *)a.W;
-
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  U128 ra[A_CHUNKS], rb[B_CHUNKS];
-  const int KT = (a.K + BK - 1) / BK;
-
-  auto g_load = [&](int kt) {
-    const int k0 = kt * BK;
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      int c = tid + i * 256;
-      int row = c / CPR, kc = (c % CPR) * 8;
-      int m = m0 + row, k = k0 + kc;
-      U128 v = {{0u, 0u, 0u, 0u}};
-      if (m < a.M && k < a.K) v = *reinterpret_cast<const U128 *>(A + (int64_t)m * a.lda + k);
-      ra[i] = v;
-    }
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      int c = tid + i * 256;
-      int row = c / CPR, kc = (c % CPR) * 8;
-      int n = n0 + row, k = k0 + kc;
-      U128 v = {{0u, 0u, 0u, 0u}};
-      if (n < a.N && k < a.K) v = *reinterpret_cast<const U128 *>(W + (int64_t)n * a.ldw + k);
-      rb[i] = v;
-    }
-  };
-  auto s_store = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      int c = tid + i * 256;
-      int row = c / CPR, kc = (c % CPR) * 8;
-      *reinterpret_cast<U128 *>(As + (buf * BM + row) * PITCH + kc) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      int c = tid + i * 256;
-      int row = c / CPR, kc = (c % CPR) * 8;
-      *reinterpret_cast<U128 *>(Bs + (buf * BN + row) * PITCH + kc) = rb[i];
-    }
-  };
-
-  g_load(0);
-  s_store(0);
-  __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) g_load(kt + 1);
-    const uint16_t *as = As + (buf * BM + wm * WM + (lane & 31)) * PITCH + (lane >> 5) * 8;
-    const uint16_t *bs = Bs + (buf * BN + wn * WN + (lane & 31)) * PITCH + (lane >> 5) * 8;
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8 fa[MT], fb[NT];
-#pragma unroll
-      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + ks * 16);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + ks * 16);
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < KT) s_store(buf ^ 1);
-    __syncthreads();
-  }
-
-  // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
-  const uint16_t *bias = (const uint16_t *)a.bias;
-  const uint16_t *bias2 = (const uint16_t *)a.bias2;
-  const uint16_t *res = (const uint16_t *)a.residual;
-#pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const int n = n0 + wn * WN + j * 32 + (lane & 31);
-    if (n >= a.N) continue;
-    const float bv = (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
-    const bool do_act = a.act >= 0 && n >= a.act_from;
-    uint16_t *dst;
-    int64_t ld;
-    int col;
-    if (n < a.n_split) { dst = (uint16_t *)a.out1; ld = a.ld1; col = n; }
-    else { dst = (uint16_t *)a.out2; ld = a.ld2; col = n - a.n_split; }
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m >= a.M) continue;
-        float v = acc[i][j][r] + bv;
-        if (do_act) v = act_eval(a.act, v);
-        if (res) v += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
-        dst[(int64_t)m * ld + col] = f32_to_bf16_bits(v);
-      }
-    }
-  }
-}
 
 // ============================================================ bf16 skinny (decode) kernel
 // M <= MROWS rows of A.  Each wave owns R consecutive weight rows at a time and
@@ -556,19 +425,6 @@ __global__ void __launch_bounds__(256) k_matmul_generic(T *out, const T *A, cons
 }
 
 // ============================================================ launchers
-template <int BM, int BN, int BK> static int launch_mfma_cfg(hipStream_t st, const LinearArgs &a) {
-  constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(uint16_t);
-  static bool attr_set = false;
-  if (lds > 64 * 1024 && !attr_set) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma<BM, BN, BK>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
-  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  hipLaunchKernelGGL((k_linear_bf16_mfma<BM, BN, BK>), dim3(tiles), dim3(256), lds, st, a);
-  return launch_check("linear_bf16_mfma");
-}
-
 static int check_linear_args(const LinearArgs &a, size_t es) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
   RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
@@ -580,13 +436,6 @@ static int check_linear_args(const LinearArgs &a, size_t es) {
   RAI_REQUIRE((uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0, RAI_ERR_BAD_STRIDE,
               "linear: operands must be 16-byte aligned");
   return RAI_OK;
-}
-
-int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
-  RAI_TRY(check_linear_args(a, 2));
-  RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear: fused norm only on the skinny path");
-  if (a.M <= 64) return launch_mfma_cfg<64, 128, 64>(st, a);
-  return launch_mfma_cfg<128, 128, 64>(st, a);
 }
 
 template <int MROWS, int R, int U> static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a, int rows_per_wave) {
@@ -658,6 +507,18 @@ int launch_linear_f32(hipStream_t st, const LinearArgs &a) {
   return launch_check("linear_f32");
 }
 
+// Lends the device's scratch block to a tile GEMM that may split K.
+static int splitk_workspace(int dev, LinearArgs *la) {
+  const size_t want = (size_t)8 * la->M * la->N * sizeof(float);
+  const size_t cap = (size_t)256 << 20;
+  const size_t bytes = want < cap ? want : cap;
+  void *ws = nullptr;
+  RAI_TRY(workspace(dev, bytes, &ws));
+  la->splitk_ws = ws;
+  la->splitk_ws_bytes = bytes;
+  return RAI_OK;
+}
+
 }  // namespace rai
 
 using namespace rai;
@@ -721,10 +582,13 @@ int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, co
       la.N = (int)N;
       la.K = (int)K;
       la.n_split = (int)N;
+      if (a->dtype == RAI_BF16 && la.M > 8 && la.K % 32 != 0) goto generic;
+      if (a->dtype == RAI_BF16 && la.M > 8) RAI_TRY(splitk_workspace(dev, &la));
       return a->dtype == RAI_BF16 ? launch_linear_bf16(st, la) : launch_linear_f32(st, la);
     }
   }
 
+generic:
   MatmulArgs g;
   g.M = M; g.N = N; g.K = K;
   g.a_rs = a->stride[r - 2]; g.a_cs = a->stride[r - 1];
@@ -801,6 +665,10 @@ int rai_hip_linear(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, co
   la.act_from = 0;
   hipStream_t st = stream_of(dev);
   if (!st) return RAI_ERR_HIP;
+  if (x->dtype == RAI_BF16 && la.M > 8) {
+    RAI_REQUIRE(K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear: bf16 with M > 8 needs K %% 32 == 0 (K=%lld)", (long long)K);
+    RAI_TRY(splitk_workspace(dev, &la));
+  }
   return x->dtype == RAI_BF16 ? launch_linear_bf16(st, la) : launch_linear_f32(st, la);
 }
 

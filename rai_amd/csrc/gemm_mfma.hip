@@ -1,0 +1,270 @@
+// bf16 x bf16 -> f32 MFMA GEMM for the Linear layout (out = A[M,K] . W[N,K]^T),
+// gfx950 v_mfma_f32_32x32x16_bf16.
+//
+//   - block tile BM x BN, 4 waves in a 2x2 grid, each wave (BM/2) x (BN/2) made of
+//     32x32 MFMA tiles; K step BK.
+//   - global -> registers -> LDS with a two-deep LDS buffer: the loads of tile
+//     k+1 are in flight while tile k is multiplied; one barrier per K step.
+//     Rows are clamped instead of predicated, so the main loop has no branches.
+//   - LDS rows are padded by 16 bytes: the 16-byte fragment reads of 16 lanes hit
+//     64 distinct banks.
+//   - blockIdx -> tile mapping is XCD-aware: hardware hands consecutive blocks to
+//     the 8 XCDs round-robin, so each XCD is given a contiguous run of tiles and
+//     the tiles that share a weight panel share one L2.
+//   - epilogue through LDS: every wave stages 32 x (BN/2) accumulators at a time
+//     and writes 16-byte rows with bias / activation / residual applied (or raw
+//     f32 partial sums when K is split over several blocks).
+#include "gemm.h"
+
+namespace rai {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kXcds = 8;
+
+__device__ __forceinline__ int xcd_remap(int bid, int total) {
+  // blocks bid, bid+8, bid+16, ... run on the same XCD; give them consecutive tiles
+  const int per = (total + kXcds - 1) / kXcds;
+  return (bid % kXcds) * per + bid / kXcds;
+}
+
+template <int BM, int BN, int BK>
+__global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits, int k_per_split, float *partial) {
+  constexpr int PITCH = BK + 8;
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int MT = WM / 32, NT = WN / 32;
+  constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
+  constexpr int A_CH = BM * CPR / 256;      // chunks per thread
+  constexpr int B_CH = BN * CPR / 256;
+  constexpr int EP = WN + 4;                // epilogue staging pitch (floats)
+  static_assert(A_CH >= 1 && B_CH >= 1, "tile too small for 256 threads");
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  uint16_t *As = lds;                       // [2][BM][PITCH]
+  uint16_t *Bs = lds + 2 * BM * PITCH;      // [2][BN][PITCH]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int tile = xcd_remap(blockIdx.x, total);
+  if (tile >= total) return;
+  const int tile_n = tile / tiles_m, tile_m = tile % tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int split = blockIdx.y;
+  const int k_begin = split * k_per_split;
+  const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
+  const int KT = (k_end - k_begin) / BK;
+
+  // per-thread source pointers (rows clamped into range; results of clamped rows are never stored)
+  const uint16_t *ga[A_CH], *gb[B_CH];
+  int sa[A_CH], sb[B_CH];
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) {
+    const int c = tid + i * 256, row = c / CPR, kc = (c % CPR) * 8;
+    int m = m0 + row;
+    m = m < a.M ? m : a.M - 1;
+    ga[i] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + kc;
+    sa[i] = row * PITCH + kc;
+  }
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) {
+    const int c = tid + i * 256, row = c / CPR, kc = (c % CPR) * 8;
+    int n = n0 + row;
+    n = n < a.N ? n : a.N - 1;
+    gb[i] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + kc;
+    sb[i] = row * PITCH + kc;
+  }
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  u32x4 ra[A_CH], rb[B_CH];
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(ga[i]);
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(gb[i]);
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4 *>(As + sa[i]) = ra[i];
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u32x4 *>(Bs + sb[i]) = rb[i];
+  __syncthreads();
+
+  const int frag = (lane & 31) * PITCH + (lane >> 5) * 8;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    const bool more = kt + 1 < KT;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(ga[i] + (kt + 1) * BK);
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(gb[i] + (kt + 1) * BK);
+    }
+    const uint16_t *as = As + buf * BM * PITCH + wm * WM * PITCH + frag;
+    const uint16_t *bs = Bs + buf * BN * PITCH + wn * WN * PITCH + frag;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 fa[MT], fb[NT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + ks * 16);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + ks * 16);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      uint16_t *ad = As + (buf ^ 1) * BM * PITCH, *bd = Bs + (buf ^ 1) * BN * PITCH;
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4 *>(ad + sa[i]) = ra[i];
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u32x4 *>(bd + sb[i]) = rb[i];
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: stage 32 x WN accumulators per wave in LDS, write 8 columns per lane
+  float *stage = reinterpret_cast<float *>(lds) + wave * 32 * EP;
+  static_assert(4 * 32 * EP * 4 <= 2 * (BM + BN) * PITCH * 2, "epilogue staging does not fit the tile buffers");
+  constexpr int CG = WN / 8;                 // 8-column groups per staged row
+  constexpr int ITEMS = 32 * CG / 64;        // per lane
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+  const bool vec_out = (a.ld1 % 8 == 0) && (a.n_split % 8 == 0) && (a.n_split == a.N || a.ld2 % 8 == 0) &&
+                       ((uintptr_t)a.out1 % 16 == 0) && (a.n_split == a.N || (uintptr_t)a.out2 % 16 == 0) &&
+                       (!res || (a.ldr % 8 == 0 && (uintptr_t)res % 16 == 0)) && a.N % 8 == 0;
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    // accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32]
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+    // LDS operations of one wave complete in order; no block barrier is needed for a wave-private region
+#pragma unroll 1
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = lane + it * 64;
+      const int row = item / CG, cg = item % CG;
+      const int m = m0 + wm * WM + i * 32 + row;
+      const int n = n0 + wn * WN + cg * 8;
+      if (m >= a.M || n >= a.N) continue;
+      const f32x4 v0 = *reinterpret_cast<const f32x4 *>(stage + row * EP + cg * 8);
+      const f32x4 v1 = *reinterpret_cast<const f32x4 *>(stage + row * EP + cg * 8 + 4);
+      float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      if (partial) {
+        float *p = partial + ((int64_t)split * a.M + m) * a.N + n;
+        if (a.N % 4 == 0) {
+          *reinterpret_cast<f32x4 *>(p) = v0;
+          if (n + 4 < a.N) *reinterpret_cast<f32x4 *>(p + 4) = v1;
+        } else {
+          for (int e = 0; e < 8 && n + e < a.N; ++e) p[e] = v[e];
+        }
+        continue;
+      }
+      const int lim = a.N - n < 8 ? a.N - n : 8;
+      for (int e = 0; e < lim; ++e) {
+        const int nn = n + e;
+        float x = v[e] + (bias ? bf16_bits_to_f32(bias[nn]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[nn]) : 0.f);
+        if (a.act >= 0 && nn >= a.act_from) x = act_eval(a.act, x);
+        if (res) x += bf16_bits_to_f32(res[(int64_t)m * a.ldr + nn]);
+        v[e] = x;
+      }
+      if (vec_out) {
+        u32x4 o;
+        o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+        o.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+        o.z = (uint32_t)f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
+        o.w = (uint32_t)f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
+        uint16_t *dst = n < a.n_split ? (uint16_t *)a.out1 + (int64_t)m * a.ld1 + n
+                                      : (uint16_t *)a.out2 + (int64_t)m * a.ld2 + (n - a.n_split);
+        *reinterpret_cast<u32x4 *>(dst) = o;
+      } else {
+        for (int e = 0; e < lim; ++e) {
+          const int nn = n + e;
+          if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = f32_to_bf16_bits(v[e]);
+          else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = f32_to_bf16_bits(v[e]);
+        }
+      }
+    }
+  }
+}
+
+// Sums the per-split partial products and applies the Linear epilogue.
+__global__ void __launch_bounds__(256) k_splitk_epilogue(LinearArgs a, int splits, const float *partial) {
+  const int64_t total = (int64_t)a.M * a.N;
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+  for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
+    const int m = (int)(e / a.N), n = (int)(e % a.N);
+    float x = 0.f;
+    for (int s = 0; s < splits; ++s) x += partial[(int64_t)s * total + e];
+    x += (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
+    if (a.act >= 0 && n >= a.act_from) x = act_eval(a.act, x);
+    if (res) x += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
+    if (n < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + n] = f32_to_bf16_bits(x);
+    else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (n - a.n_split)] = f32_to_bf16_bits(x);
+  }
+}
+
+template <int BM, int BN, int BK> static int launch_cfg(hipStream_t st, const LinearArgs &a, int splits) {
+  constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(uint16_t);
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma<BM, BN, BK>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  const int grid_x = ((tiles + kXcds - 1) / kXcds) * kXcds;  // whole rounds over the XCDs
+  int k_per_split = a.K;
+  float *partial = nullptr;
+  if (splits > 1) {
+    const int k_tiles = a.K / BK, per = (k_tiles + splits - 1) / splits;
+    splits = (k_tiles + per - 1) / per;  // every split gets at least one K tile
+    k_per_split = per * BK;
+    partial = (float *)a.splitk_ws;
+  }
+  hipLaunchKernelGGL((k_gemm_bf16_mfma<BM, BN, BK>), dim3(grid_x, splits), dim3(256), lds, st, a, splits, k_per_split,
+                     partial);
+  RAI_TRY(launch_check("gemm_bf16_mfma"));
+  if (splits > 1) {
+    int64_t total = (int64_t)a.M * a.N;
+    int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);
+    RAI_TRY(launch_check("splitk_epilogue"));
+  }
+  return RAI_OK;
+}
+
+int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
+  RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
+  RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
+  RAI_REQUIRE(a.n_split >= 0 && a.n_split <= a.N && (a.n_split == a.N || a.out2), RAI_ERR_BAD_ARG,
+              "linear: bad output split");
+  RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear: fused norm only on the skinny path");
+  RAI_REQUIRE(a.K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear mfma: K=%d must be a multiple of 32", a.K);
+  RAI_REQUIRE(a.lda % 8 == 0 && a.ldw % 8 == 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0,
+              RAI_ERR_BAD_STRIDE, "linear mfma: operands must be 16-byte aligned with row strides multiple of 8");
+  // Split K when the tile count alone cannot fill the GPU and a workspace was provided.
+  const int tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
+  int splits = 1;
+  if (a.splitk_ws && tiles < kNumCU) {
+    while (splits < 8 && tiles * splits * 2 <= 2 * kNumCU && a.K / (splits * 2) >= 512) splits *= 2;
+    while (splits > 1 && (size_t)splits * a.M * a.N * sizeof(float) > a.splitk_ws_bytes) splits /= 2;
+  }
+  return launch_cfg<128, 128, 32>(st, a, splits);
+}
+
+}  // namespace rai
