@@ -336,11 +336,196 @@ template <typename T> static int launch_row(hipStream_t st, const AttnArgs &a) {
   return launch_check("attention_row");
 }
 
+// ============================================================ prefill: flash attention on MFMA (bf16)
+// Block = NW waves, each owning 32 query rows; keys/values are streamed in
+// tiles of 64 through LDS and shared by the waves.  Both products run on
+// v_mfma_f32_32x32x16_bf16 in the transposed orientation
+//     S^T = K . Q^T        (rows = keys, columns = queries)
+//     O^T = V^T . P^T      (rows = head features, columns = queries)
+// so every lane owns one query column: the online-softmax statistics are
+// per-lane scalars, and the accumulator registers of S^T are, in order, exactly
+// the B-operand fragments of the second product (no cross-lane movement).
+// V is transposed while it is staged into LDS.  The score matrix never exists
+// in memory (the reference materialises [B,H,S,T]).
+typedef __attribute__((ext_vector_type(8))) __bf16 fa_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float fa_f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t fa_u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t fa_u32x2;
+
+template <int NW, int D>
+__global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
+  constexpr int KS = D / 16;            // K steps of the score product
+  constexpr int DT = (D + 31) / 32;     // 32-row tiles of O^T
+  constexpr int KP = D + 8;             // K tile pitch (elements)
+  constexpr int VP = 64 + 4;            // V^T tile pitch (elements)
+  constexpr int NT = NW * 64;
+  constexpr int CPR = D / 8;            // 16-byte chunks per key row
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[64 * KP];
+  __shared__ __attribute__((aligned(16))) uint16_t Vt[DT * 32 * VP];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / (a.Hq / a.Hkv);
+  const int q0 = blockIdx.x * (NW * 32);
+  const int off = a.T - a.S;  // absolute position of query row 0
+  const uint16_t *Kg = (const uint16_t *)a.k + b * a.ks[0] + hk * a.ks[1];
+  const uint16_t *Vg = (const uint16_t *)a.v + b * a.vs[0] + hk * a.vs[1];
+
+  const int qrow = q0 + wave * 32 + l32;
+  const int qrow_c = qrow < a.S ? qrow : a.S - 1;
+  const uint16_t *qp = (const uint16_t *)a.q + b * a.qs[0] + h * a.qs[1] + (int64_t)qrow_c * a.qs[2] + half * 8;
+  fa_bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const fa_bf16x8 *>(qp + ks * 16);
+
+  fa_f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  int kv_end = a.T;
+  if (a.causal) {
+    int last_q = q0 + NW * 32 < a.S ? q0 + NW * 32 : a.S;
+    kv_end = off + last_q < a.T ? off + last_q : a.T;
+  }
+  const int wave_last_key = a.causal ? off + q0 + wave * 32 + 31 : a.T - 1;  // newest key any row of this wave may see
+  const float scale_r = round_to<bf16_raw>(a.scale);
+
+  for (int k0 = 0; k0 < kv_end; k0 += 64) {
+    __syncthreads();
+    // ---- stage K [64][D] and V^T [D][64]; rows past the context re-read its last row (masked below)
+    for (int c = tid; c < 64 * CPR; c += NT) {
+      const int key = c / CPR, dc = (c % CPR) * 8;
+      int t = k0 + key;
+      t = t < a.T ? t : a.T - 1;
+      const fa_u32x4 kv = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
+      *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kv;
+      const fa_u32x4 vv = *reinterpret_cast<const fa_u32x4 *>(Vg + (int64_t)t * a.vs[2] + dc);
+      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        Vt[(dc + 2 * e) * VP + key] = (uint16_t)(w[e] & 0xffffu);
+        Vt[(dc + 2 * e + 1) * VP + key] = (uint16_t)(w[e] >> 16);
+      }
+    }
+    __syncthreads();
+    if (k0 > wave_last_key) continue;  // every key of this tile is masked for this wave (barriers stay uniform)
+
+    // ---- S^T tile: 64 keys x 32 queries
+    fa_f32x16 sc[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[u][r] = 0.f;
+      const uint16_t *kr = Ks + (u * 32 + l32) * KP + half * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const fa_bf16x8 *>(kr + ks * 16), qf[ks], sc[u],
+                                                        0, 0, 0);
+    }
+    // ---- scale, mask, online softmax (register r of sub-tile u is key k0 + 32u + 8*(r/4) + 4*half + r%4)
+    const int q_abs = off + qrow;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + u * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        float v = a.f32_scores ? sc[u][r] * a.scale : round_to<bf16_raw>(round_to<bf16_raw>(sc[u][r]) * scale_r);
+        if (key >= a.T || (a.causal && key > q_abs)) v = -INFINITY;
+        sc[u][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // fully masked so far: every p is exp(-inf) = 0
+    const float alpha = __expf(m_run - m_safe);
+    float psum = 0.f;
+    fa_bf16x8 pf[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __expf(sc[u][r] - m_safe);
+        psum += p;
+        pf[u][r >> 3][r & 7] = (__bf16)p;
+      }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const uint16_t *vr = Vt + (dt * 32 + l32) * VP + 4 * half;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const fa_u32x2 lo = *reinterpret_cast<const fa_u32x2 *>(vr + u * 32 + 16 * s2);
+          const fa_u32x2 hi = *reinterpret_cast<const fa_u32x2 *>(vr + u * 32 + 16 * s2 + 8);
+          const fa_u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(fa_bf16x8, va), pf[u][s2], o[dt], 0, 0, 0);
+        }
+    }
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if (qrow < a.S) {
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    uint16_t *op = (uint16_t *)a.out + ((int64_t)b * a.S + qrow) * a.out_row_stride + (int64_t)h * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = dt * 32 + 8 * g + 4 * half;
+        if (d < D) {
+          fa_u32x2 w;
+          w.x = (uint32_t)f32_to_bf16_bits(o[dt][4 * g] * inv) | ((uint32_t)f32_to_bf16_bits(o[dt][4 * g + 1] * inv) << 16);
+          w.y = (uint32_t)f32_to_bf16_bits(o[dt][4 * g + 2] * inv) | ((uint32_t)f32_to_bf16_bits(o[dt][4 * g + 3] * inv) << 16);
+          *reinterpret_cast<fa_u32x2 *>(op + d) = w;
+        }
+      }
+  }
+}
+
+template <int D> static int launch_flash(hipStream_t st, const AttnArgs &a) {
+  const int tiles4 = (a.S + 127) / 128;
+  if ((int64_t)tiles4 * a.Hq * a.B >= kNumCU) {
+    hipLaunchKernelGGL((k_flash_prefill_bf16<4, D>), dim3(tiles4, a.Hq, a.B), dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((k_flash_prefill_bf16<2, D>), dim3((a.S + 63) / 64, a.Hq, a.B), dim3(128), 0, st, a);
+  }
+  return launch_check("flash_prefill");
+}
+
+static bool flash_eligible(const AttnArgs &a) {
+  if (a.dtype != RAI_BF16 || a.S < 16 || a.t_dev) return false;
+  if (a.D != 64 && a.D != 80 && a.D != 128 && a.D != 256) return false;
+  auto al = [](const void *p, const int64_t *s) {
+    return (uintptr_t)p % 16 == 0 && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0;
+  };
+  return al(a.q, a.qs) && al(a.k, a.ks) && al(a.v, a.vs) && (uintptr_t)a.out % 8 == 0 && a.out_row_stride % 4 == 0 &&
+         a.Hq <= 65535 && a.B <= 65535;
+}
+
 int launch_attention(hipStream_t st, const AttnArgs &a) {
   RAI_REQUIRE(a.B > 0 && a.Hq > 0 && a.Hkv > 0 && a.S > 0 && a.T > 0 && a.D > 0, RAI_ERR_BAD_SHAPE,
               "attention: empty problem");
   RAI_REQUIRE(a.Hq % a.Hkv == 0, RAI_ERR_BAD_SHAPE, "attention: %d query heads not divisible by %d kv heads", a.Hq,
               a.Hkv);
+  if (flash_eligible(a)) {
+    switch (a.D) {
+      case 64: return launch_flash<64>(st, a);
+      case 80: return launch_flash<80>(st, a);
+      case 128: return launch_flash<128>(st, a);
+      default: return launch_flash<256>(st, a);
+    }
+  }
   switch (a.dtype) {
     case RAI_F32: return launch_row<float>(st, a);
     case RAI_BF16: return launch_row<bf16_raw>(st, a);

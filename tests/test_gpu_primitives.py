@@ -429,7 +429,10 @@ def test_rope_matches_phi2_reference_chain(R, dt):
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("hq,hkv,s,t,d,causal,f32s", [(4, 4, 16, 16, 80, 1, 1), (4, 4, 1, 37, 80, 0, 1),
-                                                     (6, 2, 9, 20, 128, 1, 0), (8, 1, 1, 50, 256, 0, 0)])
+                                                     (6, 2, 9, 20, 128, 1, 0), (8, 1, 1, 50, 256, 0, 0),
+                                                     (4, 4, 200, 200, 80, 1, 1), (3, 3, 70, 333, 80, 1, 1),
+                                                     (6, 2, 129, 129, 128, 1, 0), (4, 1, 65, 100, 256, 1, 0),
+                                                     (2, 2, 100, 160, 64, 0, 1), (40, 40, 130, 130, 80, 1, 1)])
 def test_attention(R, dt, hq, hkv, s, t, d, causal, f32s):
     import math
     g = rng(28)
