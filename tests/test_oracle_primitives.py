@@ -1,0 +1,250 @@
+"""Pins the CPU oracle (oracle/ops.py, oracle/nn.py) before it is trusted as the
+checker of the HIP path.  Nothing here re-types an oracle formula: every check
+is a known answer readable from the reference's own tests, a brute-force loop on
+tiny inputs, a mathematical invariant, or an independent library routine
+(torch CPU, scipy)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import nn as onn
+from oracle import ops as oo
+from oracle.dtypes import bf16_bits_to_f32, f32_to_bf16_bits, rnd
+
+
+def rng(seed=0):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+# ------------------------------------------------------------------ dtype rounding
+def test_bf16_rounding_equals_torch_and_is_nearest_even():
+    x = rng(1).standard_normal(100000).astype(np.float32) * np.float32(37.0)
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(rnd(x, "bf16"), want)
+    bits = np.array([0x3F808000, 0x3F818000, 0x3F80FFFF, 0x7F7FFFFF, 0xBF808000, 0x00000001], np.uint32)
+    assert list(f32_to_bf16_bits(bits.view(np.float32))) == [0x3F80, 0x3F82, 0x3F81, 0x7F80, 0xBF80, 0x0000]
+    assert np.isnan(bf16_bits_to_f32(f32_to_bf16_bits(np.array([np.nan], np.float32))))[0]
+    h = rng(2).standard_normal(1000).astype(np.float32)
+    assert np.array_equal(rnd(h, "f16"), torch.from_numpy(h).half().float().numpy())
+
+
+def test_to_dtype_float_to_int_follows_rust_as():
+    x = np.array([0.5, -0.5, 255.7, 300.0, -3.9, np.nan, np.inf, -np.inf, 1e20], np.float32)
+    assert list(oo.to_dtype(x, "f32", "u8")) == [0, 0, 255, 255, 0, 0, 255, 0, 255]
+    assert list(oo.to_dtype(x, "f32", "u32")) == [0, 0, 255, 300, 0, 0, 4294967295, 0, 4294967295]
+    got = oo.to_dtype(x, "f32", "i64")
+    assert list(got[:5]) == [0, 0, 255, 300, -3] and got[5] == 0 and got[6] == np.iinfo(np.int64).max
+    assert got[7] == np.iinfo(np.int64).min and got[8] == np.iinfo(np.int64).max
+    assert np.array_equal(oo.to_dtype(np.array([0, 255, 256, 70000], np.uint32), "u32", "u8"), [0, 255, 0, 112])
+
+
+# ------------------------------------------------------------------ reference known answers
+def test_reference_known_answers():
+    # rai-core/tests/ops.rs:80-91 ones[2,3] @ ones[3,2] == 3 ; tests/eval.rs:4-12 ; tests/eval.rs:30-47
+    assert np.array_equal(oo.matmul(np.ones((2, 3)), np.ones((3, 2)), "f32"), np.full((2, 2), 3.0))
+    z = oo.add(oo.add(np.ones((2, 3)), np.ones((2, 3)), "f32"), np.ones(3), "f32")
+    assert np.array_equal(z, np.full((2, 3), 3.0))
+    f = lambda v: oo.full(v, (2, 2), "f32")
+    z = oo.sub(oo.add(oo.div(f(1), f(2), "f32"), oo.mul(f(2), f(3), "f32"), "f32"), oo.add(f(3.1), f(3.2), "f32"), "f32")
+    assert np.allclose(z, 0.2, atol=1e-6)
+    # rai-core/tests/ops.rs:167-175
+    t = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    assert np.array_equal(oo.index_select(t, 0, np.array([1, 1, 0, 0], np.uint32)), t[[1, 1, 0, 0]])
+    # rai-core/tests/ops.rs:19-29
+    assert np.array_equal(oo.arange(10.0, 20.0, 2.0, "f32"), [10, 12, 14, 16, 18])
+    assert np.array_equal(oo.arange(0, 10, 3, "u8"), np.array([0, 3, 6, 9], np.uint8))
+
+
+# ------------------------------------------------------------------ brute force
+def test_index_select_brute_force_and_errors():
+    g = rng(3)
+    x = g.standard_normal((4, 5, 6)).astype(np.float32)
+    for dim in range(3):
+        idx = g.integers(0, x.shape[dim], 7)
+        got = oo.index_select(x, dim, idx.astype(np.uint32))
+        for p, i in enumerate(idx):
+            sl = [slice(None)] * 3
+            sl[dim] = p
+            src = [slice(None)] * 3
+            src[dim] = i
+            assert np.array_equal(got[tuple(sl)], x[tuple(src)])
+    with pytest.raises(IndexError):
+        oo.index_select(x, 0, np.array([4], np.uint32))
+
+
+def test_argmax_sequential_scan_semantics():
+    g = rng(4)
+    x = np.round(g.standard_normal((6, 50)) * 2).astype(np.float32)   # many ties
+
+    def scan(row, better):
+        best, bi = row[0], 0
+        for i in range(1, len(row)):
+            if better(row[i], best):
+                best, bi = row[i], i
+        return bi
+
+    assert list(oo.argmax(x, 1)) == [scan(r, lambda a, b: a > b) for r in x]
+    assert list(oo.argmin(x, 1)) == [scan(r, lambda a, b: a < b) for r in x]
+    assert oo.argmax(x, 1).dtype == np.uint32 and oo.argmax(x, 1, True).shape == (6, 1)
+    assert list(oo.argmax(x, 0)) == [scan(c, lambda a, b: a > b) for c in x.T]
+    y = np.array([[0, np.nan, 1, 1], [np.nan, 5, 1, 1], [-np.inf, -np.inf, -np.inf, -np.inf], [-0.0, 0.0, 0.0, -0.0]],
+                 np.float32)
+    assert list(oo.argmax(y, 1)) == [scan(r, lambda a, b: a > b) for r in y] == [2, 0, 0, 0]
+
+
+def test_matmul_triple_loop_and_batch_broadcast():
+    g = rng(5)
+    a, b = g.standard_normal((3, 4, 5)), g.standard_normal((1, 5, 2))
+    want = np.zeros((3, 4, 2))
+    for n in range(3):
+        for i in range(4):
+            for j in range(2):
+                for k in range(5):
+                    want[n, i, j] += a[n, i, k] * b[0, k, j]
+    assert np.allclose(oo.matmul(a, b, "f64"), want, rtol=1e-12)
+    assert np.allclose(oo.matmul(a, b, "f32"), want, rtol=1e-5)
+    # bf16: product of the rounded inputs, one rounding of the f32 result
+    ab, bb = rnd(a.astype(np.float32), "bf16"), rnd(b.astype(np.float32), "bf16")
+    exact = np.matmul(ab.astype(np.float64), bb.astype(np.float64))
+    got = oo.matmul(ab, bb, "bf16")
+    assert np.max(np.abs(got - exact)) <= 2 ** -8 * np.max(np.abs(exact)) * 1.01
+    assert np.array_equal(got, rnd(got, "bf16"))
+
+
+# ------------------------------------------------------------------ library routines / invariants
+@pytest.mark.parametrize("dt,tol", [("f32", 2e-6), ("f64", 1e-12)])
+def test_elementwise_against_torch(dt, tol):
+    g = rng(6)
+    tdt = torch.float32 if dt == "f32" else torch.float64
+    x = g.standard_normal((7, 33)).astype(np.float32 if dt == "f32" else np.float64)
+    t = torch.from_numpy(x)
+    pos = np.abs(x) + 0.1
+    tp = torch.from_numpy(pos)
+    pairs = [(oo.sin(x, dt), torch.sin(t)), (oo.cos(x, dt), torch.cos(t)), (oo.exp(x, dt), torch.exp(t)),
+             (oo.tanh(x, dt), torch.tanh(t)), (oo.erf(x, dt), torch.erf(t)), (oo.log(pos, dt), torch.log(tp)),
+             (oo.sqrt(pos, dt), torch.sqrt(tp)), (oo.rsqrt(pos, dt), torch.rsqrt(tp)), (oo.square(x, dt), t * t),
+             (oo.powf(pos, 3.0, dt), tp ** 3), (oo.log2(pos, dt), torch.log2(tp)), (oo.log10(pos, dt), torch.log10(tp)),
+             (oo.abs_(x, dt), torch.abs(t)), (oo.neg(x, dt), -t), (oo.sign(x, dt), torch.sign(t))]
+    for got, want in pairs:
+        assert np.allclose(got, want.to(tdt).numpy(), rtol=tol * 10, atol=tol)
+    y = g.standard_normal((33,)).astype(x.dtype)
+    ty = torch.from_numpy(y)
+    for got, want in [(oo.add(x, y, dt), t + ty), (oo.sub(x, y, dt), t - ty), (oo.mul(x, y, dt), t * ty),
+                      (oo.div(x, np.abs(y) + 1, dt), t / (ty.abs() + 1)), (oo.maximum(x, y, dt), torch.maximum(t, ty)),
+                      (oo.minimum(x, y, dt), torch.minimum(t, ty))]:
+        assert np.allclose(got, want.numpy(), rtol=tol, atol=tol)
+    assert np.array_equal(oo.gt(x, y, dt), (t > ty).numpy().astype(np.uint8))
+    assert np.array_equal(oo.where(oo.gt(x, y, dt), x, np.broadcast_to(y, x.shape), dt), torch.where(t > ty, t, ty).numpy())
+
+
+def test_softmax_invariants_and_torch():
+    g = rng(7)
+    x = (g.standard_normal((5, 9, 200)) * 3).astype(np.float32)
+    for dim in (0, 1, -1):
+        s = oo.softmax(x, dim, "f32")
+        assert np.allclose(s.sum(dim), 1.0, atol=1e-5)
+        assert np.allclose(s, torch.softmax(torch.from_numpy(x), dim).numpy(), atol=1e-6)
+        assert np.allclose(oo.softmax(x + 100.0, dim, "f32"), s, atol=2e-5)               # shift invariance
+        assert np.allclose(oo.log_softmax(x, dim, "f32"), torch.log_softmax(torch.from_numpy(x), dim).numpy(), atol=1e-5)
+    assert np.allclose(oo.softmax(np.full((3, 8), 2.5, np.float32), -1, "f32"), 1 / 8)
+    big = np.array([[1e4, 1e4 - 1, -1e4]], np.float32)
+    assert np.allclose(oo.softmax(big, -1, "f32"), [[1 / (1 + math.exp(-1)), math.exp(-1) / (1 + math.exp(-1)), 0]], atol=1e-6)
+    # bf16: every one of the five steps rounds, result stays within bf16 resolution of the f32 softmax
+    xb = rnd(x, "bf16")
+    sb = oo.softmax(xb, -1, "bf16")
+    assert np.array_equal(sb, rnd(sb, "bf16"))
+    assert np.max(np.abs(sb - torch.softmax(torch.from_numpy(xb), -1).numpy())) < 2 ** -7
+
+
+def test_reductions_against_numpy_float64():
+    g = rng(8)
+    x = g.standard_normal((4, 30, 50)).astype(np.float32)
+    for dims in [(0,), (1,), (2,), (0, 2), None]:
+        for keep in (False, True):
+            want = x.astype(np.float64).sum(axis=dims, keepdims=keep)
+            assert np.allclose(oo.reduce_sum(x, dims, keep, "f32"), want, rtol=1e-5, atol=1e-4)
+    assert np.array_equal(oo.reduce_max(x, (1,), True, "f32"), x.max(1, keepdims=True))
+    assert np.array_equal(oo.reduce_min(x, (2,), False, "f32"), x.min(2))
+
+
+def test_layer_norm_rms_norm_against_torch():
+    g = rng(9)
+    x = g.standard_normal((3, 5, 64)).astype(np.float32) * 2 + 0.5
+    w = (1 + 0.1 * g.standard_normal(64)).astype(np.float32)
+    b = (0.1 * g.standard_normal(64)).astype(np.float32)
+    t = torch.from_numpy(x)
+    want = torch.nn.functional.layer_norm(t, (64,), torch.from_numpy(w), torch.from_numpy(b), 1e-5).numpy()
+    got = onn.layer_norm(x, w, b, 1e-5, "f32")
+    assert np.allclose(got, want, atol=2e-5)
+    plain = onn.layer_norm(x, None, None, 1e-5, "f32")
+    assert np.allclose(plain.mean(-1), 0, atol=1e-5) and np.allclose(plain.var(-1), 1, atol=1e-3)   # population var
+    # rai-nn RmsNorm is algebraically x * w / sqrt(mean(x^2) + eps)
+    want = (t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6) * torch.from_numpy(w)).numpy()
+    assert np.allclose(onn.rms_norm(x, w, 1e-6, "f32"), want, atol=2e-5)
+    if hasattr(torch.nn.functional, "rms_norm"):
+        assert np.allclose(onn.rms_norm(x, w, 1e-6, "f32"),
+                           torch.nn.functional.rms_norm(t, (64,), torch.from_numpy(w), 1e-6).numpy(), atol=2e-5)
+    # Gemma variant == HF GemmaRMSNorm: f32 internal, x * (1 + w)
+    w0 = w - 1
+    want = (t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6) * (1 + torch.from_numpy(w0))).numpy()
+    assert np.allclose(onn.gemma_rms_norm(x, w0, 1e-6, "f32"), want, atol=2e-5)
+    xb = rnd(x, "bf16")
+    gb = onn.gemma_rms_norm(xb, rnd(w0, "bf16"), 1e-6, "bf16")
+    tb = torch.from_numpy(xb)
+    hf = (tb * torch.rsqrt(tb.pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16).float() * \
+        (1 + torch.from_numpy(rnd(w0, "bf16"))).to(torch.bfloat16).float()
+    assert np.allclose(gb, hf.to(torch.bfloat16).float().numpy(), atol=2 ** -6)
+
+
+def test_activations_against_torch():
+    x = np.linspace(-6, 6, 1001).astype(np.float32)
+    t = torch.from_numpy(x)
+    F = torch.nn.functional
+    assert np.allclose(onn.new_gelu(x, "f32"), F.gelu(t, approximate="tanh").numpy(), atol=2e-6)
+    assert np.allclose(onn.gelu(x, "f32"), F.gelu(t).numpy(), atol=2e-6)
+    assert np.allclose(onn.silu(x, "f32"), F.silu(t).numpy(), atol=2e-6)
+    assert np.array_equal(onn.relu(x, "f32"), F.relu(t).numpy())
+    for f in (onn.new_gelu, onn.gelu, onn.silu, onn.relu):
+        assert f(np.zeros(3, np.float32), "f32").tolist() == [0, 0, 0]
+        assert np.allclose(f(np.array([30.0], np.float32), "f32"), 30.0) and abs(f(np.array([-30.0], np.float32), "f32")[0]) < 1e-6
+    # bf16 chain stays within a few bf16 ulps of the f32 function
+    xb = rnd(x, "bf16")
+    assert np.max(np.abs(onn.new_gelu(xb, "bf16") - F.gelu(torch.from_numpy(xb), approximate="tanh").numpy())) < 0.05
+
+
+def test_linear_and_embedding_against_torch():
+    g = rng(10)
+    x, w, b = (g.standard_normal(s).astype(np.float32) for s in [(2, 7, 16), (24, 16), (24,)])
+    want = torch.nn.functional.linear(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(b)).numpy()
+    assert np.allclose(onn.linear(x, w, b, "f32"), want, atol=1e-5)
+    ids = g.integers(0, 24, (2, 5)).astype(np.uint32)
+    assert np.array_equal(onn.embedding(ids, w), torch.nn.functional.embedding(torch.from_numpy(ids.astype(np.int64)), torch.from_numpy(w)).numpy())
+
+
+def test_rope_properties():
+    from oracle import phi2
+    cfg = phi2.Config(max_position_embeddings=128)
+    sin, cos = phi2.rotary_tables(cfg, "f32")
+    rot, half = cfg.rotary_dim, cfg.rotary_dim // 2
+    g = rng(11)
+    x = g.standard_normal((1, 2, 6, 80)).astype(np.float32)
+    y0 = phi2.rotary(x[:, :, :1], sin, cos, rot, 0, "f32")
+    assert np.allclose(y0, x[:, :, :1], atol=1e-7)                                   # position 0 is the identity
+    y = phi2.rotary(x, sin, cos, rot, 17, "f32")
+    assert np.array_equal(y[..., rot:], x[..., rot:])                                 # pass-through dims untouched
+    n_in = x[..., :half] ** 2 + x[..., half:rot] ** 2
+    n_out = y[..., :half] ** 2 + y[..., half:rot] ** 2
+    assert np.allclose(n_in, n_out, rtol=1e-5)                                        # each (i, i+half) pair is rotated
+    # closed form: complex rotation of the pair (x_i, x_{i+half}) by pos * theta^(-2i/rot)
+    inv = 10000.0 ** (-np.arange(0, rot, 2) / rot)
+    pos = 17 + np.arange(6)
+    ang = pos[:, None] * inv[None, :]
+    z = (x[..., :half] + 1j * x[..., half:rot]) * np.exp(1j * ang)
+    assert np.allclose(y[..., :half], z.real, atol=1e-4) and np.allclose(y[..., half:rot], z.imag, atol=1e-4)
+    # relative-position property: <R_m q, R_n k> depends on m - n only
+    q, k = g.standard_normal((1, 1, 1, 80)).astype(np.float32), g.standard_normal((1, 1, 1, 80)).astype(np.float32)
+    dots = [float(np.sum(phi2.rotary(q, sin, cos, rot, m, "f32") * phi2.rotary(k, sin, cos, rot, m - 5, "f32")))
+            for m in (5, 40, 100)]
+    assert np.allclose(dots, dots[0], atol=1e-3)
