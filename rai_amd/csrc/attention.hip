@@ -144,16 +144,17 @@ __device__ __forceinline__ float rope_feature(const T *head, int d, int rot, con
 }
 
 // Decode attention: one 1024-thread block per (head, batch) streams the head's
-// cached K and V once.  Sixty-four 16-lane groups each keep 4 key rows (16-byte
-// loads) in flight, so a 640-token context is covered in three rounds of loads.
-// The new token's rotated key and value are appended to the cache by the block
-// and used from LDS.  Probabilities stay in f32 until the product with V (the
-// reference rounds them to V's dtype first).
+// cached K and V once.  Every 16-lane group keeps UK key rows and every thread
+// UV value chunks (16-byte loads) in flight, and the first round of both is
+// issued before anything else is computed, so a context of up to 64*UK keys
+// costs one HBM round trip for K and V together.  The new token's rotated key
+// and value are appended to the cache by the block and used from LDS.
+// Probabilities stay in f32 until the product with V (the reference rounds them
+// to V's dtype first).
 constexpr int kDecodeThreads = 1024;
-template <typename T>
+template <typename T, int CC, int UK, int UV>
 __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a) {
   constexpr int V = AttnVec<T>::V;
-  constexpr int CC = 4;  // 16-byte chunks of one key row handled by one lane of a 16-lane group
   constexpr int NW = kDecodeThreads / 64, NG = kDecodeThreads / 16;
   extern __shared__ __attribute__((aligned(16))) float smem[];
   // layout: q[D] | knew[D] | vnew[D] | red[groups*D] | scores[Tmax+1]
@@ -176,16 +177,41 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a
   T *Kc = (T *)a.kcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   T *Vc = (T *)a.vcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   const T *cos_t = (const T *)a.cos_t, *sin_t = (const T *)a.sin_t;
+  const int g = tid >> 4, gl = tid & 15;
+  const int col = tid % ncol, grp = tid / ncol;
 
-  for (int d = tid; d < D; d += kDecodeThreads) {
-    qf[d] = rope_feature<T>(row + h * D, d, a.rot, cos_t, sin_t, pos);
-    float kn = rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos);
-    float vn = (float)Scalar<T>::load(row + QD + KD + hk * D + d);
-    knew[d] = kn;
-    vnew[d] = vn;
+  // Loads return in issue order.  The few values of the new token (q, k, v and
+  // their rotary factors) are requested first, the first round of cached K and V
+  // right behind them, so the rotary prologue runs while K and V are in flight.
+  float q_rot = 0.f, k_rot = 0.f, v_new = 0.f;
+  const int d0 = tid;  // one feature per thread (D <= 1024)
+  if (d0 < D) {
+    q_rot = rope_feature<T>(row + h * D, d0, a.rot, cos_t, sin_t, pos);
+    k_rot = rope_feature<T>(row + QD + hk * D, d0, a.rot, cos_t, sin_t, pos);
+    v_new = (float)Scalar<T>::load(row + QD + KD + hk * D + d0);
+  }
+  APack<T, V> kreg[UK][CC], vreg[UV];
+#pragma unroll
+  for (int u = 0; u < UK; ++u) {
+    const int t = g + NG * u;
+#pragma unroll
+    for (int cc = 0; cc < CC; ++cc) {
+      const int c = gl + 16 * cc;
+      if (t < pos && c < ncol) kreg[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UV; ++u) {
+    const int t = grp + u * groups;
+    if (grp < groups && t < pos) vreg[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+  }
+  if (d0 < D) {
+    qf[d0] = q_rot;
+    knew[d0] = k_rot;
+    vnew[d0] = v_new;
     if (h % n_rep == 0) {
-      Scalar<T>::store(Kc + (int64_t)pos * D + d, (typename Scalar<T>::compute)kn);
-      Scalar<T>::store(Vc + (int64_t)pos * D + d, (typename Scalar<T>::compute)vn);
+      Scalar<T>::store(Kc + (int64_t)pos * D + d0, (typename Scalar<T>::compute)k_rot);
+      Scalar<T>::store(Vc + (int64_t)pos * D + d0, (typename Scalar<T>::compute)v_new);
     }
   }
   __syncthreads();
@@ -194,45 +220,43 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a
     if (a.f32_scores) return acc * a.scale;
     return round_to<T>(round_to<T>(acc) * round_to<T>(a.scale));
   };
-  // ---- scores against the cached keys [0, pos)
-  {
-    const int g = tid >> 4, gl = tid & 15;
-    for (int tb = g; tb < pos; tb += 4 * NG) {
-      APack<T, V> pk[4][CC];
+  // ---- scores against the cached keys [0, pos): round 0 from the prefetched registers
+  for (int tb = g; tb < pos; tb += UK * NG) {
+    if (tb != g) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < UK; ++u) {
         const int t = tb + NG * u;
 #pragma unroll
         for (int cc = 0; cc < CC; ++cc) {
           const int c = gl + 16 * cc;
-          if (t < pos && c < ncol) pk[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
+          if (t < pos && c < ncol) kreg[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
         }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int t = tb + NG * u;
-        float acc = 0.f;
-#pragma unroll
-        for (int cc = 0; cc < CC; ++cc) {
-          const int c = gl + 16 * cc;
-          if (t < pos && c < ncol) {
-#pragma unroll
-            for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&pk[u][cc].v[j]), acc);
-          }
-        }
-        acc += __shfl_xor(acc, 8, 64);
-        acc += __shfl_xor(acc, 4, 64);
-        acc += __shfl_xor(acc, 2, 64);
-        acc += __shfl_xor(acc, 1, 64);
-        if (gl == 0 && t < pos) scores[t] = finish_score(acc);
       }
     }
-    if (wave == NW - 1) {  // the new token's own key, still in LDS
+#pragma unroll
+    for (int u = 0; u < UK; ++u) {
+      const int t = tb + NG * u;
       float acc = 0.f;
-      for (int d = lane; d < D; d += 64) acc = fmaf(qf[d], knew[d], acc);
-      acc = wave_sum(acc);
-      if (lane == 0) scores[pos] = finish_score(acc);
+#pragma unroll
+      for (int cc = 0; cc < CC; ++cc) {
+        const int c = gl + 16 * cc;
+        if (t < pos && c < ncol) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&kreg[u][cc].v[j]), acc);
+        }
+      }
+      acc += __shfl_xor(acc, 8, 64);
+      acc += __shfl_xor(acc, 4, 64);
+      acc += __shfl_xor(acc, 2, 64);
+      acc += __shfl_xor(acc, 1, 64);
+      if (gl == 0 && t < pos) scores[t] = finish_score(acc);
     }
+  }
+  if (wave == NW - 1) {  // the new token's own key, still in LDS
+    float acc = 0.f;
+    for (int d = lane; d < D; d += 64) acc = fmaf(qf[d], knew[d], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) scores[pos] = finish_score(acc);
   }
   __syncthreads();
   const int cnt = pos + 1;
@@ -254,27 +278,27 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a
   __syncthreads();
   sum = 0.f;
   for (int w = 0; w < NW; ++w) sum += sh[NW + w];
-  // ---- unnormalised P.V over the cached values, 4 rows in flight per thread
+  // ---- unnormalised P.V over the cached values: round 0 from the prefetched registers
   {
-    const int col = tid % ncol, grp = tid / ncol;
     float acc[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) acc[j] = 0.f;
     if (grp < groups) {
-      for (int tb = grp; tb < pos; tb += 4 * groups) {
-        APack<T, V> pk[4];
+      for (int tb = grp; tb < pos; tb += UV * groups) {
+        if (tb != grp) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int t = tb + u * groups;
-          if (t < pos) pk[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+          for (int u = 0; u < UV; ++u) {
+            const int t = tb + u * groups;
+            if (t < pos) vreg[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+          }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < UV; ++u) {
           const int t = tb + u * groups;
           if (t < pos) {
             const float p = scores[t];
 #pragma unroll
-            for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&pk[u].v[j]), acc[j]);
+            for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&vreg[u].v[j]), acc[j]);
           }
         }
       }
@@ -287,25 +311,34 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a
   const float p_new = scores[pos], inv = 1.0f / sum;
   for (int d = tid; d < D; d += kDecodeThreads) {
     float r = p_new * vnew[d];
-    for (int g = 0; g < groups; ++g) r += red[g * D + d];
+    for (int gg = 0; gg < groups; ++gg) r += red[gg * D + d];
     Scalar<T>::store(o + d, (typename Scalar<T>::compute)(r * inv));
   }
 }
 
-template <typename T> static int launch_decode(hipStream_t st, const AttnDecodeArgs &a) {
+template <typename T, int CC, int UK, int UV> static int launch_decode_cfg(hipStream_t st, const AttnDecodeArgs &a) {
   constexpr int V = AttnVec<T>::V;
-  RAI_REQUIRE(a.D % V == 0 && a.D / V <= 64, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
   const int ncol = a.D / V, groups = kDecodeThreads / ncol;
   const size_t lds = sizeof(float) * (3 * (size_t)a.D + (size_t)groups * a.D + (size_t)a.Tmax + 1);
   RAI_REQUIRE(lds <= 150 * 1024, RAI_ERR_UNSUPPORTED, "attention: context %d too long for the decode kernel", a.Tmax);
   static size_t attr_bytes = 0;
   if (lds > 64 * 1024 && lds > attr_bytes) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_decode<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    150 * 1024));
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_decode<T, CC, UK, UV>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024));
     attr_bytes = 150 * 1024;
   }
-  hipLaunchKernelGGL((k_attn_decode<T>), dim3(a.Hq, a.B), dim3(kDecodeThreads), lds, st, a);
+  hipLaunchKernelGGL((k_attn_decode<T, CC, UK, UV>), dim3(a.Hq, a.B), dim3(kDecodeThreads), lds, st, a);
   return launch_check("attention_decode");
+}
+
+template <typename T> static int launch_decode(hipStream_t st, const AttnDecodeArgs &a) {
+  constexpr int V = AttnVec<T>::V;
+  RAI_REQUIRE(a.D % V == 0 && a.D / V <= 64, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
+  const int ncol = a.D / V;
+  // register budget at 1024 threads per block is 128 VGPRs: (UK*CC + UV) 16-byte packs
+  if (ncol <= 16) return launch_decode_cfg<T, 1, 10, 7>(st, a);
+  if (ncol <= 32) return launch_decode_cfg<T, 2, 5, 6>(st, a);
+  return launch_decode_cfg<T, 4, 2, 6>(st, a);
 }
 
 int launch_attention_decode(hipStream_t st, const AttnDecodeArgs &a) {

@@ -7,6 +7,8 @@
 //
 // Reference semantics: rai-core/src/backend/candle.rs:327-443 (MatMul, stride rule),
 // rai-core/src/shape.rs:130-160 (batch broadcast), rai-nn/src/linear.rs:59-69.
+#include <cstdlib>
+
 #include "gemm.h"
 
 namespace rai {
@@ -40,48 +42,87 @@ __device__ __forceinline__ float dot8_bf16(u32x4 a, u32x4 b, float c) {
 // Every wave owns `rows_per_wave` consecutive weight rows (so all waves stream
 // the same number of bytes and are co-resident: no tail), R rows at a time, with
 // U 16-byte loads per row in flight per lane.
-template <int MROWS, int R, int U>
-__global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a, int rows_per_wave) {
+template <int MROWS, int R, int U, int NWV>
+__global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, int rows_per_wave) {
+  constexpr int NT = NWV * 64;
   extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [MROWS][K]
-  __shared__ float red[8];
+  __shared__ float red[2 * NWV];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint16_t *A = (const uint16_t *)a.A;
   const uint16_t *W = (const uint16_t *)a.W;
   const int K = a.K;
+
+  // Loads return in issue order: the activation rows (L2-resident) are requested
+  // first, the first set of weight loads right behind them, so the staging into
+  // LDS completes while the weights are still in flight.
+  constexpr int XCH = 8;  // staged 16-byte chunks per thread per row that are prefetched in registers
+  const int n_begin = (blockIdx.x * NWV + wave) * rows_per_wave;
+  const int n_end = n_begin + rows_per_wave < a.N ? n_begin + rows_per_wave : a.N;
+  u32x4 xpre[XCH];
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) {
+    const int k = (tid + i * NT) * 8;
+    xpre[i] = k < K ? *reinterpret_cast<const u32x4 *>(A + k) : u32x4{0u, 0u, 0u, 0u};
+  }
+  u32x4 wv[U][R];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int k = lane * 8 + u * 512;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int n = n_begin + r < n_end ? n_begin + r : n_end - 1;
+      if (k < K && n_begin < a.N) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(W + (int64_t)n * a.ldw + k));
+      else wv[u][r] = u32x4{0u, 0u, 0u, 0u};
+    }
+  }
 
   // ---- stage activations, optionally normalising each row over K
   for (int m = 0; m < MROWS; ++m) {
     if (m >= a.M) break;
     const uint16_t *xr = A + (int64_t)m * a.lda;
     uint16_t *xd = xs + m * K;
-    for (int k = tid * 8; k < K; k += 256 * 8)
-      *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(xr + k);
+    if (m == 0) {
+#pragma unroll
+      for (int i = 0; i < XCH; ++i) {
+        const int k = (tid + i * NT) * 8;
+        if (k < K) *reinterpret_cast<u32x4 *>(xd + k) = xpre[i];
+      }
+      for (int k = (tid + XCH * NT) * 8; k < K; k += NT * 8)
+        *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(xr + k);
+    } else {
+      for (int k = tid * 8; k < K; k += NT * 8)
+        *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(xr + k);
+    }
     if (a.ln_kind >= 0) {
       __syncthreads();
       float s = 0.f;
-      for (int k = tid; k < K; k += 256) {
+      for (int k = tid; k < K; k += NT) {
         float v = bf16_bits_to_f32(xd[k]);
         s += a.ln_kind == 0 ? v : v * v;
       }
       s = wave_sum(s);
       if (lane == 0) red[wave] = s;
       __syncthreads();
-      s = red[0] + red[1] + red[2] + red[3];
+      s = 0.f;
+#pragma unroll
+      for (int w = 0; w < NWV; ++w) s += red[w];
       float mean = 0.f, scale;
       if (a.ln_kind == 0) {
         mean = s / (float)K;
         float q = 0.f;
-        for (int k = tid; k < K; k += 256) { float d = bf16_bits_to_f32(xd[k]) - mean; q += d * d; }
+        for (int k = tid; k < K; k += NT) { float d = bf16_bits_to_f32(xd[k]) - mean; q += d * d; }
         q = wave_sum(q);
-        if (lane == 0) red[4 + wave] = q;
+        if (lane == 0) red[NWV + wave] = q;
         __syncthreads();
-        q = red[4] + red[5] + red[6] + red[7];
+        q = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWV; ++w) q += red[NWV + w];
         scale = 1.0f / sqrtf(q / (float)K + a.ln_eps);
       } else {
         scale = 1.0f / sqrtf(s / (float)K + a.ln_eps);
       }
       const uint16_t *lw = (const uint16_t *)a.ln_w, *lb = (const uint16_t *)a.ln_b;
-      for (int k = tid; k < K; k += 256) {
+      for (int k = tid; k < K; k += NT) {
         float y = (bf16_bits_to_f32(xd[k]) - mean) * scale;
         float wv = bf16_bits_to_f32(lw[k]);
         y *= a.ln_kind == 2 ? 1.0f + wv : wv;
@@ -97,70 +138,80 @@ __global__ void __launch_bounds__(256) k_linear_bf16_skinny(LinearArgs a, int ro
   const uint16_t *bias = (const uint16_t *)a.bias;
   const uint16_t *bias2 = (const uint16_t *)a.bias2;
   const uint16_t *res = (const uint16_t *)a.residual;
-  const int n_begin = (blockIdx.x * 4 + wave) * rows_per_wave;
-  const int n_end = n_begin + rows_per_wave < a.N ? n_begin + rows_per_wave : a.N;
-  for (int n_base = n_begin; n_base < n_end; n_base += R) {
-    float acc[R][MROWS];
+  // Flattened (row group, K step) loop in rotated form: multiply the set in
+  // registers, then fetch the next set.
+  if (n_begin >= n_end) return;
+  float acc[R][MROWS];
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+  for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int m = 0; m < MROWS; ++m) acc[r][m] = 0.f;
-    const uint16_t *wrow[R];
+    for (int m = 0; m < MROWS; ++m) acc[r][m] = 0.f;
+  int n_base = n_begin, k0 = lane * 8;
+  while (true) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      int n = n_base + r < n_end ? n_base + r : n_end - 1;  // tail rows re-read the last row; never stored
-      wrow[r] = W + (int64_t)n * a.ldw;
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * 512;
+      if (k < K) {
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) {
+          const u32x4 xv = *reinterpret_cast<const u32x4 *>(xs + m * K + k);
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[r][m] = dot8_bf16(wv[u][r], xv, acc[r][m]);
+        }
+      }
     }
-    for (int k0 = lane * 8; k0 < K; k0 += 64 * 8 * U) {
-      u32x4 wv[U][R];
+    k0 += 64 * 8 * U;
+    const bool row_done = k0 >= K;
+    const int n_cur = n_base;
+    if (row_done) {
+      n_base += R;
+      k0 = lane * 8;
+    }
+    const bool more = n_base < n_end;
+    if (more) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int k = k0 + u * 512;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          if (k < K) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[r] + k));
-          else wv[u][r] = u32x4{0u, 0u, 0u, 0u};
+          const int n = n_base + r < n_end ? n_base + r : n_end - 1;  // tail rows re-read the last row; never stored
+          if (k < K) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(W + (int64_t)n * a.ldw + k));
         }
       }
+    }
+    if (row_done) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int k = k0 + u * 512;
-        if (k < K) {
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) acc[r][m] = wave_sum(acc[r][m]);
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int n = n_cur + r;
+          if (n >= n_end) break;
+          const float bv = (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
+          const bool do_act = a.act >= 0 && n >= a.act_from;
+          uint16_t *dst;
+          int64_t ld;
+          int col;
+          if (n < a.n_split) { dst = (uint16_t *)a.out1; ld = a.ld1; col = n; }
+          else { dst = (uint16_t *)a.out2; ld = a.ld2; col = n - a.n_split; }
 #pragma unroll
           for (int m = 0; m < MROWS; ++m) {
-            const u32x4 xv = *reinterpret_cast<const u32x4 *>(xs + m * K + k);
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r][m] = dot8_bf16(wv[u][r], xv, acc[r][m]);
+            if (m >= a.M) break;
+            float v = acc[r][m] + bv;
+            if (do_act) v = act_eval(a.act, v);
+            if (res) v += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
+            dst[(int64_t)m * ld + col] = f32_to_bf16_bits(v);
           }
         }
       }
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) acc[r][m] = 0.f;
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int m = 0; m < MROWS; ++m) acc[r][m] = wave_sum(acc[r][m]);
-    if (lane == 0) {
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int n = n_base + r;
-        if (n >= n_end) break;
-        const float bv = (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
-        const bool do_act = a.act >= 0 && n >= a.act_from;
-        uint16_t *dst;
-        int64_t ld;
-        int col;
-        if (n < a.n_split) { dst = (uint16_t *)a.out1; ld = a.ld1; col = n; }
-        else { dst = (uint16_t *)a.out2; ld = a.ld2; col = n - a.n_split; }
-#pragma unroll
-        for (int m = 0; m < MROWS; ++m) {
-          if (m >= a.M) break;
-          float v = acc[r][m] + bv;
-          if (do_act) v = act_eval(a.act, v);
-          if (res) v += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
-          dst[(int64_t)m * ld + col] = f32_to_bf16_bits(v);
-        }
-      }
-    }
+    if (!more) break;
   }
 }
 
@@ -194,15 +245,26 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
       }
     }
   };
+  // Loads return in issue order, so the small L2-resident vectors (activations,
+  // norm parameters) are requested first and the weight stream right after: the
+  // norm prologue then runs while the weights are still in flight.
+  u32x4 xv[KC], lwv[KC], lbv[KC];
+  {
+    const uint16_t *xr = (const uint16_t *)a.A + lane * 8;
+    const uint16_t *lw = a.ln_kind >= 0 ? (const uint16_t *)a.ln_w + lane * 8 : nullptr;
+    const uint16_t *lb = (a.ln_kind >= 0 && a.ln_b) ? (const uint16_t *)a.ln_b + lane * 8 : nullptr;
+#pragma unroll
+    for (int u = 0; u < KC; ++u) {
+      const bool in = lane * 8 + u * 512 < K;
+      xv[u] = in ? *reinterpret_cast<const u32x4 *>(xr + u * 512) : u32x4{0u, 0u, 0u, 0u};
+      lwv[u] = (in && lw) ? *reinterpret_cast<const u32x4 *>(lw + u * 512) : u32x4{0u, 0u, 0u, 0u};
+      lbv[u] = (in && lb) ? *reinterpret_cast<const u32x4 *>(lb + u * 512) : u32x4{0u, 0u, 0u, 0u};
+    }
+  }
   load_group(n_begin);
 
   // ---- activation vector (optionally normalised over K), packed bf16 in registers
-  u32x4 xv[KC];
   {
-    const uint16_t *xr = (const uint16_t *)a.A + lane * 8;
-#pragma unroll
-    for (int u = 0; u < KC; ++u)
-      xv[u] = (lane * 8 + u * 512 < K) ? *reinterpret_cast<const u32x4 *>(xr + u * 512) : u32x4{0u, 0u, 0u, 0u};
     if (a.ln_kind >= 0) {
       float xf[KC][8];
       float s = 0.f;
@@ -233,13 +295,11 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
       } else {
         scale = 1.0f / sqrtf(s / (float)K + a.ln_eps);
       }
-      const uint16_t *lw = (const uint16_t *)a.ln_w + lane * 8;
-      const uint16_t *lb = a.ln_b ? (const uint16_t *)a.ln_b + lane * 8 : nullptr;
 #pragma unroll
       for (int u = 0; u < KC; ++u) {
         if (lane * 8 + u * 512 < K) {
-          const u32x4 wq = *reinterpret_cast<const u32x4 *>(lw + u * 512);
-          const u32x4 bq = lb ? *reinterpret_cast<const u32x4 *>(lb + u * 512) : u32x4{0u, 0u, 0u, 0u};
+          const u32x4 wq = lwv[u];
+          const u32x4 bq = lbv[u];
           const uint32_t ww[4] = {wq.x, wq.y, wq.z, wq.w}, bb[4] = {bq.x, bq.y, bq.z, bq.w};
           uint32_t o[4];
 #pragma unroll
@@ -263,7 +323,6 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
   const uint16_t *bias2 = (const uint16_t *)a.bias2;
   const uint16_t *res = (const uint16_t *)a.residual;
   for (int n_base = n_begin; n_base < n_end; n_base += R) {
-    if (n_base != n_begin) load_group(n_base);
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -271,6 +330,8 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
 #pragma unroll
       for (int u = 0; u < KC; ++u) acc[r] = dot8_bf16(wv[r][u], xv[u], acc[r]);
     }
+    // the next group's loads go out before this group's reduction and stores
+    if (n_base + R < n_end) load_group(n_base + R);
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
     if (lane == 0) {
@@ -438,26 +499,31 @@ static int check_linear_args(const LinearArgs &a, size_t es) {
   return RAI_OK;
 }
 
-template <int MROWS, int R, int U> static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a, int rows_per_wave) {
+template <int MROWS, int R, int U, int NWV = 4>
+static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a, int rows_per_wave) {
   const size_t lds = (size_t)MROWS * a.K * sizeof(uint16_t);
   static size_t attr_bytes = 0;
   if (lds > 64 * 1024 && lds > attr_bytes) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_skinny<MROWS, R, U>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_skinny<MROWS, R, U, NWV>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_bytes = lds;
   }
   const int waves = (a.N + rows_per_wave - 1) / rows_per_wave;
-  const int blocks = (waves + 3) / 4;
-  hipLaunchKernelGGL((k_linear_bf16_skinny<MROWS, R, U>), dim3(blocks), dim3(256), lds, st, a, rows_per_wave);
+  const int blocks = (waves + NWV - 1) / NWV;
+  hipLaunchKernelGGL((k_linear_bf16_skinny<MROWS, R, U, NWV>), dim3(blocks), dim3(NWV * 64), lds, st, a, rows_per_wave);
   return launch_check("linear_bf16_skinny");
 }
 
-template <int KC, int R> static int launch_gemv_reg(hipStream_t st, const LinearArgs &a) {
-  // about 10 waves per CU (the register budget allows 12), all co-resident, each
-  // with a whole number of R-row groups
-  const int target_waves = kNumCU * 10;
-  int rpw = (a.N + target_waves - 1) / target_waves;
-  rpw = ((rpw + R - 1) / R) * R;
+template <int KC, int R>
+static int launch_gemv_reg(hipStream_t st, const LinearArgs &a, int waves_per_cu, int rows_per_wave = 0) {
+  // every wave co-resident (waves_per_cu follows the kernel's register budget),
+  // each with a whole number of R-row groups
+  int rpw = rows_per_wave;
+  if (rpw <= 0) {
+    const int target_waves = kNumCU * waves_per_cu;
+    rpw = (a.N + target_waves - 1) / target_waves;
+    rpw = ((rpw + R - 1) / R) * R;
+  }
   const int waves = (a.N + rpw - 1) / rpw;
   hipLaunchKernelGGL((k_gemv_bf16_reg<KC, R>), dim3((waves + 3) / 4), dim3(256), 0, st, a, rpw);
   return launch_check("gemv_bf16_reg");
@@ -469,14 +535,39 @@ int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE((size_t)a.M * a.K * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
   if (a.M == 1 && a.K <= 4096 && a.N >= 1024) {
     // activation vector in registers (at most 8 chunks of 16 bytes per lane)
-    if (a.K <= 2048) return launch_gemv_reg<4, 4>(st, a);
-    if (a.K <= 2560) return launch_gemv_reg<5, 4>(st, a);
-    return launch_gemv_reg<8, 2>(st, a);
+    if (a.K <= 2048) return launch_gemv_reg<4, 4>(st, a, 8);
+    if (a.K <= 2560) {
+      static const char *gk = getenv("RAI_HIP_GEMV");  // tuning aid: "R,rows_per_wave"
+      if (gk) {
+        int r = 0, rp = 0;
+        if (sscanf(gk, "%d,%d", &r, &rp) == 2 && rp > 0) {
+          if (r == 4) return launch_gemv_reg<5, 4>(st, a, 0, rp);
+          if (r == 2) return launch_gemv_reg<5, 2>(st, a, 0, rp);
+        }
+      }
+      return launch_gemv_reg<5, 2>(st, a, 0, a.N >= 8192 ? 4 : 2);  // short-lived waves, two row groups each
+    }
+    return launch_gemv_reg<8, 2>(st, a, 8);
   }
   // About 10 waves per CU, all co-resident, each with the same number of rows.
   const int target_waves = kNumCU * 10;
   int rpw = (a.N + target_waves - 1) / target_waves;
   if (a.M == 1) {
+    static const char *knob = getenv("RAI_HIP_SKINNY");  // tuning aid: "R,NWV,rows_per_wave,U"
+    if (knob) {
+      int r = 0, nwv = 0, rp = 0, u = 0;
+      if (sscanf(knob, "%d,%d,%d,%d", &r, &nwv, &rp, &u) == 4 && rp > 0) {
+        if (r == 1 && nwv == 4 && u == 8) return launch_skinny_cfg<1, 1, 8, 4>(st, a, rp);
+        if (r == 1 && nwv == 4 && u == 13) return launch_skinny_cfg<1, 1, 13, 4>(st, a, rp);
+        if (r == 1 && nwv == 4 && u == 25) return launch_skinny_cfg<1, 1, 25, 4>(st, a, rp);
+        if (r == 1 && nwv == 8 && u == 25) return launch_skinny_cfg<1, 1, 25, 8>(st, a, rp);
+        if (r == 1 && nwv == 16 && u == 25) return launch_skinny_cfg<1, 1, 25, 16>(st, a, rp);
+        if (r == 2 && nwv == 4 && u == 13) return launch_skinny_cfg<1, 2, 13, 4>(st, a, rp);
+        if (r == 2 && nwv == 4 && u == 8) return launch_skinny_cfg<1, 2, 8, 4>(st, a, rp);
+      }
+    }
+    // one row per wave with the whole row in flight when it fits the register budget
+    if (a.N <= kNumCU * 16 && a.K <= 25 * 512) return launch_skinny_cfg<1, 1, 25>(st, a, 1);
     if (rpw >= 4) { rpw = (rpw / 4) * 4; return launch_skinny_cfg<1, 4, 5>(st, a, rpw); }
     if (rpw >= 2) { rpw = 2; return launch_skinny_cfg<1, 2, 8>(st, a, rpw); }
     return launch_skinny_cfg<1, 1, 8>(st, a, 1);
