@@ -263,58 +263,52 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
   }
   load_group(n_begin);
 
-  // ---- activation vector (optionally normalised over K), packed bf16 in registers
-  {
-    if (a.ln_kind >= 0) {
-      float xf[KC][8];
-      float s = 0.f;
+  // ---- fused LayerNorm / RMSNorm of the activation vector, kept as packed bf16 in registers.
+  // Sum and sum of squares come from v_dot2_f32_bf16 on the packed pairs (exact
+  // products, f32 accumulation); the variance is E[x^2] - mean^2.
+  if (a.ln_kind >= 0) {
+    const uint32_t ones = 0x3f803f80u;  // (1.0bf16, 1.0bf16)
+    float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-      for (int u = 0; u < KC; ++u) {
-        const uint32_t w4[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+    for (int u = 0; u < KC; ++u) {
+      const uint32_t w4[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s1 = dot2_bf16(w4[j], ones, s1);
+        s2 = dot2_bf16(w4[j], w4[j], s2);
+      }
+    }
+    if (a.ln_kind == 0) s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    float mean = 0.f, scale;
+    if (a.ln_kind == 0) {
+      mean = s1 / (float)K;
+      float var = s2 / (float)K - mean * mean;
+      var = var > 0.f ? var : 0.f;
+      scale = 1.0f / sqrtf(var + a.ln_eps);
+    } else {
+      scale = 1.0f / sqrtf(s2 / (float)K + a.ln_eps);
+    }
+    const float shift = -mean * scale;
+#pragma unroll
+    for (int u = 0; u < KC; ++u) {
+      if (lane * 8 + u * 512 < K) {
+        const uint32_t xx[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+        const uint32_t ww[4] = {lwv[u].x, lwv[u].y, lwv[u].z, lwv[u].w};
+        const uint32_t bb[4] = {lbv[u].x, lbv[u].y, lbv[u].z, lbv[u].w};
+        uint32_t o[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          xf[u][2 * j] = __uint_as_float(w4[j] << 16);
-          xf[u][2 * j + 1] = __uint_as_float(w4[j] & 0xffff0000u);
-          s += a.ln_kind == 0 ? xf[u][2 * j] + xf[u][2 * j + 1]
-                              : xf[u][2 * j] * xf[u][2 * j] + xf[u][2 * j + 1] * xf[u][2 * j + 1];
+          float w0 = __uint_as_float(ww[j] << 16), w1 = __uint_as_float(ww[j] & 0xffff0000u);
+          if (a.ln_kind == 2) { w0 += 1.0f; w1 += 1.0f; }
+          // ((x - mean) * scale) * w + b
+          const float y0 = fmaf(fmaf(__uint_as_float(xx[j] << 16), scale, shift), w0, __uint_as_float(bb[j] << 16));
+          const float y1 = fmaf(fmaf(__uint_as_float(xx[j] & 0xffff0000u), scale, shift), w1,
+                                __uint_as_float(bb[j] & 0xffff0000u));
+          // the reference materialises the normalised activations in bf16 too
+          o[j] = pack_bf16x2(y0, y1);
         }
-      }
-      s = wave_sum(s);
-      float mean = 0.f, scale;
-      if (a.ln_kind == 0) {
-        mean = s / (float)K;
-        float q = 0.f;
-#pragma unroll
-        for (int u = 0; u < KC; ++u)
-          if (lane * 8 + u * 512 < K) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) { float d = xf[u][j] - mean; q += d * d; }
-          }
-        q = wave_sum(q);
-        scale = 1.0f / sqrtf(q / (float)K + a.ln_eps);
-      } else {
-        scale = 1.0f / sqrtf(s / (float)K + a.ln_eps);
-      }
-#pragma unroll
-      for (int u = 0; u < KC; ++u) {
-        if (lane * 8 + u * 512 < K) {
-          const u32x4 wq = lwv[u];
-          const u32x4 bq = lbv[u];
-          const uint32_t ww[4] = {wq.x, wq.y, wq.z, wq.w}, bb[4] = {bq.x, bq.y, bq.z, bq.w};
-          uint32_t o[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float y0 = (xf[u][2 * j] - mean) * scale, y1 = (xf[u][2 * j + 1] - mean) * scale;
-            float w0 = __uint_as_float(ww[j] << 16), w1 = __uint_as_float(ww[j] & 0xffff0000u);
-            y0 *= a.ln_kind == 2 ? 1.0f + w0 : w0;
-            y1 *= a.ln_kind == 2 ? 1.0f + w1 : w1;
-            y0 += __uint_as_float(bb[j] << 16);
-            y1 += __uint_as_float(bb[j] & 0xffff0000u);
-            // the reference materialises the normalised activations in bf16 too
-            o[j] = (uint32_t)f32_to_bf16_bits(y0) | ((uint32_t)f32_to_bf16_bits(y1) << 16);
-          }
-          xv[u] = u32x4{o[0], o[1], o[2], o[3]};
-        }
+        xv[u] = u32x4{o[0], o[1], o[2], o[3]};
       }
     }
   }
