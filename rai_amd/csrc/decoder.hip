@@ -33,7 +33,11 @@ struct ParamSlot {
 };
 
 struct Layer {
+  // Phi-2 (parallel block)
   char *Wa, *ba, *Wb, *bd, *bf, *ln_w, *ln_b;
+  // Qwen2 / Gemma (sequential block): Wqkv [QD+2KD, H] (+bqkv), Wo [H, QD] (+bo),
+  // Wgu [2I, H] with gate/up rows interleaved, Wdown [H, I], two RMSNorm weights
+  char *Wqkv, *bqkv, *Wo, *bo, *Wgu, *Wdown, *n1_w, *n2_w;
 };
 
 struct DevState {
@@ -60,6 +64,8 @@ struct rai_hip_decoder {
   char *kcache, *vcache;
   // activations (sized for max_batch * max_context rows)
   char *x, *x2, *ln, *qkv, *cat, *last, *logits;
+  char *attn, *glu;   // sequential block: attention output [rows, QD], gated MLP activation [rows, I]
+  float embed_scale;  // Gemma: sqrt(hidden) rounded to the model dtype; 1 otherwise
   uint32_t *ids, *tokens, *history;
   char *splitk_ws;        // f32 scratch for prefill GEMMs that split K
   size_t splitk_ws_bytes;
@@ -78,7 +84,8 @@ namespace rai {
 // ------------------------------------------------------------------ small kernels
 template <typename T>
 __global__ void __launch_bounds__(256)
-k_embed(T *out, const T *table, const uint32_t *ids, int64_t rows, int H, int vocab, unsigned long long *errors) {
+k_embed(T *out, const T *table, const uint32_t *ids, int64_t rows, int H, int vocab, unsigned long long *errors,
+        float scale) {
   for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < rows * H; e += (int64_t)gridDim.x * blockDim.x) {
     int64_t r = e / H;
     int c = (int)(e - r * H);
@@ -86,6 +93,8 @@ k_embed(T *out, const T *table, const uint32_t *ids, int64_t rows, int H, int vo
     if (id >= (uint32_t)vocab) {
       if (c == 0) atomicAdd(errors, 1ull);
       memset(&out[e], 0, sizeof(T));
+    } else if (scale != 1.0f) {  // Gemma: xs * sqrt(hidden), the scalar rounded to the model dtype (gemma.rs:379)
+      Scalar<T>::store(out + e, (typename Scalar<T>::compute)((float)Scalar<T>::load(table + (int64_t)id * H + c) * scale));
     } else {
       out[e] = table[(int64_t)id * H + c];
     }
@@ -164,7 +173,7 @@ __global__ void k_set_state(DevState *st, int pos, int step) {
 template <typename T>
 __global__ void __launch_bounds__(1024)
 k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
-               int dstep, const T *embed, T *x_next, int H) {
+               int dstep, const T *embed, T *x_next, int H, float embed_scale) {
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   __shared__ uint32_t chosen;
@@ -200,7 +209,12 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
   __syncthreads();
   if (x_next) {
     const T *row = embed + (int64_t)chosen * H;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) x_next[(int64_t)b * H + c] = row[c];
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+      if (embed_scale != 1.0f)
+        Scalar<T>::store(x_next + (int64_t)b * H + c, (typename Scalar<T>::compute)((float)Scalar<T>::load(row + c) * embed_scale));
+      else
+        x_next[(int64_t)b * H + c] = row[c];
+    }
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -338,10 +352,59 @@ static int create_phi2(rai_hip_decoder *d) {
   return RAI_OK;
 }
 
+// Qwen2 (rai-models/src/llm/qwen2.rs:276-300) and Gemma (gemma.rs:309-338) parameter slots.
+static int create_seq(rai_hip_decoder *d) {
+  const size_t es = d->es;
+  const int H = d->H, I = d->I, QD = d->QD, KD = d->KD, V = d->V;
+  const bool qwen = d->cfg.arch == RAI_ARCH_QWEN2;
+  RAI_TRY(dalloc(d, (size_t)V * H * es, &d->embed));
+  add_slot(d, "model.embed_tokens.weight", V, H, d->embed, H);
+  d->layers.resize(d->L);
+  for (int l = 0; l < d->L; ++l) {
+    Layer &ly = d->layers[l];
+    memset(&ly, 0, sizeof(ly));
+    const int NQ = QD + 2 * KD;
+    RAI_TRY(dalloc(d, (size_t)NQ * H * es, &ly.Wqkv));
+    RAI_TRY(dalloc(d, (size_t)H * QD * es, &ly.Wo));
+    RAI_TRY(dalloc(d, (size_t)2 * I * H * es, &ly.Wgu));
+    RAI_TRY(dalloc(d, (size_t)H * I * es, &ly.Wdown));
+    RAI_TRY(dalloc(d, (size_t)H * es, &ly.n1_w));
+    RAI_TRY(dalloc(d, (size_t)H * es, &ly.n2_w));
+    const std::string p = "model.layers." + std::to_string(l) + ".";
+    add_slot(d, p + "self_attn.q_proj.weight", QD, H, ly.Wqkv, H);
+    add_slot(d, p + "self_attn.k_proj.weight", KD, H, ly.Wqkv + (size_t)QD * H * es, H);
+    add_slot(d, p + "self_attn.v_proj.weight", KD, H, ly.Wqkv + (size_t)(QD + KD) * H * es, H);
+    if (qwen) {  // q/k/v carry a bias, o_proj does not (qwen2.rs:137-140)
+      RAI_TRY(dalloc(d, (size_t)NQ * es, &ly.bqkv));
+      add_slot(d, p + "self_attn.q_proj.bias", 1, QD, ly.bqkv, QD);
+      add_slot(d, p + "self_attn.k_proj.bias", 1, KD, ly.bqkv + (size_t)QD * es, KD);
+      add_slot(d, p + "self_attn.v_proj.bias", 1, KD, ly.bqkv + (size_t)(QD + KD) * es, KD);
+    }
+    add_slot(d, p + "self_attn.o_proj.weight", H, QD, ly.Wo, QD);
+    // gate row n -> packed row 2n, up row n -> packed row 2n+1 (pitch of two rows)
+    add_slot(d, p + "mlp.gate_proj.weight", I, H, ly.Wgu, 2 * (int64_t)H);
+    add_slot(d, p + "mlp.up_proj.weight", I, H, ly.Wgu + (size_t)H * es, 2 * (int64_t)H);
+    add_slot(d, p + "mlp.down_proj.weight", H, I, ly.Wdown, I);
+    add_slot(d, p + "input_layernorm.weight", 1, H, ly.n1_w, H);
+    add_slot(d, p + "post_attention_layernorm.weight", 1, H, ly.n2_w, H);
+  }
+  RAI_TRY(dalloc(d, (size_t)H * es, &d->lnf_w));
+  d->lnf_b = nullptr;
+  add_slot(d, "model.norm.weight", 1, H, d->lnf_w, H);
+  d->head_b = nullptr;
+  if (d->cfg.arch == RAI_ARCH_GEMMA || d->cfg.tie_word_embeddings) {
+    d->head_w = d->embed;  // gemma.rs:330 lm_head shares the embedding matrix
+  } else {
+    RAI_TRY(dalloc(d, (size_t)V * H * es, &d->head_w));
+    add_slot(d, "lm_head.weight", V, H, d->head_w, H);
+  }
+  return RAI_OK;
+}
+
 // ------------------------------------------------------------------ forward
 template <typename T> static void launch_embed(rai_hip_decoder *d, hipStream_t st, int64_t rows) {
   hipLaunchKernelGGL((k_embed<T>), dim3(grid1d(rows * d->H)), dim3(256), 0, st, (T *)d->x, (const T *)d->embed, d->ids,
-                     rows, d->H, d->V, index_error_counter(d->dev));
+                     rows, d->H, d->V, index_error_counter(d->dev), d->embed_scale);
 }
 template <typename T> static void launch_rope_append(rai_hip_decoder *d, hipStream_t st, int l, int B, int S) {
   const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
@@ -487,13 +550,155 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H);
+                       (bf16_raw *)d->x, H, d->embed_scale);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
-                       d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H);
+                       d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
+                       d->embed_scale);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
+}
+
+// Sequential pre-norm block of Qwen2 (qwen2.rs:253-266) and Gemma (gemma.rs:286-299):
+// x1 = x + o_proj(attn(norm1(x))); x = x1 + down(act(gate(norm2(x1))) * up(norm2(x1))).
+static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool from_tokens = false) {
+  hipStream_t st = stream_of(d->dev);
+  if (!st) return RAI_ERR_HIP;
+  const int dt = d->cfg.dtype;
+  const int H = d->H, QD = d->QD, KD = d->KD, I = d->I;
+  const int64_t M = (int64_t)B * S;
+  const int ldq = QD + 2 * KD;
+  const bool fuse_norm = dt == RAI_BF16 && M <= 8;
+  const int kind = d->cfg.arch == RAI_ARCH_GEMMA ? 2 : 1;
+  const int T_after = d->ctx_len + S;
+  const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
+
+  if (!from_tokens) {
+    if (dt == RAI_BF16) launch_embed<bf16_raw>(d, st, M); else launch_embed<float>(d, st, M);
+    RAI_TRY(launch_check("embed"));
+  }
+  auto norm_rows = [&](char *src, char *w, char *dst, int64_t rows, int64_t src_stride) -> int {
+    rai_hip_tensor tx = desc2(src, dt, rows, H, src_stride), tw = desc1(w, dt, H), to = desc2(dst, dt, rows, H, H);
+    return rai_hip_rms_norm(d->dev, &tx, &tw, d->cfg.norm_eps, kind == 2, &to);
+  };
+  char *x = d->x, *x1 = d->x2;
+  for (int l = 0; l < d->L; ++l) {
+    const Layer &ly = d->layers[l];
+    LinearArgs a = linear_args_default();
+    if (fuse_norm) {
+      a.A = x; a.lda = H;
+      a.ln_kind = kind; a.ln_w = ly.n1_w; a.ln_eps = (float)d->cfg.norm_eps;
+    } else {
+      RAI_TRY(norm_rows(x, ly.n1_w, d->ln, M, H));
+      a.A = d->ln; a.lda = H;
+    }
+    a.W = ly.Wqkv; a.ldw = H; a.bias = ly.bqkv;
+    a.out1 = d->qkv; a.ld1 = ldq;
+    a.M = (int)M; a.N = ldq; a.K = H; a.n_split = ldq;
+    a.splitk_ws = d->splitk_ws; a.splitk_ws_bytes = d->splitk_ws_bytes;
+    RAI_TRY(linear(d, st, a));
+
+    if (S == 1) {
+      AttnDecodeArgs t;
+      memset(&t, 0, sizeof(t));
+      t.qkv = d->qkv;
+      t.kcache = d->kcache + per_layer * l * d->es;
+      t.vcache = d->vcache + per_layer * l * d->es;
+      t.out = d->attn;
+      t.out_row_stride = QD;
+      t.cos_t = d->cos_t; t.sin_t = d->sin_t; t.rot = d->cfg.rotary_dim;
+      t.pos_dev = &d->state->pos;
+      t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.D = d->D; t.Tmax = d->cfg.max_context;
+      t.scale = (float)(1.0 / sqrt((double)d->D));
+      t.f32_scores = 0; t.dtype = dt;
+      RAI_TRY(launch_attention_decode(st, t));
+    } else {
+      if (dt == RAI_BF16) launch_rope_append<bf16_raw>(d, st, l, B, S); else launch_rope_append<float>(d, st, l, B, S);
+      RAI_TRY(launch_check("rope_append"));
+      AttnArgs t;
+      memset(&t, 0, sizeof(t));
+      t.q = d->qkv;
+      t.k = d->kcache + per_layer * l * d->es;
+      t.v = d->vcache + per_layer * l * d->es;
+      t.out = d->attn;
+      t.qs[0] = (int64_t)S * ldq; t.qs[1] = d->D; t.qs[2] = ldq;
+      t.ks[0] = t.vs[0] = (int64_t)d->Hkv * d->cfg.max_context * d->D;
+      t.ks[1] = t.vs[1] = (int64_t)d->cfg.max_context * d->D;
+      t.ks[2] = t.vs[2] = d->D;
+      t.out_row_stride = QD;
+      t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.S = S; t.D = d->D;
+      t.scale = (float)(1.0 / sqrt((double)d->D));
+      t.causal = 1; t.f32_scores = 0; t.dtype = dt;
+      t.T = T_after;
+      RAI_TRY(launch_attention(st, t));
+    }
+
+    LinearArgs o = linear_args_default();
+    o.A = d->attn; o.lda = QD;
+    o.W = ly.Wo; o.ldw = QD; o.bias = ly.bo;
+    o.residual = x; o.ldr = H;
+    o.out1 = x1; o.ld1 = H;
+    o.M = (int)M; o.N = H; o.K = QD; o.n_split = H;
+    o.splitk_ws = d->splitk_ws; o.splitk_ws_bytes = d->splitk_ws_bytes;
+    RAI_TRY(linear(d, st, o));
+
+    LinearArgs g = linear_args_default();
+    if (fuse_norm) {
+      g.A = x1; g.lda = H;
+      g.ln_kind = kind; g.ln_w = ly.n2_w; g.ln_eps = (float)d->cfg.norm_eps;
+    } else {
+      RAI_TRY(norm_rows(x1, ly.n2_w, d->ln, M, H));
+      g.A = d->ln; g.lda = H;
+    }
+    g.W = ly.Wgu; g.ldw = H;
+    g.out1 = d->glu; g.ld1 = I;
+    g.M = (int)M; g.N = 2 * I; g.K = H; g.n_split = 2 * I;
+    g.act = d->cfg.hidden_act; g.act_from = 0; g.glu = 1;
+    RAI_TRY(linear(d, st, g));
+
+    LinearArgs dn = linear_args_default();
+    dn.A = d->glu; dn.lda = I;
+    dn.W = ly.Wdown; dn.ldw = I;
+    dn.residual = x1; dn.ldr = H;
+    dn.out1 = x; dn.ld1 = H;
+    dn.M = (int)M; dn.N = H; dn.K = I; dn.n_split = H;
+    dn.splitk_ws = d->splitk_ws; dn.splitk_ws_bytes = d->splitk_ws_bytes;
+    RAI_TRY(linear(d, st, dn));
+  }
+
+  // last position -> final norm -> lm_head (qwen2.rs:355-357, gemma.rs:383-385)
+  LinearArgs h = linear_args_default();
+  char *last_rows = x + (size_t)(S - 1) * H * d->es;
+  if (dt == RAI_BF16 && B <= 8) {
+    h.A = last_rows; h.lda = (int64_t)S * H;
+    h.ln_kind = kind; h.ln_w = d->lnf_w; h.ln_eps = (float)d->cfg.norm_eps;
+  } else {
+    RAI_TRY(norm_rows(last_rows, d->lnf_w, d->last, B, (int64_t)S * H));
+    h.A = d->last; h.lda = H;
+  }
+  h.W = d->head_w; h.ldw = H;
+  h.out1 = d->logits; h.ld1 = d->V;
+  h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
+  RAI_TRY(linear(d, st, h));
+
+  uint32_t *hist = advance_step ? d->history : nullptr;
+  if (dt == RAI_BF16)
+    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
+                       (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
+                       (bf16_raw *)d->x, H, d->embed_scale);
+  else
+    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
+                       d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
+                       d->embed_scale);
+  RAI_TRY(launch_check("select_token"));
+  d->ctx_len = T_after;
+  return RAI_OK;
+}
+
+static int forward_any(rai_hip_decoder *d, int B, int S, bool advance_step, bool from_tokens = false) {
+  return d->cfg.arch == RAI_ARCH_PHI2 ? forward_phi2(d, B, S, advance_step, from_tokens)
+                                       : forward_seq(d, B, S, advance_step, from_tokens);
 }
 
 static int check_call(rai_hip_decoder *d, int B, int S) {
@@ -515,7 +720,8 @@ extern "C" {
 
 int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_decoder **out) {
   RAI_REQUIRE(cfg && out, RAI_ERR_BAD_ARG, "decoder_create: null argument");
-  RAI_REQUIRE(cfg->arch == RAI_ARCH_PHI2, RAI_ERR_UNSUPPORTED, "decoder_create: architecture %d not available", cfg->arch);
+  RAI_REQUIRE(cfg->arch == RAI_ARCH_PHI2 || cfg->arch == RAI_ARCH_QWEN2 || cfg->arch == RAI_ARCH_GEMMA,
+              RAI_ERR_UNSUPPORTED, "decoder_create: architecture %d not available", cfg->arch);
   RAI_REQUIRE(cfg->dtype == RAI_BF16 || cfg->dtype == RAI_F32, RAI_ERR_BAD_DTYPE, "decoder_create: bf16 or f32");
   RAI_REQUIRE(cfg->hidden_size > 0 && cfg->num_attention_heads > 0 && cfg->num_key_value_heads > 0 &&
                   cfg->num_attention_heads % cfg->num_key_value_heads == 0 && cfg->head_dim > 0 &&
@@ -549,7 +755,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   };
   if (d->H % vec || d->QD % vec || d->KD % vec || d->I % vec || d->D % vec)
     return bail(fail(RAI_ERR_BAD_SHAPE, "decoder_create: sizes must be multiples of %d elements", vec));
-  if ((st = create_phi2(d)) != RAI_OK) return bail(st);
+  d->embed_scale = 1.0f;
+  if (cfg->arch == RAI_ARCH_GEMMA) d->embed_scale = round_dt((float)sqrt((double)d->H), cfg->dtype);
+  if ((st = (cfg->arch == RAI_ARCH_PHI2 ? create_phi2(d) : create_seq(d))) != RAI_OK) return bail(st);
   const size_t es = d->es;
   d->max_rows = (int64_t)cfg->max_batch * cfg->max_context;
   const size_t kv = (size_t)d->L * cfg->max_batch * d->Hkv * cfg->max_context * d->D * es;
@@ -560,7 +768,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
       (st = dalloc(d, rope, &d->sin_t)) || (st = dalloc(d, d->max_rows * d->H * es, &d->x)) ||
       (st = dalloc(d, d->max_rows * d->H * es, &d->x2)) || (st = dalloc(d, d->max_rows * d->H * es, &d->ln)) ||
       (st = dalloc(d, d->max_rows * (d->QD + 2 * d->KD) * es, &d->qkv)) ||
-      (st = dalloc(d, d->max_rows * d->KB * es, &d->cat)) || (st = dalloc(d, (size_t)cfg->max_batch * d->H * es, &d->last)) ||
+      (st = dalloc(d, cfg->arch == RAI_ARCH_PHI2 ? d->max_rows * d->KB * es : 16, &d->cat)) ||
+      (st = dalloc(d, cfg->arch == RAI_ARCH_PHI2 ? 16 : d->max_rows * d->QD * es, &d->attn)) ||
+      (st = dalloc(d, cfg->arch == RAI_ARCH_PHI2 ? 16 : d->max_rows * d->I * es, &d->glu)) || (st = dalloc(d, (size_t)cfg->max_batch * d->H * es, &d->last)) ||
       (st = dalloc(d, (size_t)cfg->max_batch * d->V * es, &d->logits)))
     return bail(st);
   if ((st = dalloc(d, d->max_rows * sizeof(uint32_t), &tmp))) return bail(st);
@@ -643,7 +853,7 @@ int rai_hip_decoder_forward(rai_hip_decoder *d, const uint32_t *ids_host, int32_
   RAI_TRY(check_call(d, batch, seq));
   hipStream_t st = stream_of(d->dev);
   RAI_HIP_TRY(hipMemcpyAsync(d->ids, ids_host, (size_t)batch * seq * sizeof(uint32_t), hipMemcpyHostToDevice, st));
-  RAI_TRY(forward_phi2(d, batch, seq, false));
+  RAI_TRY(forward_any(d, batch, seq, false));
   if (logits_host) {
     // widen on device, then one synchronous copy
     void *ws = nullptr;
@@ -681,7 +891,7 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   RAI_HIP_TRY(hipMemcpyAsync(d->ids, prompt_host, (size_t)batch * prompt_len * sizeof(uint32_t), hipMemcpyHostToDevice, st));
   RAI_HIP_TRY(hipStreamSynchronize(st));
   RAI_HIP_TRY(hipEventRecord(e0, st));
-  int rc = forward_phi2(d, batch, prompt_len, true);
+  int rc = forward_any(d, batch, prompt_len, true);
   if (rc == RAI_OK) rc = hipEventRecord(e1, st) == hipSuccess ? RAI_OK : fail(RAI_ERR_HIP, "event record");
   // Single-token steps: the previous step left the next input embedding, the
   // token and the advanced context length on the device, so every step is the
@@ -702,7 +912,7 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
         rc = fail(RAI_ERR_HIP, "generate: begin capture failed");
         break;
       }
-      int frc = forward_phi2(d, batch, 1, true, true);
+      int frc = forward_any(d, batch, 1, true, true);
       hipError_t ce = hipStreamEndCapture(st, &g);
       if (frc != RAI_OK) { rc = frc; if (g) (void)hipGraphDestroy(g); break; }
       if (ce != hipSuccess || !g) { rc = fail(RAI_ERR_HIP, "generate: end capture failed: %s", hipGetErrorString(ce)); break; }
@@ -714,7 +924,7 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
       --step;  // run this step through the graph
       continue;
     }
-    rc = forward_phi2(d, batch, 1, true, true);
+    rc = forward_any(d, batch, 1, true, true);
   }
   if (rc == RAI_OK && hipEventRecord(e2, st) != hipSuccess) rc = fail(RAI_ERR_HIP, "event record");
   if (rc == RAI_OK && hipStreamSynchronize(st) != hipSuccess) rc = fail(RAI_ERR_HIP, "generate: stream sync failed");
@@ -742,7 +952,8 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
 int rai_hip_decoder_time_decode_linear(rai_hip_decoder *d, int32_t sweeps, float *us_per_launch,
                                        double *bytes_per_launch) {
   RAI_REQUIRE(d && us_per_launch && bytes_per_launch && sweeps > 0, RAI_ERR_BAD_ARG, "bad argument");
-  RAI_REQUIRE(d->cfg.dtype == RAI_BF16, RAI_ERR_UNSUPPORTED, "time_decode_linear: bf16 models only");
+  RAI_REQUIRE(d->cfg.dtype == RAI_BF16 && d->cfg.arch == RAI_ARCH_PHI2, RAI_ERR_UNSUPPORTED,
+              "time_decode_linear: bf16 Phi-2 models only");
   hipStream_t st = stream_of(d->dev);
   hipEvent_t e0, e1;
   RAI_HIP_TRY(hipEventCreate(&e0));

@@ -28,6 +28,10 @@ struct LinearArgs {
   int n_split;   // first column written to out2
   int act;       // rai_hip_unary_op activation or -1
   int act_from;  // activation applies to columns >= act_from
+  // Gated MLP (rai-models/src/llm/qwen2.rs:100-104: act(gate(x)) * up(x)): W rows are
+  // interleaved gate_0, up_0, gate_1, up_1, ...; N counts the interleaved rows and
+  // N/2 columns are written to out1.  No residual, no output split.
+  int glu;
   // Optional fused LayerNorm / RMSNorm of the rows of A before the product
   // (skinny path only): A is normalised with ln_w / ln_b over K.
   const void *ln_w;
@@ -56,6 +60,14 @@ int launch_linear_bf16(hipStream_t st, const LinearArgs &a);
 
 // f32 tile kernel for the same NT contraction, FMA in f32.
 int launch_linear_f32(hipStream_t st, const LinearArgs &a);
+
+__device__ __forceinline__ float act_eval(int act, float x);
+// act(gate) * up with the reference's roundings of gate, act(gate) and up to bf16.
+__device__ __forceinline__ float glu_bf16(int act, float g, float u) {
+  const float gr = bf16_bits_to_f32(f32_to_bf16_bits(g));
+  const float ar = bf16_bits_to_f32(f32_to_bf16_bits(act_eval(act, gr)));
+  return ar * bf16_bits_to_f32(f32_to_bf16_bits(u));
+}
 
 __device__ __forceinline__ float act_eval(int act, float x) {
   switch (act) {

@@ -184,7 +184,22 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
       for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int m = 0; m < MROWS; ++m) acc[r][m] = wave_sum(acc[r][m]);
-      if (lane == 0) {
+      if (lane == 0 && a.glu) {
+        if constexpr (R % 2 == 0) {
+#pragma unroll
+          for (int r = 0; r < R; r += 2) {
+            const int n = n_cur + r;
+            if (n + 1 >= n_end) break;
+            const float bg = bias ? bf16_bits_to_f32(bias[n]) : 0.f, bu = bias ? bf16_bits_to_f32(bias[n + 1]) : 0.f;
+#pragma unroll
+            for (int m = 0; m < MROWS; ++m) {
+              if (m >= a.M) break;
+              ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + (n >> 1)] =
+                  f32_to_bf16_bits(glu_bf16(a.act, acc[r][m] + bg, acc[r + 1][m] + bu));
+            }
+          }
+        }
+      } else if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           const int n = n_cur + r;
@@ -328,7 +343,17 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
     if (n_base + R < n_end) load_group(n_base + R);
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-    if (lane == 0) {
+    if (lane == 0 && a.glu) {
+      if constexpr (R % 2 == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r += 2) {
+          const int n = n_base + r;
+          if (n + 1 >= a.N || n >= n_end) break;
+          const float bg = bias ? bf16_bits_to_f32(bias[n]) : 0.f, bu = bias ? bf16_bits_to_f32(bias[n + 1]) : 0.f;
+          ((uint16_t *)a.out1)[n >> 1] = f32_to_bf16_bits(glu_bf16(a.act, acc[r] + bg, acc[r + 1] + bu));
+        }
+      }
+    } else if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int n = n_base + r;
@@ -393,6 +418,21 @@ __global__ void __launch_bounds__(256) k_linear_f32(LinearArgs a) {
   const float *bias = (const float *)a.bias;
   const float *bias2 = (const float *)a.bias2;
   const float *res = (const float *)a.residual;
+  if (a.glu) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int m = m0 + ty * 4 + i;
+      if (m >= a.M) continue;
+#pragma unroll
+      for (int j = 0; j < 4; j += 2) {
+        int n = n0 + tx * 4 + j;
+        if (n + 1 >= a.N) continue;
+        float g = acc[i][j] + (bias ? bias[n] : 0.f), u = acc[i][j + 1] + (bias ? bias[n + 1] : 0.f);
+        ((float *)a.out1)[(int64_t)m * a.ld1 + (n >> 1)] = act_eval(a.act, g) * u;
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     int m = m0 + ty * 4 + i;
@@ -527,6 +567,8 @@ int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   RAI_TRY(check_linear_args(a, 2));
   RAI_REQUIRE(a.M <= 8, RAI_ERR_BAD_SHAPE, "linear skinny: M=%d > 8", a.M);
   RAI_REQUIRE((size_t)a.M * a.K * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
+  if (a.glu) RAI_REQUIRE(a.N % 2 == 0 && !a.residual && a.n_split == a.N && a.act >= 0, RAI_ERR_BAD_ARG,
+                         "linear: bad gated-MLP arguments");
   if (a.M == 1 && a.K <= 4096 && a.N >= 1024) {
     // activation vector in registers (at most 8 chunks of 16 bytes per lane)
     if (a.K <= 2048) return launch_gemv_reg<4, 4>(st, a, 8);
@@ -546,6 +588,14 @@ int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   // About 10 waves per CU, all co-resident, each with the same number of rows.
   const int target_waves = kNumCU * 10;
   int rpw = (a.N + target_waves - 1) / target_waves;
+  if (a.glu) {  // gate/up row pairs must stay inside one row group
+    RAI_REQUIRE(a.N % 2 == 0 && !a.residual && a.n_split == a.N, RAI_ERR_BAD_ARG, "linear: bad gated-MLP arguments");
+    rpw = rpw < 2 ? 2 : (rpw / 2) * 2;
+    if (a.M == 1) return launch_skinny_cfg<1, 2, 8>(st, a, rpw);
+    if (a.M == 2) return launch_skinny_cfg<2, 2, 8>(st, a, rpw);
+    if (a.M <= 4) return launch_skinny_cfg<4, 2, 4>(st, a, rpw);
+    return launch_skinny_cfg<8, 2, 4>(st, a, rpw);
+  }
   if (a.M == 1) {
     static const char *knob = getenv("RAI_HIP_SKINNY");  // tuning aid: "R,NWV,rows_per_wave,U"
     if (knob) {

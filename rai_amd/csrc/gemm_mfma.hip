@@ -172,6 +172,23 @@ __global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits
         }
         continue;
       }
+      if (a.glu) {  // columns n..n+7 are four (gate, up) pairs -> four outputs at column n/2
+        uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
+        float gl[4];
+        for (int e = 0; e < 8; e += 2) {
+          const float g = v[e] + (bias ? bf16_bits_to_f32(bias[n + e]) : 0.f);
+          const float u = v[e + 1] + (bias ? bf16_bits_to_f32(bias[n + e + 1]) : 0.f);
+          gl[e >> 1] = glu_bf16(a.act, g, u);
+        }
+        if (n + 8 <= a.N && a.ld1 % 4 == 0 && (uintptr_t)a.out1 % 8 == 0) {
+          typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+          u32x2 o = {pack_bf16x2(gl[0], gl[1]), pack_bf16x2(gl[2], gl[3])};
+          *reinterpret_cast<u32x2 *>(dst) = o;
+        } else {
+          for (int e = 0; e < 4 && n + 2 * e + 1 < a.N; ++e) dst[e] = f32_to_bf16_bits(gl[e]);
+        }
+        continue;
+      }
       const int lim = a.N - n < 8 ? a.N - n : 8;
       for (int e = 0; e < lim; ++e) {
         const int nn = n + e;
@@ -208,6 +225,15 @@ __global__ void __launch_bounds__(256) k_splitk_epilogue(LinearArgs a, int split
   const uint16_t *res = (const uint16_t *)a.residual;
   for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
     const int m = (int)(e / a.N), n = (int)(e % a.N);
+    if (a.glu) {
+      if (n & 1) continue;
+      float g = 0.f, u = 0.f;
+      for (int s = 0; s < splits; ++s) { g += partial[(int64_t)s * total + e]; u += partial[(int64_t)s * total + e + 1]; }
+      g += bias ? bf16_bits_to_f32(bias[n]) : 0.f;
+      u += bias ? bf16_bits_to_f32(bias[n + 1]) : 0.f;
+      ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + (n >> 1)] = f32_to_bf16_bits(glu_bf16(a.act, g, u));
+      continue;
+    }
     float x = 0.f;
     for (int s = 0; s < splits; ++s) x += partial[(int64_t)s * total + e];
     x += (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
@@ -254,6 +280,8 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.n_split >= 0 && a.n_split <= a.N && (a.n_split == a.N || a.out2), RAI_ERR_BAD_ARG,
               "linear: bad output split");
   RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear: fused norm only on the skinny path");
+  if (a.glu) RAI_REQUIRE(a.N % 8 == 0 && !a.residual && a.n_split == a.N && a.act >= 0, RAI_ERR_BAD_ARG,
+                         "linear mfma: bad gated-MLP arguments");
   RAI_REQUIRE(a.K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear mfma: K=%d must be a multiple of 32", a.K);
   RAI_REQUIRE(a.lda % 8 == 0 && a.ldw % 8 == 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0,
               RAI_ERR_BAD_STRIDE, "linear mfma: operands must be 16-byte aligned with row strides multiple of 8");
