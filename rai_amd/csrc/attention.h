@@ -42,7 +42,14 @@ struct AttnDecodeArgs {
   float scale;
   int f32_scores;
   int dtype;
+  // Partial results of the context splits: ws holds attention_decode_ws_bytes()
+  // bytes, counters attention_decode_counter_bytes() bytes that are zero between launches.
+  float *ws;
+  int *counters;
+  int ns, chunk_cap;  // filled in by the launcher
 };
+size_t attention_decode_ws_bytes(int B, int Hq, int D);
+size_t attention_decode_counter_bytes(int B, int Hq);
 int launch_attention_decode(hipStream_t st, const AttnDecodeArgs &a);
 
 }  // namespace rai

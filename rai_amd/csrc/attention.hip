@@ -8,6 +8,8 @@
 // f32 softmax, P cast to V's dtype), qwen2.rs:205-221 and gemma.rs:238-254
 // (scores, scale and softmax rounded to the model dtype), repeat_kv
 // gemma.rs:191-201 (query head h reads kv head h / (Hq/Hkv)).
+#include <cstdlib>
+
 #include "attention.h"
 
 namespace rai {
@@ -143,35 +145,65 @@ __device__ __forceinline__ float rope_feature(const T *head, int d, int rot, con
   return round_to<T>(round_to<T>(v * c) + round_to<T>(other * s));
 }
 
-// Decode attention: one 1024-thread block per (head, batch) streams the head's
-// cached K and V once.  Every 16-lane group keeps UK key rows and every thread
-// UV value chunks (16-byte loads) in flight, and the first round of both is
-// issued before anything else is computed, so a context of up to 64*UK keys
-// costs one HBM round trip for K and V together.  The new token's rotated key
-// and value are appended to the cache by the block and used from LDS.
-// Probabilities stay in f32 until the product with V (the reference rounds them
-// to V's dtype first).
-constexpr int kDecodeThreads = 1024;
-template <typename T, int CC, int UK, int UV>
-__global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a) {
-  constexpr int V = AttnVec<T>::V;
-  constexpr int NW = kDecodeThreads / 64, NG = kDecodeThreads / 16;
-  extern __shared__ __attribute__((aligned(16))) float smem[];
-  // layout: q[D] | knew[D] | vnew[D] | red[groups*D] | scores[Tmax+1]
-  const int D = a.D, ncol = D / V;
-  const int groups = kDecodeThreads / ncol;
-  float *qf = smem;
-  float *knew = qf + D;
-  float *vnew = knew + D;
-  float *red = vnew + D;
-  float *scores = red + groups * D;
-  __shared__ float sh[2 * NW];
+// Decode attention, split over the context ("flash decoding"): block
+// (split, kv-head group, batch) handles ceil((pos+1)/NS) consecutive keys for
+// the R query heads that share one KV head, so the cached K and V are read once
+// per KV head (repeat_kv is never materialised) and NS * Hkv * B blocks keep
+// every CU busy even at batch 1.  All of a block's first K and V loads are
+// issued before anything is computed: a short context costs one HBM round trip.
+// Each block writes an unnormalised partial (running max m, sum l, o[D]) per
+// query head; the last block of a head group to finish (device-scope counter)
+// merges the NS partials and writes the output row.  The new token's rotated
+// key and value are appended to the cache by the block that owns position pos
+// and are used from LDS.  Probabilities stay in f32 until the product with V.
+constexpr int kDecodeThreads = 256;
+constexpr int kDecodeMaxSplits = 64;
+constexpr int kDecodeCounterStride = 32;
 
-  const int h = blockIdx.x, b = blockIdx.y;
+// Device-scope accesses for data handed from one block to another inside a
+// kernel.  The L2 of each XCD is not coherent with the others for ordinary
+// accesses, and a device-scope fence writes back and invalidates a whole L2;
+// relaxed device-scope atomics instead write through / read around the L2 for
+// just the words involved.
+__device__ __forceinline__ void store_device(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_device(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T, int R, int CC, int UK, int UV>
+__global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_split(AttnDecodeArgs a) {
+  constexpr int V = AttnVec<T>::V;
+  constexpr int NT = kDecodeThreads, NW = NT / 64;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int D = a.D, ncol = D / V, groups = NT / ncol;
+  const int NS = a.ns, CH = a.chunk_cap;
+  // layout: q[R*D] | knew[D] | vnew[D] | scores[R*CH] | red[groups*R*D]
+  float *qf = smem;
+  float *knew = qf + R * D;
+  float *vnew = knew + D;
+  float *scores = vnew + D;
+  float *red = scores + R * CH;
+  __shared__ float sh_m[R], sh_l[R];
+  __shared__ int sh_last;
+
+  const int s = blockIdx.x, b = blockIdx.z;
+  const int hq0 = blockIdx.y * R;           // first query head of this block
+  const int n_rep = a.Hq / a.Hkv, hk = hq0 / n_rep;
+  const bool writer = hq0 % n_rep == 0;     // one block per KV head appends the new token
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_rep = a.Hq / a.Hkv, hk = h / n_rep;
   int pos = *a.pos_dev;
-  if (pos > a.Tmax - 1) pos = a.Tmax - 1;  // capacity is checked on the host; never write past the cache
+  if (pos > a.Tmax - 1) pos = a.Tmax - 1;   // capacity is checked on the host; never write past the cache
+  const int cnt = pos + 1;
+  int chunk = (cnt + NS - 1) / NS;
+  if (chunk > CH) chunk = CH;
+  const int t0 = s * chunk;
+  const int t1 = t0 + chunk < cnt ? t0 + chunk : cnt;
+  const int n = t1 > t0 ? t1 - t0 : 0;      // keys of this split (the new token included when it falls inside)
+  const bool has_new = pos >= t0 && pos < t1;
+  const int t1c = has_new ? pos : t1;       // cached keys are [t0, t1c)
+
   const int QD = a.Hq * D, KD = a.Hkv * D;
   const T *row = (const T *)a.qkv + (int64_t)b * (QD + 2 * KD);
   T *Kc = (T *)a.kcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
@@ -180,38 +212,37 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a
   const int g = tid >> 4, gl = tid & 15;
   const int col = tid % ncol, grp = tid / ncol;
 
-  // Loads return in issue order.  The few values of the new token (q, k, v and
-  // their rotary factors) are requested first, the first round of cached K and V
-  // right behind them, so the rotary prologue runs while K and V are in flight.
-  float q_rot = 0.f, k_rot = 0.f, v_new = 0.f;
-  const int d0 = tid;  // one feature per thread (D <= 1024)
-  if (d0 < D) {
-    q_rot = rope_feature<T>(row + h * D, d0, a.rot, cos_t, sin_t, pos);
-    k_rot = rope_feature<T>(row + QD + hk * D, d0, a.rot, cos_t, sin_t, pos);
-    v_new = (float)Scalar<T>::load(row + QD + KD + hk * D + d0);
-  }
+  // ---- first round of K and V loads
   APack<T, V> kreg[UK][CC], vreg[UV];
 #pragma unroll
   for (int u = 0; u < UK; ++u) {
-    const int t = g + NG * u;
+    const int t = t0 + g + 16 * u;
 #pragma unroll
     for (int cc = 0; cc < CC; ++cc) {
       const int c = gl + 16 * cc;
-      if (t < pos && c < ncol) kreg[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
+      if (t < t1c && c < ncol) kreg[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
     }
   }
 #pragma unroll
   for (int u = 0; u < UV; ++u) {
-    const int t = grp + u * groups;
-    if (grp < groups && t < pos) vreg[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+    const int t = t0 + grp + u * groups;
+    if (grp < groups && t < t1c) vreg[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
   }
-  if (d0 < D) {
-    qf[d0] = q_rot;
-    knew[d0] = k_rot;
-    vnew[d0] = v_new;
-    if (h % n_rep == 0) {
-      Scalar<T>::store(Kc + (int64_t)pos * D + d0, (typename Scalar<T>::compute)k_rot);
-      Scalar<T>::store(Vc + (int64_t)pos * D + d0, (typename Scalar<T>::compute)v_new);
+  // ---- rotary embedding of the R query rows (and of the new key where it is needed)
+  for (int e = tid; e < R * D; e += NT) {
+    const int r = e / D, d = e - r * D;
+    qf[e] = rope_feature<T>(row + (hq0 + r) * D, d, a.rot, cos_t, sin_t, pos);
+  }
+  if (has_new) {
+    for (int d = tid; d < D; d += NT) {
+      const float kr = rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos);
+      const float vr = (float)Scalar<T>::load(row + QD + KD + hk * D + d);
+      knew[d] = kr;
+      vnew[d] = vr;
+      if (writer) {
+        Scalar<T>::store(Kc + (int64_t)pos * D + d, (typename Scalar<T>::compute)kr);
+        Scalar<T>::store(Vc + (int64_t)pos * D + d, (typename Scalar<T>::compute)vr);
+      }
     }
   }
   __syncthreads();
@@ -220,131 +251,232 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode(AttnDecodeArgs a
     if (a.f32_scores) return acc * a.scale;
     return round_to<T>(round_to<T>(acc) * round_to<T>(a.scale));
   };
-  // ---- scores against the cached keys [0, pos): round 0 from the prefetched registers
-  for (int tb = g; tb < pos; tb += UK * NG) {
-    if (tb != g) {
+  // ---- scores against the cached keys: 16 lanes per key row, round 0 from the prefetched registers
+  for (int tb = t0 + g; tb < t1c; tb += 16 * UK) {
+    if (tb != t0 + g) {
 #pragma unroll
       for (int u = 0; u < UK; ++u) {
-        const int t = tb + NG * u;
+        const int t = tb + 16 * u;
 #pragma unroll
         for (int cc = 0; cc < CC; ++cc) {
           const int c = gl + 16 * cc;
-          if (t < pos && c < ncol) kreg[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
+          if (t < t1c && c < ncol) kreg[u][cc] = *reinterpret_cast<const APack<T, V> *>(Kc + (int64_t)t * D + c * V);
         }
       }
     }
 #pragma unroll
     for (int u = 0; u < UK; ++u) {
-      const int t = tb + NG * u;
-      float acc = 0.f;
+      const int t = tb + 16 * u;
+      float kf[CC][V];
 #pragma unroll
-      for (int cc = 0; cc < CC; ++cc) {
-        const int c = gl + 16 * cc;
-        if (t < pos && c < ncol) {
+      for (int cc = 0; cc < CC; ++cc)
 #pragma unroll
-          for (int j = 0; j < V; ++j) acc = fmaf(qf[c * V + j], (float)Scalar<T>::load(&kreg[u][cc].v[j]), acc);
+        for (int j = 0; j < V; ++j) kf[cc][j] = (float)Scalar<T>::load(&kreg[u][cc].v[j]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float acc = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < CC; ++cc) {
+          const int c = gl + 16 * cc;
+          if (t < t1c && c < ncol) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc = fmaf(qf[r * D + c * V + j], kf[cc][j], acc);
+          }
         }
+        acc += __shfl_xor(acc, 8, 64);
+        acc += __shfl_xor(acc, 4, 64);
+        acc += __shfl_xor(acc, 2, 64);
+        acc += __shfl_xor(acc, 1, 64);
+        if (gl == 0 && t < t1c) scores[r * CH + (t - t0)] = finish_score(acc);
       }
-      acc += __shfl_xor(acc, 8, 64);
-      acc += __shfl_xor(acc, 4, 64);
-      acc += __shfl_xor(acc, 2, 64);
-      acc += __shfl_xor(acc, 1, 64);
-      if (gl == 0 && t < pos) scores[t] = finish_score(acc);
     }
   }
-  if (wave == NW - 1) {  // the new token's own key, still in LDS
-    float acc = 0.f;
-    for (int d = lane; d < D; d += 64) acc = fmaf(qf[d], knew[d], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) scores[pos] = finish_score(acc);
+  if (has_new && wave == NW - 1) {  // the new token's own key, still in LDS
+    for (int r = 0; r < R; ++r) {
+      float acc = 0.f;
+      for (int d = lane; d < D; d += 64) acc = fmaf(qf[r * D + d], knew[d], acc);
+      acc = wave_sum(acc);
+      if (lane == 0) scores[r * CH + (pos - t0)] = finish_score(acc);
+    }
   }
   __syncthreads();
-  const int cnt = pos + 1;
-  float m = -INFINITY;
-  for (int t = tid; t < cnt; t += kDecodeThreads) m = fmaxf(m, scores[t]);
-  m = wave_max(m);
-  if (lane == 0) sh[wave] = m;
-  __syncthreads();
-  m = sh[0];
-  for (int w = 1; w < NW; ++w) m = fmaxf(m, sh[w]);
-  float sum = 0.f;
-  for (int t = tid; t < cnt; t += kDecodeThreads) {
-    float e = expf(scores[t] - m);
-    scores[t] = e;
-    sum += e;
+  // ---- partial softmax statistics, one wave per query head
+  for (int r = wave; r < R; r += NW) {
+    float m = -INFINITY;
+    for (int t = lane; t < n; t += 64) m = fmaxf(m, scores[r * CH + t]);
+    m = wave_max(m);
+    float l = 0.f;
+    for (int t = lane; t < n; t += 64) {
+      const float e = expf(scores[r * CH + t] - m);
+      scores[r * CH + t] = e;
+      l += e;
+    }
+    l = wave_sum(l);
+    if (lane == 0) { sh_m[r] = m; sh_l[r] = l; }
   }
-  sum = wave_sum(sum);
-  if (lane == 0) sh[NW + wave] = sum;
   __syncthreads();
-  sum = 0.f;
-  for (int w = 0; w < NW; ++w) sum += sh[NW + w];
   // ---- unnormalised P.V over the cached values: round 0 from the prefetched registers
   {
-    float acc[V];
+    float acc[R][V];
 #pragma unroll
-    for (int j = 0; j < V; ++j) acc[j] = 0.f;
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < V; ++j) acc[r][j] = 0.f;
     if (grp < groups) {
-      for (int tb = grp; tb < pos; tb += UV * groups) {
-        if (tb != grp) {
+      for (int tb = t0 + grp; tb < t1c; tb += UV * groups) {
+        if (tb != t0 + grp) {
 #pragma unroll
           for (int u = 0; u < UV; ++u) {
             const int t = tb + u * groups;
-            if (t < pos) vreg[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
+            if (t < t1c) vreg[u] = *reinterpret_cast<const APack<T, V> *>(Vc + (int64_t)t * D + col * V);
           }
         }
 #pragma unroll
         for (int u = 0; u < UV; ++u) {
           const int t = tb + u * groups;
-          if (t < pos) {
-            const float p = scores[t];
+          if (t < t1c) {
+            float vf[V];
 #pragma unroll
-            for (int j = 0; j < V; ++j) acc[j] = fmaf(p, (float)Scalar<T>::load(&vreg[u].v[j]), acc[j]);
+            for (int j = 0; j < V; ++j) vf[j] = (float)Scalar<T>::load(&vreg[u].v[j]);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const float p = scores[r * CH + (t - t0)];
+#pragma unroll
+              for (int j = 0; j < V; ++j) acc[r][j] = fmaf(p, vf[j], acc[r][j]);
+            }
           }
         }
       }
 #pragma unroll
-      for (int j = 0; j < V; ++j) red[grp * D + col * V + j] = acc[j];
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < V; ++j) red[(grp * R + r) * D + col * V + j] = acc[r][j];
     }
   }
   __syncthreads();
-  T *o = (T *)a.out + (int64_t)b * a.out_row_stride + (int64_t)h * D;
-  const float p_new = scores[pos], inv = 1.0f / sum;
-  for (int d = tid; d < D; d += kDecodeThreads) {
-    float r = p_new * vnew[d];
-    for (int gg = 0; gg < groups; ++gg) r += red[gg * D + d];
-    Scalar<T>::store(o + d, (typename Scalar<T>::compute)(r * inv));
+  // ---- partial (m, l, o[D]) of every query head of the block
+  const int PW = D + 2;
+  float *part = a.ws + (((int64_t)b * a.Hq + hq0) * NS + s) * PW;  // head r at part + r*NS*PW
+  for (int e = tid; e < R * D; e += NT) {
+    const int r = e / D, d = e - r * D;
+    float o = has_new ? scores[r * CH + (pos - t0)] * vnew[d] : 0.f;
+    for (int gg = 0; gg < groups; ++gg) o += red[(gg * R + r) * D + d];
+    store_device(part + (int64_t)r * NS * PW + 2 + d, o);
   }
+  if (tid < R) {
+    store_device(part + (int64_t)tid * NS * PW, sh_m[tid]);
+    store_device(part + (int64_t)tid * NS * PW + 1, sh_l[tid]);
+  }
+  // ---- the last block of this head group merges the partials: every thread's
+  //      write-through stores have completed before the block's arrival is counted
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  int *counter = a.counters + ((int64_t)b * a.Hq + hq0) * kDecodeCounterStride;  // one 128-byte line each
+  if (tid == 0) sh_last = atomicAdd(counter, 1) == NS - 1;
+  __syncthreads();
+  if (!sh_last) return;
+  // All loads of a batch of splits are in flight together (statistics and the
+  // thread's output feature), so the merge costs one memory round trip per
+  // batch of kMergeBatch splits rather than one per split.
+  constexpr int kMergeBatch = 8;
+  const float *all = a.ws + ((int64_t)b * a.Hq + hq0) * NS * PW;
+  for (int e = tid; e < R * D; e += NT) {
+    const int r = e / D, d = e - r * D;
+    const float *pr = all + (int64_t)r * NS * PW;
+    float M = -INFINITY, L = 0.f, O = 0.f;
+    for (int s0 = 0; s0 < NS; s0 += kMergeBatch) {
+      float mv[kMergeBatch], lv[kMergeBatch], ov[kMergeBatch];
+#pragma unroll
+      for (int j = 0; j < kMergeBatch; ++j) {
+        const int ss = s0 + j < NS ? s0 + j : NS - 1;
+        mv[j] = load_device(pr + ss * PW);
+        lv[j] = load_device(pr + ss * PW + 1);
+        ov[j] = load_device(pr + ss * PW + 2 + d);
+      }
+      float mb = M;
+#pragma unroll
+      for (int j = 0; j < kMergeBatch; ++j) mb = fmaxf(mb, mv[j]);
+      const float rescale = expf(M - mb);  // M = -inf on the first batch: 0 (split 0 always holds a key, so mb is finite)
+      L *= rescale;
+      O *= rescale;
+      M = mb;
+#pragma unroll
+      for (int j = 0; j < kMergeBatch; ++j) {
+        if (s0 + j < NS) {
+          const float w = expf(mv[j] - M);  // an empty split has m = -inf: weight 0
+          L = fmaf(w, lv[j], L);
+          O = fmaf(w, ov[j], O);
+        }
+      }
+    }
+    Scalar<T>::store((T *)a.out + (int64_t)b * a.out_row_stride + (int64_t)(hq0 + r) * D + d,
+                     (typename Scalar<T>::compute)(O / L));
+  }
+  if (tid == 0) *counter = 0;  // ready for the next launch (stream order)
 }
 
-template <typename T, int CC, int UK, int UV> static int launch_decode_cfg(hipStream_t st, const AttnDecodeArgs &a) {
+// Number of context splits: enough blocks to fill the chip, bounded so that a
+// block's share of the longest context fits the LDS score buffer.
+static int decode_splits(const AttnDecodeArgs &a, int head_groups) {
+  static const int forced = getenv("RAI_HIP_ATTN_SPLITS") ? atoi(getenv("RAI_HIP_ATTN_SPLITS")) : 0;
+  int ns = forced > 0 ? forced : (2 * kNumCU + head_groups * a.B - 1) / (head_groups * a.B);
+  const int need = (a.Tmax + 1023) / 1024;
+  if (ns < need) ns = need;
+  if (ns > kDecodeMaxSplits) ns = kDecodeMaxSplits;
+  if (ns > a.Tmax) ns = a.Tmax;
+  return ns < 1 ? 1 : ns;
+}
+
+size_t attention_decode_ws_bytes(int B, int Hq, int D) {
+  return sizeof(float) * (size_t)B * Hq * kDecodeMaxSplits * (D + 2);
+}
+size_t attention_decode_counter_bytes(int B, int Hq) { return sizeof(int) * (size_t)B * Hq * kDecodeCounterStride; }
+
+template <typename T, int R, int CC, int UK, int UV> static int launch_decode_cfg(hipStream_t st, AttnDecodeArgs a) {
   constexpr int V = AttnVec<T>::V;
   const int ncol = a.D / V, groups = kDecodeThreads / ncol;
-  const size_t lds = sizeof(float) * (3 * (size_t)a.D + (size_t)groups * a.D + (size_t)a.Tmax + 1);
+  const int head_groups = a.Hq / R;
+  a.ns = decode_splits(a, head_groups);
+  a.chunk_cap = (a.Tmax + a.ns - 1) / a.ns;
+  const size_t lds = sizeof(float) * ((size_t)R * a.D + 2 * (size_t)a.D + (size_t)R * a.chunk_cap + (size_t)groups * R * a.D);
   RAI_REQUIRE(lds <= 150 * 1024, RAI_ERR_UNSUPPORTED, "attention: context %d too long for the decode kernel", a.Tmax);
   static size_t attr_bytes = 0;
   if (lds > 64 * 1024 && lds > attr_bytes) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_decode<T, CC, UK, UV>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_decode_split<T, R, CC, UK, UV>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024));
     attr_bytes = 150 * 1024;
   }
-  hipLaunchKernelGGL((k_attn_decode<T, CC, UK, UV>), dim3(a.Hq, a.B), dim3(kDecodeThreads), lds, st, a);
+  RAI_REQUIRE(head_groups <= 65535 && a.B <= 65535, RAI_ERR_UNSUPPORTED, "attention decode: grid too large");
+  hipLaunchKernelGGL((k_attn_decode_split<T, R, CC, UK, UV>), dim3(a.ns, head_groups, a.B), dim3(kDecodeThreads), lds, st, a);
   return launch_check("attention_decode");
+}
+
+template <typename T, int R> static int launch_decode_r(hipStream_t st, const AttnDecodeArgs &a) {
+  constexpr int V = AttnVec<T>::V;
+  const int ncol = a.D / V;
+  if (ncol <= 16) return launch_decode_cfg<T, R, 1, 3, 3>(st, a);
+  if (ncol <= 32) return launch_decode_cfg<T, R, 2, 2, 4>(st, a);
+  return launch_decode_cfg<T, R, 4, 1, 2>(st, a);
 }
 
 template <typename T> static int launch_decode(hipStream_t st, const AttnDecodeArgs &a) {
   constexpr int V = AttnVec<T>::V;
   RAI_REQUIRE(a.D % V == 0 && a.D / V <= 64, RAI_ERR_BAD_SHAPE, "attention: head_dim %d unsupported", a.D);
-  const int ncol = a.D / V;
-  // register budget at 1024 threads per block is 128 VGPRs: (UK*CC + UV) 16-byte packs
-  if (ncol <= 16) return launch_decode_cfg<T, 1, 10, 7>(st, a);
-  if (ncol <= 32) return launch_decode_cfg<T, 2, 5, 6>(st, a);
-  return launch_decode_cfg<T, 4, 2, 6>(st, a);
+  // the query heads of one KV head share a block when their count has an instantiation
+  switch (a.Hq / a.Hkv) {
+    case 2: return launch_decode_r<T, 2>(st, a);
+    case 4: return launch_decode_r<T, 4>(st, a);
+    case 6: return launch_decode_r<T, 6>(st, a);
+    case 8: return launch_decode_r<T, 8>(st, a);
+    default: return launch_decode_r<T, 1>(st, a);
+  }
 }
 
 int launch_attention_decode(hipStream_t st, const AttnDecodeArgs &a) {
   RAI_REQUIRE(a.B > 0 && a.Hq > 0 && a.Hkv > 0 && a.D > 0 && a.Tmax > 0 && a.Hq % a.Hkv == 0, RAI_ERR_BAD_SHAPE,
               "attention decode: bad problem");
   RAI_REQUIRE(a.rot > 0 && a.rot % 2 == 0 && a.rot <= a.D, RAI_ERR_BAD_ARG, "attention decode: rot %d", a.rot);
+  RAI_REQUIRE(a.ws && a.counters, RAI_ERR_BAD_ARG, "attention decode: partial-result workspace missing");
   switch (a.dtype) {
     case RAI_F32: return launch_decode<float>(st, a);
     case RAI_BF16: return launch_decode<bf16_raw>(st, a);

@@ -65,6 +65,8 @@ struct rai_hip_decoder {
   // activations (sized for max_batch * max_context rows)
   char *x, *x2, *ln, *qkv, *cat, *last, *logits;
   char *attn, *glu;   // sequential block: attention output [rows, QD], gated MLP activation [rows, I]
+  char *attn_ws;      // partial results of the decode attention's context splits
+  int *attn_counters; // per (batch, head) arrival counters of those splits (zero between launches)
   float embed_scale;  // Gemma: sqrt(hidden) rounded to the model dtype; 1 otherwise
   uint32_t *ids, *tokens, *history;
   char *splitk_ws;        // f32 scratch for prefill GEMMs that split K
@@ -494,6 +496,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
       t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.D = d->D; t.Tmax = d->cfg.max_context;
       t.scale = (float)(1.0 / sqrt((double)d->D));
       t.f32_scores = 1; t.dtype = dt;
+      t.ws = (float *)d->attn_ws; t.counters = d->attn_counters;
       RAI_TRY(launch_attention_decode(st, t));
     } else {
       if (dt == RAI_BF16) launch_rope_append<bf16_raw>(d, st, l, B, S); else launch_rope_append<float>(d, st, l, B, S);
@@ -612,6 +615,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
       t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.D = d->D; t.Tmax = d->cfg.max_context;
       t.scale = (float)(1.0 / sqrt((double)d->D));
       t.f32_scores = 0; t.dtype = dt;
+      t.ws = (float *)d->attn_ws; t.counters = d->attn_counters;
       RAI_TRY(launch_attention_decode(st, t));
     } else {
       if (dt == RAI_BF16) launch_rope_append<bf16_raw>(d, st, l, B, S); else launch_rope_append<float>(d, st, l, B, S);
@@ -784,6 +788,11 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->splitk_ws_bytes = (size_t)8 * d->max_rows * d->H * sizeof(float);
   if (d->splitk_ws_bytes > ((size_t)256 << 20)) d->splitk_ws_bytes = (size_t)256 << 20;
   if ((st = dalloc(d, d->splitk_ws_bytes, &d->splitk_ws))) return bail(st);
+  if ((st = dalloc(d, attention_decode_ws_bytes(cfg->max_batch, d->Hq, d->D), &d->attn_ws))) return bail(st);
+  if ((st = dalloc(d, attention_decode_counter_bytes(cfg->max_batch, d->Hq), &tmp))) return bail(st);
+  d->attn_counters = (int *)tmp;
+  if (hipMemset(d->attn_counters, 0, attention_decode_counter_bytes(cfg->max_batch, d->Hq)) != hipSuccess)
+    return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
 
   if (hipMemset(d->state, 0, sizeof(DevState)) != hipSuccess || hipMemset(d->kcache, 0, kv) != hipSuccess ||
       hipMemset(d->vcache, 0, kv) != hipSuccess)
