@@ -1,0 +1,43 @@
+// Launcher of the persistent per-token decode kernel (Phi-2 architecture,
+// batch 1, bf16) and the device-side decode state shared with the decoder
+// drivers.
+#pragma once
+#include "common.h"
+
+namespace rai {
+
+struct DevState {
+  int pos;    // tokens already in the KV cache
+  int step;   // greedy steps taken by the current generate call
+  int done;   // blocks of the token-selection kernel that have finished (reset by the last one)
+  int fault;  // set by a grid barrier that timed out; checked by the host after a generate call
+};
+
+struct MegaLayer {
+  const uint16_t *Wa, *ba;            // [NA, H] rows q | k | v | fc1, and their biases
+  const uint16_t *Wb, *bd, *bf;       // [H, QD + I] row n = dense[n, :] | fc2[n, :], and both biases
+  const uint16_t *ln_w, *ln_b;
+};
+
+struct MegaArgs {
+  const MegaLayer *layers;  // device array [L]
+  int L, H, I, QD, NA, n_qkv, Hq, rot, Tmax;
+  uint16_t *x;              // [H] residual stream, updated in place
+  uint16_t *qkv;            // [3 * QD]
+  uint16_t *act_buf;        // [I] gelu(fc1)
+  uint16_t *attn;           // [QD]
+  uint16_t *kcache, *vcache;
+  int64_t kv_layer_stride;  // elements between consecutive layers of the cache
+  const uint16_t *cos_t, *sin_t;
+  DevState *state;
+  unsigned *barrier;        // arrival counter, zero at launch
+  float ln_eps, scale;
+  int act;
+  int rows_attn;            // rows of phases B/C given to each attention block
+  unsigned long long *prof; // optional [blocks][L][8] time stamps (debugging aid), or null
+};
+
+bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why);
+int launch_phi2_decode_step(hipStream_t st, const MegaArgs &a, int D, int num_cu);
+
+}  // namespace rai

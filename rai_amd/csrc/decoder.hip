@@ -20,6 +20,7 @@
 #include <vector>
 
 #include "attention.h"
+#include "decode_mega.h"
 #include "gemm.h"
 
 namespace rai {
@@ -38,13 +39,6 @@ struct Layer {
   // Qwen2 / Gemma (sequential block): Wqkv [QD+2KD, H] (+bqkv), Wo [H, QD] (+bo),
   // Wgu [2I, H] with gate/up rows interleaved, Wdown [H, I], two RMSNorm weights
   char *Wqkv, *bqkv, *Wo, *bo, *Wgu, *Wdown, *n1_w, *n2_w;
-};
-
-struct DevState {
-  int pos;    // tokens already in the KV cache
-  int step;   // greedy steps taken by the current generate call
-  int done;   // blocks of the token-selection kernel that have finished (reset by the last one)
-  int pad;
 };
 
 }  // namespace rai
@@ -76,6 +70,12 @@ struct rai_hip_decoder {
   int ctx_len;
   int64_t max_rows;
   int history_cap;
+  // persistent per-token kernel (Phi-2, bf16, batch 1): per-layer pointer table, barrier counter
+  MegaLayer *mega_layers;
+  unsigned *mega_barrier;
+  unsigned long long *mega_prof;  // time stamps of the persistent kernel when RAI_HIP_MEGA_PROF is set
+  bool mega_ok;
+  int num_cu;
   hipGraphExec_t step_graph;  // one captured single-token step (batch step_graph_batch)
   int step_graph_batch;
   bool x_holds_next;          // d->x already holds the embedding of d->tokens
@@ -175,7 +175,7 @@ __global__ void k_set_state(DevState *st, int pos, int step) {
 template <typename T>
 __global__ void __launch_bounds__(1024)
 k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
-               int dstep, const T *embed, T *x_next, int H, float embed_scale) {
+               int dstep, const T *embed, T *x_next, int H, float embed_scale, unsigned *grid_barrier) {
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   __shared__ uint32_t chosen;
@@ -223,6 +223,7 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
     __threadfence();
     int prev = atomicAdd(&state->done, 1);
     if (prev == B - 1) {  // every block has read `step` and written its outputs
+      if (grid_barrier) *grid_barrier = 0;  // the persistent decode kernel of this step has finished
       state->done = 0;
       state->pos += dpos;
       state->step += dstep;
@@ -443,6 +444,26 @@ static int linear(rai_hip_decoder *d, hipStream_t st, const LinearArgs &a) {
   return d->cfg.dtype == RAI_BF16 ? launch_linear_bf16(st, a) : launch_linear_f32(st, a);
 }
 
+static MegaArgs mega_args(rai_hip_decoder *d) {
+  MegaArgs m;
+  memset(&m, 0, sizeof(m));
+  m.layers = d->mega_layers;
+  m.L = d->L; m.H = d->H; m.I = d->I; m.QD = d->QD; m.NA = d->NA; m.n_qkv = d->QD + 2 * d->KD;
+  m.Hq = d->Hq; m.rot = d->cfg.rotary_dim; m.Tmax = d->cfg.max_context;
+  m.x = (uint16_t *)d->x; m.qkv = (uint16_t *)d->qkv;
+  m.attn = (uint16_t *)d->cat; m.act_buf = (uint16_t *)d->cat + d->QD;
+  m.kcache = (uint16_t *)d->kcache; m.vcache = (uint16_t *)d->vcache;
+  m.kv_layer_stride = (int64_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
+  m.cos_t = (const uint16_t *)d->cos_t; m.sin_t = (const uint16_t *)d->sin_t;
+  m.state = d->state; m.barrier = d->mega_barrier;
+  m.ln_eps = (float)d->cfg.norm_eps; m.scale = (float)(1.0 / sqrt((double)d->D));
+  m.act = d->cfg.hidden_act;
+  static const int rows_attn = getenv("RAI_HIP_MEGA_ROWS_ATTN") ? atoi(getenv("RAI_HIP_MEGA_ROWS_ATTN")) : 4;
+  m.rows_attn = rows_attn;
+  m.prof = d->mega_prof;
+  return m;
+}
+
 // ids (B*S u32) are already in d->ids; device state holds the context length.
 // With from_tokens the input embeddings were already written to d->x by the
 // previous step's token selection (single-token steps only).
@@ -462,7 +483,12 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   }
 
   char *x = d->x, *xn = d->x2;
-  for (int l = 0; l < d->L; ++l) {
+  const bool use_mega = S == 1 && B == 1 && d->mega_ok;
+  if (use_mega) {
+    MegaArgs m = mega_args(d);
+    RAI_TRY(launch_phi2_decode_step(st, m, d->D, d->num_cu));
+  }
+  for (int l = 0; l < (use_mega ? 0 : d->L); ++l) {
     const Layer &ly = d->layers[l];
     LinearArgs a = linear_args_default();
     if (fuse_ln) {
@@ -553,11 +579,11 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale);
+                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale);
+                       d->embed_scale, d->mega_barrier);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
@@ -690,11 +716,11 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale);
+                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale);
+                       d->embed_scale, d->mega_barrier);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
@@ -703,6 +729,33 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
 static int forward_any(rai_hip_decoder *d, int B, int S, bool advance_step, bool from_tokens = false) {
   return d->cfg.arch == RAI_ARCH_PHI2 ? forward_phi2(d, B, S, advance_step, from_tokens)
                                        : forward_seq(d, B, S, advance_step, from_tokens);
+}
+
+// A grid barrier of the persistent decode kernel that timed out leaves
+// DevState::fault set; the results of that step are not valid.
+static int check_fault(rai_hip_decoder *d) {
+  if (!d->mega_ok) return RAI_OK;
+  DevState hs;
+  RAI_TRY(rai_hip_d2h(d->dev, &hs, d->state, sizeof(hs)));
+  if (d->mega_prof) {  // phase timings of the last token: mean over layers, for three blocks
+    std::vector<unsigned long long> t((size_t)d->num_cu * d->L * 8);
+    RAI_HIP_TRY(hipMemcpy(t.data(), d->mega_prof, t.size() * 8, hipMemcpyDeviceToHost));
+    const int blocks[4] = {0, d->Hq - 1, d->Hq, d->num_cu - 1};
+    for (int bi = 0; bi < 4; ++bi) {
+      double iv[7] = {0, 0, 0, 0, 0, 0, 0};
+      const int b = blocks[bi];
+      for (int l = 0; l < d->L; ++l)
+        for (int k = 0; k < 7; ++k)
+          iv[k] += (double)(t[((size_t)b * d->L + l) * 8 + k + 1] - t[((size_t)b * d->L + l) * 8 + k]) * 0.01 / d->L;
+      fprintf(stderr, "mega prof block %3d: A %.2f | bar %.2f | B-pre(attn) %.2f | B-stream %.2f | bar %.2f | C %.2f | bar %.2f us\n",
+              b, iv[0], iv[1], iv[2], iv[3], iv[4], iv[5], iv[6]);
+    }
+  }
+  if (hs.fault == 0) return RAI_OK;
+  hs.fault = 0;
+  RAI_HIP_TRY(hipMemcpy(&d->state->fault, &hs.fault, sizeof(int), hipMemcpyHostToDevice));
+  RAI_HIP_TRY(hipMemset(d->mega_barrier, 0, sizeof(unsigned)));
+  return fail(RAI_ERR_HIP, "decoder: a grid barrier of the persistent decode kernel timed out");
 }
 
 static int check_call(rai_hip_decoder *d, int B, int S) {
@@ -794,6 +847,34 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   if (hipMemset(d->attn_counters, 0, attention_decode_counter_bytes(cfg->max_batch, d->Hq)) != hipSuccess)
     return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
 
+  d->mega_layers = nullptr;
+  d->mega_ok = false;
+  d->mega_prof = nullptr;
+  {
+    hipDeviceProp_t prop;
+    d->num_cu = hipGetDeviceProperties(&prop, dev) == hipSuccess ? prop.multiProcessorCount : kNumCU;
+  }
+  if ((st = dalloc(d, 128, &tmp))) return bail(st);
+  d->mega_barrier = (unsigned *)tmp;
+  if (hipMemset(d->mega_barrier, 0, 128) != hipSuccess) return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
+  if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_MEGA") != nullptr) {
+    std::vector<MegaLayer> ml(d->L);
+    for (int l = 0; l < d->L; ++l) {
+      const Layer &ly = d->layers[l];
+      ml[l] = MegaLayer{(const uint16_t *)ly.Wa, (const uint16_t *)ly.ba, (const uint16_t *)ly.Wb, (const uint16_t *)ly.bd,
+                        (const uint16_t *)ly.bf, (const uint16_t *)ly.ln_w, (const uint16_t *)ly.ln_b};
+    }
+    if ((st = dalloc(d, ml.size() * sizeof(MegaLayer), &tmp))) return bail(st);
+    d->mega_layers = (MegaLayer *)tmp;
+    if (hipMemcpy(d->mega_layers, ml.data(), ml.size() * sizeof(MegaLayer), hipMemcpyHostToDevice) != hipSuccess)
+      return bail(fail(RAI_ERR_HIP, "decoder_create: layer table upload failed"));
+    if (getenv("RAI_HIP_MEGA_PROF")) {
+      if ((st = dalloc(d, (size_t)d->num_cu * d->L * 8 * sizeof(unsigned long long), &tmp))) return bail(st);
+      d->mega_prof = (unsigned long long *)tmp;
+    }
+    MegaArgs m = mega_args(d);
+    d->mega_ok = mega_eligible(m, d->D, d->num_cu, nullptr);
+  }
   if (hipMemset(d->state, 0, sizeof(DevState)) != hipSuccess || hipMemset(d->kcache, 0, kv) != hipSuccess ||
       hipMemset(d->vcache, 0, kv) != hipSuccess)
     return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
@@ -877,6 +958,7 @@ int rai_hip_decoder_forward(rai_hip_decoder *d, const uint32_t *ids_host, int32_
   }
   if (tokens_host) RAI_TRY(rai_hip_d2h(d->dev, tokens_host, d->tokens, (size_t)batch * sizeof(uint32_t)));
   if (logits_host || tokens_host) {
+    RAI_TRY(check_fault(d));
     uint64_t bad = 0;
     RAI_TRY(rai_hip_index_errors(d->dev, &bad));
     RAI_REQUIRE(bad == 0, RAI_ERR_INDEX, "decoder: %llu token ids outside the vocabulary", (unsigned long long)bad);
@@ -951,6 +1033,7 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   (void)hipEventDestroy(e1);
   (void)hipEventDestroy(e2);
   if (rc == RAI_OK) {
+    RAI_TRY(check_fault(d));
     uint64_t bad = 0;
     RAI_TRY(rai_hip_index_errors(d->dev, &bad));
     RAI_REQUIRE(bad == 0, RAI_ERR_INDEX, "decoder: %llu token ids outside the vocabulary", (unsigned long long)bad);
