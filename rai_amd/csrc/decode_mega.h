@@ -19,8 +19,12 @@ struct MegaLayer {
   const uint16_t *ln_w, *ln_b;
 };
 
+constexpr int kMegaFlagWords = 256;  // one barrier flag per block of the persistent kernel
+
 struct MegaArgs {
   const MegaLayer *layers;  // device array [L]
+  const uint16_t *Wa0, *Wb0;      // layer 0; layer l sits wa_stride / wb_stride elements further
+  int64_t wa_stride, wb_stride;
   int L, H, I, QD, NA, n_qkv, Hq, rot, Tmax;
   uint16_t *x;              // [H] residual stream, updated in place
   uint16_t *qkv;            // [3 * QD]
@@ -30,7 +34,7 @@ struct MegaArgs {
   int64_t kv_layer_stride;  // elements between consecutive layers of the cache
   const uint16_t *cos_t, *sin_t;
   DevState *state;
-  unsigned *barrier;        // arrival counter, zero at launch
+  unsigned *barrier;        // kMegaFlagWords flags: [0, blocks) zero at launch, the rest 0xffffffff
   float ln_eps, scale;
   int act;
   int rows_attn;            // rows of phases B/C given to each attention block

@@ -5,21 +5,21 @@
 // One 512-thread block per CU stays resident for the whole token.  A layer is
 // three weight-streaming phases separated by grid-wide barriers:
 //   A  LayerNorm(x) . Wa^T + bias   -> q | k | v | gelu(fc1)      (rows split over blocks)
-//   B  head h attention on block h  ||  fc2 partial products on every block
+//   B  head h attention on block h  ||  fc2 partial products on the other blocks
 //   C  dense(attn) partial + fc2 partial + biases + residual -> x (same rows as B)
-// Weights do not depend on activations, so each wave issues the first loads of
-// the next phase before it arrives at the barrier: HBM keeps streaming across
-// the dependency instead of draining at a kernel boundary.  Attention (latency
-// bound, 0.2 MB per head) hides behind the 52 MB fc2 stream of phase B.
+// Weights do not depend on activations: every wave keeps a ring of weight tiles
+// in flight that runs ahead across the phase boundaries, so HBM keeps streaming
+// through a barrier instead of draining at a kernel boundary.  Attention
+// (latency bound, 0.2 MB per head) hides behind the 52 MB fc2 stream of phase B.
 //
-// Values that cross blocks inside the launch (x, q|k|v, act, attn) are written
-// with device-scope write-through stores and read with device-scope loads: the
-// per-XCD L2s are not coherent for ordinary accesses, and a device-scope fence
-// would write back and invalidate a whole L2.  Weights, biases, rotary tables
-// and the KV cache rows of earlier tokens are read-only here and use ordinary
-// (non-temporal) loads.
+// Values that cross blocks inside the launch (x, q|k|v, act, attn, barrier flags)
+// are written with device-scope write-through stores and read with device-scope
+// loads: the per-XCD L2s are not coherent for ordinary accesses, and a
+// device-scope fence would write back and invalidate a whole L2.  Weights,
+// biases, rotary tables and the KV cache rows of earlier tokens are read-only
+// here and use ordinary (non-temporal) loads.
 //
-// The grid barrier spins on a device counter; every block of the grid is
+// The grid barrier spins on flags in device memory; every block of the grid is
 // resident (grid <= number of CUs) so the spin always ends, and it is bounded:
 // on timeout the block raises DevState::fault and every later barrier falls
 // through, so the kernel always terminates and the host reports the fault.
@@ -33,11 +33,13 @@ typedef __attribute__((ext_vector_type(2))) __bf16 mg_bf16x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t mg_u32x4;
 
 constexpr int kMegaThreads = 512, kMegaWaves = 8;
+
+constexpr int kMegaStream = kMegaWaves - 1, kMegaService = kMegaWaves - 1;
 constexpr unsigned kMegaSpinLimit = 1u << 20;
-constexpr int kMegaSlots = 4;     // phase A: weight rows in flight per wave
-constexpr int kMegaRing = 8;      // phases B, C: 1 KB weight tiles in flight per wave
-constexpr int kMegaRowsMax = 16;  // phases B, C: rows per block
-constexpr int kMegaUK = 6, kMegaUV = 6;
+constexpr int kMegaRing = 16;
+constexpr int kMegaRowsAMax = 96;
+constexpr int kMegaRowsMax = 16;
+constexpr int kMegaUK = 13, kMegaUV = 13;
 
 __device__ __forceinline__ float mg_dot2(uint32_t a, uint32_t b, float c) {
   mg_bf16x2 p, q;
@@ -54,7 +56,7 @@ __device__ __forceinline__ float mg_dot8(mg_u32x4 a, mg_u32x4 b, float c) {
 __device__ __forceinline__ mg_u32x4 mg_ldw(const uint16_t *p) {
   return __builtin_nontemporal_load(reinterpret_cast<const mg_u32x4 *>(p));
 }
-// device-scope accesses (see the header comment)
+
 __device__ __forceinline__ uint64_t ld_dev64(const void *p) {
   return __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -71,34 +73,15 @@ __device__ __forceinline__ uint16_t ld_dev16(const void *p) {
 __device__ __forceinline__ void st_dev16(void *p, uint16_t v) {
   __hip_atomic_store((uint16_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void st_dev64(void *p, uint64_t v) {
+  __hip_atomic_store((uint64_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ void st_dev32(void *p, uint32_t v) {
   __hip_atomic_store((uint32_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float mg_round(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
-// Block barrier that leaves vector-memory loads in flight (only LDS traffic is drained).
 __device__ __forceinline__ void wg_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
-// Grid barrier number `index` (0-based, counted from the start of the launch).
-// The caller's write-through stores are complete before the arrival is counted.
-__device__ __forceinline__ void grid_sync(unsigned *ctr, unsigned index, int *fault) {
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  if (threadIdx.x == 0) {
-    const unsigned target = (index + 1u) * gridDim.x;
-    __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    unsigned spins = 0;
-    while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      __builtin_amdgcn_s_sleep(1);
-      ++spins;
-      if (spins > kMegaSpinLimit) {
-        __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-      if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-    }
-  }
-  asm volatile("s_barrier" ::: "memory");
-}
 
 // Rotary embedding of feature d of a head whose D features sit in LDS as f32,
 // with the reference's three roundings (phi2.rs:75).
@@ -110,28 +93,25 @@ __device__ __forceinline__ float mg_rope(const float *head, int d, int rot, floa
   return mg_round(mg_round(v * c) + mg_round(other * s));
 }
 
-// Sums over lanes with DPP (register-to-register, no LDS crossbar).
 template <int CTRL> __device__ __forceinline__ float mg_dpp(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-// every lane of a 16-lane row receives the row's sum
+
 __device__ __forceinline__ float mg_row_sum(float v) {
-  v += mg_dpp<0xB1>(v);   // quad_perm [1,0,3,2]
-  v += mg_dpp<0x4E>(v);   // quad_perm [2,3,0,1]
-  v += mg_dpp<0x124>(v);  // row_ror:4
-  v += mg_dpp<0x128>(v);  // row_ror:8
+  v += mg_dpp<0xB1>(v);
+  v += mg_dpp<0x4E>(v);
+  v += mg_dpp<0x124>(v);
+  v += mg_dpp<0x128>(v);
   return v;
 }
-// wave-uniform sum of all 64 lanes
+
 __device__ __forceinline__ float mg_wave_sum(float v) {
   v = mg_row_sum(v);
   const int b = __builtin_bit_cast(int, v);
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16)) +
          (__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48)));
 }
-// Hides a value's origin from the optimiser, so that everything derived from it
-// is recomputed where it is used instead of being kept in registers across the
-// whole layer loop (this kernel lives at the register limit).
+
 __device__ __forceinline__ int mg_opaque(int v) {
   asm volatile("" : "+v"(v));
   return v;
@@ -139,47 +119,178 @@ __device__ __forceinline__ int mg_opaque(int v) {
 
 #define MG_ZERO4 mg_u32x4{0u, 0u, 0u, 0u}
 
-// KTA = H / 512 (K tiles of the phase A rows), D = head_dim.
+// Rotates the ring so that entry R becomes entry 0 (all of its loads have landed).
+template <int R> __device__ __forceinline__ void mg_rotate(mg_u32x4 (&ring)[kMegaRing]) {
+  mg_u32x4 tmp[kMegaRing];
+#pragma unroll
+  for (int p = 0; p < kMegaRing; ++p) tmp[p] = ring[(p + R) % kMegaRing];
+#pragma unroll
+  for (int p = 0; p < kMegaRing; ++p) ring[p] = tmp[p];
+}
+
+struct MgSplit {
+  const uint16_t *Wa0, *Wb0;
+  int64_t wa_stride, wb_stride;
+  int L, H, KB, QD, KTA, KTB, KTC;
+  int nA0, n0;
+  int tA0, tA1, tB0, tB1, tC0, tC1;
+};
+
+struct MgCursor {
+  int layer, seg, kc, KT, t, t1;
+  int64_t ld;
+  const uint16_t *ptr;
+  bool done;
+};
+
+__device__ __forceinline__ bool mg_seg_next(MgCursor &c, const MgSplit &sp) {
+  int layer = c.layer, seg = c.seg;
+
+  const int tA0 = sp.tA0, tA1 = sp.tA1, tB0 = sp.tB0, tB1 = sp.tB1, tC0 = sp.tC0, tC1 = sp.tC1;
+  const int KTA = sp.KTA, KTB = sp.KTB, KTC = sp.KTC;
+  for (;;) {
+    if (++seg == 3) { seg = 0; ++layer; }
+    if (layer >= sp.L) return false;
+    const int t0 = seg == 0 ? tA0 : seg == 1 ? tB0 : tC0;
+    const int t1 = seg == 0 ? tA1 : seg == 1 ? tB1 : tC1;
+    if (t1 <= t0) continue;
+    const int KT = seg == 0 ? KTA : seg == 1 ? KTB : KTC;
+    const int row = t0 / KT;
+    c.layer = layer; c.seg = seg; c.KT = KT; c.t = t0; c.t1 = t1;
+    c.kc = t0 - row * KT;
+    if (seg == 0) {
+      c.ld = sp.H;
+      c.ptr = sp.Wa0 + layer * sp.wa_stride + (int64_t)(sp.nA0 + row) * sp.H;
+    } else {
+      c.ld = sp.KB;
+      c.ptr = sp.Wb0 + layer * sp.wb_stride + (int64_t)(sp.n0 + row) * sp.KB + (seg == 1 ? sp.QD : 0);
+    }
+    return true;
+  }
+}
+// requests the tile under the cursor and advances the cursor (past the end of the
+// stream the last tile is requested again: the ring stays full, nothing is stored)
+__device__ __forceinline__ mg_u32x4 mg_next_load(MgCursor &c, const MgSplit &sp, int lane) {
+  const mg_u32x4 v = mg_ldw(c.ptr + c.kc * 512 + lane * 8);
+  if (!c.done) {
+    if (c.t + 1 == c.t1) {
+      if (!mg_seg_next(c, sp)) c.done = true;
+    } else {
+      ++c.t;
+      if (++c.kc == c.KT) { c.kc = 0; c.ptr += c.ld; }
+    }
+  }
+  return v;
+}
+// Consumes tiles [t0, t1) of a [rows][KT] tile grid from the ring (entry 0 first),
+// multiplying them with the activation vector in LDS; leaves one partial sum per
+// (row, wave).  Returns how many entries the ring must be rotated afterwards.
+__device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCursor &c, const MgSplit &sp, int t0, int t1,
+                                            int KT, const uint16_t *xv, float *part, int lane, int wave) {
+  float acc = 0.f;
+  int t = t0, row = t0 / KT;
+  int kc = t0 - row * KT;
+#define MG_STEP(r)                                                                         \
+  {                                                                                        \
+    const mg_u32x4 x4 = *reinterpret_cast<const mg_u32x4 *>(xv + kc * 512 + lane * 8);     \
+    acc = mg_dot8(r, x4, acc);                                                             \
+    r = mg_next_load(c, sp, lane);                                                         \
+    ++t;                                                                                   \
+    ++kc;                                                                                  \
+    if (kc == KT || t == t1) {                                                             \
+      const float total = mg_wave_sum(acc);                                                \
+      if (lane == 0) part[row * kMegaWaves + wave] = total;                                \
+      acc = 0.f;                                                                           \
+      if (kc == KT) { kc = 0; ++row; }                                                     \
+    }                                                                                      \
+  }
+  while (t + kMegaRing <= t1) {
+#pragma unroll
+    for (int p = 0; p < kMegaRing; ++p) MG_STEP(ring[p])
+  }
+#pragma unroll
+  for (int p = 0; p < kMegaRing; ++p)
+    if (t < t1) MG_STEP(ring[p])
+#undef MG_STEP
+  return t1 > t0 ? (t1 - t0) % kMegaRing : 0;
+}
+__device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r) {
+  static_assert((kMegaRing & (kMegaRing - 1)) == 0 && kMegaRing <= 16, "rotation is composed from powers of two");
+  if (r & 1) mg_rotate<1>(ring);
+  if (r & 2) mg_rotate<2 % kMegaRing>(ring);
+  if (r & 4) mg_rotate<4 % kMegaRing>(ring);
+  if (r & 8) mg_rotate<8 % kMegaRing>(ring);
+}
+
+__device__ __forceinline__ void mg_grid_arrive(unsigned *flags, unsigned index, bool service, int lane) {
+  if (service) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane == 0) __hip_atomic_store(flags + blockIdx.x, index + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+__device__ __forceinline__ void mg_grid_wait(const unsigned *flags, unsigned index, int *fault, bool service, int lane) {
+  if (service) {
+    const unsigned target = index + 1u;
+    const int G = gridDim.x;
+    unsigned spins = 0;
+    for (;;) {
+      bool ok = true;
+      if (lane * 4 < G) {
+        const uint64_t lo = ld_dev64(flags + lane * 4), hi = ld_dev64(flags + lane * 4 + 2);
+        ok = (uint32_t)lo >= target && (uint32_t)(lo >> 32) >= target && (uint32_t)hi >= target &&
+             (uint32_t)(hi >> 32) >= target;
+      }
+      if (__all(ok)) break;
+      ++spins;
+      if (spins > kMegaSpinLimit) {
+        if (lane == 0) __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 template <int KTA, int D, bool PROF>
 __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
-  constexpr int NCOL = D / 8;                     // 16-byte packs per key / value row
-  constexpr int NG_K = kMegaThreads / 16;         // key rows per round of the score loop
-  constexpr int NG_V = kMegaThreads / NCOL;       // value rows per round of the P.V loop
+  constexpr int NCOL = D / 8;
+  constexpr int NG_V = kMegaThreads / NCOL;
   extern __shared__ __attribute__((aligned(16))) unsigned char mg_smem[];
   const int H = KTA * 512, I = a.I, QD = a.QD, KB = QD + I;
   const int KTB = I / 512, KTC = QD / 512;
-  // LDS layout
-  uint16_t *xs = reinterpret_cast<uint16_t *>(mg_smem);           // [I] act, then [QD] attn
+
+  uint16_t *xs = reinterpret_cast<uint16_t *>(mg_smem);
   uint16_t *xa = xs + I;
-  float *partB = reinterpret_cast<float *>(xa + QD);               // [rows][waves]
+  uint16_t *xn = xa + QD;
+  float *partA = reinterpret_cast<float *>(xn + H);
+  float *partB = partA + kMegaRowsAMax * kMegaWaves;
   float *partC = partB + kMegaRowsMax * kMegaWaves;
-  float *qf = partC + kMegaRowsMax * kMegaWaves;                   // attention scratch
-  float *raw = qf + D;                                             // [3*D] q | k | v before rotary
+  float *qf = partC + kMegaRowsMax * kMegaWaves;
+  float *raw = qf + D;
   float *knew = raw + 3 * D;
   float *vnew = knew + D;
-  float *red = vnew + D;                                           // [NG_V * D]
-  float *sh = red + NG_V * D;                                      // [2 * waves]
-  float *red2 = sh + 2 * kMegaWaves;                               // [4 * D]
-  float *scores = red2 + 4 * D;                                    // [Tmax + 1]
+  float *red = vnew + D;
+  float *sh = red + NG_V * D;
+  float *red2 = sh + 2 * kMegaWaves;
+  float *scores = red2 + 4 * D;
+  float *pd = scores + a.Tmax + 1;
 
   const int tid0 = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid0 >> 6);      // wave-uniform: lives in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid0 >> 6);
   const int wg = blockIdx.x, G = gridDim.x;
   int *fault = &a.state->fault;
   int pos = a.state->pos;
   if (pos > a.Tmax - 1) pos = a.Tmax - 1;
-  // rotary factors of this position (the same for every layer)
+
   float rope_c = 1.f, rope_s = 0.f;
   if (tid0 < a.rot) {
     rope_c = bf16_bits_to_f32(a.cos_t[(int64_t)pos * a.rot + tid0]);
     rope_s = bf16_bits_to_f32(a.sin_t[(int64_t)pos * a.rot + tid0]);
   }
 
-  // ---- static work split (all wave-uniform)
-  // phase A: rows [nA0, nA1) of Wa; wave w takes rows nA0 + w + 8 i
-  const int nA0 = (int)((int64_t)a.NA * wg / G), nA1 = (int)((int64_t)a.NA * (wg + 1) / G);
-  const int cntA = nA1 - nA0 > wave ? (nA1 - nA0 - wave + kMegaWaves - 1) / kMegaWaves : 0;
-  // phases B, C: the attention blocks (wg < Hq) take rows_attn rows each, the rest is split evenly
+  const int nA0 = 4 * (int)((int64_t)(a.NA / 4) * wg / G), nA1 = 4 * (int)((int64_t)(a.NA / 4) * (wg + 1) / G);
+  const int rowsA = nA1 - nA0;
+
   int n0, n1;
   const bool is_attn = wg < a.Hq;
   {
@@ -191,114 +302,80 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       n1 = n0 + ra;
     } else {
       const int base = n_attn_blocks * ra, rem = H - base, o = wg - n_attn_blocks;
-      n0 = base + (int)((int64_t)rem * o / others);
-      n1 = base + (int)((int64_t)rem * (o + 1) / others);
+      n0 = base + 4 * (int)((int64_t)(rem / 4) * o / others);
+      n1 = base + 4 * (int)((int64_t)(rem / 4) * (o + 1) / others);
     }
     if (n0 > H) n0 = H;
     if (n1 > H) n1 = H;
   }
-  const int nrows = n1 - n0;  // <= kMegaRowsMax (checked on the host)
-  // contiguous tile ranges of this wave in phases B and C
-  const int ttB = nrows * KTB, ttC = nrows * KTC;
-  const int tB0 = ttB * wave / kMegaWaves, tB1 = ttB * (wave + 1) / kMegaWaves;
-  const int tC0 = ttC * wave / kMegaWaves, tC1 = ttC * (wave + 1) / kMegaWaves;
+  const int nrows = n1 - n0;
 
-  mg_u32x4 slot[kMegaSlots][KTA];
+  const int ttA = rowsA * KTA, ttB = nrows * KTB, ttC = nrows * KTC;
+  const bool streams = wave < kMegaStream;
+  const int tA0 = streams ? ttA * wave / kMegaStream : 0, tA1 = streams ? ttA * (wave + 1) / kMegaStream : 0;
+  const int tB0 = streams ? ttB * wave / kMegaStream : 0, tB1 = streams ? ttB * (wave + 1) / kMegaStream : 0;
+  const int tC0 = streams ? ttC * wave / kMegaStream : 0, tC1 = streams ? ttC * (wave + 1) / kMegaStream : 0;
+
   mg_u32x4 ring[kMegaRing];
-  mg_u32x4 kreg[2][kMegaUK], vreg[2][kMegaUV];
+  mg_u32x4 kreg[kMegaUK], vreg[kMegaUV];
 
-  auto load_row = [&](mg_u32x4(&dst)[KTA], const uint16_t *W, int i, int lane) {
-    const uint16_t *wr = W + (int64_t)(nA0 + wave + kMegaWaves * i) * H + lane * 8;
+  MgSplit sp;
+  sp.Wa0 = a.Wa0; sp.Wb0 = a.Wb0; sp.wa_stride = a.wa_stride; sp.wb_stride = a.wb_stride; sp.L = a.L; sp.H = H; sp.KB = KB; sp.QD = QD; sp.KTA = KTA; sp.KTB = KTB; sp.KTC = KTC;
+  sp.nA0 = nA0; sp.n0 = n0;
+  sp.tA0 = tA0; sp.tA1 = tA1; sp.tB0 = tB0; sp.tB1 = tB1; sp.tC0 = tC0; sp.tC1 = tC1;
+  MgCursor cur;
+  cur.layer = 0; cur.seg = -1; cur.kc = 0; cur.KT = 1; cur.t = 0; cur.t1 = 0; cur.ld = 0;
+  cur.ptr = a.Wa0;
+  cur.done = !mg_seg_next(cur, sp);
+  unsigned bar = 0;
+  unsigned *const barrier = a.barrier;
+  const float att_scale = a.scale;
+  unsigned long long *const prof = a.prof;
+  const int n_layers = a.L;
+
+  auto k_load = [&](const uint16_t *Kc, int q0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < KTA; ++u) dst[u] = mg_ldw(wr + u * 512);
-  };
-  auto prime_A = [&](const uint16_t *W, int lane) {
-#pragma unroll
-    for (int s = 0; s < kMegaSlots; ++s) {
-      // (the else branch ends the live range of the previous contents)
-      if (s < cntA) load_row(slot[s], W, s, lane);
-      else
-#pragma unroll
-        for (int u = 0; u < KTA; ++u) slot[s][u] = MG_ZERO4;
+    for (int u = 0; u < kMegaUK; ++u) {
+      const int q = q0 + kMegaThreads * u;
+      kreg[u] = q < pos * NCOL ? mg_ldw(Kc + (int64_t)q * 8) : MG_ZERO4;
     }
   };
-  // tile t of a [rows][KT] tile grid whose K origin is column col0 of Wb
-  auto tile_ptr = [&](const uint16_t *Wb, int t, int KT, int col0, int lane) -> const uint16_t * {
-    const int row = t / KT, kc = t - row * KT;
-    return Wb + (int64_t)(n0 + row) * KB + col0 + kc * 512 + lane * 8;
-  };
-  auto prime_ring = [&](const uint16_t *Wb, int t0, int t1, int KT, int col0, int lane) {
+
+  auto k_partials = [&](int q0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int p = 0; p < kMegaRing; ++p)
-      ring[p] = t0 + p < t1 ? mg_ldw(tile_ptr(Wb, t0 + p, KT, col0, lane)) : MG_ZERO4;
-  };
-  // Streams tiles [t0, t1) (the first kMegaRing are already in the ring), multiplies
-  // them with the activation vector in LDS and leaves one partial per (row, wave).
-  auto run_ring = [&](const uint16_t *Wb, int t0, int t1, int KT, int col0, const uint16_t *xv, float *part, int lane) {
-    float acc = 0.f;
-    int row = t0 / KT, kc = t0 - row * KT;                    // tile being consumed
-    int lrow = (t0 + kMegaRing) / KT, lkc = t0 + kMegaRing - lrow * KT;  // tile being requested
-    for (int tb = t0; tb < t1; tb += kMegaRing) {
-#pragma unroll
-      for (int p = 0; p < kMegaRing; ++p) {
-        const int t = tb + p;
-        if (t < t1) {
-          const mg_u32x4 x4 = *reinterpret_cast<const mg_u32x4 *>(xv + kc * 512 + lane * 8);
-          acc = mg_dot8(ring[p], x4, acc);
-          if (t + kMegaRing < t1) {
-            ring[p] = mg_ldw(Wb + (int64_t)(n0 + lrow) * KB + col0 + lkc * 512 + lane * 8);
-            if (++lkc == KT) { lkc = 0; ++lrow; }
-          }
-          ++kc;
-          if (kc == KT || t + 1 == t1) {
-            const float total = mg_wave_sum(acc);
-            if (lane == 0) part[row * kMegaWaves + wave] = total;
-            acc = 0.f;
-            if (kc == KT) { kc = 0; ++row; }
-          }
-        }
+    for (int u = 0; u < kMegaUK; ++u) {
+      const int q = q0 + kMegaThreads * u;
+      if (q < pos * NCOL) {
+        const int c = q % NCOL;
+        const float4 qa = *reinterpret_cast<const float4 *>(qf + c * 8);
+        const float4 qb = *reinterpret_cast<const float4 *>(qf + c * 8 + 4);
+        const uint32_t w4[4] = {kreg[u].x, kreg[u].y, kreg[u].z, kreg[u].w};
+        float acc = qa.x * __uint_as_float(w4[0] << 16);
+        acc = fmaf(qa.y, __uint_as_float(w4[0] & 0xffff0000u), acc);
+        acc = fmaf(qa.z, __uint_as_float(w4[1] << 16), acc);
+        acc = fmaf(qa.w, __uint_as_float(w4[1] & 0xffff0000u), acc);
+        acc = fmaf(qb.x, __uint_as_float(w4[2] << 16), acc);
+        acc = fmaf(qb.y, __uint_as_float(w4[2] & 0xffff0000u), acc);
+        acc = fmaf(qb.z, __uint_as_float(w4[3] << 16), acc);
+        acc = fmaf(qb.w, __uint_as_float(w4[3] & 0xffff0000u), acc);
+        pd[q] = acc;
       }
     }
   };
-  // cached keys tb + NG_K u (u < UK) of one round, 16 lanes per key row of which NCOL load
-  auto k_load = [&](mg_u32x4(&kr)[kMegaUK], const uint16_t *Kc, int tb, int gl) {
-#pragma unroll
-    for (int u = 0; u < kMegaUK; ++u) {
-      const int t = tb + NG_K * u;
-      kr[u] = (t < pos && gl < NCOL) ? mg_ldw(Kc + (int64_t)t * D + gl * 8) : MG_ZERO4;
-    }
-  };
-  auto k_scores = [&](const mg_u32x4(&kr)[kMegaUK], int tb, int gl) {
-    float q8[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) q8[j] = gl < NCOL ? qf[gl * 8 + j] : 0.f;
-#pragma unroll
-    for (int u = 0; u < kMegaUK; ++u) {
-      const int t = tb + NG_K * u;
-      const uint32_t w4[4] = {kr[u].x, kr[u].y, kr[u].z, kr[u].w};
-      float acc = 0.f;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc = fmaf(q8[2 * j], __uint_as_float(w4[j] << 16), acc);
-        acc = fmaf(q8[2 * j + 1], __uint_as_float(w4[j] & 0xffff0000u), acc);
-      }
-      acc = mg_row_sum(acc);
-      if (gl == 0 && t < pos) scores[t] = acc * a.scale;
-    }
-  };
-  auto v_load = [&](mg_u32x4(&vr)[kMegaUV], const uint16_t *Vc, int tb, int col, bool active) {
+
+  auto v_load = [&](const uint16_t *Vc, int tb, int col, bool active) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < kMegaUV; ++u) {
       const int t = tb + NG_V * u;
-      vr[u] = (active && t < pos) ? mg_ldw(Vc + (int64_t)t * D + col * 8) : MG_ZERO4;
+      vreg[u] = (active && t < pos) ? mg_ldw(Vc + (int64_t)t * D + col * 8) : MG_ZERO4;
     }
   };
-  auto v_accum = [&](const mg_u32x4(&vr)[kMegaUV], int tb, float(&acc)[8]) {
+  auto v_accum = [&](int tb, float(&acc)[8]) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < kMegaUV; ++u) {
       const int t = tb + NG_V * u;
-      const float p = t < pos ? scores[t] : 0.f;  // rows past the context hold zeros
-      const uint32_t w4[4] = {vr[u].x, vr[u].y, vr[u].z, vr[u].w};
+      const float p = t < pos ? scores[t] : 0.f;
+      const uint32_t w4[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         acc[2 * j] = fmaf(p, __uint_as_float(w4[j] << 16), acc[2 * j]);
@@ -307,52 +384,67 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     }
   };
 
-  unsigned bar = 0;
-  prime_A(a.layers[0].Wa, tid0 & 63);
-  // optional time stamps (100 MHz clock) of thread 0 of every block: [block][layer][8]
-  auto stamp = [&](int l, int k) {
+  auto stamp = [&](int l, int k) __attribute__((always_inline)) {
     if constexpr (PROF) {
-      if (threadIdx.x == 0) a.prof[((int64_t)wg * a.L + l) * 8 + k] = wall_clock64();
+      if (threadIdx.x == kMegaService * 64) prof[((int64_t)wg * n_layers + l) * 16 + k] = wall_clock64();
     }
   };
 
+  for (int e = tid0; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
+
+  {
+    const int lane = tid0 & 63;
+#pragma unroll
+    for (int p = 0; p < kMegaRing; ++p) {
+      ring[p] = streams ? mg_next_load(cur, sp, lane) : MG_ZERO4;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kMegaUK; ++u) kreg[u] = MG_ZERO4;
+#pragma unroll
+  for (int u = 0; u < kMegaUV; ++u) vreg[u] = MG_ZERO4;
+
   for (int l = 0; l < a.L; ++l) {
     const MegaLayer ly = a.layers[l];
-    uint16_t *Kc = a.kcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg * a.Tmax * D;  // attention blocks: head wg
+    uint16_t *Kc = a.kcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg * a.Tmax * D;
     uint16_t *Vc = a.vcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg * a.Tmax * D;
-    // =================================================== phase A
+
     stamp(l, 0);
     {
       const int tid = mg_opaque(tid0), lane = tid & 63;
-      // lane i keeps the bias of this wave's row i
-      const float bias_lane = lane < cntA ? bf16_bits_to_f32(ly.ba[nA0 + wave + kMegaWaves * lane]) : 0.f;
-      // activation vector of this lane: K positions lane*8 + 512 u
-      mg_u32x4 xv[KTA];
+      const bool service = wave == kMegaService;
+
+      uint64_t bias_a = 0;
+      if (service && lane * 4 < rowsA) bias_a = *reinterpret_cast<const uint64_t *>(ly.ba + nA0 + lane * 4);
+      if (tid < 2 * kMegaRowsMax * kMegaWaves) partB[tid] = 0.f;
+      if (wave < KTA) {
+
+        mg_u32x4 xv[KTA];
 #pragma unroll
-      for (int u = 0; u < KTA; ++u) xv[u] = ld_dev128(a.x + u * 512 + lane * 8);
-      // LayerNorm statistics from packed pairs (exact products, f32 accumulation)
-      const uint32_t ones = 0x3f803f80u;
-      float s1 = 0.f, s2 = 0.f;
+        for (int u = 0; u < KTA; ++u) xv[u] = ld_dev128(a.x + u * 512 + lane * 8);
+        const mg_u32x4 lw = *reinterpret_cast<const mg_u32x4 *>(ly.ln_w + wave * 512 + lane * 8);
+        const mg_u32x4 lb = *reinterpret_cast<const mg_u32x4 *>(ly.ln_b + wave * 512 + lane * 8);
+
+        const uint32_t ones = 0x3f803f80u;
+        float s1 = 0.f, s2 = 0.f;
+        mg_u32x4 mine = MG_ZERO4;
 #pragma unroll
-      for (int u = 0; u < KTA; ++u) {
-        const uint32_t w4[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+        for (int u = 0; u < KTA; ++u) {
+          const uint32_t w4[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          s1 = mg_dot2(w4[j], ones, s1);
-          s2 = mg_dot2(w4[j], w4[j], s2);
+          for (int j = 0; j < 4; ++j) {
+            s1 = mg_dot2(w4[j], ones, s1);
+            s2 = mg_dot2(w4[j], w4[j], s2);
+          }
+          if (wave == u) mine = xv[u];
         }
-      }
-      s1 = mg_wave_sum(s1);
-      s2 = mg_wave_sum(s2);
-      const float mean = s1 / (float)H;
-      float var = s2 / (float)H - mean * mean;
-      var = var > 0.f ? var : 0.f;
-      const float scale = 1.0f / sqrtf(var + a.ln_eps), shift = -mean * scale;
-#pragma unroll
-      for (int u = 0; u < KTA; ++u) {
-        const mg_u32x4 lw = *reinterpret_cast<const mg_u32x4 *>(ly.ln_w + u * 512 + lane * 8);
-        const mg_u32x4 lb = *reinterpret_cast<const mg_u32x4 *>(ly.ln_b + u * 512 + lane * 8);
-        const uint32_t xx[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+        s1 = mg_wave_sum(s1);
+        s2 = mg_wave_sum(s2);
+        const float mean = s1 / (float)H;
+        float var = s2 / (float)H - mean * mean;
+        var = var > 0.f ? var : 0.f;
+        const float scale = 1.0f / sqrtf(var + a.ln_eps), shift = -mean * scale;
+        const uint32_t xx[4] = {mine.x, mine.y, mine.z, mine.w};
         const uint32_t ww[4] = {lw.x, lw.y, lw.z, lw.w};
         const uint32_t bb[4] = {lb.x, lb.y, lb.z, lb.w};
         uint32_t o[4];
@@ -362,77 +454,57 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
                                 __uint_as_float(bb[j] << 16));
           const float y1 = fmaf(fmaf(__uint_as_float(xx[j] & 0xffff0000u), scale, shift),
                                 __uint_as_float(ww[j] & 0xffff0000u), __uint_as_float(bb[j] & 0xffff0000u));
-          o[j] = pack_bf16x2(y0, y1);  // the reference materialises the normalised activations in bf16
+          o[j] = pack_bf16x2(y0, y1);
         }
-        xv[u] = mg_u32x4{o[0], o[1], o[2], o[3]};
-      }
-      // rows of this wave, kMegaSlots at a time: products, next loads, then the four
-      // reductions together; lane s finishes row i0 + s.  Results are staged in LDS
-      // (the act buffer is free until phase B).
-      float *stage = reinterpret_cast<float *>(xs);  // [nA1 - nA0] f32
-      for (int i0 = 0; i0 < cntA; i0 += kMegaSlots) {
-        float acc[kMegaSlots];
-#pragma unroll
-        for (int s = 0; s < kMegaSlots; ++s) {
-          acc[s] = 0.f;
-#pragma unroll
-          for (int u = 0; u < KTA; ++u) acc[s] = mg_dot8(slot[s][u], xv[u], acc[s]);
-        }
-#pragma unroll
-        for (int s = 0; s < kMegaSlots; ++s)
-          if (i0 + s + kMegaSlots < cntA) load_row(slot[s], ly.Wa, i0 + s + kMegaSlots, lane);
-        float mine = 0.f;
-#pragma unroll
-        for (int s = 0; s < kMegaSlots; ++s) {
-          const float total = mg_wave_sum(acc[s]);
-          if (lane == s) mine = total;
-        }
-        const float bias = __shfl(bias_lane, i0 + lane, 64);
-        if (lane < kMegaSlots && i0 + lane < cntA) {
-          const int n = nA0 + wave + kMegaWaves * (i0 + lane);
-          float v = mine + bias;
-          if (n >= a.n_qkv) v = act_eval(a.act, v);
-          stage[n - nA0] = v;
-        }
-      }
-      // first loads of phase B: this wave's fc2 tiles; the attention blocks also fetch
-      // the first two rounds of cached keys and values of their head
-      prime_ring(ly.Wb, tB0, tB1, KTB, QD, lane);
-      if (is_attn) {
-        const int g = tid >> 4, gl = tid & 15, col = tid % NCOL, grp = tid / NCOL;
-        k_load(kreg[0], Kc, g, gl);
-        k_load(kreg[1], Kc, g + NG_K * kMegaUK, gl);
-        v_load(vreg[0], Vc, grp, col, grp < NG_V);
-        v_load(vreg[1], Vc, grp + NG_V * kMegaUV, col, grp < NG_V);
-      } else {
-#pragma unroll
-        for (int u = 0; u < kMegaUK; ++u) kreg[0][u] = kreg[1][u] = MG_ZERO4;
-#pragma unroll
-        for (int u = 0; u < kMegaUV; ++u) vreg[0][u] = vreg[1][u] = MG_ZERO4;
+        *reinterpret_cast<mg_u32x4 *>(xn + wave * 512 + lane * 8) = mg_u32x4{o[0], o[1], o[2], o[3]};
       }
       wg_sync();
-      // write q|k|v and act with write-through stores
-      for (int e = tid; e < nA1 - nA0; e += kMegaThreads) {
-        const int n = nA0 + e;
-        st_dev16(n < a.n_qkv ? a.qkv + n : a.act_buf + (n - a.n_qkv), f32_to_bf16_bits(stage[e]));
+      const int rot = mg_run_phase(ring, cur, sp, tA0, tA1, KTA, xn, partA, lane, wave);
+      wg_sync();
+
+      if (service && lane * 4 < rowsA) {
+        const int n = nA0 + lane * 4;
+        uint32_t packed[2];
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          float v[2];
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            const int e = lane * 4 + h2 * 2 + k;
+            float s4 = __uint_as_float((uint32_t)((bias_a >> (16 * (h2 * 2 + k))) & 0xffffu) << 16);
+#pragma unroll
+            for (int w = 0; w < kMegaStream; ++w) s4 += partA[e * kMegaWaves + w];
+            if (n >= a.n_qkv) s4 = act_eval(a.act, s4);
+            v[k] = s4;
+          }
+          packed[h2] = pack_bf16x2(v[0], v[1]);
+        }
+        st_dev64(n < a.n_qkv ? a.qkv + n : a.act_buf + (n - a.n_qkv), (uint64_t)packed[0] | ((uint64_t)packed[1] << 32));
       }
       stamp(l, 1);
-      grid_sync(a.barrier, bar++, fault);
+      mg_grid_arrive(barrier, bar, service, lane);
+      stamp(l, 8);
+      mg_rotate_by(ring, rot);
+      if (is_attn) {
+        const int col = tid % NCOL, grp = tid / NCOL;
+        k_load(Kc, tid);
+        v_load(Vc, grp, col, grp < NG_V);
+      }
+      mg_grid_wait(barrier, bar++, fault, service, lane);
       stamp(l, 2);
     }
 
-    // =================================================== phase B
     {
       const int tid = mg_opaque(tid0), lane = tid & 63;
-      if (tid < 2 * kMegaRowsMax * kMegaWaves) partB[tid] = 0.f;  // partB and partC are adjacent
-      // act -> LDS
+      for (int e = tid; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
+
       for (int k = tid * 4; k < I; k += kMegaThreads * 4) {
         const uint64_t v = ld_dev64(a.act_buf + k);
         *reinterpret_cast<uint64_t *>(xs + k) = v;
       }
       if (is_attn) {
         const int h = wg;
-        // q, k, v of the new token
+
         if (tid < 3 * D / 2) {
           const int which = tid / (D / 2), e = (tid - which * (D / 2)) * 2;
           const uint32_t w = ld_dev32(a.qkv + which * QD + h * D + e);
@@ -450,28 +522,30 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           Vc[(int64_t)pos * D + tid] = f32_to_bf16_bits(vr);
         }
         wg_sync();
-        // scores against the cached keys, two rounds of NG_K * UK keys in flight
+
         {
-          const int g = tid >> 4, gl = tid & 15;
-          constexpr int RK = NG_K * kMegaUK;
-          for (int tb = 0; tb < pos; tb += 2 * RK) {
-            k_scores(kreg[0], tb + g, gl);
-            if (tb + 2 * RK < pos) k_load(kreg[0], Kc, tb + 2 * RK + g, gl);
-            if (tb + RK < pos) {
-              k_scores(kreg[1], tb + RK + g, gl);
-              if (tb + 3 * RK < pos) k_load(kreg[1], Kc, tb + 3 * RK + g, gl);
-            }
+          constexpr int RKP = kMegaThreads * kMegaUK;
+          for (int qb = 0; qb < pos * NCOL; qb += RKP) {
+            if (qb > 0) k_load(Kc, qb + tid);
+            k_partials(qb + tid);
           }
         }
-        if (wave == kMegaWaves - 1) {  // the new token's own key
+        wg_sync();
+        for (int t = tid; t < pos; t += kMegaThreads) {
+          float sc = 0.f;
+#pragma unroll
+          for (int c = 0; c < NCOL; ++c) sc += pd[t * NCOL + c];
+          scores[t] = sc * att_scale;
+        }
+        if (wave == kMegaWaves - 1) {
           float acc = 0.f;
           for (int d = lane; d < D; d += 64) acc = fmaf(qf[d], knew[d], acc);
           acc = mg_wave_sum(acc);
-          if (lane == 0) scores[pos] = acc * a.scale;
+          if (lane == 0) scores[pos] = acc * att_scale;
         }
         wg_sync();
         const int cnt = pos + 1;
-        float m = -INFINITY;
+        float m = -(__builtin_inff ());
         for (int t = tid; t < cnt; t += kMegaThreads) m = fmaxf(m, scores[t]);
         m = wave_max(m);
         if (lane == 0) sh[wave] = m;
@@ -491,7 +565,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         sum = 0.f;
 #pragma unroll
         for (int w = 0; w < kMegaWaves; ++w) sum += sh[kMegaWaves + w];
-        // unnormalised P.V over the cached values, two rounds of NG_V * UV rows in flight
+
         {
           const int col = tid % NCOL, grp = tid / NCOL;
           const bool active = grp < NG_V;
@@ -499,13 +573,9 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           float acc[8];
 #pragma unroll
           for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-          for (int tb = 0; tb < pos; tb += 2 * RV) {
-            v_accum(vreg[0], tb + grp, acc);
-            if (tb + 2 * RV < pos) v_load(vreg[0], Vc, tb + 2 * RV + grp, col, active);
-            if (tb + RV < pos) {
-              v_accum(vreg[1], tb + RV + grp, acc);
-              if (tb + 3 * RV < pos) v_load(vreg[1], Vc, tb + 3 * RV + grp, col, active);
-            }
+          for (int tb = 0; tb < pos; tb += RV) {
+            if (tb > 0) v_load(Vc, tb + grp, col, active);
+            v_accum(tb + grp, acc);
           }
           if (active) {
 #pragma unroll
@@ -513,7 +583,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           }
         }
         wg_sync();
-        // two-level sum over the NG_V groups, then the head's D outputs as D/2 packed pairs
+
         if (tid < 4 * D) {
           const int d = tid % D, q4 = tid / D;
           float r = 0.f;
@@ -521,56 +591,67 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           red2[tid] = r;
         }
         wg_sync();
-        if (tid < D / 2) {
+        if (wave == kMegaService && lane < D / 2) {
           const float inv = 1.0f / sum, p_new = scores[pos];
           float o[2];
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
-            const int d = 2 * tid + k;
+            const int d = 2 * lane + k;
             o[k] = (p_new * vnew[d] + red2[d] + red2[D + d] + red2[2 * D + d] + red2[3 * D + d]) * inv;
           }
-          st_dev32(a.attn + h * D + 2 * tid, pack_bf16x2(o[0], o[1]));
+          st_dev32(a.attn + h * D + 2 * lane, pack_bf16x2(o[0], o[1]));
         }
       }
       wg_sync();
       stamp(l, 3);
-      run_ring(ly.Wb, tB0, tB1, KTB, QD, xs, partB, lane);
-      // first loads of phase C: the dense columns of the same rows
-      prime_ring(ly.Wb, tC0, tC1, KTC, 0, lane);
+      const int rot = mg_run_phase(ring, cur, sp, tB0, tB1, KTB, xs, partB, lane, wave);
       stamp(l, 4);
-      grid_sync(a.barrier, bar++, fault);
+      mg_grid_arrive(barrier, bar, wave == kMegaService, lane);
+      mg_rotate_by(ring, rot);
+      mg_grid_wait(barrier, bar++, fault, wave == kMegaService, lane);
       stamp(l, 5);
     }
 
-    // =================================================== phase C
     {
       const int tid = mg_opaque(tid0), lane = tid & 63;
-      // epilogue operands of this thread's row, requested before the stream
-      float bsum = 0.f, res = 0.f;
-      if (tid < nrows) {
-        res = bf16_bits_to_f32(ld_dev16(a.x + n0 + tid));
-        bsum = bf16_bits_to_f32(ly.bd[n0 + tid]) + bf16_bits_to_f32(ly.bf[n0 + tid]);
+      const bool service = wave == kMegaService;
+
+      uint64_t res4 = 0, bd4 = 0, bf4 = 0;
+      if (service && lane * 4 < nrows) {
+        res4 = ld_dev64(a.x + n0 + lane * 4);
+        bd4 = *reinterpret_cast<const uint64_t *>(ly.bd + n0 + lane * 4);
+        bf4 = *reinterpret_cast<const uint64_t *>(ly.bf + n0 + lane * 4);
       }
       for (int k = tid * 4; k < QD; k += kMegaThreads * 4) {
         const uint64_t v = ld_dev64(a.attn + k);
         *reinterpret_cast<uint64_t *>(xa + k) = v;
       }
       wg_sync();
-      run_ring(ly.Wb, tC0, tC1, KTC, 0, xa, partC, lane);
-      if (l + 1 < a.L) prime_A(a.layers[l + 1].Wa, lane);
+      const int rot = mg_run_phase(ring, cur, sp, tC0, tC1, KTC, xa, partC, lane, wave);
       wg_sync();
-      // x[n] += dense + fc2 + biases for the rows of this block.
-      // Fixed summation order: fc2 partials of the waves, then the dense partials.
-      if (tid < nrows) {
-        float sacc = 0.f;
+
+      if (service && lane * 4 < nrows) {
+        auto elem = [](uint64_t v, int k) { return __uint_as_float((uint32_t)((v >> (16 * k)) & 0xffffu) << 16); };
+        float v[4];
 #pragma unroll
-        for (int w = 0; w < kMegaWaves; ++w) sacc += partB[tid * kMegaWaves + w];
+        for (int k = 0; k < 4; ++k) {
+          const int e = lane * 4 + k;
+          float sacc = 0.f;
 #pragma unroll
-        for (int w = 0; w < kMegaWaves; ++w) sacc += partC[tid * kMegaWaves + w];
-        st_dev16(a.x + n0 + tid, f32_to_bf16_bits(sacc + bsum + res));
+          for (int w = 0; w < kMegaStream; ++w) sacc += partB[e * kMegaWaves + w];
+#pragma unroll
+          for (int w = 0; w < kMegaStream; ++w) sacc += partC[e * kMegaWaves + w];
+          v[k] = sacc + (elem(bd4, k) + elem(bf4, k)) + elem(res4, k);
+        }
+        st_dev64(a.x + n0 + lane * 4,
+                 (uint64_t)pack_bf16x2(v[0], v[1]) | ((uint64_t)pack_bf16x2(v[2], v[3]) << 32));
       }
       stamp(l, 6);
-      if (l + 1 < a.L) grid_sync(a.barrier, bar++, fault);
+      if (l + 1 < a.L) {
+        mg_grid_arrive(barrier, bar, service, lane);
+        mg_rotate_by(ring, rot);
+        mg_grid_wait(barrier, bar++, fault, service, lane);
+      }
       stamp(l, 7);
     }
   }
@@ -578,9 +659,9 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
 
 size_t mega_lds_bytes(const MegaArgs &a, int D) {
   const int NG_V = kMegaThreads / (D / 8);
-  size_t n = (size_t)(a.I + a.QD) * 2;
-  n += sizeof(float) * (2 * kMegaRowsMax * kMegaWaves + 6 * (size_t)D + (size_t)NG_V * D + 2 * kMegaWaves +
-                        4 * (size_t)D + (size_t)a.Tmax + 1);
+  size_t n = (size_t)(a.I + a.QD + a.H) * 2;
+  n += sizeof(float) * ((kMegaRowsAMax + 2 * kMegaRowsMax) * kMegaWaves + 6 * (size_t)D + (size_t)NG_V * D +
+                        2 * kMegaWaves + 4 * (size_t)D + (size_t)a.Tmax + 1 + (size_t)a.Tmax * (D / 8));
   return (n + 15) & ~(size_t)15;
 }
 
@@ -589,18 +670,18 @@ bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
   if (a.H != 2560) return no("hidden size is not 2560");
   if (D != 80) return no("head_dim is not 80");
   if (a.Hq * D != a.QD || a.QD % 512 || a.I % 512) return no("projection widths are not multiples of 512");
-  if (a.Hq > num_cu) return no("more heads than CUs");
-  if (a.n_qkv != 3 * a.QD || a.NA != a.n_qkv + a.I) return no("q|k|v layout");
+  if (a.Hq > num_cu || num_cu > 256) return no("more heads than CUs, or more than 256 CUs");
+  if (a.n_qkv != 3 * a.QD || a.NA != a.n_qkv + a.I || a.n_qkv % 4 || a.NA % 4) return no("q|k|v layout");
   if (a.rot > D || (a.rot & 1)) return no("rotary_dim");
-  // rows per block in phases B and C
+
   const int others = num_cu - a.Hq;
   const int ra = others > 0 ? a.rows_attn : (a.H + a.Hq - 1) / a.Hq;
-  if (ra < 0 || ra > kMegaRowsMax) return no("rows_attn");
+  if (ra < 0 || ra > kMegaRowsMax || ra % 4) return no("rows_attn");
   if (others > 0) {
     const int rem = a.H - a.Hq * ra;
-    if (rem < 0 || (rem + others - 1) / others + 1 > kMegaRowsMax) return no("too many rows per block");
+    if (rem < 0 || rem / others + 4 > kMegaRowsMax) return no("too many rows per block");
   }
-  if ((size_t)(a.NA / num_cu + 2) * sizeof(float) > (size_t)a.I * 2) return no("phase A staging does not fit");
+  if (a.NA / num_cu + 4 > kMegaRowsAMax) return no("too many phase A rows per block");
   if (mega_lds_bytes(a, D) > 150 * 1024) return no("context too long for the LDS score buffer");
   return true;
 }

@@ -175,7 +175,7 @@ __global__ void k_set_state(DevState *st, int pos, int step) {
 template <typename T>
 __global__ void __launch_bounds__(1024)
 k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
-               int dstep, const T *embed, T *x_next, int H, float embed_scale, unsigned *grid_barrier) {
+               int dstep, const T *embed, T *x_next, int H, float embed_scale, unsigned *grid_barrier, int grid_blocks) {
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   __shared__ uint32_t chosen;
@@ -223,7 +223,8 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
     __threadfence();
     int prev = atomicAdd(&state->done, 1);
     if (prev == B - 1) {  // every block has read `step` and written its outputs
-      if (grid_barrier) *grid_barrier = 0;  // the persistent decode kernel of this step has finished
+      // the persistent decode kernel of this step has finished: lower its barrier flags
+      for (int i = 0; i < grid_blocks; ++i) grid_barrier[i] = 0;
       state->done = 0;
       state->pos += dpos;
       state->step += dstep;
@@ -314,11 +315,18 @@ static int create_phi2(rai_hip_decoder *d) {
   RAI_TRY(dalloc(d, (size_t)V * H * es, &d->embed));
   add_slot(d, "model.embed_tokens.weight", V, H, d->embed, H);
   d->layers.resize(d->L);
+  // The two weight matrices of all layers sit back to back (layer l at a fixed
+  // stride), so a kernel that walks through the layers computes their addresses
+  // instead of loading them.
+  char *wa_all = nullptr, *wb_all = nullptr;
+  const size_t wa_bytes = (size_t)d->NA * H * es, wb_bytes = (size_t)H * d->KB * es;
+  RAI_TRY(dalloc(d, wa_bytes * d->L, &wa_all));
+  RAI_TRY(dalloc(d, wb_bytes * d->L, &wb_all));
   for (int l = 0; l < d->L; ++l) {
     Layer &ly = d->layers[l];
-    RAI_TRY(dalloc(d, (size_t)d->NA * H * es, &ly.Wa));
+    ly.Wa = wa_all + wa_bytes * l;
     RAI_TRY(dalloc(d, (size_t)d->NA * es, &ly.ba));
-    RAI_TRY(dalloc(d, (size_t)H * d->KB * es, &ly.Wb));
+    ly.Wb = wb_all + wb_bytes * l;
     RAI_TRY(dalloc(d, (size_t)H * es, &ly.bd));
     RAI_TRY(dalloc(d, (size_t)H * es, &ly.bf));
     RAI_TRY(dalloc(d, (size_t)H * es, &ly.ln_w));
@@ -448,6 +456,8 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   MegaArgs m;
   memset(&m, 0, sizeof(m));
   m.layers = d->mega_layers;
+  m.Wa0 = (const uint16_t *)d->layers[0].Wa; m.Wb0 = (const uint16_t *)d->layers[0].Wb;
+  m.wa_stride = (int64_t)d->NA * d->H; m.wb_stride = (int64_t)d->H * d->KB;
   m.L = d->L; m.H = d->H; m.I = d->I; m.QD = d->QD; m.NA = d->NA; m.n_qkv = d->QD + 2 * d->KD;
   m.Hq = d->Hq; m.rot = d->cfg.rotary_dim; m.Tmax = d->cfg.max_context;
   m.x = (uint16_t *)d->x; m.qkv = (uint16_t *)d->qkv;
@@ -458,7 +468,7 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   m.state = d->state; m.barrier = d->mega_barrier;
   m.ln_eps = (float)d->cfg.norm_eps; m.scale = (float)(1.0 / sqrt((double)d->D));
   m.act = d->cfg.hidden_act;
-  static const int rows_attn = getenv("RAI_HIP_MEGA_ROWS_ATTN") ? atoi(getenv("RAI_HIP_MEGA_ROWS_ATTN")) : 4;
+  static const int rows_attn = getenv("RAI_HIP_MEGA_ROWS_ATTN") ? atoi(getenv("RAI_HIP_MEGA_ROWS_ATTN")) : 0;
   m.rows_attn = rows_attn;
   m.prof = d->mega_prof;
   return m;
@@ -579,11 +589,11 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier);
+                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale, d->mega_barrier);
+                       d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
@@ -716,11 +726,11 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier);
+                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale, d->mega_barrier);
+                       d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
@@ -738,23 +748,42 @@ static int check_fault(rai_hip_decoder *d) {
   DevState hs;
   RAI_TRY(rai_hip_d2h(d->dev, &hs, d->state, sizeof(hs)));
   if (d->mega_prof) {  // phase timings of the last token: mean over layers, for three blocks
-    std::vector<unsigned long long> t((size_t)d->num_cu * d->L * 8);
+    std::vector<unsigned long long> t((size_t)d->num_cu * d->L * 16);
     RAI_HIP_TRY(hipMemcpy(t.data(), d->mega_prof, t.size() * 8, hipMemcpyDeviceToHost));
     const int blocks[4] = {0, d->Hq - 1, d->Hq, d->num_cu - 1};
+    auto at = [&](int b, int l, int k) { return (double)t[((size_t)b * d->L + l) * 16 + k] * 0.01; };
     for (int bi = 0; bi < 4; ++bi) {
       double iv[7] = {0, 0, 0, 0, 0, 0, 0};
       const int b = blocks[bi];
       for (int l = 0; l < d->L; ++l)
-        for (int k = 0; k < 7; ++k)
-          iv[k] += (double)(t[((size_t)b * d->L + l) * 8 + k + 1] - t[((size_t)b * d->L + l) * 8 + k]) * 0.01 / d->L;
+        for (int k = 0; k < 7; ++k) iv[k] += (at(b, l, k + 1) - at(b, l, k)) / d->L;
       fprintf(stderr, "mega prof block %3d: A %.2f | bar %.2f | B-pre(attn) %.2f | B-stream %.2f | bar %.2f | C %.2f | bar %.2f us\n",
               b, iv[0], iv[1], iv[2], iv[3], iv[4], iv[5], iv[6]);
+    }
+    // per barrier over all blocks: spread of the arrivals, last arrival -> first exit, spread of the exits
+    const int before[3] = {1, 4, 6}, after[3] = {2, 5, 7};
+    for (int k = 0; k < 3; ++k) {
+      double spread = 0, lat = 0, espread = 0;
+      int layers = 0, last_attn = 0;
+      for (int l = 0; l + (k == 2 ? 1 : 0) < d->L; ++l, ++layers) {
+        double amin = 1e30, amax = 0, emin = 1e30, emax = 0;
+        int who = 0;
+        for (int b = 0; b < d->num_cu; ++b) {
+          const double av = at(b, l, before[k]), ev = at(b, l, after[k]);
+          if (av > amax) { amax = av; who = b; }
+          amin = av < amin ? av : amin; emin = ev < emin ? ev : emin; emax = ev > emax ? ev : emax;
+        }
+        spread += amax - amin; lat += emin - amax; espread += emax - emin;
+        last_attn += who < d->Hq;
+      }
+      fprintf(stderr, "mega prof barrier %d: arrival spread %.2f us, last arrival -> first exit %.2f us, exit spread %.2f us, last arriver was an attention block in %d of %d layers\n",
+              k, spread / layers, lat / layers, espread / layers, last_attn, layers);
     }
   }
   if (hs.fault == 0) return RAI_OK;
   hs.fault = 0;
   RAI_HIP_TRY(hipMemcpy(&d->state->fault, &hs.fault, sizeof(int), hipMemcpyHostToDevice));
-  RAI_HIP_TRY(hipMemset(d->mega_barrier, 0, sizeof(unsigned)));
+  RAI_HIP_TRY(hipMemset(d->mega_barrier, 0, sizeof(unsigned) * (d->num_cu < kMegaFlagWords ? d->num_cu : kMegaFlagWords)));
   return fail(RAI_ERR_HIP, "decoder: a grid barrier of the persistent decode kernel timed out");
 }
 
@@ -854,9 +883,14 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
     hipDeviceProp_t prop;
     d->num_cu = hipGetDeviceProperties(&prop, dev) == hipSuccess ? prop.multiProcessorCount : kNumCU;
   }
-  if ((st = dalloc(d, 128, &tmp))) return bail(st);
+  if ((st = dalloc(d, kMegaFlagWords * sizeof(unsigned), &tmp))) return bail(st);
   d->mega_barrier = (unsigned *)tmp;
-  if (hipMemset(d->mega_barrier, 0, 128) != hipSuccess) return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
+  {  // flags of blocks that exist start at 0, the padding reads as "arrived"
+    std::vector<unsigned> f(kMegaFlagWords, 0xffffffffu);
+    for (int i = 0; i < d->num_cu && i < kMegaFlagWords; ++i) f[i] = 0;
+    if (hipMemcpy(d->mega_barrier, f.data(), f.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess)
+      return bail(fail(RAI_ERR_HIP, "decoder_create: flag upload failed"));
+  }
   if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_MEGA") != nullptr) {
     std::vector<MegaLayer> ml(d->L);
     for (int l = 0; l < d->L; ++l) {
@@ -869,7 +903,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
     if (hipMemcpy(d->mega_layers, ml.data(), ml.size() * sizeof(MegaLayer), hipMemcpyHostToDevice) != hipSuccess)
       return bail(fail(RAI_ERR_HIP, "decoder_create: layer table upload failed"));
     if (getenv("RAI_HIP_MEGA_PROF")) {
-      if ((st = dalloc(d, (size_t)d->num_cu * d->L * 8 * sizeof(unsigned long long), &tmp))) return bail(st);
+      if ((st = dalloc(d, (size_t)d->num_cu * d->L * 16 * sizeof(unsigned long long), &tmp))) return bail(st);
       d->mega_prof = (unsigned long long *)tmp;
     }
     MegaArgs m = mega_args(d);
