@@ -891,7 +891,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
     if (hipMemcpy(d->mega_barrier, f.data(), f.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess)
       return bail(fail(RAI_ERR_HIP, "decoder_create: flag upload failed"));
   }
-  if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_MEGA") != nullptr) {
+  if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_NO_MEGA") == nullptr) {
     std::vector<MegaLayer> ml(d->L);
     for (int l = 0; l < d->L; ++l) {
       const Layer &ly = d->layers[l];

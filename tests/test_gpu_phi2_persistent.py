@@ -21,8 +21,7 @@ def wide_cfg(**kw):
     return phi2.Config(**base)
 
 
-def test_persistent_step_logits_match_oracle(hip, monkeypatch):
-    monkeypatch.setenv("RAI_HIP_MEGA", "1")
+def test_persistent_step_logits_match_oracle(hip):
     cfg = wide_cfg()
     dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
     ids = np.random.Generator(np.random.PCG64(11)).integers(0, cfg.vocab_size, (1, 21)).astype(np.uint32)
@@ -43,10 +42,10 @@ def test_persistent_step_logits_match_oracle(hip, monkeypatch):
 def test_persistent_generate_equals_per_primitive_path(hip, monkeypatch):
     cfg = wide_cfg(num_hidden_layers=3)
     prompt = np.random.Generator(np.random.PCG64(12)).integers(0, cfg.vocab_size, (1, 37)).astype(np.uint32)
+    monkeypatch.setenv("RAI_HIP_NO_MEGA", "1")
     plain, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
-    monkeypatch.setenv("RAI_HIP_MEGA", "1")
+    monkeypatch.delenv("RAI_HIP_NO_MEGA")
     mega, _ = make(cfg, "bf16", hip, max_batch=1, max_context=96)
-    monkeypatch.delenv("RAI_HIP_MEGA")
     a, _, _ = plain.generate(prompt, 24)
     b, _, _ = mega.generate(prompt, 24)
     want, logits_all = phi2.greedy_decode(ref, prompt, 24)
