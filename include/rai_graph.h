@@ -102,6 +102,9 @@ int rai_tensor_storage(const rai_tensor *t, rai_hip_tensor *out);
  * (device, op) pair without a rule (Error::Unimplemented), RAI_ERR_BAD_SHAPE when
  * the graph contains an Err node (Error::Op), or a kernel failure status. */
 int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph);
+/* The order in which rai_eval would visit the un-evaluated nodes behind `outputs`
+ * (utils.rs:35-66): writes up to `capacity` node ids, *count receives the tape length. */
+int rai_graph_eval_order(rai_tensor *const *outputs, int32_t n, uint64_t *ids, int32_t capacity, int32_t *count);
 /* Tensor::as_vec / as_bytes: evaluates if needed, copies the contiguous contents to the host. */
 int rai_tensor_to_host(rai_tensor *t, void *dst, size_t bytes);
 

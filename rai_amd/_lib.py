@@ -123,6 +123,59 @@ PROTOTYPES = {
     "rai_hip_decoder_context_len": [_vp, C.POINTER(_i32)],
 }
 
+class GraphStats(C.Structure):
+    _fields_ = [("nodes_evaluated", C.c_uint64), ("kernel_launches", C.c_uint64), ("fused_regions", C.c_uint64),
+                ("fused_nodes", C.c_uint64)]
+
+
+_T = C.c_void_p  # rai_tensor *
+_I64P = C.POINTER(_i64)
+_I32P = C.POINTER(_i32)
+# include/rai_graph.h: name -> (restype, argtypes)
+GRAPH_PROTOTYPES = {
+    "rai_full": (_T, [_dbl, _i32, _I64P, _i32, _i32]),
+    "rai_arange": (_T, [_dbl, _dbl, _dbl, _i32, _i32]),
+    "rai_from_array": (_T, [_vp, _i32, _I64P, _i32, _i32]),
+    "rai_to_dtype": (_T, [_T, _i32]),
+    "rai_unary": (_T, [_i32, _T, _dbl]),
+    "rai_binary": (_T, [_i32, _T, _T]),
+    "rai_matmul": (_T, [_T, _T]),
+    "rai_softmax": (_T, [_T, _i32]),
+    "rai_log_softmax": (_T, [_T, _i32]),
+    "rai_reduce": (_T, [_i32, _T, _I32P, _i32, _i32]),
+    "rai_argmax": (_T, [_T, _i32, _i32]),
+    "rai_argmin": (_T, [_T, _i32, _i32]),
+    "rai_index_select": (_T, [_T, _i32, _T]),
+    "rai_narrow": (_T, [_T, _i32, _i64, _i64]),
+    "rai_concatenate": (_T, [C.POINTER(_T), _i32, _i32]),
+    "rai_where": (_T, [_T, _T, _T]),
+    "rai_transpose": (_T, [_T, _i32, _i32]),
+    "rai_reshape": (_T, [_T, _I64P, _i32]),
+    "rai_permute": (_T, [_T, _I32P, _i32]),
+    "rai_broadcast_to": (_T, [_T, _I64P, _i32]),
+    "rai_to_contiguous": (_T, [_T]),
+    "rai_tensor_retain": (None, [_T]),
+    "rai_tensor_release": (None, [_T]),
+    "rai_tensor_rank": (_i32, [_T]),
+    "rai_tensor_dtype": (_i32, [_T]),
+    "rai_tensor_device": (_i32, [_T]),
+    "rai_tensor_op": (_i32, [_T]),
+    "rai_tensor_shape": (_i32, [_T, _I64P]),
+    "rai_tensor_is_evaluated": (_i32, [_T]),
+    "rai_tensor_num_inputs": (_i32, [_T]),
+    "rai_tensor_id": (C.c_uint64, [_T]),
+    "rai_tensor_error": (C.c_char_p, [_T]),
+    "rai_tensor_storage": (C.c_int, [_T, _TP]),
+    "rai_eval": (C.c_int, [C.POINTER(_T), _i32, _i32]),
+    "rai_graph_eval_order": (C.c_int, [C.POINTER(_T), _i32, C.POINTER(C.c_uint64), _i32, _I32P]),
+    "rai_tensor_to_host": (C.c_int, [_T, _vp, C.c_size_t]),
+    "rai_dispatch_unregister": (C.c_int, [_i32]),
+    "rai_dispatch_register_builtin": (C.c_int, [_i32]),
+    "rai_dispatch_has_rule": (_i32, [_i32]),
+    "rai_graph_set_fusion": (C.c_int, [_i32]),
+    "rai_graph_get_stats": (C.c_int, [C.POINTER(GraphStats), _i32]),
+}
+
 _lib = None
 
 
@@ -139,6 +192,10 @@ def load():
     for name, args in PROTOTYPES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is missing
         fn.restype = C.c_int
+        fn.argtypes = args
+    for name, (res, args) in GRAPH_PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
         fn.argtypes = args
     _lib = lib
     return lib

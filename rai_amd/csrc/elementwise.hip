@@ -6,6 +6,7 @@
 // :445-473,525-553,608-656,947-978 (unary), :658-774 (compare, max/min, cast),
 // :901-915 (where), :980-988 (contiguous).
 #include "common.h"
+#include "fused.h"
 
 namespace rai {
 
@@ -329,6 +330,61 @@ __global__ void __launch_bounds__(256) k_cast(IterSpace s, D *out, const S *in) 
   }
 }
 
+// ------------------------------------------------------------------ fused elementwise regions
+__device__ __forceinline__ float fused_round(float v, int dtype) {
+  if (dtype == RAI_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  if (dtype == RAI_F16) return __half2float(__float2half_rn(v));
+  return v;
+}
+__device__ __forceinline__ float fused_load(const void *base, int dtype, int64_t off) {
+  if (dtype == RAI_BF16) return bf16_bits_to_f32(((const uint16_t *)base)[off]);
+  if (dtype == RAI_F16) return __half2float(__ushort_as_half(((const uint16_t *)base)[off]));
+  return ((const float *)base)[off];
+}
+// One element per thread per step; the register file of the little machine
+// lives in LDS (one column per thread) because its indices are only known at
+// run time.  Each instruction is evaluated in f32 by the same routines as the
+// single-op kernels and rounded to the dtype of its node.
+__global__ void __launch_bounds__(256) k_fused_elementwise(FusedProgram p) {
+  __shared__ float regs[kFusedMaxInstr][256];
+  const int tid = threadIdx.x;
+  for (int64_t e = blockIdx.x * (int64_t)blockDim.x + tid; e < p.numel; e += (int64_t)gridDim.x * blockDim.x) {
+    int64_t loff[kFusedMaxLeaves];
+#pragma unroll
+    for (int l = 0; l < kFusedMaxLeaves; ++l) loff[l] = 0;
+    int64_t rem = e;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      const int64_t c = rem % p.shape[d];
+      rem /= p.shape[d];
+#pragma unroll
+      for (int l = 0; l < kFusedMaxLeaves; ++l)
+        if (l < p.n_leaves) loff[l] += c * p.lstride[l][d];
+    }
+    float v = 0.f;
+    for (int i = 0; i < p.n_instr; ++i) {
+      const FusedInstr in = p.instr[i];
+      switch (in.kind) {
+        case FUSED_LEAF: {
+          int64_t off = 0;
+#pragma unroll
+          for (int l = 0; l < kFusedMaxLeaves; ++l)
+            if (l == in.a) off = loff[l];
+          v = fused_load(p.leaf[in.a], p.leaf_dtype[in.a], off);
+          break;
+        }
+        case FUSED_CONST: v = in.param; break;
+        case FUSED_UNARY: v = fused_round(unary_eval<float>(in.op, regs[in.a][tid], in.param), in.dtype); break;
+        case FUSED_BINARY: v = fused_round(arith_eval<float>(in.op, regs[in.a][tid], regs[in.b][tid]), in.dtype); break;
+        default: v = fused_round(regs[in.a][tid], in.dtype); break;  // FUSED_CAST
+      }
+      regs[i][tid] = v;
+    }
+    if (p.out_dtype == RAI_BF16) ((uint16_t *)p.out)[e] = f32_to_bf16_bits(v);
+    else if (p.out_dtype == RAI_F16) ((uint16_t *)p.out)[e] = __half_as_ushort(__float2half_rn(v));
+    else ((float *)p.out)[e] = v;
+  }
+}
+
 // ------------------------------------------------------------------ host side
 static int grid_for(int64_t work_items) {
   int64_t blocks = (work_items + 255) / 256;
@@ -374,6 +430,16 @@ static int build_space(int nops, const rai_hip_tensor *const *ts, int max_v, Ite
 }
 
 template <typename T> static int max_pack() { return (int)(16 / sizeof(T)); }
+
+int launch_fused_elementwise(int dev, const FusedProgram &p) {
+  hipStream_t st = stream_of(dev);
+  if (!st) return RAI_ERR_HIP;
+  if (p.numel == 0) return RAI_OK;
+  RAI_REQUIRE(p.n_instr >= 1 && p.n_instr <= kFusedMaxInstr && p.n_leaves <= kFusedMaxLeaves, RAI_ERR_BAD_ARG,
+              "fused region: %d instructions, %d leaves", p.n_instr, p.n_leaves);
+  hipLaunchKernelGGL(k_fused_elementwise, dim3(grid_for(p.numel)), dim3(256), 0, st, p);
+  return launch_check("fused_elementwise");
+}
 
 }  // namespace rai
 

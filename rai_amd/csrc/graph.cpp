@@ -1,0 +1,919 @@
+// Lazy tensor graph, dispatcher and evaluator for the Hip device: the host-side
+// machinery of rai-core that sits in front of the kernels.
+//   rai-core/src/tensor.rs:28-37,229   Tensor = ref-counted node {device, dtype, shape, op, inputs, data}
+//   rai-core/src/ops/*.rs               one builder per primitive; a bad shape yields an Err node
+//   rai-core/src/utils.rs:35-66         iterative DFS topological sort that skips evaluated nodes
+//   rai-core/src/dispatch.rs:159-212    (device, op) -> rule table with runtime registration
+//   rai-core/src/eval.rs:31-51          eval(): per node look up the rule, run it, detach
+// On top of that an elementwise-fusion pass: a chain of elementwise primitives
+// (unary, arithmetic binary, float casts, constants) whose intermediate results
+// nobody else can observe is evaluated by one launch of a small register-machine
+// kernel (fused.h) that rounds exactly where node-by-node evaluation would.
+#include <cmath>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "fused.h"
+#include "rai_graph.h"
+
+using namespace rai;
+
+struct rai_tensor {
+  int refs;
+  uint64_t id;
+  int dev, dtype;
+  std::vector<int64_t> shape;
+  int op, sub;                    // rai_op_kind and its sub-kind (unary / binary / reduce op)
+  double p0, p1, p2;              // scalar parameters (fill value, arange start/step, powf exponent)
+  std::vector<int64_t> ip;        // integer parameters (dims, target shape, narrow start/len, keep_dim)
+  std::vector<rai_tensor *> inputs;
+  std::string err;                // message of an Err node
+  std::vector<uint8_t> host;      // FromArray payload
+  bool evaluated;
+  rai_hip_tensor view;            // storage once evaluated (may alias an input's buffer)
+  void *buf;                      // retained allocation the view points into
+};
+
+namespace {
+
+uint64_t g_next_id = 1;
+bool g_fusion = true;
+rai_graph_stats g_stats = {0, 0, 0, 0};
+
+int64_t numel_of(const std::vector<int64_t> &s) {
+  int64_t n = 1;
+  for (int64_t d : s) n *= d;
+  return n;
+}
+
+rai_tensor *new_node(int dev, int dtype, const std::vector<int64_t> &shape, int op, std::vector<rai_tensor *> inputs) {
+  rai_tensor *t = new rai_tensor();
+  t->refs = 1;
+  t->id = g_next_id++;
+  t->dev = dev;
+  t->dtype = dtype;
+  t->shape = shape;
+  t->op = op;
+  t->sub = 0;
+  t->p0 = t->p1 = t->p2 = 0.0;
+  t->inputs = std::move(inputs);
+  for (rai_tensor *i : t->inputs) ++i->refs;
+  t->evaluated = false;
+  memset(&t->view, 0, sizeof(t->view));
+  t->buf = nullptr;
+  return t;
+}
+
+// Err node (rai-core/src/ops/err.rs): keeps the op it replaces and its inputs; eval reports it.
+rai_tensor *err_node(int dev, int dtype, const std::vector<int64_t> &shape, std::vector<rai_tensor *> inputs,
+                     const std::string &msg) {
+  rai_tensor *t = new_node(dev, dtype, shape, RAI_OP_ERR, std::move(inputs));
+  t->err = msg;
+  return t;
+}
+
+std::string shape_str(const std::vector<int64_t> &s) {
+  std::string r = "[";
+  for (size_t i = 0; i < s.size(); ++i) r += (i ? ", " : "") + std::to_string(s[i]);
+  return r + "]";
+}
+std::string incompatible(const rai_tensor *a, const rai_tensor *b) {
+  return "IncompatibleShape { lhs: " + shape_str(a->shape) + ", rhs: " + shape_str(b->shape) + " }";
+}
+
+// numpy-style right-aligned broadcast (rai-core/src/shape.rs:88-127)
+bool broadcast_shapes(const std::vector<int64_t> &l, const std::vector<int64_t> &r, std::vector<int64_t> *out, bool *lb,
+                      bool *rb) {
+  std::vector<int64_t> a = l, b = r;
+  *lb = *rb = false;
+  if (a.size() < b.size()) { a.insert(a.begin(), b.size() - a.size(), 1); *lb = true; }
+  else if (b.size() < a.size()) { b.insert(b.begin(), a.size() - b.size(), 1); *rb = true; }
+  out->clear();
+  for (size_t i = 0; i < a.size(); ++i) {
+    if (a[i] == b[i]) out->push_back(a[i]);
+    else if (a[i] == 1) { out->push_back(b[i]); *lb = true; }
+    else if (b[i] == 1) { out->push_back(a[i]); *rb = true; }
+    else return false;
+  }
+  return true;
+}
+
+int norm_dim(int d, int rank) { return d < 0 ? d + rank : d; }
+
+// ------------------------------------------------------------------ storage helpers
+void drop_storage(rai_tensor *t) {
+  if (t->buf) (void)rai_hip_release(t->buf);
+  t->buf = nullptr;
+  t->evaluated = false;
+}
+
+void contiguous_view(rai_tensor *t, void *data) {
+  rai_hip_tensor &v = t->view;
+  memset(&v, 0, sizeof(v));
+  v.data = data;
+  v.dtype = t->dtype;
+  v.rank = (int32_t)t->shape.size();
+  int64_t st = 1;
+  for (int i = v.rank - 1; i >= 0; --i) {
+    v.shape[i] = t->shape[i];
+    v.stride[i] = st;
+    st *= t->shape[i];
+  }
+  v.offset = 0;
+}
+
+// Fresh contiguous output for a node (functional semantics: outputs never alias inputs).
+int alloc_output(rai_tensor *t) {
+  void *p = nullptr;
+  const size_t bytes = (size_t)numel_of(t->shape) * dtype_size(t->dtype);
+  RAI_TRY(rai_hip_alloc(t->dev, bytes ? bytes : 1, &p));
+  t->buf = p;
+  contiguous_view(t, p);
+  return RAI_OK;
+}
+
+// The node's data becomes a view of `src`'s buffer.
+void alias_storage(rai_tensor *t, const rai_tensor *src, const rai_hip_tensor &v) {
+  t->view = v;
+  t->buf = src->buf;
+  if (t->buf) (void)rai_hip_retain(t->buf);
+}
+
+// ------------------------------------------------------------------ evaluation rules (one per primitive)
+typedef int (*rule_fn)(rai_tensor *);
+
+int ev_full(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_fill(t->dev, &t->view, t->p0);
+}
+int ev_arange(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_arange(t->dev, &t->view, t->p0, t->p2);
+}
+int ev_from_array(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  return rai_hip_h2d(t->dev, t->view.data, t->host.data(), t->host.size());
+}
+int ev_to_dtype(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_cast(t->dev, &t->inputs[0]->view, &t->view);
+}
+int ev_unary(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_unary(t->dev, t->sub, &t->inputs[0]->view, &t->view, t->p0);
+}
+int ev_binary(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_binary(t->dev, t->sub, &t->inputs[0]->view, &t->inputs[1]->view, &t->view);
+}
+int ev_matmul(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_matmul(t->dev, &t->inputs[0]->view, &t->inputs[1]->view, &t->view);
+}
+int ev_softmax(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_softmax(t->dev, &t->inputs[0]->view, (int32_t)t->ip[0], &t->view);
+}
+int ev_log_softmax(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_log_softmax(t->dev, &t->inputs[0]->view, (int32_t)t->ip[0], &t->view);
+}
+int ev_reduce(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  std::vector<int32_t> dims(t->ip.begin() + 1, t->ip.end());
+  return rai_hip_reduce(t->dev, t->sub, &t->inputs[0]->view, dims.data(), (int32_t)dims.size(), (int32_t)t->ip[0], &t->view);
+}
+int ev_argmax(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_argmax(t->dev, &t->inputs[0]->view, (int32_t)t->ip[0], (int32_t)t->ip[1], &t->view);
+}
+int ev_argmin(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_argmin(t->dev, &t->inputs[0]->view, (int32_t)t->ip[0], (int32_t)t->ip[1], &t->view);
+}
+int ev_index_select(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_index_select(t->dev, &t->inputs[0]->view, &t->inputs[1]->view, (int32_t)t->ip[0], &t->view);
+}
+int ev_where(rai_tensor *t) {  // inputs are ordered [on_true, on_false, cond] (ops/where.rs:37-45)
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_where(t->dev, &t->inputs[2]->view, &t->inputs[0]->view, &t->inputs[1]->view, &t->view);
+}
+int ev_to_contiguous(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_copy(t->dev, &t->inputs[0]->view, &t->view);
+}
+int ev_concatenate(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  const int dim = (int)t->ip[0];
+  int64_t at = 0;
+  for (rai_tensor *in : t->inputs) {
+    rai_hip_tensor dst = t->view;  // the slice of the output this input fills
+    dst.shape[dim] = in->shape[dim];
+    dst.offset += at * dst.stride[dim];
+    at += in->shape[dim];
+    if (numel_of(in->shape) == 0) continue;
+    ++g_stats.kernel_launches;
+    RAI_TRY(rai_hip_copy(t->dev, &in->view, &dst));
+  }
+  return RAI_OK;
+}
+// ---- views: no launch, the node shares the input's buffer
+int ev_transpose(rai_tensor *t) {
+  rai_hip_tensor v = t->inputs[0]->view;
+  const int a = (int)t->ip[0], b = (int)t->ip[1];
+  std::swap(v.shape[a], v.shape[b]);
+  std::swap(v.stride[a], v.stride[b]);
+  alias_storage(t, t->inputs[0], v);
+  return RAI_OK;
+}
+int ev_permute(rai_tensor *t) {
+  const rai_hip_tensor &s = t->inputs[0]->view;
+  rai_hip_tensor v = s;
+  for (int i = 0; i < v.rank; ++i) {
+    v.shape[i] = s.shape[t->ip[i]];
+    v.stride[i] = s.stride[t->ip[i]];
+  }
+  alias_storage(t, t->inputs[0], v);
+  return RAI_OK;
+}
+int ev_narrow(rai_tensor *t) {
+  rai_hip_tensor v = t->inputs[0]->view;
+  const int dim = (int)t->ip[0];
+  v.offset += t->ip[1] * v.stride[dim];
+  v.shape[dim] = t->ip[2];
+  alias_storage(t, t->inputs[0], v);
+  return RAI_OK;
+}
+int ev_broadcast(rai_tensor *t) {
+  const rai_hip_tensor &s = t->inputs[0]->view;
+  rai_hip_tensor v = s;
+  v.rank = (int32_t)t->shape.size();
+  const int lead = v.rank - s.rank;
+  for (int i = 0; i < v.rank; ++i) {
+    v.shape[i] = t->shape[i];
+    if (i < lead) v.stride[i] = 0;
+    else v.stride[i] = s.shape[i - lead] == t->shape[i] ? s.stride[i - lead] : 0;
+  }
+  alias_storage(t, t->inputs[0], v);
+  return RAI_OK;
+}
+int ev_reshape(rai_tensor *t) {
+  rai_tensor *in = t->inputs[0];
+  if (is_contiguous(&in->view)) {
+    rai_hip_tensor v;
+    memset(&v, 0, sizeof(v));
+    v.data = in->view.data;
+    v.dtype = in->view.dtype;
+    v.offset = in->view.offset;
+    v.rank = (int32_t)t->shape.size();
+    int64_t st = 1;
+    for (int i = v.rank - 1; i >= 0; --i) {
+      v.shape[i] = t->shape[i];
+      v.stride[i] = st;
+      st *= t->shape[i];
+    }
+    alias_storage(t, in, v);
+    return RAI_OK;
+  }
+  // a reshape of a non-contiguous view has to materialise it first
+  RAI_TRY(alloc_output(t));
+  rai_hip_tensor as_in = t->view;
+  as_in.rank = in->view.rank;
+  int64_t st = 1;
+  for (int i = as_in.rank - 1; i >= 0; --i) {
+    as_in.shape[i] = in->view.shape[i];
+    as_in.stride[i] = st;
+    st *= in->view.shape[i];
+  }
+  ++g_stats.kernel_launches;
+  return rai_hip_copy(t->dev, &in->view, &as_in);
+}
+
+const rule_fn kBuiltin[RAI_OP_COUNT_] = {
+    ev_full, ev_arange, ev_from_array, ev_to_dtype, ev_unary, ev_binary, ev_matmul, ev_softmax, ev_log_softmax, ev_reduce,
+    ev_argmax, ev_argmin, ev_index_select, ev_narrow, ev_concatenate, ev_where, ev_transpose, ev_reshape, ev_permute,
+    ev_broadcast, ev_to_contiguous, nullptr /* Err nodes never reach a rule */};
+rule_fn g_rules[RAI_OP_COUNT_];
+bool g_rules_init = false;
+void init_rules() {
+  if (g_rules_init) return;
+  for (int i = 0; i < RAI_OP_COUNT_; ++i) g_rules[i] = kBuiltin[i];
+  g_rules_init = true;
+}
+
+const char *op_name(int op) {
+  static const char *n[RAI_OP_COUNT_] = {"Full", "Arange", "FromArray", "ToDType", "Unary", "Binary", "MatMul", "Softmax",
+                                         "LogSoftmax", "Reduce", "ArgMax", "ArgMin", "IndexSelect", "Narrow",
+                                         "Concatenate", "Where", "Transpose", "Reshape", "Permute", "Broadcast",
+                                         "ToContiguous", "Err"};
+  return op >= 0 && op < RAI_OP_COUNT_ ? n[op] : "?";
+}
+
+// ------------------------------------------------------------------ topological order (utils.rs:35-66)
+int topo_sort(rai_tensor *const *outputs, int n, std::vector<rai_tensor *> *tape) {
+  std::unordered_set<uint64_t> visited;
+  std::vector<std::pair<rai_tensor *, bool>> stack;
+  for (int o = 0; o < n; ++o) {
+    stack.push_back({outputs[o], outputs[o]->inputs.empty()});
+    while (!stack.empty()) {
+      auto [t, inputs_done] = stack.back();
+      stack.pop_back();
+      if (visited.count(t->id) || t->evaluated) continue;
+      if (t->op == RAI_OP_ERR) return fail(RAI_ERR_BAD_SHAPE, "eval: %s", t->err.c_str());
+      if (inputs_done) {
+        visited.insert(t->id);
+        tape->push_back(t);
+      } else {
+        stack.push_back({t, true});
+        for (rai_tensor *in : t->inputs) stack.push_back({in, in->inputs.empty()});
+      }
+    }
+  }
+  return RAI_OK;
+}
+
+// ------------------------------------------------------------------ fusion pass
+bool fusable_dtype(int dt) { return dt == RAI_F32 || dt == RAI_BF16 || dt == RAI_F16; }
+bool elementwise(const rai_tensor *t) {
+  if (!fusable_dtype(t->dtype)) return false;
+  switch (t->op) {
+    case RAI_OP_UNARY: return fusable_dtype(t->inputs[0]->dtype);
+    case RAI_OP_BINARY:
+      return t->sub <= RAI_BIN_MINIMUM && fusable_dtype(t->inputs[0]->dtype) && t->inputs[1]->dtype == t->inputs[0]->dtype;
+    case RAI_OP_TO_DTYPE: return fusable_dtype(t->inputs[0]->dtype);
+    case RAI_OP_FULL: return true;
+    default: return false;
+  }
+}
+
+struct FusionPlan {
+  std::unordered_set<uint64_t> inlined;  // nodes that never receive data: they live inside a consumer's region
+};
+
+// A node is folded into its consumer when it is elementwise, exactly one edge of
+// the tape uses it, that user is elementwise too, it is not a requested output,
+// and no handle outside the tape refers to it (refs == that one edge).
+void plan_fusion(const std::vector<rai_tensor *> &tape, rai_tensor *const *outputs, int n_out, FusionPlan *plan) {
+  std::unordered_map<uint64_t, int> uses;
+  std::unordered_map<uint64_t, const rai_tensor *> user;
+  for (const rai_tensor *t : tape)
+    for (const rai_tensor *in : t->inputs) {
+      ++uses[in->id];
+      user[in->id] = t;
+    }
+  std::unordered_set<uint64_t> is_output;
+  for (int i = 0; i < n_out; ++i) is_output.insert(outputs[i]->id);
+  for (const rai_tensor *t : tape) {
+    if (!elementwise(t) || is_output.count(t->id) || !g_rules[t->op]) continue;  // fusion never hides a missing rule
+    auto u = uses.find(t->id);
+    if (u == uses.end() || u->second != 1 || t->refs != 1) continue;
+    const rai_tensor *c = user[t->id];
+    if (!elementwise(c) || numel_of(c->shape) != numel_of(t->shape) || c->shape != t->shape) continue;
+    plan->inlined.insert(t->id);
+  }
+}
+
+// Emits the instructions of `t` (post-order) into the program; returns its register or -1 when the region is too large.
+int emit(const rai_tensor *t, const FusionPlan &plan, bool root, FusedProgram *p, std::unordered_map<uint64_t, int> *leaf_reg,
+         std::vector<const rai_tensor *> *members) {
+  auto push = [&](FusedInstr in) -> int {
+    if (p->n_instr >= kFusedMaxInstr) return -1;
+    p->instr[p->n_instr] = in;
+    return p->n_instr++;
+  };
+  if (!root && !plan.inlined.count(t->id)) {  // a materialised input: leaf
+    auto it = leaf_reg->find(t->id);
+    if (it != leaf_reg->end()) return it->second;
+    if (p->n_leaves >= kFusedMaxLeaves) return -1;
+    const int l = p->n_leaves++;
+    p->leaf[l] = base_ptr(&t->view);
+    p->leaf_dtype[l] = t->dtype;
+    for (int d = 0; d < p->rank; ++d) p->lstride[l][d] = t->view.shape[d] == 1 ? 0 : t->view.stride[d];
+    FusedInstr in = {};
+    in.kind = FUSED_LEAF;
+    in.a = (uint8_t)l;
+    in.dtype = (uint8_t)t->dtype;
+    const int r = push(in);
+    if (r >= 0) (*leaf_reg)[t->id] = r;
+    return r;
+  }
+  if (!root) members->push_back(t);
+  FusedInstr in = {};
+  in.dtype = (uint8_t)t->dtype;
+  switch (t->op) {
+    case RAI_OP_FULL: {
+      in.kind = FUSED_CONST;
+      float v = (float)t->p0;  // rounded to the node's dtype like the fill kernel does
+      if (t->dtype == RAI_BF16) {
+        uint32_t u;
+        memcpy(&u, &v, 4);
+        if ((u & 0x7fffffffu) <= 0x7f800000u) { u += 0x7fffu + ((u >> 16) & 1u); u &= 0xffff0000u; }
+        memcpy(&v, &u, 4);
+      } else if (t->dtype == RAI_F16) {
+        v = (float)(_Float16)v;
+      }
+      in.param = v;
+      return push(in);
+    }
+    case RAI_OP_UNARY: {
+      const int a = emit(t->inputs[0], plan, false, p, leaf_reg, members);
+      if (a < 0) return -1;
+      in.kind = FUSED_UNARY;
+      in.op = (uint8_t)t->sub;
+      in.a = (uint8_t)a;
+      in.param = (float)t->p0;
+      return push(in);
+    }
+    case RAI_OP_BINARY: {
+      const int a = emit(t->inputs[0], plan, false, p, leaf_reg, members);
+      if (a < 0) return -1;
+      const int b = emit(t->inputs[1], plan, false, p, leaf_reg, members);
+      if (b < 0) return -1;
+      in.kind = FUSED_BINARY;
+      in.op = (uint8_t)t->sub;
+      in.a = (uint8_t)a;
+      in.b = (uint8_t)b;
+      return push(in);
+    }
+    default: {  // RAI_OP_TO_DTYPE
+      const int a = emit(t->inputs[0], plan, false, p, leaf_reg, members);
+      if (a < 0) return -1;
+      in.kind = FUSED_CAST;
+      in.a = (uint8_t)a;
+      return push(in);
+    }
+  }
+}
+
+bool has_inlined_input(const rai_tensor *t, const FusionPlan &plan) {
+  for (const rai_tensor *in : t->inputs)
+    if (plan.inlined.count(in->id)) return true;
+  return false;
+}
+
+// Evaluates the region rooted at t with one launch.  RAI_ERR_UNSUPPORTED means
+// "too large for one program": the caller falls back to node-by-node evaluation.
+int eval_region(rai_tensor *t, const FusionPlan &plan) {
+  FusedProgram p;
+  memset(&p, 0, sizeof(p));
+  p.rank = (int)t->shape.size();
+  p.numel = numel_of(t->shape);
+  for (int d = 0; d < p.rank; ++d) p.shape[d] = t->shape[d];
+  std::unordered_map<uint64_t, int> leaf_reg;
+  std::vector<const rai_tensor *> members;
+  if (emit(t, plan, true, &p, &leaf_reg, &members) < 0) return RAI_ERR_UNSUPPORTED;
+  RAI_TRY(alloc_output(t));
+  p.out = t->view.data;
+  p.out_dtype = t->dtype;
+  ++g_stats.kernel_launches;
+  ++g_stats.fused_regions;
+  g_stats.fused_nodes += members.size() + 1;
+  return launch_fused_elementwise(t->dev, p);
+}
+
+// Node-by-node evaluation of an inlined sub-tree (used when a region did not fit).
+int eval_plain(rai_tensor *t, const FusionPlan &plan);
+int eval_inputs_plain(rai_tensor *t, const FusionPlan &plan) {
+  for (rai_tensor *in : t->inputs)
+    if (!in->evaluated && plan.inlined.count(in->id)) RAI_TRY(eval_plain(in, plan));
+  return RAI_OK;
+}
+int eval_plain(rai_tensor *t, const FusionPlan &plan) {
+  RAI_TRY(eval_inputs_plain(t, plan));
+  rule_fn rule = g_rules[t->op];
+  RAI_REQUIRE(rule, RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op));
+  RAI_TRY(rule(t));
+  t->evaluated = true;
+  ++g_stats.nodes_evaluated;
+  return RAI_OK;
+}
+
+void detach(rai_tensor *t) {  // tensor.rs: drop the inputs so the graph behind an evaluated node can be freed
+  std::vector<rai_tensor *> ins;
+  ins.swap(t->inputs);
+  for (rai_tensor *i : ins) rai_tensor_release(i);
+}
+
+}  // namespace
+
+extern "C" {
+
+// ------------------------------------------------------------------ creation
+rai_tensor *rai_full(double value, int32_t dtype, const int64_t *shape, int32_t rank, int32_t dev) {
+  rai_tensor *t = new_node(dev, dtype, std::vector<int64_t>(shape, shape + rank), RAI_OP_FULL, {});
+  t->p0 = value;
+  return t;
+}
+
+rai_tensor *rai_arange(double start, double stop, double step, int32_t dtype, int32_t dev) {
+  // ops/arange.rs:102-117: ceil((stop - start) / step) elements
+  int64_t n = step != 0.0 ? (int64_t)ceil((stop - start) / step) : 0;
+  if (n < 0) n = 0;
+  rai_tensor *t = new_node(dev, dtype, {n}, RAI_OP_ARANGE, {});
+  t->p0 = start;
+  t->p1 = stop;
+  t->p2 = step;
+  return t;
+}
+
+rai_tensor *rai_from_array(const void *host, int32_t dtype, const int64_t *shape, int32_t rank, int32_t dev) {
+  rai_tensor *t = new_node(dev, dtype, std::vector<int64_t>(shape, shape + rank), RAI_OP_FROM_ARRAY, {});
+  const size_t bytes = (size_t)numel_of(t->shape) * dtype_size(dtype);
+  t->host.assign((const uint8_t *)host, (const uint8_t *)host + bytes);
+  return t;
+}
+
+// ------------------------------------------------------------------ primitives
+rai_tensor *rai_to_dtype(rai_tensor *x, int32_t dtype) {
+  if (x->dtype == dtype) {  // ops/to_dtype.rs:45-55: same dtype returns the tensor itself
+    ++x->refs;
+    return x;
+  }
+  return new_node(x->dev, dtype, x->shape, RAI_OP_TO_DTYPE, {x});
+}
+
+rai_tensor *rai_unary(int32_t op, rai_tensor *x, double param) {
+  rai_tensor *t = new_node(x->dev, x->dtype, x->shape, RAI_OP_UNARY, {x});
+  t->sub = op;
+  t->p0 = param;
+  return t;
+}
+
+rai_tensor *rai_binary(int32_t op, rai_tensor *lhs, rai_tensor *rhs) {
+  // ops/mod.rs:298-340: operands are wrapped in Broadcast nodes where needed; the output takes lhs' dtype
+  // (comparisons: U8)
+  const int out_dtype = op >= RAI_BIN_EQ ? RAI_U8 : lhs->dtype;
+  std::vector<int64_t> shape;
+  bool lb, rb;
+  if (!broadcast_shapes(lhs->shape, rhs->shape, &shape, &lb, &rb))
+    return err_node(lhs->dev, out_dtype, {}, {lhs, rhs}, incompatible(lhs, rhs));
+  rai_tensor *l = lb ? rai_broadcast_to(lhs, shape.data(), (int32_t)shape.size()) : lhs;
+  rai_tensor *r = rb ? rai_broadcast_to(rhs, shape.data(), (int32_t)shape.size()) : rhs;
+  rai_tensor *t = new_node(lhs->dev, out_dtype, shape, RAI_OP_BINARY, {l, r});
+  t->sub = op;
+  if (lb) rai_tensor_release(l);
+  if (rb) rai_tensor_release(r);
+  return t;
+}
+
+rai_tensor *rai_matmul(rai_tensor *lhs, rai_tensor *rhs) {
+  // ops/matmul.rs:34-70 + shape.rs:130-160: rank-1 operands are promoted, leading dims broadcast
+  rai_tensor *a = lhs, *b = rhs;
+  const bool a1 = lhs->shape.size() == 1, b1 = rhs->shape.size() == 1;
+  if (lhs->shape.empty() || rhs->shape.empty()) return err_node(lhs->dev, lhs->dtype, {}, {lhs, rhs}, incompatible(lhs, rhs));
+  if (a1) { int64_t s[2] = {1, lhs->shape[0]}; a = rai_reshape(lhs, s, 2); }
+  if (b1) { int64_t s[2] = {rhs->shape[0], 1}; b = rai_reshape(rhs, s, 2); }
+  auto done = [&](rai_tensor *res) {
+    if (a1) rai_tensor_release(a);
+    if (b1) rai_tensor_release(b);
+    return res;
+  };
+  const size_t ra = a->shape.size(), rbk = b->shape.size();
+  const int64_t m = a->shape[ra - 2], k = a->shape[ra - 1], k2 = b->shape[rbk - 2], n = b->shape[rbk - 1];
+  if (k != k2) return done(err_node(lhs->dev, lhs->dtype, {}, {lhs, rhs}, incompatible(lhs, rhs)));
+  std::vector<int64_t> batch;
+  bool lb = false, rb = false;
+  if (ra > 2 || rbk > 2) {
+    std::vector<int64_t> ab(a->shape.begin(), a->shape.end() - 2), bb(b->shape.begin(), b->shape.end() - 2);
+    if (!broadcast_shapes(ab, bb, &batch, &lb, &rb)) return done(err_node(lhs->dev, lhs->dtype, {}, {lhs, rhs}, incompatible(lhs, rhs)));
+  }
+  std::vector<int64_t> sa = batch, sb = batch, so = batch;
+  sa.push_back(m); sa.push_back(k);
+  sb.push_back(k); sb.push_back(n);
+  so.push_back(m); so.push_back(n);
+  rai_tensor *aa = lb ? rai_broadcast_to(a, sa.data(), (int32_t)sa.size()) : a;
+  rai_tensor *bb2 = rb ? rai_broadcast_to(b, sb.data(), (int32_t)sb.size()) : b;
+  rai_tensor *t = new_node(lhs->dev, lhs->dtype, so, RAI_OP_MATMUL, {aa, bb2});
+  if (lb) rai_tensor_release(aa);
+  if (rb) rai_tensor_release(bb2);
+  if (a1 || b1) {  // drop the promoted dims again
+    std::vector<int64_t> s = so;
+    if (b1) s.pop_back();
+    if (a1) s.erase(s.end() - (b1 ? 1 : 2));
+    rai_tensor *r = rai_reshape(t, s.data(), (int32_t)s.size());
+    rai_tensor_release(t);
+    t = r;
+  }
+  return done(t);
+}
+
+static rai_tensor *softmax_like(int op, rai_tensor *x, int32_t dim) {
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank) return err_node(x->dev, x->dtype, x->shape, {x}, "dim out of range");
+  rai_tensor *t = new_node(x->dev, x->dtype, x->shape, op, {x});
+  t->ip = {d};
+  return t;
+}
+rai_tensor *rai_softmax(rai_tensor *x, int32_t dim) { return softmax_like(RAI_OP_SOFTMAX, x, dim); }
+rai_tensor *rai_log_softmax(rai_tensor *x, int32_t dim) { return softmax_like(RAI_OP_LOG_SOFTMAX, x, dim); }
+
+rai_tensor *rai_reduce(int32_t op, rai_tensor *x, const int32_t *dims, int32_t ndims, int32_t keep_dim) {
+  // shape.rs:162-173 shape_reduce
+  const int rank = (int)x->shape.size();
+  std::vector<int64_t> nd;
+  for (int i = 0; i < ndims; ++i) {
+    const int d = norm_dim(dims[i], rank);
+    if (d < 0 || d >= rank) return err_node(x->dev, x->dtype, {}, {x}, "dim out of range");
+    nd.push_back(d);
+  }
+  std::vector<int64_t> shape;
+  for (int i = 0; i < rank; ++i) {
+    bool red = false;
+    for (int64_t d : nd) red |= d == i;
+    if (!red) shape.push_back(x->shape[i]);
+    else if (keep_dim) shape.push_back(1);
+  }
+  rai_tensor *t = new_node(x->dev, x->dtype, shape, RAI_OP_REDUCE, {x});
+  t->sub = op;
+  t->ip.push_back(keep_dim);
+  for (int64_t d : nd) t->ip.push_back(d);
+  return t;
+}
+
+static rai_tensor *arg_like(int op, rai_tensor *x, int32_t dim, int32_t keep_dim) {
+  // ops/argmax.rs:48-61: output dtype U32
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank) return err_node(x->dev, RAI_U32, {}, {x}, "dim out of range");
+  std::vector<int64_t> shape;
+  for (int i = 0; i < rank; ++i) {
+    if (i != d) shape.push_back(x->shape[i]);
+    else if (keep_dim) shape.push_back(1);
+  }
+  rai_tensor *t = new_node(x->dev, RAI_U32, shape, op, {x});
+  t->ip = {d, keep_dim};
+  return t;
+}
+rai_tensor *rai_argmax(rai_tensor *x, int32_t dim, int32_t keep_dim) { return arg_like(RAI_OP_ARGMAX, x, dim, keep_dim); }
+rai_tensor *rai_argmin(rai_tensor *x, int32_t dim, int32_t keep_dim) { return arg_like(RAI_OP_ARGMIN, x, dim, keep_dim); }
+
+rai_tensor *rai_index_select(rai_tensor *x, int32_t dim, rai_tensor *index) {
+  // ops/index_select.rs:52-61: the selected dim becomes index.elem_count()
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank) return err_node(x->dev, x->dtype, {}, {x, index}, "dim out of range");
+  std::vector<int64_t> shape = x->shape;
+  shape[d] = numel_of(index->shape);
+  rai_tensor *t = new_node(x->dev, x->dtype, shape, RAI_OP_INDEX_SELECT, {x, index});
+  t->ip = {d};
+  return t;
+}
+
+rai_tensor *rai_narrow(rai_tensor *x, int32_t dim, int64_t start, int64_t len) {
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank || start < 0 || len < 0 || start + len > x->shape[d])
+    return err_node(x->dev, x->dtype, x->shape, {x}, "narrow out of range");
+  std::vector<int64_t> shape = x->shape;
+  shape[d] = len;
+  rai_tensor *t = new_node(x->dev, x->dtype, shape, RAI_OP_NARROW, {x});
+  t->ip = {d, start, len};
+  return t;
+}
+
+rai_tensor *rai_concatenate(rai_tensor *const *xs, int32_t n, int32_t dim) {
+  // ops/concatenate.rs:54-67
+  rai_tensor *t1 = xs[0];
+  const int rank = (int)t1->shape.size();
+  const int d = norm_dim(dim, rank);
+  std::vector<rai_tensor *> ins(xs, xs + n);
+  if (d < 0 || d >= rank) return err_node(t1->dev, t1->dtype, t1->shape, ins, "dim out of range");
+  std::vector<int64_t> shape = t1->shape;
+  shape[d] = 0;
+  for (int i = 0; i < n; ++i) {
+    if ((int)xs[i]->shape.size() != rank || xs[i]->dtype != t1->dtype)
+      return err_node(t1->dev, t1->dtype, t1->shape, ins, incompatible(t1, xs[i]));
+    for (int k = 0; k < rank; ++k)
+      if (k != d && xs[i]->shape[k] != t1->shape[k]) return err_node(t1->dev, t1->dtype, t1->shape, ins, incompatible(t1, xs[i]));
+    shape[d] += xs[i]->shape[d];
+  }
+  rai_tensor *t = new_node(t1->dev, t1->dtype, shape, RAI_OP_CONCATENATE, ins);
+  t->ip = {d};
+  return t;
+}
+
+rai_tensor *rai_where(rai_tensor *cond, rai_tensor *on_true, rai_tensor *on_false) {
+  // ops/where.rs:37-45: shape of the condition, dtype of the branches, inputs [on_true, on_false, cond]
+  if (on_true->dtype != on_false->dtype || on_true->shape != cond->shape || on_false->shape != cond->shape)
+    return err_node(cond->dev, on_true->dtype, cond->shape, {on_true, on_false, cond}, incompatible(on_true, on_false));
+  return new_node(cond->dev, on_true->dtype, cond->shape, RAI_OP_WHERE, {on_true, on_false, cond});
+}
+
+rai_tensor *rai_transpose(rai_tensor *x, int32_t dim0, int32_t dim1) {
+  const int rank = (int)x->shape.size();
+  const int a = norm_dim(dim0, rank), b = norm_dim(dim1, rank);
+  if (a < 0 || a >= rank || b < 0 || b >= rank) return err_node(x->dev, x->dtype, x->shape, {x}, "dim out of range");
+  std::vector<int64_t> shape = x->shape;
+  std::swap(shape[a], shape[b]);
+  rai_tensor *t = new_node(x->dev, x->dtype, shape, RAI_OP_TRANSPOSE, {x});
+  t->ip = {a, b};
+  return t;
+}
+
+rai_tensor *rai_reshape(rai_tensor *x, const int64_t *shape, int32_t rank) {
+  // ops/reshape.rs:50-78: an equal shape returns the tensor itself; a different element count is an Err node
+  std::vector<int64_t> s(shape, shape + rank);
+  if (s == x->shape) {
+    ++x->refs;
+    return x;
+  }
+  if (numel_of(s) != numel_of(x->shape)) {
+    rai_tensor *e = err_node(x->dev, x->dtype, s, {x},
+                             "IncompatibleShape { lhs: " + shape_str(x->shape) + ", rhs: " + shape_str(s) + " }");
+    return e;
+  }
+  rai_tensor *t = new_node(x->dev, x->dtype, s, RAI_OP_RESHAPE, {x});
+  t->ip = s;
+  return t;
+}
+
+rai_tensor *rai_permute(rai_tensor *x, const int32_t *dims, int32_t rank) {
+  if (rank != (int32_t)x->shape.size()) return err_node(x->dev, x->dtype, x->shape, {x}, "permute rank mismatch");
+  std::vector<int64_t> shape(rank), ip(rank);
+  std::vector<bool> seen(rank, false);
+  for (int i = 0; i < rank; ++i) {
+    const int d = norm_dim(dims[i], rank);
+    if (d < 0 || d >= rank || seen[d]) return err_node(x->dev, x->dtype, x->shape, {x}, "permute dims are not a permutation");
+    seen[d] = true;
+    shape[i] = x->shape[d];
+    ip[i] = d;
+  }
+  rai_tensor *t = new_node(x->dev, x->dtype, shape, RAI_OP_PERMUTE, {x});
+  t->ip = ip;
+  return t;
+}
+
+rai_tensor *rai_broadcast_to(rai_tensor *x, const int64_t *shape, int32_t rank) {
+  std::vector<int64_t> s(shape, shape + rank), out;
+  bool lb, rb;
+  if (!broadcast_shapes(x->shape, s, &out, &lb, &rb) || out != s)
+    return err_node(x->dev, x->dtype, s, {x},
+                    "IncompatibleShape { lhs: " + shape_str(x->shape) + ", rhs: " + shape_str(s) + " }");
+  return new_node(x->dev, x->dtype, s, RAI_OP_BROADCAST, {x});
+}
+
+rai_tensor *rai_to_contiguous(rai_tensor *x) { return new_node(x->dev, x->dtype, x->shape, RAI_OP_TO_CONTIGUOUS, {x}); }
+
+// ------------------------------------------------------------------ handles and metadata
+void rai_tensor_retain(rai_tensor *t) {
+  if (t) ++t->refs;
+}
+
+void rai_tensor_release(rai_tensor *t) {
+  // iterative: a long chain of nodes must not recurse once per node
+  std::vector<rai_tensor *> work;
+  if (t) work.push_back(t);
+  while (!work.empty()) {
+    rai_tensor *n = work.back();
+    work.pop_back();
+    if (--n->refs > 0) continue;
+    for (rai_tensor *i : n->inputs) work.push_back(i);
+    if (n->buf) (void)rai_hip_release(n->buf);
+    delete n;
+  }
+}
+
+int32_t rai_tensor_rank(const rai_tensor *t) { return (int32_t)t->shape.size(); }
+int32_t rai_tensor_dtype(const rai_tensor *t) { return t->dtype; }
+int32_t rai_tensor_device(const rai_tensor *t) { return t->dev; }
+int32_t rai_tensor_op(const rai_tensor *t) { return t->op; }
+int32_t rai_tensor_shape(const rai_tensor *t, int64_t *shape_out) {
+  for (size_t i = 0; i < t->shape.size(); ++i) shape_out[i] = t->shape[i];
+  return (int32_t)t->shape.size();
+}
+int32_t rai_tensor_is_evaluated(const rai_tensor *t) { return t->evaluated ? 1 : 0; }
+int32_t rai_tensor_num_inputs(const rai_tensor *t) { return (int32_t)t->inputs.size(); }
+uint64_t rai_tensor_id(const rai_tensor *t) { return t->id; }
+const char *rai_tensor_error(const rai_tensor *t) { return t->op == RAI_OP_ERR ? t->err.c_str() : nullptr; }
+
+int rai_tensor_storage(const rai_tensor *t, rai_hip_tensor *out) {
+  RAI_REQUIRE(t && out, RAI_ERR_BAD_ARG, "null argument");
+  RAI_REQUIRE(t->evaluated, RAI_ERR_BAD_ARG, "tensor %llu is not evaluated", (unsigned long long)t->id);
+  *out = t->view;
+  return RAI_OK;
+}
+
+// ------------------------------------------------------------------ evaluation
+int rai_graph_eval_order(rai_tensor *const *outputs, int32_t n, uint64_t *ids, int32_t capacity, int32_t *count) {
+  RAI_REQUIRE(outputs && count && n >= 0, RAI_ERR_BAD_ARG, "null argument");
+  std::vector<rai_tensor *> tape;
+  RAI_TRY(topo_sort(outputs, n, &tape));
+  *count = (int32_t)tape.size();
+  for (int i = 0; i < *count && i < capacity; ++i) ids[i] = tape[i]->id;
+  return RAI_OK;
+}
+
+int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
+  RAI_REQUIRE(outputs && n >= 0, RAI_ERR_BAD_ARG, "null argument");
+  init_rules();
+  std::vector<rai_tensor *> tape;
+  RAI_TRY(topo_sort(outputs, n, &tape));
+  FusionPlan plan;
+  if (g_fusion) plan_fusion(tape, outputs, n, &plan);
+  for (rai_tensor *t : tape) {
+    if (t->evaluated || plan.inlined.count(t->id)) continue;
+    rule_fn rule = g_rules[t->op];
+    RAI_REQUIRE(rule, RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op));
+    int st = RAI_ERR_UNSUPPORTED;
+    if (elementwise(t) && has_inlined_input(t, plan)) {
+      // the rules of the inlined members must exist too: fusion never hides a missing rule
+      st = eval_region(t, plan);
+      if (st == RAI_ERR_UNSUPPORTED) {  // region too large for one program: evaluate its members one by one
+        drop_storage(t);
+        st = eval_inputs_plain(t, plan);
+        if (st == RAI_OK) st = rule(t);
+      }
+    } else {
+      st = rule(t);
+    }
+    if (st != RAI_OK) {
+      drop_storage(t);
+      return st;
+    }
+    t->evaluated = true;
+    ++g_stats.nodes_evaluated;
+  }
+  if (!retain_graph)
+    for (rai_tensor *t : tape)
+      if (t->evaluated) detach(t);
+  return RAI_OK;
+}
+
+int rai_tensor_to_host(rai_tensor *t, void *dst, size_t bytes) {
+  RAI_REQUIRE(t && dst, RAI_ERR_BAD_ARG, "null argument");
+  if (!t->evaluated) {
+    rai_tensor *outs[1] = {t};
+    RAI_TRY(rai_eval(outs, 1, 0));
+  }
+  const size_t want = (size_t)numel_of(t->shape) * dtype_size(t->dtype);
+  RAI_REQUIRE(bytes == want, RAI_ERR_BAD_SHAPE, "to_host: tensor holds %zu bytes, buffer has %zu", want, bytes);
+  if (want == 0) return RAI_OK;
+  if (is_contiguous(&t->view)) return rai_hip_d2h(t->dev, dst, base_ptr(&t->view), want);
+  // Tensor::as_vec of a strided view: contiguous copy first
+  void *tmp = nullptr;
+  RAI_TRY(rai_hip_alloc(t->dev, want, &tmp));
+  rai_hip_tensor c;
+  memset(&c, 0, sizeof(c));
+  c.data = tmp;
+  c.dtype = t->dtype;
+  c.rank = t->view.rank;
+  int64_t st = 1;
+  for (int i = c.rank - 1; i >= 0; --i) {
+    c.shape[i] = t->view.shape[i];
+    c.stride[i] = st;
+    st *= c.shape[i];
+  }
+  int rc = rai_hip_copy(t->dev, &t->view, &c);
+  if (rc == RAI_OK) rc = rai_hip_d2h(t->dev, dst, tmp, want);
+  (void)rai_hip_release(tmp);
+  return rc;
+}
+
+// ------------------------------------------------------------------ dispatcher
+int rai_dispatch_unregister(int32_t op_kind) {
+  RAI_REQUIRE(op_kind >= 0 && op_kind < RAI_OP_COUNT_, RAI_ERR_BAD_ARG, "op kind %d", op_kind);
+  init_rules();
+  g_rules[op_kind] = nullptr;
+  return RAI_OK;
+}
+int rai_dispatch_register_builtin(int32_t op_kind) {
+  RAI_REQUIRE(op_kind >= 0 && op_kind < RAI_OP_COUNT_, RAI_ERR_BAD_ARG, "op kind %d", op_kind);
+  init_rules();
+  g_rules[op_kind] = kBuiltin[op_kind];
+  return RAI_OK;
+}
+int32_t rai_dispatch_has_rule(int32_t op_kind) {
+  init_rules();
+  return op_kind >= 0 && op_kind < RAI_OP_COUNT_ && g_rules[op_kind] != nullptr;
+}
+
+// ------------------------------------------------------------------ fusion control and counters
+int rai_graph_set_fusion(int32_t enabled) {
+  g_fusion = enabled != 0;
+  return RAI_OK;
+}
+int rai_graph_get_stats(rai_graph_stats *out, int32_t reset) {
+  if (out) *out = g_stats;
+  if (reset) g_stats = rai_graph_stats{0, 0, 0, 0};
+  return RAI_OK;
+}
+
+}  // extern "C"

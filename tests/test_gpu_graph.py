@@ -1,0 +1,181 @@
+"""The lazy-graph evaluator on the device against the CPU oracle: rai's own
+decompositions (LayerNorm, RMSNorm, new_gelu / gelu / silu, Linear, Embedding, a
+softmax attention block) built node by node and evaluated through the dispatcher;
+the elementwise-fusion pass must give bit-identical results with fewer launches."""
+import numpy as np
+import pytest
+
+from oracle import nn as onn, ops as oo
+from oracle.dtypes import from_storage, rnd, to_storage
+from rai_amd import graph as g
+from rai_amd.graph import Tensor
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(arr, dt):
+    return Tensor.from_array(to_storage(arr, dt), dt)
+
+
+def rand(rng, shape, dt, scale=1.0):
+    return rnd(rng.standard_normal(shape).astype(np.float32) * scale, dt)
+
+
+def run(build, fusion):
+    g.set_fusion(fusion)
+    g.stats(reset=True)
+    out = build()
+    storage = out.as_storage()
+    st = g.stats()
+    g.set_fusion(True)
+    return storage, st, out
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_layer_norm_chain_matches_oracle_and_fuses(hip, dt):
+    rng = np.random.default_rng(0)
+    x, w, b = rand(rng, (6, 37, 96), dt), rand(rng, (96,), dt), rand(rng, (96,), dt)
+    build = lambda: g.layer_norm(dev(x, dt), dev(w, dt), dev(b, dt), 1e-5)
+    fused, st_f, _ = run(build, True)
+    plain, st_p, _ = run(build, False)
+    assert np.array_equal(fused, plain), "fusion changed the result"
+    assert st_f["fused_regions"] >= 2 and st_f["kernel_launches"] < st_p["kernel_launches"]
+    assert st_p["fused_regions"] == 0
+    want = onn.layer_norm(x, w, b, 1e-5, dt)
+    assert_close(from_storage(fused, dt), want, dt, "layer_norm")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("act", ["new_gelu", "gelu", "silu", "relu"])
+def test_activations_fuse_into_one_launch(hip, dt, act):
+    rng = np.random.default_rng(1)
+    x = rand(rng, (5, 1000), dt, 2.0)
+    build = lambda: getattr(dev(x, dt), act)()
+    fused, st_f, _ = run(build, True)
+    plain, st_p, _ = run(build, False)
+    assert np.array_equal(fused, plain), "fusion changed the result"
+    assert st_f["kernel_launches"] == 1 and st_f["fused_regions"] == 1     # the whole chain is one region
+    assert st_p["kernel_launches"] >= (5 if act != "relu" else 2)
+    want = getattr(onn, act)(x, dt)
+    assert_close(from_storage(fused, dt), want, dt, act)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_rms_norm_linear_embedding(hip, dt):
+    rng = np.random.default_rng(2)
+    table = rand(rng, (50, 64), dt)
+    ids = rng.integers(0, 50, (2, 7)).astype(np.uint32)
+    w, wl, bl = rand(rng, (64,), dt), rand(rng, (48, 64), dt, 0.2), rand(rng, (48,), dt)
+
+    def build():
+        h = g.embedding(Tensor.from_array(ids, "u32"), dev(table, dt))
+        h = g.rms_norm(h, dev(w, dt), 1e-6)
+        return g.linear(h, dev(wl, dt), dev(bl, dt))
+
+    fused, st_f, out = run(build, True)
+    plain, _, _ = run(build, False)
+    assert out.shape == (2, 7, 48)
+    assert np.array_equal(fused, plain)
+    h = onn.embedding(ids, table)
+    h = onn.rms_norm(h, w, 1e-6, dt)
+    want = onn.linear(h, wl, bl, dt)
+    assert_close(from_storage(fused, dt), want, dt, "embedding -> rms_norm -> linear")
+
+
+def test_attention_block_through_the_graph(hip):
+    # q k^T * scale, causal mask by where, softmax, p v: the node sequence of phi2.rs:244-262 (f32)
+    rng = np.random.default_rng(3)
+    B, H, S, D = 2, 3, 9, 16
+    q, k, v = (rand(rng, (B, H, S, D), "f32") for _ in range(3))
+    mask = np.triu(np.ones((S, S), np.uint8), 1)
+
+    def build():
+        scores = dev(q, "f32").matmul(dev(k, "f32").transpose(-2, -1) * (1.0 / np.sqrt(D)))
+        m = Tensor.from_array(mask, "u8").broadcast_to((B, H, S, S))
+        scores = m.where_cond(scores.full_like(float("-inf")), scores)
+        return scores.softmax(-1).matmul(dev(v, "f32")).transpose(1, 2).reshape((B, S, H * D))
+
+    got, _, _ = run(build, True)
+    s = np.einsum("bhsd,bhtd->bhst", q, k * np.float32(1.0 / np.sqrt(D)))
+    s = np.where(mask.astype(bool), -np.inf, s)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    want = np.einsum("bhst,bhtd->bhsd", p, v).transpose(0, 2, 1, 3).reshape(B, S, H * D)
+    assert_close(got, want, "f32", "attention through the graph")
+
+
+def test_views_share_storage_and_detach_drops_inputs(hip):
+    x = dev(np.arange(24, dtype=np.float32).reshape(2, 3, 4), "f32")
+    y = x.transpose(0, 2).narrow(1, 1, 2)          # views only
+    g.stats(reset=True)
+    y.eval(retain_graph=True)
+    assert g.stats()["kernel_launches"] == 0 and y.num_inputs() == 1     # retain_graph keeps the inputs
+    assert x.is_evaluated() and y.storage().data == x.storage().data      # zero-copy views
+    np.testing.assert_array_equal(y.as_storage(), np.arange(24, dtype=np.float32).reshape(2, 3, 4).transpose(2, 1, 0)[:, 1:3])
+    z = (y + 1.0).sum(0)
+    z.eval()
+    assert z.num_inputs() == 0                      # eval.rs:47-49 detach
+    np.testing.assert_array_equal(z.as_storage(), (np.arange(24, dtype=np.float32).reshape(2, 3, 4).transpose(2, 1, 0)[:, 1:3] + 1).sum(0))
+
+
+def test_shared_intermediates_are_materialised_not_inlined(hip):
+    rng = np.random.default_rng(4)
+    x = rand(rng, (64, 33), "f32")
+
+    def build():
+        y = dev(x, "f32").exp()                      # three consumers: must receive data
+        return (y + y.tanh()) * y
+
+    fused, st, _ = run(build, True)
+    plain, _, _ = run(build, False)
+    assert np.array_equal(fused, plain)
+    y = np.exp(x)
+    assert_close(fused, (y + np.tanh(y)) * y, "f32", "shared intermediate")
+
+
+def test_held_intermediate_is_not_folded_away(hip):
+    x = dev(np.linspace(-2, 2, 40, dtype=np.float32), "f32")
+    mid = x.tanh()                                   # a handle stays alive: it must be evaluated
+    out = (mid * 2.0).exp()
+    out.eval(retain_graph=True)
+    assert mid.is_evaluated()
+    np.testing.assert_allclose(mid.as_storage(), np.tanh(np.linspace(-2, 2, 40, dtype=np.float32)), rtol=1e-6)
+
+
+def test_unimplemented_rule_and_err_node_fail_eval(hip):
+    x = dev(np.ones((3, 5), np.float32), "f32")
+    g.dispatch_unregister("Softmax")
+    try:
+        with pytest.raises(g.RaiHipError) as e:
+            x.softmax(-1).eval()
+        assert e.value.status == -7 and "Unimplemented" in str(e.value) and "Softmax" in str(e.value)
+        # fusion never hides a missing rule of a node it would fold
+        g.dispatch_unregister("Unary")
+        with pytest.raises(g.RaiHipError):
+            ((x.tanh() + 1.0) * 2.0).eval()
+    finally:
+        g.dispatch_register_builtin("Softmax")
+        g.dispatch_register_builtin("Unary")
+    np.testing.assert_allclose(x.softmax(-1).as_storage(), np.full((3, 5), 0.2, np.float32), rtol=1e-6)
+    with pytest.raises(g.RaiHipError) as e:
+        (x.matmul(x) + 1.0).eval()
+    assert e.value.status == -2
+
+
+def test_large_region_falls_back_to_node_by_node(hip):
+    x0 = np.linspace(0.1, 1.0, 128, dtype=np.float32)
+
+    def build():
+        t = dev(x0, "f32")
+        for _ in range(40):                          # longer than one fused program
+            t = (t * 1.01).tanh()
+        return t
+
+    fused, _, _ = run(build, True)
+    plain, _, _ = run(build, False)
+    assert np.array_equal(fused, plain)
+    want = x0.astype(np.float64)
+    for _ in range(40):
+        want = np.tanh(want * np.float64(np.float32(1.01)))
+    assert_close(fused, want, "f32", "long chain")
