@@ -179,3 +179,29 @@ def test_large_region_falls_back_to_node_by_node(hip):
     for _ in range(40):
         want = np.tanh(want * np.float64(np.float32(1.01)))
     assert_close(fused, want, "f32", "long chain")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_phi2_through_the_graph_matches_oracle(hip, dt):
+    # the model code of phi2.rs recorded as a lazy graph and evaluated node by node on the
+    # device (the reference's own execution scheme), prefill then two cached decode steps
+    from oracle import phi2
+    from rai_amd.graph_models import Phi2Graph
+    cfg = phi2.Config(vocab_size=300, hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                      num_attention_heads=4, max_position_embeddings=64)
+    params = phi2.random_params(cfg, dt, seed=0)
+    ref = phi2.Model(cfg, params, dt)
+    model = Phi2Graph(cfg, {k: dev(v, dt) for k, v in params.items()}, dt)
+    ids = np.random.Generator(np.random.PCG64(1)).integers(0, cfg.vocab_size, (2, 10)).astype(np.uint32)
+    for step in range(3):
+        g.stats(reset=True)
+        logits = model.fwd(Tensor.from_array(ids, "u32"))
+        got = from_storage(logits.as_storage(), dt)[:, 0, :]
+        want = ref.fwd(ids)
+        assert_close(got, want, dt, f"graph phi2 step {step}")
+        st = g.stats()
+        assert st["fused_regions"] > 0 and st["kernel_launches"] < st["nodes_evaluated"]
+        ids = np.argmax(want, -1).astype(np.uint32).reshape(2, 1)
+    # greedy ids through the graph: argmax node, u32, bit-exact against the oracle on the same logits
+    tok = logits.argmax(-1).as_storage()[:, 0]
+    assert tok.dtype == np.uint32 and np.array_equal(tok, np.argmax(got, -1))
