@@ -29,6 +29,10 @@ PHI2 = dict(vocab_size=51200, hidden_size=2560, intermediate_size=10240, num_hid
             num_attention_heads=32, rotary_dim=32, max_position_embeddings=2048, hidden_act="gelu_new",
             rope_theta=10000.0, norm_eps=1e-5)
 PROMPT, NEW = 512, 128
+# HBM traffic of the dominant kernel relative to its algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs), each scaled by what the same counter reads for a plain 256 MiB copy kernel
+# (profiles/phi2_decode_step_hbm_traffic_pmc.md): 5.247 GB fetched + 2.8 MB written against 5.224 GB.
+TRAFFIC_OVER_ALGORITHMIC = 1.0049
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
@@ -112,6 +116,9 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="also run a plain device copy of 256 MiB three times (k_copy): the known-size reference "
+                         "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     ap.add_argument("--layers", type=int, default=PHI2["num_hidden_layers"],
                     help="debug only: fewer layers (the JSON line then says so and is not the headline workload)")
     args = ap.parse_args()
@@ -147,9 +154,12 @@ def main():
     decode_tok_s = (NEW - 1) / (dcd / 1e3)     # the prefill produces token 0; NEW-1 single-token steps follow
     prefill_tok_s = PROMPT / (pre / 1e3)
 
-    # dominant kernel: the M=1 weight-streaming kernel, timed live with hipEvents on the library's stream
-    us, bytes_per_launch = dec.time_decode_linear(sweeps=20)
+    # dominant kernel: the persistent per-token kernel that runs all layers of a decode step (weights, biases,
+    # norm parameters and the KV cache of the current context once per launch), timed live with one hipEvent
+    # pair per launch on the library's stream, at the context length the generate call ended with
+    us, bytes_per_launch = dec.time_decode_step(sweeps=20)
     achieved = bytes_per_launch / (us * 1e-6) / 1e9
+    gemv_us, gemv_bytes = dec.time_decode_linear(sweeps=10)   # the launch-per-primitive path's streaming kernels
     mean_ctx = PROMPT + (NEW - 1) / 2.0 + 1
     step_bytes = decode_bytes_per_token(cfg, mean_ctx)
     out = {
@@ -176,18 +186,31 @@ def main():
         "weights_load_s": round(load_s, 1),
         "first_tokens": [int(t) for t in toks[0, :8]],
         "roofline": {
-            "kernel": "k_linear_bf16_skinny<1,4> (decode: fused LayerNorm + q|k|v|fc1 GEMV, dense|fc2 GEMV)",
+            "kernel": "k_phi2_decode_step (persistent kernel: all 32 layers of one decode step, grid barriers, "
+                      "weight ring prefetched across phases)",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": int(bytes_per_launch * TRAFFIC_OVER_ALGORITHMIC),
             "us_per_launch": round(us, 3),
             "bytes_per_launch": int(bytes_per_launch),
         },
+        "decode_gemv_kernels": {"us_per_launch": round(gemv_us, 3), "bytes_per_launch": int(gemv_bytes),
+                                "GB_per_s": round(gemv_bytes / (gemv_us * 1e-6) / 1e9, 1)},
     }
     dec.close()
+    if args.pmc_calibrate:
+        import ctypes as C
+
+        from rai_amd import _lib, ops
+        from rai_amd.hip import HipTensor
+        src = ops.full(1.0, (64 * 1024 * 1024,), "f32")
+        dst = HipTensor.empty((64 * 1024 * 1024,), "f32")
+        for _ in range(3):
+            _lib.call("rai_hip_copy", 0, C.byref(src.desc()), C.byref(dst.desc()))
+        sync()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)

@@ -328,6 +328,14 @@ int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *dec);
 /* Current cached context length. */
 int rai_hip_decoder_context_len(rai_hip_decoder *dec, int32_t *len);
 
+/* Measurement aid: mean duration (hipEvents on the library's stream, one pair per launch) of the
+ * persistent per-token kernel that runs all layers of a single-token step (Phi-2 architecture, bf16,
+ * batch 1), launched `sweeps` times at the current context length, and the algorithmic bytes one launch
+ * moves (weights, biases, norm parameters, cached K/V).  The residual stream and the cache row at the
+ * current position are overwritten: clear the KV cache before the decoder is used again.
+ * No counterpart in the reference (it has no kernels of its own). */
+int rai_hip_decoder_time_decode_step(rai_hip_decoder *dec, int32_t sweeps, float *us_per_launch,
+                                     double *bytes_per_launch);
 /* Measurement only (no counterpart in the reference): launches the decode-step
  * weight-streaming kernel back to back over every layer's two packed matrices
  * (q|k|v|fc1 with the fused LayerNorm, then dense|fc2 with the residual; 2*L

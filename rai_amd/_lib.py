@@ -119,6 +119,7 @@ PROTOTYPES = {
     "rai_hip_decoder_generate": [_vp, C.POINTER(C.c_uint32), _i32, _i32, _i32, C.POINTER(C.c_uint32),
                                  C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "rai_hip_decoder_time_decode_linear": [_vp, _i32, C.POINTER(C.c_float), C.POINTER(C.c_double)],
+    "rai_hip_decoder_time_decode_step": [_vp, _i32, C.POINTER(C.c_float), C.POINTER(C.c_double)],
     "rai_hip_decoder_clear_kv_cache": [_vp],
     "rai_hip_decoder_context_len": [_vp, C.POINTER(_i32)],
 }

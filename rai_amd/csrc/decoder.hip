@@ -1075,6 +1075,45 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   return rc;
 }
 
+int rai_hip_decoder_time_decode_step(rai_hip_decoder *d, int32_t sweeps, float *us_per_launch,
+                                     double *bytes_per_launch) {
+  RAI_REQUIRE(d && us_per_launch && bytes_per_launch && sweeps > 0, RAI_ERR_BAD_ARG, "bad argument");
+  RAI_REQUIRE(d->mega_ok, RAI_ERR_UNSUPPORTED, "time_decode_step: the persistent decode kernel does not serve this model");
+  RAI_REQUIRE(d->ctx_len >= 1 && d->ctx_len < d->cfg.max_context, RAI_ERR_BAD_SHAPE,
+              "time_decode_step: needs a context of 1..%d tokens", d->cfg.max_context - 1);
+  hipStream_t st = stream_of(d->dev);
+  hipEvent_t e0, e1;
+  RAI_HIP_TRY(hipEventCreate(&e0));
+  RAI_HIP_TRY(hipEventCreate(&e1));
+  const MegaArgs m = mega_args(d);
+  const size_t flag_bytes = sizeof(unsigned) * (size_t)(d->num_cu < kMegaFlagWords ? d->num_cu : kMegaFlagWords);
+  double total_ms = 0.0;
+  int rc = RAI_OK;
+  for (int s = 0; s < sweeps + 2 && rc == RAI_OK; ++s) {  // two warm-up launches
+    if (hipEventRecord(e0, st) != hipSuccess) { rc = fail(RAI_ERR_HIP, "event record"); break; }
+    rc = launch_phi2_decode_step(st, m, d->D, d->num_cu);
+    if (rc != RAI_OK) break;
+    if (hipEventRecord(e1, st) != hipSuccess || hipMemsetAsync(d->mega_barrier, 0, flag_bytes, st) != hipSuccess ||
+        hipEventSynchronize(e1) != hipSuccess) { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    if (s >= 2) total_ms += ms;
+  }
+  (void)hipStreamSynchronize(st);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  RAI_TRY(rc);
+  RAI_TRY(check_fault(d));
+  *us_per_launch = (float)(total_ms * 1000.0 / sweeps);
+  // algorithmic bytes of one launch: every layer's weights, biases and LayerNorm parameters once, plus the
+  // cached keys and values of the current context
+  const double es = (double)d->es;
+  const double per_layer = (double)d->NA * d->H + d->NA + (double)d->H * d->KB + 2.0 * d->H + 2.0 * d->H;
+  const double kv = 2.0 * d->Hkv * d->D * (double)d->ctx_len;
+  *bytes_per_launch = es * d->L * (per_layer + kv);
+  return RAI_OK;
+}
+
 int rai_hip_decoder_time_decode_linear(rai_hip_decoder *d, int32_t sweeps, float *us_per_launch,
                                        double *bytes_per_launch) {
   RAI_REQUIRE(d && us_per_launch && bytes_per_launch && sweeps > 0, RAI_ERR_BAD_ARG, "bad argument");

@@ -102,6 +102,12 @@ class Decoder:
         call("rai_hip_decoder_context_len", self._h, C.byref(n))
         return n.value
 
+    def time_decode_step(self, sweeps=20):
+        """Mean launch time (us) and algorithmic bytes of the persistent per-token decode kernel."""
+        us, by = C.c_float(0), C.c_double(0)
+        call("rai_hip_decoder_time_decode_step", self._h, int(sweeps), C.byref(us), C.byref(by))
+        return us.value, by.value
+
     def time_decode_linear(self, sweeps=20):
         """Mean launch time (us) and algorithmic bytes of the decode weight-streaming kernel."""
         us, by = C.c_float(0), C.c_double(0)
