@@ -110,6 +110,183 @@ def cpu_baseline(steps_decode=2, layers=2):
     }
 
 
+# ------------------------------------------------------------------------------------------------
+# Secondary workloads (not the headline line): the other configurations of the same hot path.
+QWEN2_15B = dict(vocab_size=151936, hidden_size=1536, intermediate_size=8960, num_hidden_layers=28,
+                 num_attention_heads=12, num_key_value_heads=2, head_dim=128, rotary_dim=128,
+                 max_position_embeddings=2048, hidden_act="silu", rope_theta=1e6, norm_eps=1e-6)
+GEMMA_2B = dict(vocab_size=256000, hidden_size=2048, intermediate_size=16384, num_hidden_layers=18,
+                num_attention_heads=8, num_key_value_heads=1, head_dim=256, rotary_dim=256,
+                max_position_embeddings=4096, hidden_act="gelu", rope_theta=10000.0, norm_eps=1e-6,
+                tie_word_embeddings=True)
+
+
+def _line(metric, value, unit, steps, warmup, ms_per_step, workload, extra):
+    out = {"metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+           "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16", "data": "synthetic", "config": {"workload": workload}}
+    out.update(extra)
+    print(json.dumps(out), flush=True)
+
+
+def run_qwen2_prefill(args):
+    """Qwen2-1.5B architecture, bf16, batched prefill 16 x 1024 with causal mask."""
+    from rai_amd import synthetic
+    from rai_amd.hip import sync
+    from rai_amd.models import Decoder
+    B, S = 16, 1024
+    cfg = QWEN2_15B
+    dec = Decoder("qwen2", "bf16", max_batch=B, max_context=S, **cfg)
+    synthetic.load_random_params(dec, seed=0)
+    ids = synthetic.prompt(cfg["vocab_size"], B, S, seed=1)
+    times = []
+    for it in range(args.warmup + args.steps):
+        dec.clear_kv_cache()
+        sync()
+        t0 = time.perf_counter()
+        _, tok = dec.forward(ids, want_logits=False)   # returns after the tokens are on the host
+        dt = time.perf_counter() - t0
+        if it >= args.warmup:
+            times.append(dt)
+    t = float(np.mean(times))
+    h, i, v, l = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    qd, kd = cfg["num_attention_heads"] * cfg["head_dim"], cfg["num_key_value_heads"] * cfg["head_dim"]
+    lin = 2.0 * (h * (qd + 2 * kd) + qd * h + 3 * h * i) * l * B * S
+    attn = l * 4.0 * cfg["num_attention_heads"] * B * S * S * cfg["head_dim"]
+    flops = lin + attn + 2.0 * B * v * h
+    _line("Qwen2-1.5B bf16 batched prefill tok/s on 1 MI355X", B * S / t, "tokens/s", args.steps, args.warmup, t * 1e3,
+          "Qwen2-1.5B architecture 28L bf16, prefill batch 16 x 1024 tokens, causal, GQA 12/2 (random-init N(0,0.02))",
+          {"prefill_ms": round(t * 1e3, 3), "prefill_tflops": round(flops / t / 1e12, 1),
+           "prefill_frac_of_bf16_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+           "first_tokens": [int(x) for x in tok[:8]]})
+    dec.close()
+
+
+def run_gemma_decode(args):
+    """Gemma-2B architecture, bf16, greedy decode at batch 32 on a 2048-token context per sequence, 64 steps."""
+    from rai_amd import synthetic
+    from rai_amd.models import Decoder
+    B, CTX, NEWT = 32, 2048, 64
+    cfg = GEMMA_2B
+    dec = Decoder("gemma", "bf16", max_batch=B, max_context=CTX + NEWT, **cfg)
+    synthetic.load_random_params(dec, seed=0)
+    prompt = synthetic.prompt(cfg["vocab_size"], B, CTX, seed=1)
+    pre, dcd = [], []
+    wall0 = time.perf_counter()
+    for it in range(args.warmup + args.steps):
+        if it == args.warmup:
+            wall0 = time.perf_counter()
+        toks, p, d = dec.generate(prompt, NEWT)
+        if it >= args.warmup:
+            pre.append(p)
+            dcd.append(d)
+    wall = time.perf_counter() - wall0
+    d_ms = float(np.mean(dcd)) / (NEWT - 1)
+    h, i, v, l = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    qd, kd = cfg["num_attention_heads"] * cfg["head_dim"], cfg["num_key_value_heads"] * cfg["head_dim"]
+    weights = 2.0 * (l * (h * (qd + 2 * kd) + qd * h + 3 * h * i + 2 * h) + v * h + h)
+    kv = 2.0 * l * B * 2 * kd * (CTX + NEWT / 2.0)
+    step_bytes = weights + kv
+    _line("Gemma-2B bf16 batch-32 decode tok/s on 1 MI355X", B / (d_ms / 1e3), "tokens/s", args.steps, args.warmup,
+          wall * 1e3 / max(args.steps, 1),
+          "Gemma-2B architecture 18L bf16, greedy decode batch 32, 2048-token context per sequence, 64 steps, "
+          "MQA 8/1 x 256, tied 256000-way head (random-init N(0,0.02))",
+          {"decode_ms_per_step": round(d_ms, 4), "decode_step_bytes": int(step_bytes),
+           "decode_frac_of_hbm_roofline": round(step_bytes / (d_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4),
+           "prefill_tokens_per_s": round(B * CTX / (float(np.mean(pre)) / 1e3), 1),
+           "first_tokens": [int(x) for x in toks[0, :8]]})
+    dec.close()
+
+
+def run_ops(args):
+    """Primitive sweep, bf16 and f32: each op timed over a batched loop (hipEvents) and as a single launch."""
+    import ctypes as C
+
+    from rai_amd import _lib, ops
+    from rai_amd.hip import HipTensor, sync
+    _lib.call("rai_hip_init", 0)
+    rng = np.random.default_rng(0)
+
+    def rnd(shape, dt, scale=1.0):
+        a = rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)
+        if dt == "bf16":
+            return HipTensor.from_storage((a.view(np.uint32) >> 16).astype(np.uint16), "bf16")
+        return HipTensor.from_storage(a, "f32")
+
+    def timed(fn, iters):
+        t = C.c_void_p()
+        _lib.call("rai_hip_timer_create", 0, C.byref(t))
+        for _ in range(3):
+            fn()
+        _lib.call("rai_hip_timer_start", t)
+        for _ in range(iters):
+            fn()
+        _lib.call("rai_hip_timer_stop", t)
+        ms = C.c_float()
+        _lib.call("rai_hip_timer_elapsed_ms", t, C.byref(ms))
+        loop_us = ms.value * 1e3 / iters
+        _lib.call("rai_hip_timer_start", t)
+        fn()
+        _lib.call("rai_hip_timer_stop", t)
+        _lib.call("rai_hip_timer_elapsed_ms", t, C.byref(ms))
+        _lib.call("rai_hip_timer_destroy", t)
+        return loop_us, ms.value * 1e3
+
+    rows = []
+    for dt, es in (("bf16", 2), ("f32", 4)):
+        a, b = rnd((4096, 2560), dt), rnd((2560, 10240), dt)
+        lu, su = timed(lambda: ops.matmul(a, b), 10)
+        fl = 2.0 * 4096 * 2560 * 10240
+        peak = MFMA_BF16_PEAK_TFLOPS if dt == "bf16" else 157.3
+        rows.append(dict(op="matmul [4096,2560]x[2560,10240]", dtype=dt, loop_us=lu, single_us=su, bound="mfma",
+                         achieved=fl / lu / 1e6, unit="TFLOP/s", frac=fl / lu / 1e6 / peak))
+        w = rnd((10240, 2560), dt)
+        lu, su = timed(lambda: ops.linear(a, w), 10)
+        rows.append(dict(op="linear x[4096,2560] . W[10240,2560]^T", dtype=dt, loop_us=lu, single_us=su, bound="mfma",
+                         achieved=fl / lu / 1e6, unit="TFLOP/s", frac=fl / lu / 1e6 / peak))
+        del a, b, w
+        x = rnd((32, 128, 2048), dt, 3.0)
+        lu, su = timed(lambda: ops.softmax(x, -1), 50)
+        by = 2.0 * x.numel() * es
+        rows.append(dict(op="softmax [32,128,2048]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
+                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        x = rnd((4096, 2560), dt)
+        w1, b1 = rnd((2560,), dt), rnd((2560,), dt)
+        by = 2.0 * x.numel() * es
+        lu, su = timed(lambda: ops.layer_norm(x, w1, b1, 1e-5), 50)
+        rows.append(dict(op="layer_norm [4096,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
+                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        lu, su = timed(lambda: ops.rms_norm(x, w1, 1e-6), 50)
+        rows.append(dict(op="rms_norm [4096,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
+                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        x = rnd((1, 32, 2048, 80), dt)
+        cos, sin = ops.rope_tables(2048, 32, 10000.0, dt)
+        by = 2.0 * x.numel() * es
+        lu, su = timed(lambda: ops.rope(x, cos, sin, 32, 0), 50)
+        rows.append(dict(op="rope [1,32,2048,80] rot 32", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
+                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        table = rnd((51200, 2560), dt)
+        ids = HipTensor.from_storage(rng.integers(0, 51200, 4096).astype(np.uint32), "u32")
+        by = 2.0 * 4096 * 2560 * es
+        lu, su = timed(lambda: ops.index_select(table, 0, ids), 50)
+        rows.append(dict(op="index_select 4096 of [51200,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
+                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        del table
+        x = rnd((64, 51200), dt)
+        by = 1.0 * x.numel() * es
+        lu, su = timed(lambda: ops.argmax(x, -1), 50)
+        rows.append(dict(op="argmax [64,51200]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
+                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+    sync()
+    for r in rows:
+        r.update(loop_us=round(r["loop_us"], 2), single_us=round(r["single_us"], 2), achieved=round(r["achieved"], 1),
+                 frac=round(r["frac"], 4))
+    mm = rows[1]
+    _line("bf16 linear [4096,2560]x[2560,10240] TFLOP/s on 1 MI355X", mm["achieved"], "TFLOP/s", 10, 3, mm["loop_us"] / 1e3,
+          "primitive sweep, bf16 and f32: matmul / linear, softmax, LayerNorm, RMSNorm, RoPE, index_select, argmax",
+          {"ops": rows})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -121,9 +298,17 @@ def main():
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     ap.add_argument("--layers", type=int, default=PHI2["num_hidden_layers"],
                     help="debug only: fewer layers (the JSON line then says so and is not the headline workload)")
+    ap.add_argument("--workload", default="phi2-decode", choices=["phi2-decode", "qwen2-prefill", "gemma-decode", "ops"],
+                    help="phi2-decode is the headline line; the others are the remaining configurations of the path")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (multi-GPU sharding is a design note only)")
+    if args.workload == "qwen2-prefill":
+        return run_qwen2_prefill(args)
+    if args.workload == "gemma-decode":
+        return run_gemma_decode(args)
+    if args.workload == "ops":
+        return run_ops(args)
 
     from rai_amd import synthetic
     from rai_amd.hip import sync

@@ -723,6 +723,35 @@ int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, co
     }
   }
 
+  // NN layout with one shared right operand (B[K,N] row-major): transpose B once into a
+  // scratch [N,K] (one pass over B) and run the NT tile kernel on the batch folded into M.
+  if ((a->dtype == RAI_BF16 || a->dtype == RAI_F32) && b->stride[r - 1] == 1 && b->stride[r - 2] == N && N > 1 && K > 1 &&
+      (double)batch * M * N * K >= 1e8) {
+    bool b_shared = true;
+    for (int i = 0; i < r - 2; ++i)
+      if (b->shape[i] != 1 && b->stride[i] != 0) b_shared = false;
+    if (b_shared) {
+      void *tmp = nullptr;
+      RAI_TRY(rai_hip_alloc(dev, (size_t)N * K * dtype_size(b->dtype), &tmp));
+      rai_hip_tensor src;  // B^T as a strided view of B: [N, K] with strides (1, N)
+      memset(&src, 0, sizeof(src));
+      src.data = b->data; src.dtype = b->dtype; src.offset = b->offset; src.rank = 2;
+      src.shape[0] = N; src.shape[1] = K; src.stride[0] = 1; src.stride[1] = N;
+      rai_hip_tensor bt = src;  // contiguous [N, K]
+      bt.data = tmp; bt.offset = 0; bt.stride[0] = K; bt.stride[1] = 1;
+      int rc = rai_hip_copy(dev, &src, &bt);
+      if (rc == RAI_OK) {
+        rai_hip_tensor b2 = *b;  // [.., K, N] view of the transposed copy: strides (1, K), batch strides 0
+        b2.data = tmp; b2.offset = 0;
+        for (int i = 0; i < r - 2; ++i) b2.stride[i] = 0;
+        b2.stride[r - 2] = 1; b2.stride[r - 1] = K;
+        rc = rai_hip_matmul(dev, a, &b2, out);
+      }
+      (void)rai_hip_release(tmp);  // stream-ordered reuse: later work on this stream runs after the product
+      return rc;
+    }
+  }
+
 generic:
   MatmulArgs g;
   g.M = M; g.N = N; g.K = K;

@@ -274,6 +274,150 @@ template <int BM, int BN, int BK> static int launch_cfg(hipStream_t st, const Li
   return RAI_OK;
 }
 
+// ---- small M (9..64 rows): weight streaming through 16x16x32 MFMA -----------------------
+// The activations are tiny and the weights are read exactly once, so the kernel is a
+// stream over W: every wave owns 16 weight rows and reads them straight from global
+// memory in MFMA fragment order (lane l: row l%16, 8 consecutive k at 8*(l/16)), U
+// fragments ahead of the multiply.  The activation rows sit in LDS (16-byte padded
+// pitch: the fragment reads of 16 lanes hit distinct banks) and are the B operand, so
+// accumulator register r of lane l is out[m = l%16][n = 4*(l/16) + r]: four consecutive
+// columns per lane.  K may be split over blockIdx.y (f32 partial sums, summed by
+// k_splitk_epilogue) so that narrow outputs still fill the chip.
+template <int MT, int U>
+__global__ void __launch_bounds__(256) k_linear_bf16_mfma_skinny(LinearArgs a, int k_per_split, int k_chunk,
+                                                                 float *partial) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int split = blockIdx.y;
+  const int kb = split * k_per_split;
+  const int ke = kb + k_per_split < a.K ? kb + k_per_split : a.K;
+  const int pitch = k_chunk + 8;
+  const int n0 = (blockIdx.x * 4 + wave) * 16;
+  int nrow = n0 + (lane & 15);
+  nrow = nrow < a.N ? nrow : a.N - 1;  // clamped rows are computed and never stored
+  const uint16_t *wrow = (const uint16_t *)a.W + (int64_t)nrow * a.ldw + (lane >> 4) * 8;
+  const uint16_t *xfrag = lds + (lane & 15) * pitch + (lane >> 4) * 8;
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int kc0 = kb; kc0 < ke; kc0 += k_chunk) {
+    const int clen = ke - kc0 < k_chunk ? ke - kc0 : k_chunk;  // multiple of 32
+    const int cpr = clen >> 3;
+    if (kc0 != kb) __syncthreads();
+    for (int c = tid; c < MT * 16 * cpr; c += 256) {
+      const int row = c / cpr, kc = (c - row * cpr) * 8;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row < a.M) v = *reinterpret_cast<const u32x4 *>((const uint16_t *)a.A + (int64_t)row * a.lda + kc0 + kc);
+      *reinterpret_cast<u32x4 *>(lds + row * pitch + kc) = v;
+    }
+    const uint16_t *wp = wrow + kc0;
+    bf16x8 w[U];
+    const int full = clen / (32 * U);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (full > 0) w[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8 *>(wp + u * 32));
+    __syncthreads();
+    int k = 0;
+    for (int it = 0; it < full; ++it, k += 32 * U) {
+      bf16x8 cur[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) cur[u] = w[u];
+      if (it + 1 < full) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          w[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8 *>(wp + k + 32 * U + u * 32));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const bf16x8 x = *reinterpret_cast<const bf16x8 *>(xfrag + i * 16 * pitch + k + u * 32);
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], x, acc[i], 0, 0, 0);
+        }
+    }
+    for (; k < clen; k += 32) {
+      const bf16x8 wv = __builtin_nontemporal_load(reinterpret_cast<const bf16x8 *>(wp + k));
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8 *>(xfrag + i * 16 * pitch + k);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, x, acc[i], 0, 0, 0);
+      }
+    }
+  }
+
+  const int n = n0 + 4 * (lane >> 4);
+  if (n >= a.N) return;
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const int m = i * 16 + (lane & 15);
+    if (m >= a.M) continue;
+    const float v[4] = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+    if (partial) {
+      float *p = partial + ((int64_t)split * a.M + m) * a.N + n;
+      if (a.N % 4 == 0) *reinterpret_cast<f32x4 *>(p) = acc[i];
+      else for (int e = 0; e < 4 && n + e < a.N; ++e) p[e] = v[e];
+      continue;
+    }
+    if (a.glu) {  // columns n..n+3 are two (gate, up) pairs
+      uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
+      for (int e = 0; e < 4 && n + e + 1 < a.N; e += 2) {
+        const float g = v[e] + (bias ? bf16_bits_to_f32(bias[n + e]) : 0.f);
+        const float u = v[e + 1] + (bias ? bf16_bits_to_f32(bias[n + e + 1]) : 0.f);
+        dst[e >> 1] = f32_to_bf16_bits(glu_bf16(a.act, g, u));
+      }
+      continue;
+    }
+    for (int e = 0; e < 4 && n + e < a.N; ++e) {
+      const int nn = n + e;
+      float x = v[e] + (bias ? bf16_bits_to_f32(bias[nn]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[nn]) : 0.f);
+      if (a.act >= 0 && nn >= a.act_from) x = act_eval(a.act, x);
+      if (res) x += bf16_bits_to_f32(res[(int64_t)m * a.ldr + nn]);
+      if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = f32_to_bf16_bits(x);
+      else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = f32_to_bf16_bits(x);
+    }
+  }
+}
+
+template <int MT> static int launch_mfma_skinny(hipStream_t st, const LinearArgs &a) {
+  constexpr int U = 8;
+  constexpr int kcap = MT == 1 ? 2048 : MT == 2 ? 1024 : 512;  // LDS: MT*16 rows of (chunk + 8) bf16, about 64 KB
+  const int blocks_x = ((a.N + 15) / 16 + 3) / 4;
+  // Split K until there are about four blocks per CU, keeping at least 256 columns per split.
+  int splits = 1;
+  if (a.splitk_ws) {
+    while (blocks_x * splits < 4 * kNumCU && a.K / (splits * 2) >= 256 &&
+           (size_t)(splits * 2) * a.M * a.N * sizeof(float) <= a.splitk_ws_bytes)
+      splits *= 2;
+  }
+  int kps = (a.K + splits - 1) / splits;
+  kps = (kps + 127) / 128 * 128;
+  splits = (a.K + kps - 1) / kps;
+  const int chunk = kps < kcap ? kps : kcap;
+  const size_t lds = (size_t)MT * 16 * (chunk + 8) * sizeof(uint16_t);
+  static bool attr_set = false;
+  if (!attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma_skinny<MT, U>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024));
+    attr_set = true;
+  }
+  float *partial = splits > 1 ? (float *)a.splitk_ws : nullptr;
+  hipLaunchKernelGGL((k_linear_bf16_mfma_skinny<MT, U>), dim3(blocks_x, splits), dim3(256), lds, st, a, kps, chunk,
+                     partial);
+  RAI_TRY(launch_check("linear_bf16_mfma_skinny"));
+  if (splits > 1) {
+    const int64_t total = (int64_t)a.M * a.N;
+    const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);
+    RAI_TRY(launch_check("splitk_epilogue"));
+  }
+  return RAI_OK;
+}
+
 int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
   RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
@@ -285,6 +429,14 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear mfma: K=%d must be a multiple of 32", a.K);
   RAI_REQUIRE(a.lda % 8 == 0 && a.ldw % 8 == 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0,
               RAI_ERR_BAD_STRIDE, "linear mfma: operands must be 16-byte aligned with row strides multiple of 8");
+  static const bool no_skinny = getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr;
+  if (a.M <= 64 && !no_skinny) {
+    const int mt = (a.M + 15) / 16;
+    if (mt == 1) return launch_mfma_skinny<1>(st, a);
+    if (mt == 2) return launch_mfma_skinny<2>(st, a);
+    if (mt == 3) return launch_mfma_skinny<3>(st, a);
+    return launch_mfma_skinny<4>(st, a);
+  }
   // Split K when the tile count alone cannot fill the GPU and a workspace was provided.
   const int tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
   int splits = 1;

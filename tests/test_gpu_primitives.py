@@ -381,7 +381,7 @@ def test_matmul_batched_strided(R, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
-@pytest.mark.parametrize("m", [1, 4, 130])
+@pytest.mark.parametrize("m", [1, 4, 9, 16, 33, 48, 64, 130])
 def test_fused_linear_bias_act_residual(R, dt, m):
     g = rng(25)
     k, n = 512, 384
@@ -390,6 +390,21 @@ def test_fused_linear_bias_act_residual(R, dt, m):
     got = down(R.linear(up(x, dt), up(w, dt), up(b, dt), "new_gelu", up(r, dt)))
     assert_close(got, want, dt, f"linear fused m={m}")
     assert_close(down(R.linear(up(x, dt), up(w, dt))), onn.linear(x, w, None, dt), dt, "linear plain")
+
+
+@pytest.mark.parametrize("m", [9, 16, 31, 64])
+@pytest.mark.parametrize("k,n", [(4096, 200), (1056, 2048), (16384, 64), (96, 50)])
+def test_linear_small_batch_deep_k(R, m, k, n):
+    # batched-decode shapes: 9..64 activation rows against a weight matrix read once; K deep enough
+    # to be split over blocks and staged in several chunks, N not a multiple of the 16-row tile
+    g = rng(125)
+    x, w, b = rand(g, (m, k), "bf16"), rand(g, (n, k), "bf16", 0.03), rand(g, (n,), "bf16")
+    r = rand(g, (m, n), "bf16")
+    assert_close(down(R.linear(up(x, "bf16"), up(w, "bf16"), up(b, "bf16"))), onn.linear(x, w, b, "bf16"), "bf16",
+                 f"linear {m}x{k}x{n}")
+    want = oo.add(onn.new_gelu(onn.linear(x, w, b, "bf16"), "bf16"), r, "bf16")
+    got = down(R.linear(up(x, "bf16"), up(w, "bf16"), up(b, "bf16"), "new_gelu", up(r, "bf16")))
+    assert_close(got, want, "bf16", f"linear fused {m}x{k}x{n}")
 
 
 # ------------------------------------------------------------------ norms / rope / attention

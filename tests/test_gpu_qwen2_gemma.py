@@ -88,3 +88,23 @@ def test_greedy_generate_matches_oracle(hip, arch):
     toks2, _, _ = dec.generate(prompt, 10)
     assert np.array_equal(toks, toks2)
     dec.close()
+
+
+@pytest.mark.parametrize("arch", ["qwen2", "gemma"])
+def test_batched_decode_many_sequences_bf16(hip, arch):
+    # 24 sequences decoded together: 9..64 activation rows take the weight-streaming MFMA path
+    # (gated-MLP epilogue, q/k/v bias, output split, residual) and the split decode attention
+    cfg = CFGS[arch]()
+    dec, ref = make(cfg, "bf16", max_batch=24, max_context=64)
+    ids = np.random.Generator(np.random.PCG64(4)).integers(0, cfg.vocab_size, (24, 5)).astype(np.uint32)
+    logits, tok = dec.forward(ids)
+    want = ref.fwd(ids)
+    assert_close(logits, want, "bf16", f"{arch} prefill 24x5")
+    nxt = np.argmax(want, -1).astype(np.uint32).reshape(24, 1)
+    for step in range(3):
+        logits, tok = dec.forward(nxt)
+        want = ref.fwd(nxt)
+        assert_close(logits, want, "bf16", f"{arch} batched decode step {step}")
+        check_tokens(tok, want, "bf16")
+        nxt = np.argmax(want, -1).astype(np.uint32).reshape(24, 1)
+    dec.close()
