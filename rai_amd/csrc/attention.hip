@@ -172,6 +172,75 @@ __device__ __forceinline__ float load_device(const float *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Tail of a decode-attention block: once its partials are written, the block
+// counts itself in; the last block of the head group to arrive merges the NS
+// partials of the R query heads starting at hq0 and writes their output rows.
+// wbuf is block-shared scratch of 2 * R * NS floats that no wave uses any more.
+// The merge is a chain of dependent memory round trips, so it is kept short: one
+// for all (m, l) statistics, then the per-split weights exp(m_s - M) / L are
+// computed once per head, and every thread has 64 partial-output loads in flight.
+template <typename T>
+__device__ __forceinline__ void decode_merge_last(const AttnDecodeArgs &a, int b, int hq0, int R, int *sh_last,
+                                                  float *wbuf) {
+  constexpr int NT = kDecodeThreads;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NS = a.ns, D = a.D, PW = D + 2;
+  // every thread's write-through stores have completed before the block's arrival is counted
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  int *counter = a.counters + ((int64_t)b * a.Hq + hq0) * kDecodeCounterStride;  // one 128-byte line each
+  if (tid == 0) *sh_last = atomicAdd(counter, 1) == NS - 1;
+  __syncthreads();
+  if (!*sh_last) return;
+  const float *all = a.ws + ((int64_t)b * a.Hq + hq0) * NS * PW;
+  float *wm = wbuf, *wl = wbuf + R * NS;
+  for (int i = tid; i < R * NS; i += NT) {
+    const float *st = all + (int64_t)i * PW;   // (head r, split s) at index r*NS + s
+    wm[i] = load_device(st);
+    wl[i] = load_device(st + 1);
+  }
+  __syncthreads();
+  for (int r = wave; r < R; r += NT / 64) {      // NS <= 64: one split per lane
+    const float m = lane < NS ? wm[r * NS + lane] : -INFINITY;
+    const float M = wave_max(m);                 // split 0 always holds a key, so M is finite
+    const float e = lane < NS ? expf(m - M) : 0.f;  // an empty split has m = -inf: weight 0
+    const float L = wave_sum(lane < NS ? e * wl[r * NS + lane] : 0.f);
+    if (lane < NS) wm[r * NS + lane] = e / L;
+  }
+  __syncthreads();
+  constexpr int EU = 8, SB = 8;
+  for (int e0 = tid; e0 < R * D; e0 += NT * EU) {
+    const float *po[EU];
+    int hr[EU], hd[EU];
+    float O[EU];
+#pragma unroll
+    for (int i = 0; i < EU; ++i) {
+      const int e = e0 + i * NT < R * D ? e0 + i * NT : e0;
+      hr[i] = e / D;
+      hd[i] = e - hr[i] * D;
+      po[i] = all + (int64_t)hr[i] * NS * PW + 2 + hd[i];
+      O[i] = 0.f;
+    }
+    for (int s0 = 0; s0 < NS; s0 += SB) {
+      float ov[EU][SB];
+#pragma unroll
+      for (int i = 0; i < EU; ++i)
+#pragma unroll
+        for (int j = 0; j < SB; ++j) ov[i][j] = load_device(po[i] + (s0 + j < NS ? s0 + j : NS - 1) * PW);
+#pragma unroll
+      for (int i = 0; i < EU; ++i)
+#pragma unroll
+        for (int j = 0; j < SB; ++j)
+          if (s0 + j < NS) O[i] = fmaf(wm[hr[i] * NS + s0 + j], ov[i][j], O[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < EU; ++i)
+      if (e0 + i * NT < R * D)
+        Scalar<T>::store((T *)a.out + (int64_t)b * a.out_row_stride + (int64_t)(hq0 + hr[i]) * D + hd[i],
+                         (typename Scalar<T>::compute)O[i]);
+  }
+  if (tid == 0) *counter = 0;  // ready for the next launch (stream order)
+}
+
 template <typename T, int R, int CC, int UK, int UV>
 __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_split(AttnDecodeArgs a) {
   constexpr int V = AttnVec<T>::V;
@@ -367,58 +436,14 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_split(AttnDecode
     store_device(part + (int64_t)tid * NS * PW, sh_m[tid]);
     store_device(part + (int64_t)tid * NS * PW + 1, sh_l[tid]);
   }
-  // ---- the last block of this head group merges the partials: every thread's
-  //      write-through stores have completed before the block's arrival is counted
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  int *counter = a.counters + ((int64_t)b * a.Hq + hq0) * kDecodeCounterStride;  // one 128-byte line each
-  if (tid == 0) sh_last = atomicAdd(counter, 1) == NS - 1;
-  __syncthreads();
-  if (!sh_last) return;
-  // All loads of a batch of splits are in flight together (statistics and the
-  // thread's output feature), so the merge costs one memory round trip per
-  // batch of kMergeBatch splits rather than one per split.
-  constexpr int kMergeBatch = 8;
-  const float *all = a.ws + ((int64_t)b * a.Hq + hq0) * NS * PW;
-  for (int e = tid; e < R * D; e += NT) {
-    const int r = e / D, d = e - r * D;
-    const float *pr = all + (int64_t)r * NS * PW;
-    float M = -INFINITY, L = 0.f, O = 0.f;
-    for (int s0 = 0; s0 < NS; s0 += kMergeBatch) {
-      float mv[kMergeBatch], lv[kMergeBatch], ov[kMergeBatch];
-#pragma unroll
-      for (int j = 0; j < kMergeBatch; ++j) {
-        const int ss = s0 + j < NS ? s0 + j : NS - 1;
-        mv[j] = load_device(pr + ss * PW);
-        lv[j] = load_device(pr + ss * PW + 1);
-        ov[j] = load_device(pr + ss * PW + 2 + d);
-      }
-      float mb = M;
-#pragma unroll
-      for (int j = 0; j < kMergeBatch; ++j) mb = fmaxf(mb, mv[j]);
-      const float rescale = expf(M - mb);  // M = -inf on the first batch: 0 (split 0 always holds a key, so mb is finite)
-      L *= rescale;
-      O *= rescale;
-      M = mb;
-#pragma unroll
-      for (int j = 0; j < kMergeBatch; ++j) {
-        if (s0 + j < NS) {
-          const float w = expf(mv[j] - M);  // an empty split has m = -inf: weight 0
-          L = fmaf(w, lv[j], L);
-          O = fmaf(w, ov[j], O);
-        }
-      }
-    }
-    Scalar<T>::store((T *)a.out + (int64_t)b * a.out_row_stride + (int64_t)(hq0 + r) * D + d,
-                     (typename Scalar<T>::compute)(O / L));
-  }
-  if (tid == 0) *counter = 0;  // ready for the next launch (stream order)
+  decode_merge_last<T>(a, b, hq0, R, &sh_last, smem);
 }
 
 // Number of context splits: enough blocks to fill the chip, bounded so that a
 // block's share of the longest context fits the LDS score buffer.
 static int decode_splits(const AttnDecodeArgs &a, int head_groups) {
-  static const int forced = getenv("RAI_HIP_ATTN_SPLITS") ? atoi(getenv("RAI_HIP_ATTN_SPLITS")) : 0;
+  const char *knob = getenv("RAI_HIP_ATTN_SPLITS");  // tuning and test aid, read at every launch
+  const int forced = knob ? atoi(knob) : 0;
   int ns = forced > 0 ? forced : (2 * kNumCU + head_groups * a.B - 1) / (head_groups * a.B);
   const int need = (a.Tmax + 1023) / 1024;
   if (ns < need) ns = need;
@@ -431,6 +456,297 @@ size_t attention_decode_ws_bytes(int B, int Hq, int D) {
   return sizeof(float) * (size_t)B * Hq * kDecodeMaxSplits * (D + 2);
 }
 size_t attention_decode_counter_bytes(int B, int Hq) { return sizeof(int) * (size_t)B * Hq * kDecodeCounterStride; }
+
+// Decode attention for grouped-query models in bf16, both products on
+// v_mfma_f32_16x16x32_bf16.  Block (split, kv head, batch) serves all R <= 16 query
+// heads of one KV head over at most CH (64 or 128) consecutive keys:
+//   - every K and V load of the block is issued before anything is computed.  K goes
+//     straight from global memory into MFMA A fragments (lane l: key l%16 of a 16-key
+//     tile, features 32*step + 8*(l/16) ..), two tiles per wave; V goes through LDS;
+//   - scores^T[key, head] = K . Q^T per tile; accumulator register r of lane l is key
+//     4*(l/16)+r, head l%16.  The rotated queries are the B fragments, held in registers;
+//   - per-head max / exp / sum over the block's keys (one wave per head), exp values
+//     rounded to bf16 for the second product (the reference rounds P to V's dtype);
+//   - O[head, feature] = P . V: wave w owns features [w*D/4, (w+1)*D/4), P fragments are
+//     16-byte LDS reads, V fragments are gathered from LDS two bytes at a time (the
+//     transposition costs LDS reads, of which there are few: the kernel is bound by
+//     the K/V stream);
+//   - partial (m, l, o[D]) per head, merged by the last block as in the split kernel.
+typedef __attribute__((ext_vector_type(8))) __bf16 ad_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float ad_f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t ad_u32x4;
+
+template <int D, int CH>
+__global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeArgs a) {
+  typedef bf16_raw T;
+  constexpr int KS = D / 32, KT = CH / 64;
+  constexpr int VP = D + 8, PP = CH + 8;           // LDS pitches (bf16 elements)
+  constexpr int CPR = D / 8;                        // 16-byte chunks per K/V row
+  constexpr int VL = CH * CPR / kDecodeThreads;     // V chunks per thread
+  constexpr int DT = D / 64;                        // 16-feature tiles per wave in P.V
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  uint16_t *Vs = reinterpret_cast<uint16_t *>(smem);          // [CH][VP]; the first 16 rows hold Q until the scores are done
+  const int R = a.Hq / a.Hkv;
+  float *scores = reinterpret_cast<float *>(Vs + CH * VP);    // [R][CH]
+  uint16_t *ps = reinterpret_cast<uint16_t *>(scores + R * CH);   // [16][PP]
+  uint16_t *knew = ps + 16 * PP;                              // [D]
+  uint16_t *vnew = knew + D;                                  // [D]
+  __shared__ float sh_m[16], sh_l[16];
+
+  const int s = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  const int hq0 = hk * R;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 15, lq = lane >> 4;
+  const int NS = a.ns;
+  int pos = *a.pos_dev;
+  if (pos > a.Tmax - 1) pos = a.Tmax - 1;   // capacity is checked on the host; never write past the cache
+  const int cnt = pos + 1;
+  int chunk = (cnt + NS - 1) / NS;
+  if (chunk > CH) chunk = CH;
+  const int t0 = s * chunk;
+  const int t1 = t0 + chunk < cnt ? t0 + chunk : cnt;
+  const int n = t1 > t0 ? t1 - t0 : 0;
+  const bool has_new = pos >= t0 && pos < t1;
+  const int t1c = has_new ? pos : t1;       // cached keys are [t0, t1c)
+  const int new_row = pos - t0;
+
+  const int QD = a.Hq * D, KD = a.Hkv * D;
+  const T *row = (const T *)a.qkv + (int64_t)b * (QD + 2 * KD);
+  T *Kc = (T *)a.kcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
+  T *Vc = (T *)a.vcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
+  const T *cos_t = (const T *)a.cos_t, *sin_t = (const T *)a.sin_t;
+
+  // ---- all K and V loads of the block
+  ad_bf16x8 kreg[KT][KS];
+#pragma unroll
+  for (int i = 0; i < KT; ++i) {
+    const int t = t0 + (wave + 4 * i) * 16 + lrow;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      ad_bf16x8 z = {};
+      if (t < t1c) z = *reinterpret_cast<const ad_bf16x8 *>(Kc + (int64_t)t * D + ks * 32 + lq * 8);
+      kreg[i][ks] = z;
+    }
+  }
+  ad_u32x4 vreg[VL];
+#pragma unroll
+  for (int j = 0; j < VL; ++j) {
+    const int c = tid + j * kDecodeThreads, r = c / CPR, c8 = c - r * CPR;
+    ad_u32x4 z = {0u, 0u, 0u, 0u};
+    if (t0 + r < t1c) z = *reinterpret_cast<const ad_u32x4 *>(Vc + (int64_t)(t0 + r) * D + c8 * 8);
+    vreg[j] = z;
+  }
+  // ---- rotated queries (rows >= R are zero).  Eight features per item, all loads of a thread in
+  //      flight together: one memory round trip instead of one per feature.
+  if (a.rot % 16 == 0) {
+    constexpr int QI = (16 * CPR + kDecodeThreads - 1) / kDecodeThreads;
+    const int half = a.rot >> 1;
+    ad_u32x4 qx[QI], qo[QI], qc[QI], qn[QI];
+#pragma unroll
+    for (int i = 0; i < QI; ++i) {
+      const int item = tid + i * kDecodeThreads, r = item / CPR, d = (item - r * CPR) * 8;
+      qx[i] = qo[i] = qc[i] = qn[i] = ad_u32x4{0u, 0u, 0u, 0u};
+      if (item < 16 * CPR && r < R) {
+        const T *head = row + (hq0 + r) * D;
+        qx[i] = *reinterpret_cast<const ad_u32x4 *>(head + d);
+        if (d < a.rot) {
+          qo[i] = *reinterpret_cast<const ad_u32x4 *>(head + (d < half ? d + half : d - half));
+          qc[i] = *reinterpret_cast<const ad_u32x4 *>(cos_t + (int64_t)pos * a.rot + d);
+          qn[i] = *reinterpret_cast<const ad_u32x4 *>(sin_t + (int64_t)pos * a.rot + d);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < QI; ++i) {
+      const int item = tid + i * kDecodeThreads, r = item / CPR, d = (item - r * CPR) * 8;
+      if (item >= 16 * CPR) continue;
+      ad_u32x4 out = qx[i];
+      if (r < R && d < a.rot) {
+        const float sign = d < half ? -1.f : 1.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          uint32_t packed = 0;
+#pragma unroll
+          for (int hbit = 0; hbit < 2; ++hbit) {
+            const int sh = 16 * hbit;
+            const float x = bf16_bits_to_f32((uint16_t)(qx[i][w] >> sh)), o = sign * bf16_bits_to_f32((uint16_t)(qo[i][w] >> sh));
+            const float c = bf16_bits_to_f32((uint16_t)(qc[i][w] >> sh)), sn = bf16_bits_to_f32((uint16_t)(qn[i][w] >> sh));
+            // three roundings, as rope_feature
+            const float res = round_to<T>(round_to<T>(x * c) + round_to<T>(o * sn));
+            packed |= (uint32_t)f32_to_bf16_bits(res) << sh;
+          }
+          out[w] = packed;
+        }
+      }
+      *reinterpret_cast<ad_u32x4 *>(Vs + r * VP + d) = out;
+    }
+  } else {
+    for (int e = tid; e < 16 * D; e += kDecodeThreads) {
+      const int r = e / D, d = e - r * D;
+      const float q = r < R ? rope_feature<T>(row + (hq0 + r) * D, d, a.rot, cos_t, sin_t, pos) : 0.f;
+      Vs[r * VP + d] = f32_to_bf16_bits(q);
+    }
+  }
+  for (int e = tid; e < 16 * PP; e += kDecodeThreads) ps[e] = 0;
+  if (has_new) {
+    for (int d = tid; d < D; d += kDecodeThreads) {
+      const uint16_t kr = f32_to_bf16_bits(rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos));
+      const uint16_t vr = (row + QD + KD + hk * D + d)->bits;
+      knew[d] = kr;
+      vnew[d] = vr;
+      (Kc + (int64_t)pos * D + d)->bits = kr;
+      (Vc + (int64_t)pos * D + d)->bits = vr;
+    }
+  }
+  __syncthreads();
+
+  // ---- scores
+  {
+    ad_bf16x8 qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const ad_bf16x8 *>(Vs + lrow * VP + ks * 32 + lq * 8);
+#pragma unroll
+    for (int i = 0; i < KT; ++i) {
+      const int tile = wave + 4 * i;
+      if (has_new && new_row == tile * 16 + lrow) {   // the lanes that hold the new token's key row
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kreg[i][ks] = *reinterpret_cast<const ad_bf16x8 *>(knew + ks * 32 + lq * 8);
+      }
+      ad_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[i][ks], qf[ks], acc, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int tl = tile * 16 + 4 * lq + r;
+        float sc = a.f32_scores ? acc[r] * a.scale : round_to<T>(round_to<T>(acc[r]) * round_to<T>(a.scale));
+        if (lrow < R) scores[lrow * CH + tl] = tl < n ? sc : -INFINITY;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- V into LDS (the new token's row from the activations), softmax statistics
+#pragma unroll
+  for (int j = 0; j < VL; ++j) {
+    const int c = tid + j * kDecodeThreads, r = c / CPR, c8 = c - r * CPR;
+    ad_u32x4 v = vreg[j];
+    if (has_new && r == new_row) v = *reinterpret_cast<const ad_u32x4 *>(vnew + c8 * 8);
+    *reinterpret_cast<ad_u32x4 *>(Vs + r * VP + c8 * 8) = v;
+  }
+  for (int r = wave; r < R; r += 4) {
+    float m = -INFINITY;
+    for (int t = lane; t < n; t += 64) m = fmaxf(m, scores[r * CH + t]);
+    m = wave_max(m);
+    float l = 0.f;
+    for (int t = lane; t < n; t += 64) {
+      const float e = expf(scores[r * CH + t] - m);
+      ps[r * PP + t] = f32_to_bf16_bits(e);
+      l += e;
+    }
+    l = wave_sum(l);
+    if (lane == 0) { sh_m[r] = m; sh_l[r] = l; }
+  }
+  __syncthreads();
+
+  // ---- O = P . V for this wave's features
+  const int PW = D + 2;
+  float *part = a.ws + (((int64_t)b * a.Hq + hq0) * NS + s) * PW;  // head r at part + r*NS*PW
+  {
+    ad_f32x4 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = ad_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int d0 = wave * (D / 4);
+    for (int k0 = 0; k0 < n; k0 += 32) {
+      const ad_bf16x8 pf = *reinterpret_cast<const ad_bf16x8 *>(ps + lrow * PP + k0 + lq * 8);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        typedef __attribute__((ext_vector_type(8))) uint16_t u16x8;
+        u16x8 vb;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vb[j] = Vs[(k0 + lq * 8 + j) * VP + d0 + dt * 16 + lrow];
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, __builtin_bit_cast(ad_bf16x8, vb), o[dt], 0, 0, 0);
+      }
+    }
+    // accumulator register r of lane l is head 4*(l/16)+r, feature l%16 of the tile
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int h = 4 * lq + r;
+        if (h < R) part[(int64_t)h * NS * PW + 2 + d0 + dt * 16 + lrow] = o[dt][r];
+      }
+  }
+  if (tid < R) {
+    part[(int64_t)tid * NS * PW] = sh_m[tid];
+    part[(int64_t)tid * NS * PW + 1] = sh_l[tid];
+  }
+}
+
+// Merges the NS partials of one (batch, query head): block (head, batch), one
+// thread per output feature.  Every wave computes the split weights
+// exp(m_s - M) / L with one split per lane (NS <= 64), then each thread has all
+// its partial-output loads in flight at once: two memory round trips in all.
+__global__ void __launch_bounds__(256) k_attn_decode_merge_bf16(AttnDecodeArgs a) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x, lane = threadIdx.x & 63;
+  const int NS = a.ns, D = a.D, PW = D + 2;
+  const float *pr = a.ws + ((int64_t)b * a.Hq + h) * NS * PW;
+  const float m = lane < NS ? pr[lane * PW] : -INFINITY;
+  const float l = lane < NS ? pr[lane * PW + 1] : 0.f;
+  const float M = wave_max(m);                    // split 0 always holds a key, so M is finite
+  const float e = lane < NS ? expf(m - M) : 0.f;  // an empty split has m = -inf: weight 0
+  const float L = wave_sum(e * l);
+  const float w = e / L;
+  float O = 0.f;
+  constexpr int SB = 16;
+  for (int s0 = 0; s0 < NS; s0 += SB) {
+    float ov[SB];
+#pragma unroll
+    for (int j = 0; j < SB; ++j) ov[j] = pr[(s0 + j < NS ? s0 + j : NS - 1) * PW + 2 + d];
+#pragma unroll
+    for (int j = 0; j < SB; ++j)
+      if (s0 + j < NS) O = fmaf(__shfl(w, s0 + j, 64), ov[j], O);
+  }
+  ((bf16_raw *)a.out + (int64_t)b * a.out_row_stride + (int64_t)h * D + d)->bits = f32_to_bf16_bits(O);
+}
+
+template <int D, int CH> static int launch_decode_mfma_cfg(hipStream_t st, AttnDecodeArgs a) {
+  const int R = a.Hq / a.Hkv;
+  a.ns = decode_splits(a, a.Hkv);
+  const int need = (a.Tmax + CH - 1) / CH;
+  if (a.ns < need) a.ns = need;
+  a.chunk_cap = CH;
+  const size_t lds = (size_t)CH * (D + 8) * 2 + (size_t)R * CH * 4 + 16 * (CH + 8) * 2 + 2 * D * 2;
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_attn_decode_mfma<D, CH>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)((size_t)CH * (D + 8) * 2 + 16 * CH * 4 + 16 * (CH + 8) * 2 + 2 * D * 2)));
+    attr_set = true;
+  }
+  RAI_REQUIRE(a.Hkv <= 65535 && a.B <= 65535, RAI_ERR_UNSUPPORTED, "attention decode: grid too large");
+  hipLaunchKernelGGL((k_attn_decode_mfma<D, CH>), dim3(a.ns, a.Hkv, a.B), dim3(kDecodeThreads), lds, st, a);
+  RAI_TRY(launch_check("attention_decode_mfma"));
+  hipLaunchKernelGGL(k_attn_decode_merge_bf16, dim3(a.Hq, a.B), dim3(D), 0, st, a);
+  return launch_check("attention_decode_merge");
+}
+
+// Blocks of 64 keys (four or more per CU) while the longest context fits
+// kDecodeMaxSplits of them, else blocks of 128 keys.
+constexpr int kMfmaDecodeKeysMax = 128;
+template <int D> static int launch_decode_mfma(hipStream_t st, const AttnDecodeArgs &a) {
+  const char *knob = getenv("RAI_HIP_ATTN_KEYS");  // tuning and test aid: 64 or 128 keys per block
+  const int forced = knob ? atoi(knob) : 0;
+  if (forced != 128 && (a.Tmax + 63) / 64 <= kDecodeMaxSplits) return launch_decode_mfma_cfg<D, 64>(st, a);
+  return launch_decode_mfma_cfg<D, 128>(st, a);
+}
+
+// The MFMA kernel serves bf16 grouped-query shapes whose longest context fits
+// kDecodeMaxSplits blocks of kMfmaDecodeKeysMax keys.
+static bool decode_mfma_eligible(const AttnDecodeArgs &a) {
+  static const bool off = getenv("RAI_HIP_NO_MFMA_DECODE") != nullptr;
+  const int rep = a.Hq / a.Hkv;
+  return !off && a.dtype == RAI_BF16 && rep >= 4 && rep <= 16 && (a.D == 64 || a.D == 128 || a.D == 256) &&
+         (a.Tmax + kMfmaDecodeKeysMax - 1) / kMfmaDecodeKeysMax <= kDecodeMaxSplits;
+}
 
 template <typename T, int R, int CC, int UK, int UV> static int launch_decode_cfg(hipStream_t st, AttnDecodeArgs a) {
   constexpr int V = AttnVec<T>::V;
@@ -477,6 +793,11 @@ int launch_attention_decode(hipStream_t st, const AttnDecodeArgs &a) {
               "attention decode: bad problem");
   RAI_REQUIRE(a.rot > 0 && a.rot % 2 == 0 && a.rot <= a.D, RAI_ERR_BAD_ARG, "attention decode: rot %d", a.rot);
   RAI_REQUIRE(a.ws && a.counters, RAI_ERR_BAD_ARG, "attention decode: partial-result workspace missing");
+  if (decode_mfma_eligible(a)) {
+    if (a.D == 64) return launch_decode_mfma<64>(st, a);
+    if (a.D == 128) return launch_decode_mfma<128>(st, a);
+    return launch_decode_mfma<256>(st, a);
+  }
   switch (a.dtype) {
     case RAI_F32: return launch_decode<float>(st, a);
     case RAI_BF16: return launch_decode<bf16_raw>(st, a);

@@ -108,3 +108,43 @@ def test_batched_decode_many_sequences_bf16(hip, arch):
         check_tokens(tok, want, "bf16")
         nxt = np.argmax(want, -1).astype(np.uint32).reshape(24, 1)
     dec.close()
+
+
+GQA_CFGS = {
+    # all query heads of a KV head share one block of the MFMA decode-attention kernel
+    "gemma-mqa-8x256": lambda: qwen2.Config("gemma", 500, 256, 512, 1, 8, 1, "gelu", max_position_embeddings=320,
+                                            head_dim=256),
+    "qwen2-gqa-12/2x128": lambda: qwen2.Config("qwen2", 500, 256, 512, 1, 12, 2, "silu", max_position_embeddings=320,
+                                               rope_theta=1e6, head_dim=128),
+    "qwen2-gqa-16/4x64": lambda: qwen2.Config("qwen2", 500, 256, 512, 1, 16, 4, "silu", max_position_embeddings=320,
+                                              rope_theta=1e6, head_dim=64),
+}
+
+
+@pytest.mark.parametrize("splits,keys", [(None, None), ("2", None), ("2", "128"), ("5", "128")])
+@pytest.mark.parametrize("name", list(GQA_CFGS))
+def test_grouped_query_decode_attention_long_context(hip, name, splits, keys, monkeypatch):
+    # context long enough that one block holds several 16-key tiles (few splits) or a handful of keys
+    # (default: as many splits as fill the GPU); the new token lands in different tiles and lanes
+    if splits is None:
+        monkeypatch.delenv("RAI_HIP_ATTN_SPLITS", raising=False)
+    else:
+        monkeypatch.setenv("RAI_HIP_ATTN_SPLITS", splits)
+    if keys is None:
+        monkeypatch.delenv("RAI_HIP_ATTN_KEYS", raising=False)
+    else:
+        monkeypatch.setenv("RAI_HIP_ATTN_KEYS", keys)     # keys per block of the MFMA kernel
+    cfg = GQA_CFGS[name]()
+    dec, ref = make(cfg, "bf16", max_batch=3, max_context=320)
+    ids = np.random.Generator(np.random.PCG64(5)).integers(0, cfg.vocab_size, (3, 171)).astype(np.uint32)
+    logits, tok = dec.forward(ids)
+    want = ref.fwd(ids)
+    assert_close(logits, want, "bf16", f"{name} prefill")
+    nxt = np.argmax(want, -1).astype(np.uint32).reshape(3, 1)
+    for step in range(6):
+        logits, tok = dec.forward(nxt)
+        want = ref.fwd(nxt)
+        assert_close(logits, want, "bf16", f"{name} decode step {step} splits {splits}")
+        check_tokens(tok, want, "bf16")
+        nxt = np.argmax(want, -1).astype(np.uint32).reshape(3, 1)
+    dec.close()
