@@ -418,6 +418,167 @@ template <int MT> static int launch_mfma_skinny(hipStream_t st, const LinearArgs
   return RAI_OK;
 }
 
+// ---- small M, second form: activations in registers, K split over the waves of a block ----
+// Block = 8 waves; wave w owns K columns [k0 + w*32*KS, k0 + (w+1)*32*KS) of the block's
+// K span and keeps the activation fragments of that slice in registers for the whole
+// launch (MT*KS fragments).  The block walks over 16-row weight tiles: every wave reads
+// its slice of the tile's rows straight into MFMA A fragments (one tile ahead of the
+// multiply), so the block as a whole reads one contiguous 16-row panel after another and
+// nothing is staged through LDS.  After G tiles the eight partial accumulators of each
+// output are summed through LDS and the Linear epilogue is applied.  A K span of
+// 256*KS covers K = 2048 (M <= 32) without splitting K over blocks, so the qkv / dense
+// shapes of a batched decode step need neither a partial-sum buffer nor a second kernel.
+template <int MT, int KS, int G>
+__global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, int tiles, float *partial) {
+  constexpr int NW = 8;
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  f32x4 *red = reinterpret_cast<f32x4 *>(lds);        // [NW][G*MT][64]
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 15, lq = lane >> 4;
+  const int split = blockIdx.y;
+  const int k0 = (split * NW + wave) * KS * 32;
+
+  // activation fragments of this wave's K slice (zero beyond M and K)
+  bf16x8 xf[MT][KS];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int m = mt * 16 + lrow, k = k0 + ks * 32;
+      bf16x8 z = {};
+      if (m < a.M && k < a.K)
+        z = *reinterpret_cast<const bf16x8 *>((const uint16_t *)a.A + (int64_t)m * a.lda + k + lq * 8);
+      xf[mt][ks] = z;
+    }
+  int koff[KS];   // K steps beyond K read column 0 (their activation fragments are zero)
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = k0 + ks * 32 < a.K ? k0 + ks * 32 : 0;
+  const uint16_t *wbase = (const uint16_t *)a.W + lq * 8;
+
+  bf16x8 wa[KS], wb[KS];
+  auto load_tile = [&](bf16x8 (&w)[KS], int tile) {
+    tile = tile < tiles ? tile : tiles - 1;
+    int n = tile * 16 + lrow;
+    n = n < a.N ? n : a.N - 1;
+    const uint16_t *p = wbase + (int64_t)n * a.ldw;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) w[ks] = *reinterpret_cast<const bf16x8 *>(p + koff[ks]);
+  };
+  const int stride = gridDim.x * G;
+  int g0 = blockIdx.x * G;
+  load_tile(wa, g0);
+  for (; g0 < tiles; g0 += stride) {
+    f32x4 acc[G][MT];
+#pragma unroll
+    for (int j = 0; j < G; ++j)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < G; j += 2) {
+      if (G > 1) load_tile(wb, g0 + j + 1);
+      else load_tile(wb, g0 + stride);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ks], xf[mt][ks], acc[j][mt], 0, 0, 0);
+      if (G > 1) {
+        load_tile(wa, j + 2 < G ? g0 + j + 2 : g0 + stride);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[j + 1 < G ? j + 1 : j][mt] =
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[ks], xf[mt][ks], acc[j + 1 < G ? j + 1 : j][mt], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) wa[ks] = wb[ks];
+      }
+    }
+    // ---- sum the eight K slices and write G tiles of 16 columns x 16*MT rows
+    __syncthreads();   // the previous group's sums have been read
+#pragma unroll
+    for (int j = 0; j < G; ++j)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) red[(wave * G * MT + j * MT + mt) * 64 + lane] = acc[j][mt];
+    __syncthreads();
+    const float *redf = reinterpret_cast<const float *>(red);
+    const uint16_t *bias = (const uint16_t *)a.bias;
+    const uint16_t *bias2 = (const uint16_t *)a.bias2;
+    const uint16_t *res = (const uint16_t *)a.residual;
+    for (int v = tid; v < G * MT * 256; v += 512) {
+      const int slot = v >> 8, rem = v & 255, ln = rem >> 2, r = rem & 3;
+      const int j = slot / MT, mt = slot - j * MT;
+      const int tile = g0 + j;
+      const int n = tile * 16 + 4 * (ln >> 4) + r, m = mt * 16 + (ln & 15);
+      if (tile >= tiles || n >= a.N || m >= a.M) continue;
+      float x = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) x += redf[(w * G * MT + slot) * 256 + rem];
+      if (partial) {
+        partial[((int64_t)split * a.M + m) * a.N + n] = x;
+        continue;
+      }
+      if (a.glu) {   // columns (n, n+1) are a (gate, up) pair
+        if (r & 1) continue;
+        float u = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) u += redf[(w * G * MT + slot) * 256 + rem + 1];
+        x += bias ? bf16_bits_to_f32(bias[n]) : 0.f;
+        u += bias ? bf16_bits_to_f32(bias[n + 1]) : 0.f;
+        ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + (n >> 1)] = f32_to_bf16_bits(glu_bf16(a.act, x, u));
+        continue;
+      }
+      x += (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
+      if (a.act >= 0 && n >= a.act_from) x = act_eval(a.act, x);
+      if (res) x += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
+      if (n < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + n] = f32_to_bf16_bits(x);
+      else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (n - a.n_split)] = f32_to_bf16_bits(x);
+    }
+  }
+}
+
+template <int MT, int KS, int G> static int launch_mfma_stream_cfg(hipStream_t st, const LinearArgs &a, int splits) {
+  const int tiles = (a.N + 15) / 16;
+  const int groups = (tiles + G - 1) / G;
+  int blocks_x = kNumCU / splits;
+  if (blocks_x < 1) blocks_x = 1;
+  if (blocks_x > groups) blocks_x = groups;
+  const size_t lds = (size_t)8 * G * MT * 64 * sizeof(f32x4);
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma_stream<MT, KS, G>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  float *partial = splits > 1 ? (float *)a.splitk_ws : nullptr;
+  hipLaunchKernelGGL((k_linear_bf16_mfma_stream<MT, KS, G>), dim3(blocks_x, splits), dim3(512), lds, st, a, tiles,
+                     partial);
+  RAI_TRY(launch_check("linear_bf16_mfma_stream"));
+  if (splits > 1) {
+    const int64_t total = (int64_t)a.M * a.N;
+    const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);
+    RAI_TRY(launch_check("splitk_epilogue"));
+  }
+  return RAI_OK;
+}
+
+// False when the shape needs a K split and no (or too small a) workspace was lent.
+template <int MT, int KS> static bool mfma_stream_fits(const LinearArgs &a, int *splits) {
+  const int span = 8 * KS * 32;
+  *splits = (a.K + span - 1) / span;
+  return *splits == 1 || (a.splitk_ws && (size_t)*splits * a.M * a.N * sizeof(float) <= a.splitk_ws_bytes);
+}
+
+template <int MT, int KS> static int launch_mfma_stream(hipStream_t st, const LinearArgs &a, int splits) {
+  const int tiles = (a.N + 15) / 16;
+  const int per_block = tiles * splits / kNumCU;   // tiles per block when every CU holds one block
+  if (per_block >= 4) return launch_mfma_stream_cfg<MT, KS, 4>(st, a, splits);
+  if (per_block >= 2) return launch_mfma_stream_cfg<MT, KS, 2>(st, a, splits);
+  return launch_mfma_stream_cfg<MT, KS, 1>(st, a, splits);
+}
+
 int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
   RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
@@ -430,6 +591,14 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.lda % 8 == 0 && a.ldw % 8 == 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0,
               RAI_ERR_BAD_STRIDE, "linear mfma: operands must be 16-byte aligned with row strides multiple of 8");
   static const bool no_skinny = getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr;
+  static const bool no_stream = getenv("RAI_HIP_NO_MFMA_STREAM") != nullptr;
+  if (a.M <= 64 && !no_skinny && !no_stream) {
+    int splits = 1;
+    if (a.M <= 16 && mfma_stream_fits<1, 8>(a, &splits)) return launch_mfma_stream<1, 8>(st, a, splits);
+    if (a.M > 16 && a.M <= 32 && mfma_stream_fits<2, 8>(a, &splits)) return launch_mfma_stream<2, 8>(st, a, splits);
+    if (a.M > 32 && a.M <= 48 && mfma_stream_fits<3, 4>(a, &splits)) return launch_mfma_stream<3, 4>(st, a, splits);
+    if (a.M > 48 && mfma_stream_fits<4, 4>(a, &splits)) return launch_mfma_stream<4, 4>(st, a, splits);
+  }
   if (a.M <= 64 && !no_skinny) {
     const int mt = (a.M + 15) / 16;
     if (mt == 1) return launch_mfma_skinny<1>(st, a);
