@@ -54,7 +54,9 @@ typedef enum rai_hip_status {
   RAI_ERR_HIP = -5,
   RAI_ERR_BAD_ARG = -6,
   RAI_ERR_UNSUPPORTED = -7, /* rai-core/src/error.rs:10-14 Error::Unimplemented */
-  RAI_ERR_INDEX = -8        /* gather index out of range: never silent */
+  RAI_ERR_INDEX = -8,       /* gather index out of range: never silent */
+  RAI_ERR_PARAM_NOT_FOUND = -9, /* rai-core/src/error.rs Error::ParamNotFound (nn.rs:198-204) */
+  RAI_ERR_IO = -10          /* unreadable or malformed checkpoint file */
 } rai_hip_status;
 
 /* Strided tensor view over device memory (the storage half of
@@ -308,6 +310,19 @@ int rai_hip_decoder_destroy(rai_hip_decoder *dec);
  * phi2.rs:307-313): copy one named parameter from host memory, e.g.
  * "model.layers.3.self_attn.q_proj.weight".  `data` is row-major in the model dtype. */
 int rai_hip_decoder_load_param(rai_hip_decoder *dec, const char *name, const void *host_data, size_t bytes);
+/* Module::update_by_safetensors (rai-core/src/nn.rs:39-55): reads every file, collects its tensors by
+ * name (a later file wins on a duplicate), then looks every parameter of the model up by name, converts
+ * it to the model dtype (nn.rs:198-201) and stores it.  A parameter that no file holds fails with
+ * RAI_ERR_PARAM_NOT_FOUND naming it; tensors the model does not have are ignored.  Source dtypes F32,
+ * F16, BF16 and F64 (the floating ones of hlops/from_safetensor.rs:51-91); anything else is
+ * RAI_ERR_BAD_DTYPE, a malformed file RAI_ERR_IO. */
+int rai_hip_decoder_load_safetensors(rai_hip_decoder *dec, const char *const *paths, int32_t n_paths);
+/* ext::hf::load_safetensors (rai/src/lib.rs:17-42) without the hub download: the distinct shard files
+ * named by the "weight_map" of a model.safetensors.index.json, resolved against the directory of the
+ * index file and written to buf separated by '\n'.  A missing or non-object weight_map is RAI_ERR_IO. */
+int rai_hip_safetensors_index_files(const char *index_json_path, char *buf, size_t buflen, int32_t *n_files);
+/* Dtype of the decoder's parameters (RAI_F32 or RAI_BF16). */
+int rai_hip_decoder_dtype(rai_hip_decoder *dec, int32_t *dtype);
 /* Number of parameter names the architecture expects / i-th name (for loaders). */
 int rai_hip_decoder_param_count(rai_hip_decoder *dec, int32_t *count);
 int rai_hip_decoder_param_name(rai_hip_decoder *dec, int32_t i, char *buf, size_t buflen, int64_t *numel);

@@ -113,6 +113,9 @@ PROTOTYPES = {
     "rai_hip_decoder_create": [C.c_int, C.POINTER(DecoderConfig), C.POINTER(_vp)],
     "rai_hip_decoder_destroy": [_vp],
     "rai_hip_decoder_load_param": [_vp, C.c_char_p, _vp, C.c_size_t],
+    "rai_hip_decoder_load_safetensors": [_vp, C.POINTER(C.c_char_p), _i32],
+    "rai_hip_safetensors_index_files": [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(_i32)],
+    "rai_hip_decoder_dtype": [_vp, C.POINTER(_i32)],
     "rai_hip_decoder_param_count": [_vp, C.POINTER(_i32)],
     "rai_hip_decoder_param_name": [_vp, _i32, C.c_char_p, C.c_size_t, C.POINTER(_i64)],
     "rai_hip_decoder_forward": [_vp, C.POINTER(C.c_uint32), _i32, _i32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)],

@@ -956,6 +956,12 @@ int rai_hip_decoder_load_param(rai_hip_decoder *d, const char *name, const void 
   return RAI_OK;
 }
 
+int rai_hip_decoder_dtype(rai_hip_decoder *d, int32_t *dtype) {
+  RAI_REQUIRE(d && dtype, RAI_ERR_BAD_ARG, "null argument");
+  *dtype = d->cfg.dtype;
+  return RAI_OK;
+}
+
 int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *d) {
   RAI_REQUIRE(d, RAI_ERR_BAD_ARG, "decoder is null");
   hipStream_t st = stream_of(d->dev);

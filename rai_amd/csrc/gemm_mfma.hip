@@ -463,6 +463,9 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
     const uint16_t *p = wbase + (int64_t)n * a.ldw;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) w[ks] = *reinterpret_cast<const bf16x8 *>(p + koff[ks]);
+    // keep the whole tile's loads together and ahead of the multiplies that follow: left alone,
+    // the scheduler sinks each load to just before its use and the prefetch distance collapses
+    __builtin_amdgcn_sched_barrier(0);
   };
   const int stride = gridDim.x * G;
   int g0 = blockIdx.x * G;
@@ -482,6 +485,7 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ks], xf[mt][ks], acc[j][mt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
       if (G > 1) {
         load_tile(wa, j + 2 < G ? g0 + j + 2 : g0 + stride);
 #pragma unroll
@@ -490,6 +494,7 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
           for (int mt = 0; mt < MT; ++mt)
             acc[j + 1 < G ? j + 1 : j][mt] =
                 __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[ks], xf[mt][ks], acc[j + 1 < G ? j + 1 : j][mt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       } else {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) wa[ks] = wb[ks];

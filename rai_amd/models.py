@@ -73,6 +73,12 @@ class Decoder:
         a = np.ascontiguousarray(storage)
         call("rai_hip_decoder_load_param", self._h, name.encode(), a.ctypes.data_as(C.c_void_p), a.nbytes)
 
+    def load_safetensors(self, paths):
+        """Module::update_by_safetensors (rai-core/src/nn.rs:39-55): every parameter by name from the given files."""
+        paths = [paths] if isinstance(paths, (str, bytes)) or hasattr(paths, "__fspath__") else list(paths)
+        arr = (C.c_char_p * len(paths))(*[str(p).encode() for p in paths])
+        call("rai_hip_decoder_load_safetensors", self._h, arr, len(paths))
+
     def forward(self, ids, want_logits=True):
         """Model::fwd: ids [B, S] u32 -> (logits [B, vocab] f32, greedy tokens [B] u32)."""
         ids = np.ascontiguousarray(ids, dtype=np.uint32)
@@ -113,3 +119,13 @@ class Decoder:
         us, by = C.c_float(0), C.c_double(0)
         call("rai_hip_decoder_time_decode_linear", self._h, int(sweeps), C.byref(us), C.byref(by))
         return us.value, by.value
+
+
+def safetensors_index_files(index_json_path):
+    """The shard files a model.safetensors.index.json names (rai/src/lib.rs:17-42, without the hub download)."""
+    buf = C.create_string_buffer(1 << 16)
+    n = C.c_int32(0)
+    call("rai_hip_safetensors_index_files", str(index_json_path).encode(), buf, len(buf), C.byref(n))
+    files = buf.value.decode().split("\n") if n.value else []
+    assert len(files) == n.value
+    return files

@@ -109,3 +109,26 @@ def test_bench_refuses_multi_gpu():
     import sys
     r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_safetensors_index_files_host_only(tmp_path):
+    """ext::hf::load_safetensors (rai/src/lib.rs:17-42) minus the download: distinct weight_map values,
+    resolved against the index's directory; missing / invalid weight_map is an error.  No GPU involved."""
+    import json
+
+    from rai_amd._lib import RaiHipError
+    from rai_amd.models import safetensors_index_files
+    idx = tmp_path / "model.safetensors.index.json"
+    idx.write_text(json.dumps({"metadata": {}, "weight_map": {"a.weight": "s2.safetensors", "b.weight": "s1.safetensors",
+                                                               "c.weight": "s2.safetensors", "odd": 3}}))
+    assert safetensors_index_files(idx) == [str(tmp_path / "s1.safetensors"), str(tmp_path / "s2.safetensors")]
+    idx.write_text(json.dumps({"metadata": {}}))
+    with pytest.raises(RaiHipError) as e:
+        safetensors_index_files(idx)
+    assert e.value.status == -10 and "weight_map" in str(e.value)
+    idx.write_text(json.dumps({"weight_map": ["x"]}))
+    with pytest.raises(RaiHipError):
+        safetensors_index_files(idx)
+    idx.write_text("{not json")
+    with pytest.raises(RaiHipError):
+        safetensors_index_files(idx)
