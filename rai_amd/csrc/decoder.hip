@@ -184,9 +184,37 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
   const T *x = logits + (int64_t)b * n;
   float bv = -INFINITY;
   uint32_t bi = 0xffffffffu;
-  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
-    float v = (float)Scalar<T>::load(x + i);
-    if (v > bv || (bi == 0xffffffffu && v == v)) { bv = v; bi = (uint32_t)i; }
+  constexpr int VEC = 16 / sizeof(T);
+  if (n % VEC == 0 && ((uintptr_t)x & 15) == 0) {
+    // 16-byte loads, four per thread in flight; every thread still visits its elements in
+    // increasing index order, so the first maximum wins exactly as in the scalar scan
+    struct alignas(16) Pack { T v[VEC]; };
+    const Pack *xp = reinterpret_cast<const Pack *>(x);
+    const int64_t chunks = n / VEC;
+    for (int64_t c0 = threadIdx.x; c0 < chunks; c0 += (int64_t)blockDim.x * 4) {
+      Pack pk[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + (int64_t)u * blockDim.x;
+        if (c < chunks) pk[u] = xp[c];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + (int64_t)u * blockDim.x;
+        if (c < chunks) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float v = (float)Scalar<T>::load(&pk[u].v[j]);
+            if (v > bv || (bi == 0xffffffffu && v == v)) { bv = v; bi = (uint32_t)(c * VEC + j); }
+          }
+        }
+      }
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+      float v = (float)Scalar<T>::load(x + i);
+      if (v > bv || (bi == 0xffffffffu && v == v)) { bv = v; bi = (uint32_t)i; }
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {

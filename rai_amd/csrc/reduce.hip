@@ -248,12 +248,42 @@ k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int6
   C bv = C(0);
   uint32_t bi = 0xffffffffu;
   bool have = false;
-  for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
-    C v = Scalar<T>::load(x + i * axis_stride);
-    if (!have || better<C, IS_MAX>(v, (uint32_t)i, bv, bi)) {
-      bv = v;
-      bi = (uint32_t)i;
-      have = true;
+  constexpr int VEC = 16 / sizeof(T);
+  if (axis_stride == 1 && lo % VEC == 0 && ((uintptr_t)(x + lo) & 15) == 0) {
+    // unit-stride axis: 16-byte loads, four per thread in flight, elements still visited in index order
+    struct alignas(16) Pack { T v[VEC]; };
+    const Pack *xp = reinterpret_cast<const Pack *>(x + lo);
+    const int64_t chunks = (hi - lo) / VEC;
+    for (int64_t c0 = threadIdx.x; c0 < chunks; c0 += (int64_t)blockDim.x * 4) {
+      Pack pk[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (c0 + (int64_t)u * blockDim.x < chunks) pk[u] = xp[c0 + (int64_t)u * blockDim.x];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + (int64_t)u * blockDim.x;
+        if (c < chunks) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const C v = Scalar<T>::load(&pk[u].v[j]);
+            const uint32_t i = (uint32_t)(lo + c * VEC + j);
+            if (!have || better<C, IS_MAX>(v, i, bv, bi)) { bv = v; bi = i; have = true; }
+          }
+        }
+      }
+    }
+    for (int64_t i = lo + chunks * VEC + threadIdx.x; i < hi; i += blockDim.x) {  // tail shorter than one pack
+      C v = Scalar<T>::load(x + i);
+      if (!have || better<C, IS_MAX>(v, (uint32_t)i, bv, bi)) { bv = v; bi = (uint32_t)i; have = true; }
+    }
+  } else {
+    for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+      C v = Scalar<T>::load(x + i * axis_stride);
+      if (!have || better<C, IS_MAX>(v, (uint32_t)i, bv, bi)) {
+        bv = v;
+        bi = (uint32_t)i;
+        have = true;
+      }
     }
   }
   // Lanes that saw nothing carry index 0xffffffff and a NaN so they never win.
@@ -274,9 +304,10 @@ k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int6
   }
 }
 
-template <typename C, bool IS_MAX>
+template <typename T, typename C, bool IS_MAX>
 __global__ void __launch_bounds__(64)
-k_arg_row_final(const C *pval, const uint32_t *pidx, int64_t rows, int splits, uint32_t *out) {
+k_arg_row_final(const C *pval, const uint32_t *pidx, int64_t rows, int splits, uint32_t *out, const T *in,
+                int64_t row_stride) {
   int64_t row = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (row >= rows) return;
   C bv = pval[row * splits];
@@ -287,19 +318,9 @@ k_arg_row_final(const C *pval, const uint32_t *pidx, int64_t rows, int splits, u
     if (better<C, IS_MAX>(v, i, bv, bi)) { bv = v; bi = i; }
   }
   // all-NaN row: every candidate is NaN and the smallest index (0) wins already;
-  // NaN at index 0 with finite values elsewhere must still win -> checked by caller kernel
-  out[row] = bi == 0xffffffffu ? 0u : bi;
-}
-
-// NaN at element 0 wins in the reference's sequential scan.
-template <typename T>
-__global__ void __launch_bounds__(256)
-k_arg_nan0_fix(const T *in, int64_t rows, int64_t row_stride, uint32_t *out) {
-  typedef typename Scalar<T>::compute C;
-  int64_t row = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-  if (row >= rows) return;
-  C v = Scalar<T>::load(in + row * row_stride);
-  if (v != v) out[row] = 0;
+  // NaN at element 0 wins in the reference's sequential scan even with finite values elsewhere
+  const typename Scalar<T>::compute first = Scalar<T>::load(in + row * row_stride);
+  out[row] = (bi == 0xffffffffu || first != first) ? 0u : bi;
 }
 
 // Generic strided variant: one thread per output, sequential scan like the reference.
@@ -483,15 +504,13 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
     RAI_TRY(launch_check("arg_partial"));
     int fgrid = (int)((rows + 63) / 64);
     if (in->dtype == RAI_F64)
-      hipLaunchKernelGGL((k_arg_row_final<double, IS_MAX>), dim3(fgrid), dim3(64), 0, st, pd, pi, rows, splits, o);
+      hipLaunchKernelGGL((k_arg_row_final<double, double, IS_MAX>), dim3(fgrid), dim3(64), 0, st, pd, pi, rows, splits, o,
+                         (const double *)base_ptr(in), row_stride);
     else
-      hipLaunchKernelGGL((k_arg_row_final<float, IS_MAX>), dim3(fgrid), dim3(64), 0, st, pf, pi, rows, splits, o);
-    RAI_TRY(launch_check("arg_final"));
-    int ngrid = (int)((rows + 255) / 256);
-    RAI_DISPATCH_FLOAT(in->dtype, T,
-                       hipLaunchKernelGGL((k_arg_nan0_fix<T>), dim3(ngrid), dim3(256), 0, st, (const T *)base_ptr(in),
-                                          rows, row_stride, o));
-    return launch_check("arg_nan0");
+      RAI_DISPATCH_FLOAT(in->dtype, T,
+                         hipLaunchKernelGGL((k_arg_row_final<T, float, IS_MAX>), dim3(fgrid), dim3(64), 0, st, pf, pi,
+                                            rows, splits, o, (const T *)base_ptr(in), row_stride));
+    return launch_check("arg_final");
   }
   int64_t blocks = (s.n_out + 255) / 256;
   int grid = (int)(blocks < kNumCU * 16 ? blocks : kNumCU * 16);
