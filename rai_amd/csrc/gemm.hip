@@ -634,6 +634,24 @@ int launch_linear_bf16(hipStream_t st, const LinearArgs &a) {
   return launch_linear_bf16_mfma(st, a);
 }
 
+// dst[N][K] = src[K][N]^T through a 64x64 LDS tile: both the reads (rows of src) and the
+// writes (rows of dst) are contiguous runs of 64 elements.
+template <typename T>
+__global__ void __launch_bounds__(256) k_transpose_2d(T *dst, const T *src, int K, int N) {
+  __shared__ T tile[64][64 + 2];
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int k = k0 + i, n = n0 + tx;
+    if (k < K && n < N) tile[i][tx] = src[(int64_t)k * N + n];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int n = n0 + i, k = k0 + tx;
+    if (n < N && k < K) dst[(int64_t)n * K + k] = tile[tx][i];
+  }
+}
+
 int launch_linear_f32(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem");
   RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear f32: no fused norm");
@@ -733,13 +751,15 @@ int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, co
     if (b_shared) {
       void *tmp = nullptr;
       RAI_TRY(rai_hip_alloc(dev, (size_t)N * K * dtype_size(b->dtype), &tmp));
-      rai_hip_tensor src;  // B^T as a strided view of B: [N, K] with strides (1, N)
-      memset(&src, 0, sizeof(src));
-      src.data = b->data; src.dtype = b->dtype; src.offset = b->offset; src.rank = 2;
-      src.shape[0] = N; src.shape[1] = K; src.stride[0] = 1; src.stride[1] = N;
-      rai_hip_tensor bt = src;  // contiguous [N, K]
-      bt.data = tmp; bt.offset = 0; bt.stride[0] = K; bt.stride[1] = 1;
-      int rc = rai_hip_copy(dev, &src, &bt);
+      hipStream_t tst = stream_of(dev);
+      const dim3 tgrid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
+      if (b->dtype == RAI_BF16)
+        hipLaunchKernelGGL(k_transpose_2d<uint16_t>, tgrid, dim3(256), 0, tst, (uint16_t *)tmp,
+                           (const uint16_t *)base_ptr(b), (int)K, (int)N);
+      else
+        hipLaunchKernelGGL(k_transpose_2d<float>, tgrid, dim3(256), 0, tst, (float *)tmp, (const float *)base_ptr(b),
+                           (int)K, (int)N);
+      int rc = launch_check("transpose_2d");
       if (rc == RAI_OK) {
         rai_hip_tensor b2 = *b;  // [.., K, N] view of the transposed copy: strides (1, K), batch strides 0
         b2.data = tmp; b2.offset = 0;

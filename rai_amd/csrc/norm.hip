@@ -165,6 +165,37 @@ __global__ void __launch_bounds__(256) k_rope(T *out, const T *x, const TT *cos_
   }
 }
 
+// Same operation, one thread per 16 bytes of a row: requires unit inner stride, D, rot and
+// rot/2 multiples of the pack width, 16-byte aligned rows, and fewer than 2^31 packs (all
+// index arithmetic in 32 bits; the per-element form spends most of its time in 64-bit
+// divisions).
+template <typename T, typename TT>
+__global__ void __launch_bounds__(256) k_rope_vec(T *out, const T *x, const TT *cos_t, const TT *sin_t, RopeArgs a) {
+  constexpr int VEC = 16 / sizeof(T);
+  struct alignas(16) Pack { T v[VEC]; };
+  const uint32_t cpr = (uint32_t)(a.D / VEC), S = (uint32_t)a.S, H = (uint32_t)a.H;
+  const uint32_t total = (uint32_t)(a.B * a.H * a.S) * cpr;
+  const uint32_t rot = (uint32_t)a.rot, half = (uint32_t)a.half;
+  for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+    const uint32_t row = idx / cpr, d = (idx - row * cpr) * VEC;
+    const uint32_t s = row % S, r2 = row / S, h = r2 % H, b = r2 / H;
+    const T *xp = x + (int64_t)b * a.xs[0] + (int64_t)h * a.xs[1] + (int64_t)s * a.xs[2];
+    Pack v = *reinterpret_cast<const Pack *>(xp + d);
+    if (d < rot) {
+      const Pack o = *reinterpret_cast<const Pack *>(xp + (d < half ? d + half : d - half));
+      const int64_t trow = (a.offset + s) * a.tab_row_stride + d;
+      const float sign = d < half ? -1.f : 1.f;  // rotate_half = cat(-x2, x1)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float c = (float)Scalar<TT>::load(cos_t + trow + j), sn = (float)Scalar<TT>::load(sin_t + trow + j);
+        const float r = (float)Scalar<T>::load(&v.v[j]) * c + sign * (float)Scalar<T>::load(&o.v[j]) * sn;
+        Scalar<T>::store(&v.v[j], (typename Scalar<T>::compute)r);
+      }
+    }
+    *reinterpret_cast<Pack *>(out + (int64_t)row * a.D + d) = v;
+  }
+}
+
 template <typename TT>
 __global__ void __launch_bounds__(256)
 k_rope_tables(TT *cos_t, TT *sin_t, int64_t max_pos, int rot, double theta, int f64_powf) {
@@ -296,15 +327,29 @@ int rai_hip_rope(int dev, const rai_hip_tensor *x, const rai_hip_tensor *cos_t, 
   a.B = x->shape[0]; a.H = x->shape[1]; a.S = S; a.D = D;
   for (int i = 0; i < 4; ++i) a.xs[i] = x->stride[i];
   a.rot = rot_dim; a.half = rot_dim / 2; a.offset = offset; a.tab_row_stride = cos_t->stride[0];
-  int64_t blocks = (numel(out) + 255) / 256;
+  const int vec = (int)(16 / dtype_size(x->dtype));
+  const bool vec_ok = x->stride[3] == 1 && D % vec == 0 && rot_dim % vec == 0 && (rot_dim / 2) % vec == 0 &&
+                      x->stride[0] % vec == 0 && x->stride[1] % vec == 0 && x->stride[2] % vec == 0 &&
+                      (uintptr_t)base_ptr(x) % 16 == 0 && (uintptr_t)base_ptr(out) % 16 == 0 &&
+                      numel(out) / vec < (int64_t)1 << 31;
+  int64_t blocks = ((vec_ok ? numel(out) / vec : numel(out)) + 255) / 256;
   int grid = (int)(blocks < kNumCU * 32 ? blocks : kNumCU * 32);
-#define ROPE_LAUNCH(T, TT)                                                                                   \
+#define ROPE_LAUNCH(T, TT)                                                                                       \
+  do {                                                                                                           \
+    if (vec_ok)                                                                                                  \
+      hipLaunchKernelGGL((k_rope_vec<T, TT>), dim3(grid), dim3(256), 0, st, (T *)base_ptr(out),                  \
+                         (const T *)base_ptr(x), (const TT *)base_ptr(cos_t), (const TT *)base_ptr(sin_t), a);   \
+    else                                                                                                         \
+      ROPE_LAUNCH_SCALAR(T, TT);                                                                                 \
+  } while (0)
+#define ROPE_LAUNCH_SCALAR(T, TT)                                                                                   \
   hipLaunchKernelGGL((k_rope<T, TT>), dim3(grid), dim3(256), 0, st, (T *)base_ptr(out), (const T *)base_ptr(x), \
                      (const TT *)base_ptr(cos_t), (const TT *)base_ptr(sin_t), a)
   if (x->dtype == RAI_F32) ROPE_LAUNCH(float, float);
   else if (x->dtype == RAI_BF16) { if (cos_t->dtype == RAI_F32) ROPE_LAUNCH(bf16_raw, float); else ROPE_LAUNCH(bf16_raw, bf16_raw); }
   else { if (cos_t->dtype == RAI_F32) ROPE_LAUNCH(f16_raw, float); else ROPE_LAUNCH(f16_raw, f16_raw); }
 #undef ROPE_LAUNCH
+#undef ROPE_LAUNCH_SCALAR
   return launch_check("rope");
 }
 
