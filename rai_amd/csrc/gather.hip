@@ -14,6 +14,38 @@ __global__ void __launch_bounds__(256)
 k_index_select_vec(Bytes16 *out, const Bytes16 *in, const IT *index, int64_t index_stride, int64_t outer, int64_t L,
                    int64_t D, int64_t inner_packs, unsigned long long *errors) {
   const int64_t total = outer * L * inner_packs;
+  if (total < ((int64_t)1 << 31)) {
+    // 32-bit index arithmetic, four packs per thread with their index and data loads batched
+    const uint32_t tot = (uint32_t)total, ipk = (uint32_t)inner_packs, Lu = (uint32_t)L;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t p0 = blockIdx.x * blockDim.x + threadIdx.x; p0 < tot; p0 += stride * 4) {
+      uint32_t ip[4], o[4];
+      int64_t id[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t p = p0 + u * stride;
+        const uint32_t row = (p < tot ? p : p0) / ipk;
+        ip[u] = (p < tot ? p : p0) - row * ipk;
+        o[u] = row / Lu;
+        id[u] = (int64_t)index[(int64_t)(row - o[u] * Lu) * index_stride];
+      }
+      Bytes16 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        v[u] = Bytes16{{0u, 0u, 0u, 0u}};
+        if (id[u] >= 0 && id[u] < D) v[u] = in[((int64_t)o[u] * D + id[u]) * inner_packs + ip[u]];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t p = p0 + u * stride;
+        if (p < tot) {
+          if (!(id[u] >= 0 && id[u] < D) && ip[u] == 0) atomicAdd(errors, 1ull);
+          out[p] = v[u];
+        }
+      }
+    }
+    return;
+  }
   for (int64_t p = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; p < total; p += (int64_t)gridDim.x * blockDim.x) {
     int64_t row = p / inner_packs;
     int64_t ip = p - row * inner_packs;
@@ -106,8 +138,8 @@ extern "C" int rai_hip_index_select(int dev, const rai_hip_tensor *in, const rai
   if (vec) {
     int64_t inner_packs = inner * es / 16;
     int64_t work = outer * L * inner_packs;
-    int64_t blocks = (work + 255) / 256;
-    int grid = (int)(blocks < kNumCU * 32 ? blocks : kNumCU * 32);
+    int64_t blocks = (work / 4 + 255) / 256;   // four packs per thread
+    int grid = (int)(blocks < kNumCU * 32 ? (blocks < 1 ? 1 : blocks) : kNumCU * 32);
 #define ISV(IT)                                                                                                   \
   hipLaunchKernelGGL((k_index_select_vec<IT>), dim3(grid), dim3(256), 0, st, (Bytes16 *)base_ptr(out),            \
                      (const Bytes16 *)base_ptr(in), (const IT *)base_ptr(index), index->stride[0], outer, L, D,   \
