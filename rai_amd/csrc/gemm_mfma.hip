@@ -14,6 +14,8 @@
 //   - epilogue through LDS: every wave stages 32 x (BN/2) accumulators at a time
 //     and writes 16-byte rows with bias / activation / residual applied (or raw
 //     f32 partial sums when K is split over several blocks).
+#include <cstring>
+
 #include "gemm.h"
 
 namespace rai {
@@ -25,116 +27,68 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kXcds = 8;
 
+// Tile order inside an XCD's run: bands of kGroupM tile rows swept across all tile columns, so the
+// ~100 tiles that are resident on an XCD at any moment form a block of about kGroupM x 12 tiles and
+// share their A and B panels through that XCD's L2 (a column-by-column order re-reads all of A from
+// memory for every tile column).
+constexpr int kGroupM = 8;
+__device__ __forceinline__ void tile_coords(int tile, int tiles_m, int tiles_n, int *tile_m, int *tile_n) {
+  const int band = tile / (kGroupM * tiles_n);
+  const int first_m = band * kGroupM;
+  const int height = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+  const int in_band = tile - band * kGroupM * tiles_n;
+  *tile_m = first_m + in_band % height;
+  *tile_n = in_band / height;
+}
+
 __device__ __forceinline__ int xcd_remap(int bid, int total) {
   // blocks bid, bid+8, bid+16, ... run on the same XCD; give them consecutive tiles
   const int per = (total + kXcds - 1) / kXcds;
   return (bid % kXcds) * per + bid / kXcds;
 }
 
-template <int BM, int BN, int BK>
-__global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits, int k_per_split, float *partial) {
-  constexpr int PITCH = BK + 8;
+// LDS a tile kernel needs: two stages of A and B tiles, or the epilogue staging area if that is larger.
+template <int BM, int BN, int PITCH> constexpr int gemm_lds_bytes() {
+  constexpr int tiles = 2 * (BM + BN) * PITCH * 2, staging = 4 * 32 * (BN / 2 + 4) * 4;
+  return tiles > staging ? tiles : staging;
+}
+
+// Applies activation `act` to the elements of x[8] whose column n + e is >= from.  The switch on the
+// (block-uniform) activation sits outside the element loop, so only one activation's code runs.
+__device__ __forceinline__ void act8(int act, float (&x)[8], int n, int from) {
+#define RAI_ACT_CASE(K)                                     \
+  case K:                                                   \
+    _Pragma("unroll") for (int e = 0; e < 8; ++e)           \
+      if (n + e >= from) x[e] = act_eval(K, x[e]);          \
+    break;
+  switch (act) {
+    RAI_ACT_CASE(RAI_UN_GELU)
+    RAI_ACT_CASE(RAI_UN_NEW_GELU)
+    RAI_ACT_CASE(RAI_UN_SILU)
+    RAI_ACT_CASE(RAI_UN_RELU)
+    RAI_ACT_CASE(RAI_UN_TANH)
+    default: break;
+  }
+#undef RAI_ACT_CASE
+}
+__device__ __forceinline__ void unpack8(const u32x4 &p, float (&f)[8]) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = bf16_bits_to_f32((uint16_t)(p[e >> 1] >> (16 * (e & 1))));
+}
+
+// Tile epilogue shared by the tile kernels: every wave stages 32 x WN accumulators at a time in
+// LDS (the tile buffers are free by then) and writes 16-byte rows with bias / activation /
+// residual applied, or raw f32 partial sums when K is split over several blocks.
+template <int BM, int BN, int LDS_BYTES>
+__device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (&acc)[BM / 64][BN / 64], uint16_t *lds,
+                                                   int m0, int n0, int wave, int lane, int split, float *partial) {
   constexpr int WM = BM / 2, WN = BN / 2;
   constexpr int MT = WM / 32, NT = WN / 32;
-  constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
-  constexpr int A_CH = BM * CPR / 256;      // chunks per thread
-  constexpr int B_CH = BN * CPR / 256;
   constexpr int EP = WN + 4;                // epilogue staging pitch (floats)
-  static_assert(A_CH >= 1 && B_CH >= 1, "tile too small for 256 threads");
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  uint16_t *As = lds;                       // [2][BM][PITCH]
-  uint16_t *Bs = lds + 2 * BM * PITCH;      // [2][BN][PITCH]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
-  const int total = tiles_m * tiles_n;
-  const int tile = xcd_remap(blockIdx.x, total);
-  if (tile >= total) return;
-  const int tile_n = tile / tiles_m, tile_m = tile % tiles_m;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int split = blockIdx.y;
-  const int k_begin = split * k_per_split;
-  const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
-  const int KT = (k_end - k_begin) / BK;
-
-  // per-thread source pointers (rows clamped into range; results of clamped rows are never stored)
-  const uint16_t *ga[A_CH], *gb[B_CH];
-  int sa[A_CH], sb[B_CH];
-#pragma unroll
-  for (int i = 0; i < A_CH; ++i) {
-    const int c = tid + i * 256, row = c / CPR, kc = (c % CPR) * 8;
-    int m = m0 + row;
-    m = m < a.M ? m : a.M - 1;
-    ga[i] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + kc;
-    sa[i] = row * PITCH + kc;
-  }
-#pragma unroll
-  for (int i = 0; i < B_CH; ++i) {
-    const int c = tid + i * 256, row = c / CPR, kc = (c % CPR) * 8;
-    int n = n0 + row;
-    n = n < a.N ? n : a.N - 1;
-    gb[i] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + kc;
-    sb[i] = row * PITCH + kc;
-  }
-
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  u32x4 ra[A_CH], rb[B_CH];
-#pragma unroll
-  for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(ga[i]);
-#pragma unroll
-  for (int i = 0; i < B_CH; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(gb[i]);
-#pragma unroll
-  for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4 *>(As + sa[i]) = ra[i];
-#pragma unroll
-  for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u32x4 *>(Bs + sb[i]) = rb[i];
-  __syncthreads();
-
-  const int frag = (lane & 31) * PITCH + (lane >> 5) * 8;
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    const bool more = kt + 1 < KT;
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(ga[i] + (kt + 1) * BK);
-#pragma unroll
-      for (int i = 0; i < B_CH; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(gb[i] + (kt + 1) * BK);
-    }
-    const uint16_t *as = As + buf * BM * PITCH + wm * WM * PITCH + frag;
-    const uint16_t *bs = Bs + buf * BN * PITCH + wn * WN * PITCH + frag;
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8 fa[MT], fb[NT];
-#pragma unroll
-      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + ks * 16);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + ks * 16);
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) {
-      uint16_t *ad = As + (buf ^ 1) * BM * PITCH, *bd = Bs + (buf ^ 1) * BN * PITCH;
-#pragma unroll
-      for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4 *>(ad + sa[i]) = ra[i];
-#pragma unroll
-      for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u32x4 *>(bd + sb[i]) = rb[i];
-    }
-    __syncthreads();
-  }
-
   // ---- epilogue: stage 32 x WN accumulators per wave in LDS, write 8 columns per lane
   float *stage = reinterpret_cast<float *>(lds) + wave * 32 * EP;
-  static_assert(4 * 32 * EP * 4 <= 2 * (BM + BN) * PITCH * 2, "epilogue staging does not fit the tile buffers");
+  static_assert(4 * 32 * EP * 4 <= LDS_BYTES, "epilogue staging does not fit the tile buffers");
   constexpr int CG = WN / 8;                 // 8-column groups per staged row
   constexpr int ITEMS = 32 * CG / 64;        // per lane
   const uint16_t *bias = (const uint16_t *)a.bias;
@@ -168,34 +122,77 @@ __global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits
           *reinterpret_cast<f32x4 *>(p) = v0;
           if (n + 4 < a.N) *reinterpret_cast<f32x4 *>(p + 4) = v1;
         } else {
-          for (int e = 0; e < 8 && n + e < a.N; ++e) p[e] = v[e];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < a.N) p[e] = v[e];
         }
         continue;
       }
+      // bias values of the 8 columns: one 16-byte load when the row of columns is whole and aligned
+      const bool whole = n + 8 <= a.N;
+      float bv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bv[e] = 0.f;
+      if (bias) {
+        if (whole && ((uintptr_t)(bias + n) & 15) == 0) unpack8(*reinterpret_cast<const u32x4 *>(bias + n), bv);
+        else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < a.N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+        }
+      }
+      if (bias2) {
+        float b2[8];
+        if (whole && ((uintptr_t)(bias2 + n) & 15) == 0) {
+          unpack8(*reinterpret_cast<const u32x4 *>(bias2 + n), b2);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) bv[e] += b2[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < a.N) bv[e] += bf16_bits_to_f32(bias2[n + e]);
+        }
+      }
       if (a.glu) {  // columns n..n+7 are four (gate, up) pairs -> four outputs at column n/2
         uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
-        float gl[4];
-        for (int e = 0; e < 8; e += 2) {
-          const float g = v[e] + (bias ? bf16_bits_to_f32(bias[n + e]) : 0.f);
-          const float u = v[e + 1] + (bias ? bf16_bits_to_f32(bias[n + e + 1]) : 0.f);
-          gl[e >> 1] = glu_bf16(a.act, g, u);
+        float gr[8], ga[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          gr[e] = bf16_bits_to_f32(f32_to_bf16_bits(v[e] + bv[e]));  // gate / up rounded to bf16 as the reference does
+          ga[e] = gr[e];
         }
-        if (n + 8 <= a.N && a.ld1 % 4 == 0 && (uintptr_t)a.out1 % 8 == 0) {
+        act8(a.act, ga, 0, 0);   // evaluated on all eight; only the gates (even e) are used
+        float gl[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gl[e] = bf16_bits_to_f32(f32_to_bf16_bits(ga[2 * e])) * gr[2 * e + 1];
+        if (whole && a.ld1 % 4 == 0 && (uintptr_t)a.out1 % 8 == 0) {
           typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
           u32x2 o = {pack_bf16x2(gl[0], gl[1]), pack_bf16x2(gl[2], gl[3])};
           *reinterpret_cast<u32x2 *>(dst) = o;
         } else {
-          for (int e = 0; e < 4 && n + 2 * e + 1 < a.N; ++e) dst[e] = f32_to_bf16_bits(gl[e]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + 2 * e + 1 < a.N) dst[e] = f32_to_bf16_bits(gl[e]);
         }
         continue;
       }
+      // compile-time element indices throughout: a loop bounded by a run-time count would index v[]
+      // dynamically, which the compiler lowers to a chain of selects per access
       const int lim = a.N - n < 8 ? a.N - n : 8;
-      for (int e = 0; e < lim; ++e) {
-        const int nn = n + e;
-        float x = v[e] + (bias ? bf16_bits_to_f32(bias[nn]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[nn]) : 0.f);
-        if (a.act >= 0 && nn >= a.act_from) x = act_eval(a.act, x);
-        if (res) x += bf16_bits_to_f32(res[(int64_t)m * a.ldr + nn]);
-        v[e] = x;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += bv[e];
+      if (a.act >= 0) act8(a.act, v, n, a.act_from);
+      if (res) {
+        if (vec_out) {
+          float rv[8];
+          unpack8(*reinterpret_cast<const u32x4 *>(res + (int64_t)m * a.ldr + n), rv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += rv[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e < lim) v[e] += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n + e]);
+        }
       }
       if (vec_out) {
         u32x4 o;
@@ -207,14 +204,289 @@ __global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits
                                       : (uint16_t *)a.out2 + (int64_t)m * a.ld2 + (n - a.n_split);
         *reinterpret_cast<u32x4 *>(dst) = o;
       } else {
-        for (int e = 0; e < lim; ++e) {
-          const int nn = n + e;
-          if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = f32_to_bf16_bits(v[e]);
-          else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = f32_to_bf16_bits(v[e]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (e < lim) {
+            const int nn = n + e;
+            if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = f32_to_bf16_bits(v[e]);
+            else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = f32_to_bf16_bits(v[e]);
+          }
         }
       }
     }
   }
+}
+
+template <int BM, int BN, int BK, int SH = 0>
+__global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits, int k_per_split, float *partial) {
+  // SH == 0: rows padded by 16 bytes.  SH > 0: unpadded rows, the 16-byte chunk c of row r stored at
+  // chunk c ^ ((r >> SH) & (BK/8 - 1)), so that both the row-wise stores and the column-wise
+  // fragment reads spread over the banks.
+  constexpr int PITCH = SH ? BK : BK + 8;
+  constexpr int CMASK = BK / 8 - 1;
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int MT = WM / 32, NT = WN / 32;
+  constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
+  constexpr int A_CH = BM * CPR / 256;      // chunks per thread
+  constexpr int B_CH = BN * CPR / 256;
+  static_assert(A_CH >= 1 && B_CH >= 1, "tile too small for 256 threads");
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  uint16_t *As = lds;                       // [2][BM][PITCH]
+  uint16_t *Bs = lds + 2 * BM * PITCH;      // [2][BN][PITCH]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int tile = xcd_remap(blockIdx.x, total);
+  if (tile >= total) return;
+  int tile_m, tile_n;
+  tile_coords(tile, tiles_m, tiles_n, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int split = blockIdx.y;
+  const int k_begin = split * k_per_split;
+  const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
+  const int KT = (k_end - k_begin) / BK;
+
+  // per-thread source pointers (rows clamped into range; results of clamped rows are never stored)
+  const uint16_t *ga[A_CH], *gb[B_CH];
+  int sa[A_CH], sb[B_CH];
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) {
+    const int c = tid + i * 256, row = c / CPR, kc = (c % CPR) * 8;
+    int m = m0 + row;
+    m = m < a.M ? m : a.M - 1;
+    ga[i] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + kc;
+    sa[i] = row * PITCH + (SH ? (((kc >> 3) ^ ((row >> SH) & CMASK)) << 3) : kc);
+  }
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) {
+    const int c = tid + i * 256, row = c / CPR, kc = (c % CPR) * 8;
+    int n = n0 + row;
+    n = n < a.N ? n : a.N - 1;
+    gb[i] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + kc;
+    sb[i] = row * PITCH + (SH ? (((kc >> 3) ^ ((row >> SH) & CMASK)) << 3) : kc);
+  }
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  u32x4 ra[A_CH], rb[B_CH];
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(ga[i]);
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(gb[i]);
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4 *>(As + sa[i]) = ra[i];
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u32x4 *>(Bs + sb[i]) = rb[i];
+  __syncthreads();
+
+  const int frag = (lane & 31) * PITCH + (SH ? 0 : (lane >> 5) * 8);
+  const int rsw = SH ? (((lane & 31) >> SH) & CMASK) : 0;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    const bool more = kt + 1 < KT;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(ga[i] + (kt + 1) * BK);
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(gb[i] + (kt + 1) * BK);
+    }
+    const uint16_t *as = As + buf * BM * PITCH + wm * WM * PITCH + frag;
+    const uint16_t *bs = Bs + buf * BN * PITCH + wn * WN * PITCH + frag;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 fa[MT], fb[NT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        fa[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + (SH ? (((ks * 2 + (lane >> 5)) ^ rsw) << 3) : ks * 16));
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        fb[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + (SH ? (((ks * 2 + (lane >> 5)) ^ rsw) << 3) : ks * 16));
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      uint16_t *ad = As + (buf ^ 1) * BM * PITCH, *bd = Bs + (buf ^ 1) * BN * PITCH;
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4 *>(ad + sa[i]) = ra[i];
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) *reinterpret_cast<u32x4 *>(bd + sb[i]) = rb[i];
+    }
+    __syncthreads();
+  }
+
+  gemm_tile_epilogue<BM, BN, gemm_lds_bytes<BM, BN, PITCH>()>(a, acc, lds, m0, n0, wave, lane, split, partial);
+}
+
+// Tile kernel with direct global -> LDS loads (global_load_lds_dwordx4): no registers and no
+// ds_write instructions are spent on staging, so NS LDS stages are cheap and the loads run
+// NS-1 K tiles ahead of the multiplies, which is what hides HBM/L2 latency at 2-3 blocks per CU.
+//   - one load instruction moves 64 lanes x 16 bytes into 1 KB of consecutive LDS, i.e. 16
+//     unpadded tile rows of BK = 32 bf16; bank spreading comes from a swizzle instead of padding:
+//     the 16-byte chunk c of row r lives at chunk position c ^ ((r >> SH) & 3), applied by choosing
+//     which global chunk each lane fetches;
+//   - every wave issues (BM + BN) / 64 loads per K tile; `s_waitcnt vmcnt(loads * (NS - 3))` then a
+//     bare s_barrier make tile t+1 visible to the block (and retire stage t-1 for refilling) with one
+//     barrier per K tile.  The barrier carries no fence: a fence would wait for every outstanding
+//     LDS load, i.e. drain the pipeline.
+template <int BM, int BN, int NS, int SH>
+__global__ void __launch_bounds__(256) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
+  constexpr int BK = 32, PITCH = BK;
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int MT = WM / 32, NT = WN / 32;
+  constexpr int LA = BM / 64, LB = BN / 64;          // loads per wave per K tile (16 rows each)
+  constexpr int STAGE = (BM + BN) * BK;              // elements per stage: A rows then B rows
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int tile = xcd_remap(blockIdx.x, total);
+  if (tile >= total) return;
+  int tile_m, tile_n;
+  tile_coords(tile, tiles_m, tiles_n, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int split = blockIdx.y;
+  const int k_begin = split * k_per_split;
+  const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
+  const int KT = (k_end - k_begin) / BK;
+
+  // lane -> (row within the 16-row group, swizzled chunk)
+  const int lrow = lane >> 2;
+  const uint16_t *gpa[LA], *gpb[LB];
+#pragma unroll
+  for (int j = 0; j < LA; ++j) {
+    const int r = (wave * LA + j) * 16 + lrow;   // row within the tile
+    int m = m0 + r;
+    m = m < a.M ? m : a.M - 1;
+    gpa[j] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + (((lane & 3) ^ ((r >> SH) & 3)) << 3);
+  }
+#pragma unroll
+  for (int j = 0; j < LB; ++j) {
+    const int r = (wave * LB + j) * 16 + lrow;
+    int n = n0 + r;
+    n = n < a.N ? n : a.N - 1;
+    gpb[j] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + (((lane & 3) ^ ((r >> SH) & 3)) << 3);
+  }
+  typedef __attribute__((address_space(3))) void *lds_ptr;
+  auto issue = [&](int kt, int stage) {
+    kt = kt < KT ? kt : KT - 1;   // past the end: refetch the last tile into a stage nobody reads again
+    uint16_t *sa = lds + stage * STAGE + wave * LA * 16 * BK;
+    uint16_t *sb = lds + stage * STAGE + BM * BK + wave * LB * 16 * BK;
+#pragma unroll
+    for (int j = 0; j < LA; ++j)
+      __builtin_amdgcn_global_load_lds((const void *)(gpa[j] + kt * BK), (lds_ptr)(sa + j * 16 * BK), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < LB; ++j)
+      __builtin_amdgcn_global_load_lds((const void *)(gpb[j] + kt * BK), (lds_ptr)(sb + j * 16 * BK), 16, 0, 0);
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t) issue(t, t);
+
+  // Software pipeline of one K tile (BK = 32 = two MFMA K steps, fragment sets F0 and F1):
+  //   top:  read F1 (tile t, step 1)            | multiply F0 (tile t, step 0)
+  //   mid:  wait for tile t+1, barrier, issue the loads of tile t+NS-1, read F0 (tile t+1, step 0)
+  //                                             | multiply F1
+  // so LDS reads always run one fragment set ahead of the MFMAs, the barrier sits between two
+  // batches of multiplies that are already in the pipe, and global loads are NS-2 tiles ahead.
+  const int frow = (lane & 31) * PITCH;
+  const int rsw = ((lane & 31) >> SH) & 3;
+  const int coff0 = ((0 + (lane >> 5)) ^ rsw) << 3, coff1 = ((2 + (lane >> 5)) ^ rsw) << 3;
+  const int a_off = wm * WM * PITCH + frow, b_off = BM * BK + wn * WN * PITCH + frow;
+  bf16x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];
+#define RAI_DMA_WAIT(n)                                                                        \
+  do {                                                                                         \
+    if constexpr ((n) == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                   \
+    else if constexpr ((n) == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");              \
+    else if constexpr ((n) == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");              \
+    else if constexpr ((n) == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");              \
+    else if constexpr ((n) == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");            \
+    else if constexpr ((n) == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");            \
+    else static_assert((n) < 0, "add the vmcnt immediate for this configuration");             \
+  } while (0)
+  RAI_DMA_WAIT((LA + LB) * (NS - 2));   // tile 0 has landed (this wave's part)
+  __builtin_amdgcn_s_barrier();
+  {
+    const uint16_t *as = lds + a_off, *bs = lds + b_off;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) fa0[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + coff0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) fb0[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + coff0);
+  }
+  int cur = 0, nxt = NS - 1;
+  // A wave issues in order and an MFMA issue blocks until the matrix pipe is free, so anything placed
+  // between two batches of MFMAs runs with the pipe idle.  The LDS reads and the load issues are
+  // therefore interleaved one by one between the MFMAs of each half (sched_group_barrier patterns).
+  for (int kt = 0; kt < KT; ++kt) {
+    {
+      const uint16_t *as = lds + cur * STAGE + a_off, *bs = lds + cur * STAGE + b_off;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa1[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + coff1);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb1[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + coff1);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0[i], fb0[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int g = 0; g < MT + NT; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MT * NT / (MT + NT) > 0 ? MT * NT / (MT + NT) : 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                  // one LDS read
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    RAI_DMA_WAIT((LA + LB) * (NS - 3));  // tile kt+1 has landed; NS-3 younger tiles stay in flight
+    __builtin_amdgcn_s_barrier();
+    issue(kt + NS - 1, nxt);               // into the stage of tile kt-1, which every wave has left
+    cur = cur + 1 == NS ? 0 : cur + 1;
+    nxt = nxt + 1 == NS ? 0 : nxt + 1;
+    {
+      const uint16_t *as = lds + cur * STAGE + a_off, *bs = lds + cur * STAGE + b_off;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa0[i] = *reinterpret_cast<const bf16x8 *>(as + i * 32 * PITCH + coff0);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb0[j] = *reinterpret_cast<const bf16x8 *>(bs + j * 32 * PITCH + coff0);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1[i], fb1[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int g = 0; g < MT + NT; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global -> LDS load
+      __builtin_amdgcn_sched_group_barrier(0x008, MT * NT / (MT + NT) > 1 ? MT * NT / (MT + NT) - 1 : 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#undef RAI_DMA_WAIT
+  // the refetches issued past the end must land before the stages are reused for the epilogue
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  gemm_tile_epilogue<BM, BN, gemm_lds_bytes<BM, BN, PITCH * NS / 2>()>(a, acc, lds, m0, n0, wave, lane, split, partial);
 }
 
 // Sums the per-split partial products and applies the Linear epilogue.
@@ -244,11 +516,11 @@ __global__ void __launch_bounds__(256) k_splitk_epilogue(LinearArgs a, int split
   }
 }
 
-template <int BM, int BN, int BK> static int launch_cfg(hipStream_t st, const LinearArgs &a, int splits) {
-  constexpr size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(uint16_t);
+template <int BM, int BN, int BK, int SH = 0> static int launch_cfg(hipStream_t st, const LinearArgs &a, int splits) {
+  constexpr size_t lds = gemm_lds_bytes<BM, BN, (SH ? BK : BK + 8)>();
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma<BM, BN, BK>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma<BM, BN, BK, SH>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
@@ -262,9 +534,39 @@ template <int BM, int BN, int BK> static int launch_cfg(hipStream_t st, const Li
     k_per_split = per * BK;
     partial = (float *)a.splitk_ws;
   }
-  hipLaunchKernelGGL((k_gemm_bf16_mfma<BM, BN, BK>), dim3(grid_x, splits), dim3(256), lds, st, a, splits, k_per_split,
+  hipLaunchKernelGGL((k_gemm_bf16_mfma<BM, BN, BK, SH>), dim3(grid_x, splits), dim3(256), lds, st, a, splits, k_per_split,
                      partial);
   RAI_TRY(launch_check("gemm_bf16_mfma"));
+  if (splits > 1) {
+    int64_t total = (int64_t)a.M * a.N;
+    int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);
+    RAI_TRY(launch_check("splitk_epilogue"));
+  }
+  return RAI_OK;
+}
+
+template <int BM, int BN, int NS, int SH> static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
+  constexpr size_t lds = gemm_lds_bytes<BM, BN, 32 * NS / 2>();
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma<BM, BN, NS, SH>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  const int grid_x = ((tiles + kXcds - 1) / kXcds) * kXcds;
+  int k_per_split = a.K;
+  float *partial = nullptr;
+  if (splits > 1) {
+    const int k_tiles = a.K / 32, per = (k_tiles + splits - 1) / splits;
+    splits = (k_tiles + per - 1) / per;
+    k_per_split = per * 32;
+    partial = (float *)a.splitk_ws;
+  }
+  hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH>), dim3(grid_x, splits), dim3(256), lds, st, a, splits,
+                     k_per_split, partial);
+  RAI_TRY(launch_check("gemm_bf16_mfma_dma"));
   if (splits > 1) {
     int64_t total = (int64_t)a.M * a.N;
     int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
@@ -618,7 +920,20 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     while (splits < 8 && tiles * splits * 2 <= 2 * kNumCU && a.K / (splits * 2) >= 512) splits *= 2;
     while (splits > 1 && (size_t)splits * a.M * a.N * sizeof(float) > a.splitk_ws_bytes) splits /= 2;
   }
-  return launch_cfg<128, 128, 32>(st, a, splits);
+  // Tile choice.  The LDS-DMA kernels stream K tiles straight into LDS; the 256x128 tile halves the
+  // L2 -> LDS traffic per flop for one operand and is used once there are enough tiles of that size
+  // to give every CU at least one; smaller products keep the 128x128 tile (three blocks per CU).
+  // RAI_HIP_GEMM_TILE = "128x128" | "256x128" | "256x256" | "classic" overrides (tuning aid).
+  const char *knob = getenv("RAI_HIP_GEMM_TILE");
+  if (knob) {
+    if (!strcmp(knob, "128x128")) return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
+    if (!strcmp(knob, "256x128")) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
+    if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
+    if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
+  }
+  const int big_tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
+  if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
+  return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
 }
 
 }  // namespace rai
