@@ -11,6 +11,7 @@ struct DevState {
   int step;   // greedy steps taken by the current generate call
   int done;   // blocks of the token-selection kernel that have finished (reset by the last one)
   int fault;  // set by a grid barrier that timed out; checked by the host after a generate call
+  unsigned epoch;  // launches of the persistent decode kernel so far: makes its exchange tags unique
 };
 
 struct MegaLayer {
@@ -27,9 +28,12 @@ struct MegaArgs {
   int64_t wa_stride, wb_stride;
   int L, H, I, QD, NA, n_qkv, Hq, rot, Tmax;
   uint16_t *x;              // [H] residual stream, updated in place
-  uint16_t *qkv;            // [3 * QD]
-  uint16_t *act_buf;        // [I] gelu(fc1)
-  uint16_t *attn;           // [QD]
+  // Vectors exchanged between blocks inside the launch, as 8-byte packets {two bf16 values, 32-bit tag}:
+  // a packet is valid for an exchange when its tag is epoch * 128 + exchange index + 1.
+  uint64_t *xp;             // [H / 2]      residual stream after a layer
+  uint64_t *qkvp;           // [3 * QD / 2]
+  uint64_t *actp;           // [I / 2]      gelu(fc1)
+  uint64_t *attnp;          // [QD / 2]
   uint16_t *kcache, *vcache;
   int64_t kv_layer_stride;  // elements between consecutive layers of the cache
   const uint16_t *cos_t, *sin_t;
@@ -38,7 +42,7 @@ struct MegaArgs {
   float ln_eps, scale;
   int act;
   int rows_attn;            // rows of phases B/C given to each attention block
-  unsigned long long *prof; // optional [blocks][L][8] time stamps (debugging aid), or null
+  unsigned long long *prof; // optional [blocks][L][16] time stamps (debugging aid), or null
 };
 
 bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why);

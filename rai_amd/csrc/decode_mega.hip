@@ -222,10 +222,39 @@ __device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r)
   if (r & 8) mg_rotate<8 % kMegaRing>(ring);
 }
 
+// A block announces that it has issued its stores for exchange `index`.  The flag is a hint only:
+// it is not ordered after the data stores (waiting for their acknowledgement would cost a memory
+// round trip per barrier), so consumers validate every packet by its tag and re-read the late ones.
 __device__ __forceinline__ void mg_grid_arrive(unsigned *flags, unsigned index, bool service, int lane) {
-  if (service) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (lane == 0) __hip_atomic_store(flags + blockIdx.x, index + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (service && lane == 0) __hip_atomic_store(flags + blockIdx.x, index + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Reads N packets per lane (packet i at src[idx[i]] when on[i]) until each carries `tag`; returns the
+// payloads.  The wave leaves the loop together; the spin is bounded like the barrier's.
+template <int N>
+__device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N], const bool (&on)[N], uint32_t tag,
+                                        uint32_t (&out)[N], int *fault) {
+  bool need[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) { need[i] = on[i]; out[i] = 0u; }
+  unsigned spins = 0;
+  for (;;) {
+    uint64_t pk[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) pk[i] = need[i] ? ld_dev64(src + idx[i]) : 0ull;
+    bool pending = false;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (need[i]) {
+        if ((uint32_t)(pk[i] >> 32) == tag) { out[i] = (uint32_t)pk[i]; need[i] = false; }
+        else pending = true;
+      }
+    }
+    if (!__any(pending)) break;
+    if (++spins > kMegaSpinLimit) {
+      __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
   }
 }
 __device__ __forceinline__ void mg_grid_wait(const unsigned *flags, unsigned index, int *fault, bool service, int lane) {
@@ -328,6 +357,8 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   cur.ptr = a.Wa0;
   cur.done = !mg_seg_next(cur, sp);
   unsigned bar = 0;
+  const uint32_t tagbase = a.state->epoch * 128u;   // exchange tags of this launch: tagbase + index + 1
+  uint32_t tag_x = 0;                                // tag of the residual-stream packets of the previous layer
   unsigned *const barrier = a.barrier;
   const float att_scale = a.scale;
   unsigned long long *const prof = a.prof;
@@ -417,11 +448,29 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       uint64_t bias_a = 0;
       if (service && lane * 4 < rowsA) bias_a = *reinterpret_cast<const uint64_t *>(ly.ba + nA0 + lane * 4);
       if (tid < 2 * kMegaRowsMax * kMegaWaves) partB[tid] = 0.f;
+      // the residual stream into LDS (xa is free until phase C): the plain vector for layer 0 (written
+      // before this launch), else the packets of the previous layer's last phase, polled by all threads
+      if (l == 0) {
+        for (int i = tid; i < H / 2; i += kMegaThreads) reinterpret_cast<uint32_t *>(xa)[i] = ld_dev32(a.x + 2 * i);
+      } else {
+        for (int base = 0; base < H / 2; base += kMegaThreads * 4) {
+          int idx[4];
+          bool on[4];
+          uint32_t val[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < H / 2; }
+          mg_poll<4>(a.xp, idx, on, tag_x, val, fault);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
+        }
+      }
+      wg_sync();
       if (wave < KTA) {
 
         mg_u32x4 xv[KTA];
 #pragma unroll
-        for (int u = 0; u < KTA; ++u) xv[u] = ld_dev128(a.x + u * 512 + lane * 8);
+        for (int u = 0; u < KTA; ++u) xv[u] = *reinterpret_cast<const mg_u32x4 *>(xa + u * 512 + lane * 8);
         const mg_u32x4 lw = *reinterpret_cast<const mg_u32x4 *>(ly.ln_w + wave * 512 + lane * 8);
         const mg_u32x4 lb = *reinterpret_cast<const mg_u32x4 *>(ly.ln_b + wave * 512 + lane * 8);
 
@@ -479,7 +528,10 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           }
           packed[h2] = pack_bf16x2(v[0], v[1]);
         }
-        st_dev64(n < a.n_qkv ? a.qkv + n : a.act_buf + (n - a.n_qkv), (uint64_t)packed[0] | ((uint64_t)packed[1] << 32));
+        uint64_t *dst = n < a.n_qkv ? a.qkvp + (n >> 1) : a.actp + ((n - a.n_qkv) >> 1);
+        const uint64_t tg = (uint64_t)(tagbase + bar + 1u) << 32;
+        st_dev64(dst, tg | packed[0]);
+        st_dev64(dst + 1, tg | packed[1]);
       }
       stamp(l, 1);
       mg_grid_arrive(barrier, bar, service, lane);
@@ -498,18 +550,31 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       const int tid = mg_opaque(tid0), lane = tid & 63;
       for (int e = tid; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
 
-      for (int k = tid * 4; k < I; k += kMegaThreads * 4) {
-        const uint64_t v = ld_dev64(a.act_buf + k);
-        *reinterpret_cast<uint64_t *>(xs + k) = v;
+      const uint32_t tag_a = tagbase + bar;   // bar was advanced past the A -> B exchange: its tag is index + 1
+      for (int base = 0; base < I / 2; base += kMegaThreads * 4) {
+        int idx[4];
+        bool on[4];
+        uint32_t val[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < I / 2; }
+        mg_poll<4>(a.actp, idx, on, tag_a, val, fault);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (on[i]) reinterpret_cast<uint32_t *>(xs)[idx[i]] = val[i];
       }
       if (is_attn) {
         const int h = wg;
-
-        if (tid < 3 * D / 2) {
-          const int which = tid / (D / 2), e = (tid - which * (D / 2)) * 2;
-          const uint32_t w = ld_dev32(a.qkv + which * QD + h * D + e);
-          raw[which * D + e] = __uint_as_float(w << 16);
-          raw[which * D + e + 1] = __uint_as_float(w & 0xffff0000u);
+        {
+          const int which = tid / (D / 2), pe = tid - which * (D / 2);
+          int idx[1] = {(which * QD + h * D) / 2 + pe};
+          bool on[1] = {tid < 3 * D / 2};
+          if (!on[0]) idx[0] = 0;
+          uint32_t val[1];
+          mg_poll<1>(a.qkvp, idx, on, tag_a, val, fault);
+          if (on[0]) {
+            raw[which * D + 2 * pe] = __uint_as_float(val[0] << 16);
+            raw[which * D + 2 * pe + 1] = __uint_as_float(val[0] & 0xffff0000u);
+          }
         }
         wg_sync();
         if (tid < D) {
@@ -599,16 +664,16 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
             const int d = 2 * lane + k;
             o[k] = (p_new * vnew[d] + red2[d] + red2[D + d] + red2[2 * D + d] + red2[3 * D + d]) * inv;
           }
-          st_dev32(a.attn + h * D + 2 * lane, pack_bf16x2(o[0], o[1]));
+          st_dev64(a.attnp + (h * D) / 2 + lane, ((uint64_t)(tagbase + bar + 1u) << 32) | pack_bf16x2(o[0], o[1]));
         }
       }
       wg_sync();
       stamp(l, 3);
       const int rot = mg_run_phase(ring, cur, sp, tB0, tB1, KTB, xs, partB, lane, wave);
       stamp(l, 4);
-      mg_grid_arrive(barrier, bar, wave == kMegaService, lane);
+      // no barrier here: the consumers of the attention output poll its packets
       mg_rotate_by(ring, rot);
-      mg_grid_wait(barrier, bar++, fault, wave == kMegaService, lane);
+      wg_sync();
       stamp(l, 5);
     }
 
@@ -622,9 +687,18 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         bd4 = *reinterpret_cast<const uint64_t *>(ly.bd + n0 + lane * 4);
         bf4 = *reinterpret_cast<const uint64_t *>(ly.bf + n0 + lane * 4);
       }
-      for (int k = tid * 4; k < QD; k += kMegaThreads * 4) {
-        const uint64_t v = ld_dev64(a.attn + k);
-        *reinterpret_cast<uint64_t *>(xa + k) = v;
+      const uint32_t tag_b = tagbase + bar + 1u;
+      ++bar;
+      for (int base = 0; base < QD / 2; base += kMegaThreads * 4) {
+        int idx[4];
+        bool on[4];
+        uint32_t val[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < QD / 2; }
+        mg_poll<4>(a.attnp, idx, on, tag_b, val, fault);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
       }
       wg_sync();
       const int rot = mg_run_phase(ring, cur, sp, tC0, tC1, KTC, xa, partC, lane, wave);
@@ -643,14 +717,18 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           for (int w = 0; w < kMegaStream; ++w) sacc += partC[e * kMegaWaves + w];
           v[k] = sacc + (elem(bd4, k) + elem(bf4, k)) + elem(res4, k);
         }
-        st_dev64(a.x + n0 + lane * 4,
-                 (uint64_t)pack_bf16x2(v[0], v[1]) | ((uint64_t)pack_bf16x2(v[2], v[3]) << 32));
+        const uint32_t lo = pack_bf16x2(v[0], v[1]), hi = pack_bf16x2(v[2], v[3]);
+        st_dev64(a.x + n0 + lane * 4, (uint64_t)lo | ((uint64_t)hi << 32));   // plain copy: this block's residual, and the head's input
+        const uint64_t tg = (uint64_t)(tagbase + bar + 1u) << 32;
+        st_dev64(a.xp + ((n0 + lane * 4) >> 1), tg | lo);
+        st_dev64(a.xp + ((n0 + lane * 4) >> 1) + 1, tg | hi);
       }
+      tag_x = tagbase + bar + 1u;
+      ++bar;
       stamp(l, 6);
-      if (l + 1 < a.L) {
-        mg_grid_arrive(barrier, bar, service, lane);
+      if (l + 1 < a.L) {   // no barrier: the next layer's LayerNorm polls the packets
         mg_rotate_by(ring, rot);
-        mg_grid_wait(barrier, bar++, fault, service, lane);
+        wg_sync();
       }
       stamp(l, 7);
     }

@@ -73,6 +73,7 @@ struct rai_hip_decoder {
   // persistent per-token kernel (Phi-2, bf16, batch 1): per-layer pointer table, barrier counter
   MegaLayer *mega_layers;
   unsigned *mega_barrier;
+  uint64_t *mega_xchg;    // packets exchanged between the blocks of the persistent decode kernel
   unsigned long long *mega_prof;  // time stamps of the persistent kernel when RAI_HIP_MEGA_PROF is set
   bool mega_ok;
   int num_cu;
@@ -159,6 +160,9 @@ k_rope_append(T *qkv, T *kcache, T *vcache, const T *cos_t, const T *sin_t, cons
     }
   }
 }
+
+// Between two launches of the persistent decode kernel that no token selection separates.
+__global__ void k_next_epoch(DevState *st) { st->epoch += 1u; }
 
 __global__ void k_set_state(DevState *st, int pos, int step) {
   st->pos = pos;
@@ -253,6 +257,7 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
     if (prev == B - 1) {  // every block has read `step` and written its outputs
       // the persistent decode kernel of this step has finished: lower its barrier flags
       for (int i = 0; i < grid_blocks; ++i) grid_barrier[i] = 0;
+      state->epoch += 1u;   // the next launch of the decode kernel tags its packets differently
       state->done = 0;
       state->pos += dpos;
       state->step += dstep;
@@ -488,8 +493,11 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   m.wa_stride = (int64_t)d->NA * d->H; m.wb_stride = (int64_t)d->H * d->KB;
   m.L = d->L; m.H = d->H; m.I = d->I; m.QD = d->QD; m.NA = d->NA; m.n_qkv = d->QD + 2 * d->KD;
   m.Hq = d->Hq; m.rot = d->cfg.rotary_dim; m.Tmax = d->cfg.max_context;
-  m.x = (uint16_t *)d->x; m.qkv = (uint16_t *)d->qkv;
-  m.attn = (uint16_t *)d->cat; m.act_buf = (uint16_t *)d->cat + d->QD;
+  m.x = (uint16_t *)d->x;
+  m.xp = d->mega_xchg;
+  m.qkvp = m.xp + d->H / 2;
+  m.actp = m.qkvp + (d->QD + 2 * d->KD) / 2;
+  m.attnp = m.actp + d->I / 2;
   m.kcache = (uint16_t *)d->kcache; m.vcache = (uint16_t *)d->vcache;
   m.kv_layer_stride = (int64_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
   m.cos_t = (const uint16_t *)d->cos_t; m.sin_t = (const uint16_t *)d->sin_t;
@@ -919,7 +927,15 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
     if (hipMemcpy(d->mega_barrier, f.data(), f.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess)
       return bail(fail(RAI_ERR_HIP, "decoder_create: flag upload failed"));
   }
+  d->mega_xchg = nullptr;
   if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_NO_MEGA") == nullptr) {
+    {  // zeroed: tag 0 is never a valid exchange tag
+      const size_t packets = (size_t)(d->H + d->QD + 2 * d->KD + d->I + d->QD) / 2 + 8;
+      if ((st = dalloc(d, packets * sizeof(uint64_t), &tmp))) return bail(st);
+      d->mega_xchg = (uint64_t *)tmp;
+      if (hipMemset(d->mega_xchg, 0, packets * sizeof(uint64_t)) != hipSuccess)
+        return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
+    }
     std::vector<MegaLayer> ml(d->L);
     for (int l = 0; l < d->L; ++l) {
       const Layer &ly = d->layers[l];
@@ -1127,8 +1143,10 @@ int rai_hip_decoder_time_decode_step(rai_hip_decoder *d, int32_t sweeps, float *
     if (hipEventRecord(e0, st) != hipSuccess) { rc = fail(RAI_ERR_HIP, "event record"); break; }
     rc = launch_phi2_decode_step(st, m, d->D, d->num_cu);
     if (rc != RAI_OK) break;
-    if (hipEventRecord(e1, st) != hipSuccess || hipMemsetAsync(d->mega_barrier, 0, flag_bytes, st) != hipSuccess ||
-        hipEventSynchronize(e1) != hipSuccess) { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
+    if (hipEventRecord(e1, st) != hipSuccess || hipMemsetAsync(d->mega_barrier, 0, flag_bytes, st) != hipSuccess)
+      { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
+    hipLaunchKernelGGL(k_next_epoch, dim3(1), dim3(1), 0, st, d->state);
+    if (hipEventSynchronize(e1) != hipSuccess) { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
     float ms = 0.f;
     (void)hipEventElapsedTime(&ms, e0, e1);
     if (s >= 2) total_ms += ms;
