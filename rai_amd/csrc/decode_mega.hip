@@ -250,6 +250,7 @@ __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N]
       }
     }
     if (!__any(pending)) break;
+    __builtin_amdgcn_s_sleep(4);   // a few hundred cycles between rounds: bounds the polling traffic
     if (++spins > kMegaSpinLimit) {
       __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
@@ -534,7 +535,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         st_dev64(dst + 1, tg | packed[1]);
       }
       stamp(l, 1);
-      mg_grid_arrive(barrier, bar, service, lane);
+      ++bar;   // no barrier: phase B polls the packets it needs
       stamp(l, 8);
       mg_rotate_by(ring, rot);
       if (is_attn) {
@@ -542,7 +543,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         k_load(Kc, tid);
         v_load(Vc, grp, col, grp < NG_V);
       }
-      mg_grid_wait(barrier, bar++, fault, service, lane);
+      wg_sync();
       stamp(l, 2);
     }
 
