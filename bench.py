@@ -371,8 +371,8 @@ def main():
         "weights_load_s": round(load_s, 1),
         "first_tokens": [int(t) for t in toks[0, :8]],
         "roofline": {
-            "kernel": "k_phi2_decode_step (persistent kernel: all 32 layers of one decode step, grid barriers, "
-                      "weight ring prefetched across phases)",
+            "kernel": "k_phi2_decode_step (persistent kernel: all 32 layers of one decode step, blocks exchange "
+                      "tagged packets instead of grid barriers, weight ring prefetched across phases)",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,

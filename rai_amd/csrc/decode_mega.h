@@ -10,7 +10,7 @@ struct DevState {
   int pos;    // tokens already in the KV cache
   int step;   // greedy steps taken by the current generate call
   int done;   // blocks of the token-selection kernel that have finished (reset by the last one)
-  int fault;  // set by a grid barrier that timed out; checked by the host after a generate call
+  int fault;  // set by a packet poll that timed out; checked by the host after a generate call
   unsigned epoch;  // launches of the persistent decode kernel so far: makes its exchange tags unique
 };
 
@@ -19,8 +19,6 @@ struct MegaLayer {
   const uint16_t *Wb, *bd, *bf;       // [H, QD + I] row n = dense[n, :] | fc2[n, :], and both biases
   const uint16_t *ln_w, *ln_b;
 };
-
-constexpr int kMegaFlagWords = 256;  // one barrier flag per block of the persistent kernel
 
 struct MegaArgs {
   const MegaLayer *layers;  // device array [L]
@@ -38,7 +36,6 @@ struct MegaArgs {
   int64_t kv_layer_stride;  // elements between consecutive layers of the cache
   const uint16_t *cos_t, *sin_t;
   DevState *state;
-  unsigned *barrier;        // kMegaFlagWords flags: [0, blocks) zero at launch, the rest 0xffffffff
   float ln_eps, scale;
   int act;
   int rows_attn;            // rows of phases B/C given to each attention block

@@ -3,26 +3,31 @@
 // parallel attention + MLP block) for batch 1, bf16.
 //
 // One 512-thread block per CU stays resident for the whole token.  A layer is
-// three weight-streaming phases separated by grid-wide barriers:
+// three weight-streaming phases:
 //   A  LayerNorm(x) . Wa^T + bias   -> q | k | v | gelu(fc1)      (rows split over blocks)
 //   B  head h attention on block h  ||  fc2 partial products on the other blocks
 //   C  dense(attn) partial + fc2 partial + biases + residual -> x (same rows as B)
 // Weights do not depend on activations: every wave keeps a ring of weight tiles
 // in flight that runs ahead across the phase boundaries, so HBM keeps streaming
-// through a barrier instead of draining at a kernel boundary.  Attention
-// (latency bound, 0.2 MB per head) hides behind the 52 MB fc2 stream of phase B.
+// while a block waits for its inputs.  Attention (latency bound, 0.2 MB per head)
+// hides behind the 52 MB fc2 stream of phase B.
 //
-// Values that cross blocks inside the launch (x, q|k|v, act, attn, barrier flags)
-// are written with device-scope write-through stores and read with device-scope
-// loads: the per-XCD L2s are not coherent for ordinary accesses, and a
-// device-scope fence would write back and invalidate a whole L2.  Weights,
-// biases, rotary tables and the KV cache rows of earlier tokens are read-only
-// here and use ordinary (non-temporal) loads.
+// There is no grid barrier.  The vectors that cross blocks (x, q|k|v, act, attn) are
+// written as 8-byte packets {two bf16 values, 32-bit tag}, tag = launch epoch * 128 +
+// exchange index + 1, with device-scope write-through stores, and every consumer
+// polls exactly the packets it needs with device-scope loads until their tags match
+// (an 8-byte store is single-copy atomic, so a matching tag proves the payload).
+// Data and notification are therefore one memory trip, not a store, its
+// acknowledgement, a flag and a second read; a buffer is safe to overwrite two
+// exchanges later because receiving a block's packets proves that block has left the
+// phase in which it read the older ones.  The per-XCD L2s are not coherent for
+// ordinary accesses and a device-scope fence would write back and invalidate a whole
+// L2, hence packets and no fences.  Weights, biases, rotary tables and the KV cache
+// rows of earlier tokens are read-only here and use ordinary loads.
 //
-// The grid barrier spins on flags in device memory; every block of the grid is
-// resident (grid <= number of CUs) so the spin always ends, and it is bounded:
-// on timeout the block raises DevState::fault and every later barrier falls
-// through, so the kernel always terminates and the host reports the fault.
+// Every block of the grid is resident (grid <= number of CUs), so a poll always ends,
+// and it is bounded: on timeout the wave raises DevState::fault, later polls fall
+// through, the kernel terminates and the host reports the fault.
 #include "decode_mega.h"
 
 #include "gemm.h"
@@ -222,14 +227,8 @@ __device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r)
   if (r & 8) mg_rotate<8 % kMegaRing>(ring);
 }
 
-// A block announces that it has issued its stores for exchange `index`.  The flag is a hint only:
-// it is not ordered after the data stores (waiting for their acknowledgement would cost a memory
-// round trip per barrier), so consumers validate every packet by its tag and re-read the late ones.
-__device__ __forceinline__ void mg_grid_arrive(unsigned *flags, unsigned index, bool service, int lane) {
-  if (service && lane == 0) __hip_atomic_store(flags + blockIdx.x, index + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 // Reads N packets per lane (packet i at src[idx[i]] when on[i]) until each carries `tag`; returns the
-// payloads.  The wave leaves the loop together; the spin is bounded like the barrier's.
+// payloads.  The wave leaves the loop together; the spin is bounded.
 template <int N>
 __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N], const bool (&on)[N], uint32_t tag,
                                         uint32_t (&out)[N], int *fault) {
@@ -257,29 +256,6 @@ __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N]
     }
     if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
   }
-}
-__device__ __forceinline__ void mg_grid_wait(const unsigned *flags, unsigned index, int *fault, bool service, int lane) {
-  if (service) {
-    const unsigned target = index + 1u;
-    const int G = gridDim.x;
-    unsigned spins = 0;
-    for (;;) {
-      bool ok = true;
-      if (lane * 4 < G) {
-        const uint64_t lo = ld_dev64(flags + lane * 4), hi = ld_dev64(flags + lane * 4 + 2);
-        ok = (uint32_t)lo >= target && (uint32_t)(lo >> 32) >= target && (uint32_t)hi >= target &&
-             (uint32_t)(hi >> 32) >= target;
-      }
-      if (__all(ok)) break;
-      ++spins;
-      if (spins > kMegaSpinLimit) {
-        if (lane == 0) __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-      if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-    }
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 template <int KTA, int D, bool PROF>
 __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
@@ -360,7 +336,6 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   unsigned bar = 0;
   const uint32_t tagbase = a.state->epoch * 128u;   // exchange tags of this launch: tagbase + index + 1
   uint32_t tag_x = 0;                                // tag of the residual-stream packets of the previous layer
-  unsigned *const barrier = a.barrier;
   const float att_scale = a.scale;
   unsigned long long *const prof = a.prof;
   const int n_layers = a.L;

@@ -70,9 +70,8 @@ struct rai_hip_decoder {
   int ctx_len;
   int64_t max_rows;
   int history_cap;
-  // persistent per-token kernel (Phi-2, bf16, batch 1): per-layer pointer table, barrier counter
+  // persistent per-token kernel (Phi-2, bf16, batch 1): per-layer pointer table, exchange packets
   MegaLayer *mega_layers;
-  unsigned *mega_barrier;
   uint64_t *mega_xchg;    // packets exchanged between the blocks of the persistent decode kernel
   unsigned long long *mega_prof;  // time stamps of the persistent kernel when RAI_HIP_MEGA_PROF is set
   bool mega_ok;
@@ -179,7 +178,7 @@ __global__ void k_set_state(DevState *st, int pos, int step) {
 template <typename T>
 __global__ void __launch_bounds__(1024)
 k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
-               int dstep, const T *embed, T *x_next, int H, float embed_scale, unsigned *grid_barrier, int grid_blocks) {
+               int dstep, const T *embed, T *x_next, int H, float embed_scale) {
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   __shared__ uint32_t chosen;
@@ -255,8 +254,6 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
     __threadfence();
     int prev = atomicAdd(&state->done, 1);
     if (prev == B - 1) {  // every block has read `step` and written its outputs
-      // the persistent decode kernel of this step has finished: lower its barrier flags
-      for (int i = 0; i < grid_blocks; ++i) grid_barrier[i] = 0;
       state->epoch += 1u;   // the next launch of the decode kernel tags its packets differently
       state->done = 0;
       state->pos += dpos;
@@ -501,7 +498,7 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   m.kcache = (uint16_t *)d->kcache; m.vcache = (uint16_t *)d->vcache;
   m.kv_layer_stride = (int64_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
   m.cos_t = (const uint16_t *)d->cos_t; m.sin_t = (const uint16_t *)d->sin_t;
-  m.state = d->state; m.barrier = d->mega_barrier;
+  m.state = d->state;
   m.ln_eps = (float)d->cfg.norm_eps; m.scale = (float)(1.0 / sqrt((double)d->D));
   m.act = d->cfg.hidden_act;
   static const int rows_attn = getenv("RAI_HIP_MEGA_ROWS_ATTN") ? atoi(getenv("RAI_HIP_MEGA_ROWS_ATTN")) : 0;
@@ -625,11 +622,11 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
+                       (bf16_raw *)d->x, H, d->embed_scale);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
+                       d->embed_scale);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
@@ -762,11 +759,11 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   if (dt == RAI_BF16)
     hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
+                       (bf16_raw *)d->x, H, d->embed_scale);
   else
     hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale, d->mega_barrier, d->mega_ok ? d->num_cu : 0);
+                       d->embed_scale);
   RAI_TRY(launch_check("select_token"));
   d->ctx_len = T_after;
   return RAI_OK;
@@ -777,7 +774,7 @@ static int forward_any(rai_hip_decoder *d, int B, int S, bool advance_step, bool
                                        : forward_seq(d, B, S, advance_step, from_tokens);
 }
 
-// A grid barrier of the persistent decode kernel that timed out leaves
+// A packet poll of the persistent decode kernel that timed out leaves
 // DevState::fault set; the results of that step are not valid.
 static int check_fault(rai_hip_decoder *d) {
   if (!d->mega_ok) return RAI_OK;
@@ -793,34 +790,14 @@ static int check_fault(rai_hip_decoder *d) {
       const int b = blocks[bi];
       for (int l = 0; l < d->L; ++l)
         for (int k = 0; k < 7; ++k) iv[k] += (at(b, l, k + 1) - at(b, l, k)) / d->L;
-      fprintf(stderr, "mega prof block %3d: A %.2f | bar %.2f | B-pre(attn) %.2f | B-stream %.2f | bar %.2f | C %.2f | bar %.2f us\n",
+      fprintf(stderr, "mega prof block %3d: A (wait x, LN, stream) %.2f | wave sync %.2f | B-pre (wait act, attention) %.2f | service %.2f | B stream %.2f | C (wait attn, stream) %.2f | wave sync %.2f us\n",
               b, iv[0], iv[1], iv[2], iv[3], iv[4], iv[5], iv[6]);
-    }
-    // per barrier over all blocks: spread of the arrivals, last arrival -> first exit, spread of the exits
-    const int before[3] = {1, 4, 6}, after[3] = {2, 5, 7};
-    for (int k = 0; k < 3; ++k) {
-      double spread = 0, lat = 0, espread = 0;
-      int layers = 0, last_attn = 0;
-      for (int l = 0; l + (k == 2 ? 1 : 0) < d->L; ++l, ++layers) {
-        double amin = 1e30, amax = 0, emin = 1e30, emax = 0;
-        int who = 0;
-        for (int b = 0; b < d->num_cu; ++b) {
-          const double av = at(b, l, before[k]), ev = at(b, l, after[k]);
-          if (av > amax) { amax = av; who = b; }
-          amin = av < amin ? av : amin; emin = ev < emin ? ev : emin; emax = ev > emax ? ev : emax;
-        }
-        spread += amax - amin; lat += emin - amax; espread += emax - emin;
-        last_attn += who < d->Hq;
-      }
-      fprintf(stderr, "mega prof barrier %d: arrival spread %.2f us, last arrival -> first exit %.2f us, exit spread %.2f us, last arriver was an attention block in %d of %d layers\n",
-              k, spread / layers, lat / layers, espread / layers, last_attn, layers);
     }
   }
   if (hs.fault == 0) return RAI_OK;
   hs.fault = 0;
   RAI_HIP_TRY(hipMemcpy(&d->state->fault, &hs.fault, sizeof(int), hipMemcpyHostToDevice));
-  RAI_HIP_TRY(hipMemset(d->mega_barrier, 0, sizeof(unsigned) * (d->num_cu < kMegaFlagWords ? d->num_cu : kMegaFlagWords)));
-  return fail(RAI_ERR_HIP, "decoder: a grid barrier of the persistent decode kernel timed out");
+  return fail(RAI_ERR_HIP, "decoder: an exchange of the persistent decode kernel timed out");
 }
 
 static int check_call(rai_hip_decoder *d, int B, int S) {
@@ -918,14 +895,6 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   {
     hipDeviceProp_t prop;
     d->num_cu = hipGetDeviceProperties(&prop, dev) == hipSuccess ? prop.multiProcessorCount : kNumCU;
-  }
-  if ((st = dalloc(d, kMegaFlagWords * sizeof(unsigned), &tmp))) return bail(st);
-  d->mega_barrier = (unsigned *)tmp;
-  {  // flags of blocks that exist start at 0, the padding reads as "arrived"
-    std::vector<unsigned> f(kMegaFlagWords, 0xffffffffu);
-    for (int i = 0; i < d->num_cu && i < kMegaFlagWords; ++i) f[i] = 0;
-    if (hipMemcpy(d->mega_barrier, f.data(), f.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess)
-      return bail(fail(RAI_ERR_HIP, "decoder_create: flag upload failed"));
   }
   d->mega_xchg = nullptr;
   if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_NO_MEGA") == nullptr) {
@@ -1136,15 +1105,13 @@ int rai_hip_decoder_time_decode_step(rai_hip_decoder *d, int32_t sweeps, float *
   RAI_HIP_TRY(hipEventCreate(&e0));
   RAI_HIP_TRY(hipEventCreate(&e1));
   const MegaArgs m = mega_args(d);
-  const size_t flag_bytes = sizeof(unsigned) * (size_t)(d->num_cu < kMegaFlagWords ? d->num_cu : kMegaFlagWords);
   double total_ms = 0.0;
   int rc = RAI_OK;
   for (int s = 0; s < sweeps + 2 && rc == RAI_OK; ++s) {  // two warm-up launches
     if (hipEventRecord(e0, st) != hipSuccess) { rc = fail(RAI_ERR_HIP, "event record"); break; }
     rc = launch_phi2_decode_step(st, m, d->D, d->num_cu);
     if (rc != RAI_OK) break;
-    if (hipEventRecord(e1, st) != hipSuccess || hipMemsetAsync(d->mega_barrier, 0, flag_bytes, st) != hipSuccess)
-      { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
+    if (hipEventRecord(e1, st) != hipSuccess) { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
     hipLaunchKernelGGL(k_next_epoch, dim3(1), dim3(1), 0, st, d->state);
     if (hipEventSynchronize(e1) != hipSuccess) { rc = fail(RAI_ERR_HIP, "time_decode_step: launch failed"); break; }
     float ms = 0.f;
