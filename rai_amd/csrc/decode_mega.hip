@@ -249,7 +249,7 @@ __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N]
       }
     }
     if (!__any(pending)) break;
-    __builtin_amdgcn_s_sleep(4);   // a few hundred cycles between rounds: bounds the polling traffic
+    __builtin_amdgcn_s_sleep(1);   // a short pause between rounds: bounds the polling traffic
     if (++spins > kMegaSpinLimit) {
       __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
@@ -527,7 +527,9 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       for (int e = tid; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
 
       const uint32_t tag_a = tagbase + bar;   // bar was advanced past the A -> B exchange: its tag is index + 1
-      for (int base = 0; base < I / 2; base += kMegaThreads * 4) {
+      // a block without fc2 rows (an attention block, by default) does not wait for the activations:
+      // its attention starts as soon as the few blocks that produce its head's q, k and v are done
+      for (int base = 0; nrows > 0 && base < I / 2; base += kMegaThreads * 4) {
         int idx[4];
         bool on[4];
         uint32_t val[4];
