@@ -76,12 +76,15 @@ struct rai_hip_decoder {
   unsigned long long *mega_prof;  // time stamps of the persistent kernel when RAI_HIP_MEGA_PROF is set
   bool mega_ok;
   int num_cu;
-  hipGraphExec_t step_graph;  // one captured single-token step (batch step_graph_batch)
+  hipGraphExec_t step_graph;   // one captured single-token step (batch step_graph_batch)
+  hipGraphExec_t step_graph_n; // kGraphSteps consecutive single-token steps in one graph (same batch)
   int step_graph_batch;
   bool x_holds_next;          // d->x already holds the embedding of d->tokens
 };
 
 namespace rai {
+
+constexpr int kGraphSteps = 8;  // single-token steps recorded in the multi-step decode graph
 
 // ------------------------------------------------------------------ small kernels
 template <typename T>
@@ -251,7 +254,8 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    __threadfence();
+    // no fence: `step` was read (and used for an address) before this point, and what this block wrote is
+    // consumed by later kernels only
     int prev = atomicAdd(&state->done, 1);
     if (prev == B - 1) {  // every block has read `step` and written its outputs
       state->epoch += 1u;   // the next launch of the decode kernel tags its packets differently
@@ -844,6 +848,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->KB = d->QD + d->I;
   d->ctx_len = 0;
   d->step_graph = nullptr;
+  d->step_graph_n = nullptr;
   d->step_graph_batch = 0;
   d->x_holds_next = false;
   const int vec = (int)(16 / d->es);
@@ -935,6 +940,7 @@ int rai_hip_decoder_destroy(rai_hip_decoder *d) {
   (void)hipSetDevice(d->dev);
   (void)hipStreamSynchronize(stream_of(d->dev));
   if (d->step_graph) (void)hipGraphExecDestroy(d->step_graph);
+  if (d->step_graph_n) (void)hipGraphExecDestroy(d->step_graph_n);
   for (void *p : d->allocs) (void)hipFree(p);
   delete d;
   return RAI_OK;
@@ -1040,35 +1046,55 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   // Single-token steps: the previous step left the next input embedding, the
   // token and the advanced context length on the device, so every step is the
   // same sequence of launches.  The first step runs eagerly (it also performs
-  // any one-time kernel attribute set-up), the second is captured into a
-  // hipGraph, the rest replay it.
+  // any one-time kernel attribute set-up); the rest replay captured hipGraphs,
+  // kGraphSteps steps per launch while that many remain, then one step per launch.
   const bool use_graph = d->cfg.dtype == RAI_BF16 && getenv("RAI_HIP_NO_GRAPH") == nullptr;
-  for (int step = 1; rc == RAI_OK && step < n_new; ++step) {
-    if (use_graph && d->step_graph && d->step_graph_batch == batch) {
-      if (hipGraphLaunch(d->step_graph, st) != hipSuccess) rc = fail(RAI_ERR_HIP, "generate: graph launch failed");
-      else d->ctx_len += 1;
-      continue;
-    }
-    if (use_graph && step >= 2) {
-      if (d->step_graph) { (void)hipGraphExecDestroy(d->step_graph); d->step_graph = nullptr; }
-      hipGraph_t g = nullptr;
-      if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess) {
-        rc = fail(RAI_ERR_HIP, "generate: begin capture failed");
-        break;
-      }
-      int frc = forward_any(d, batch, 1, true, true);
-      hipError_t ce = hipStreamEndCapture(st, &g);
-      if (frc != RAI_OK) { rc = frc; if (g) (void)hipGraphDestroy(g); break; }
-      if (ce != hipSuccess || !g) { rc = fail(RAI_ERR_HIP, "generate: end capture failed: %s", hipGetErrorString(ce)); break; }
-      d->ctx_len -= 1;  // capture only recorded the step; it has not run yet
-      hipError_t ie = hipGraphInstantiate(&d->step_graph, g, nullptr, nullptr, 0);
-      (void)hipGraphDestroy(g);
-      if (ie != hipSuccess) { d->step_graph = nullptr; rc = fail(RAI_ERR_HIP, "generate: graph instantiate: %s", hipGetErrorString(ie)); break; }
-      d->step_graph_batch = batch;
-      --step;  // run this step through the graph
-      continue;
-    }
+  // Captures `steps` consecutive single-token steps (they read their inputs from device state, so the
+  // recorded launches are identical for every step) into an executable graph.
+  auto capture = [&](int steps, hipGraphExec_t *exec) -> int {
+    hipGraph_t g = nullptr;
+    const int ctx0 = d->ctx_len;
+    if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess)
+      return fail(RAI_ERR_HIP, "generate: begin capture failed");
+    int frc = RAI_OK;
+    for (int i = 0; i < steps && frc == RAI_OK; ++i) frc = forward_any(d, batch, 1, true, true);
+    hipError_t ce = hipStreamEndCapture(st, &g);
+    d->ctx_len = ctx0;  // capture only recorded the steps; they have not run
+    if (frc != RAI_OK) { if (g) (void)hipGraphDestroy(g); return frc; }
+    if (ce != hipSuccess || !g) return fail(RAI_ERR_HIP, "generate: end capture failed: %s", hipGetErrorString(ce));
+    hipError_t ie = hipGraphInstantiate(exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (ie != hipSuccess) { *exec = nullptr; return fail(RAI_ERR_HIP, "generate: graph instantiate: %s", hipGetErrorString(ie)); }
+    return RAI_OK;
+  };
+  int step = 1;
+  if (rc == RAI_OK && step < n_new) {  // first step eagerly: one-time kernel attribute set-up happens outside capture
     rc = forward_any(d, batch, 1, true, true);
+    ++step;
+  }
+  if (rc == RAI_OK && use_graph && d->step_graph_batch != batch) {
+    if (d->step_graph) { (void)hipGraphExecDestroy(d->step_graph); d->step_graph = nullptr; }
+    if (d->step_graph_n) { (void)hipGraphExecDestroy(d->step_graph_n); d->step_graph_n = nullptr; }
+    d->step_graph_batch = batch;
+  }
+  while (rc == RAI_OK && step < n_new) {
+    const int left = n_new - step;
+    if (!use_graph) {
+      rc = forward_any(d, batch, 1, true, true);
+      ++step;
+      continue;
+    }
+    if (left >= kGraphSteps) {   // the gap between two graph launches is paid once per kGraphSteps tokens
+      if (!d->step_graph_n) { rc = capture(kGraphSteps, &d->step_graph_n); if (rc != RAI_OK) break; }
+      if (hipGraphLaunch(d->step_graph_n, st) != hipSuccess) { rc = fail(RAI_ERR_HIP, "generate: graph launch failed"); break; }
+      d->ctx_len += kGraphSteps;
+      step += kGraphSteps;
+    } else {
+      if (!d->step_graph) { rc = capture(1, &d->step_graph); if (rc != RAI_OK) break; }
+      if (hipGraphLaunch(d->step_graph, st) != hipSuccess) { rc = fail(RAI_ERR_HIP, "generate: graph launch failed"); break; }
+      d->ctx_len += 1;
+      ++step;
+    }
   }
   if (rc == RAI_OK && hipEventRecord(e2, st) != hipSuccess) rc = fail(RAI_ERR_HIP, "event record");
   if (rc == RAI_OK && hipStreamSynchronize(st) != hipSuccess) rc = fail(RAI_ERR_HIP, "generate: stream sync failed");
