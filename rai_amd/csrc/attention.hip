@@ -879,24 +879,61 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
   const int wave_last_key = a.causal ? off + q0 + wave * 32 + 31 : a.T - 1;  // newest key any row of this wave may see
   const float scale_r = round_to<bf16_raw>(a.scale);
 
-  for (int k0 = 0; k0 < kv_end; k0 += 64) {
-    __syncthreads();
-    // ---- stage K [64][D] and V^T [D][64]; rows past the context re-read its last row (masked below)
-    for (int c = tid; c < 64 * CPR; c += NT) {
+  // K/V tiles go global -> registers -> LDS; with PF the loads of tile t+1 are issued before tile t is
+  // multiplied, so their latency hides behind the MFMAs (register budget allows it for D <= 128)
+  constexpr int CH = (64 * CPR + NT - 1) / NT;   // 16-byte chunks of K (and of V) per thread
+  constexpr bool PF = D <= 128;
+  fa_u32x4 kreg[CH], vreg[CH];
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + i * NT;
       const int key = c / CPR, dc = (c % CPR) * 8;
       int t = k0 + key;
-      t = t < a.T ? t : a.T - 1;
-      const fa_u32x4 kv = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
-      *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kv;
-      const fa_u32x4 vv = *reinterpret_cast<const fa_u32x4 *>(Vg + (int64_t)t * a.vs[2] + dc);
-      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+      t = t < a.T ? t : a.T - 1;   // rows past the context re-read its last row (masked below)
+      if (c < 64 * CPR) {
+        kreg[i] = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
+        vreg[i] = *reinterpret_cast<const fa_u32x4 *>(Vg + (int64_t)t * a.vs[2] + dc);
+      }
+    }
+  };
+  if (PF && kv_end > 0) load_tile(0);
+  for (int k0 = 0; k0 < kv_end; k0 += 64) {
+    __syncthreads();
+    // ---- stage K [64][D] and V^T [D][64]
+    if constexpr (PF) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        Vt[(dc + 2 * e) * VP + key] = (uint16_t)(w[e] & 0xffffu);
-        Vt[(dc + 2 * e + 1) * VP + key] = (uint16_t)(w[e] >> 16);
+      for (int i = 0; i < CH; ++i) {
+        const int c = tid + i * NT;
+        const int key = c / CPR, dc = (c % CPR) * 8;
+        if (c < 64 * CPR) {
+          *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kreg[i];
+          const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            Vt[(dc + 2 * e) * VP + key] = (uint16_t)(w[e] & 0xffffu);
+            Vt[(dc + 2 * e + 1) * VP + key] = (uint16_t)(w[e] >> 16);
+          }
+        }
+      }
+    } else {
+      for (int c = tid; c < 64 * CPR; c += NT) {
+        const int key = c / CPR, dc = (c % CPR) * 8;
+        int t = k0 + key;
+        t = t < a.T ? t : a.T - 1;
+        const fa_u32x4 kv = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
+        *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kv;
+        const fa_u32x4 vv = *reinterpret_cast<const fa_u32x4 *>(Vg + (int64_t)t * a.vs[2] + dc);
+        const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          Vt[(dc + 2 * e) * VP + key] = (uint16_t)(w[e] & 0xffffu);
+          Vt[(dc + 2 * e + 1) * VP + key] = (uint16_t)(w[e] >> 16);
+        }
       }
     }
     __syncthreads();
+    if (PF && k0 + 64 < kv_end) load_tile(k0 + 64);
     if (k0 > wave_last_key) continue;  // every key of this tile is masked for this wave (barriers stay uniform)
 
     // ---- S^T tile: 64 keys x 32 queries

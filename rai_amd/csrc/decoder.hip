@@ -163,6 +163,60 @@ k_rope_append(T *qkv, T *kcache, T *vcache, const T *cos_t, const T *sin_t, cons
   }
 }
 
+// The same operation with one thread per 16-byte pack and 32-bit indexing (D, rot/2 and the row
+// length multiples of the pack width; fewer than 2^31 packs).  The pack at feature d0 < rot/2 and
+// its partner at d0 + rot/2 are rotated by one thread, so the update of q stays in place.
+template <typename T>
+__global__ void __launch_bounds__(256)
+k_rope_append_vec(T *qkv, T *kcache, T *vcache, const T *cos_t, const T *sin_t, const DevState *state, int B, int S,
+                  int Hq, int Hkv, int D, int rot, int Tmax) {
+  constexpr int VEC = 16 / sizeof(T);
+  struct alignas(16) Pack { T v[VEC]; };
+  const int pos0 = state->pos;
+  const int QD = Hq * D, KD = Hkv * D, ld = QD + 2 * KD;
+  const int half = rot / 2;
+  const uint32_t heads = Hq + 2 * Hkv, ppr = D / VEC;        // packs per head row
+  const uint32_t total = (uint32_t)B * S * heads * ppr;
+  for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < total; e += gridDim.x * blockDim.x) {
+    const uint32_t r = e / ppr, d0 = (e - r * ppr) * VEC;
+    const uint32_t hh = r % heads, r2 = r / heads, s = r2 % S, b = r2 / S;
+    T *row = qkv + ((int64_t)b * S + s) * ld;
+    const int pos = pos0 + (int)s;
+    if (hh < (uint32_t)(Hq + Hkv)) {  // q or k head
+      T *hp = row + (hh < (uint32_t)Hq ? hh * D : QD + (hh - Hq) * D);
+      T *kc = hh < (uint32_t)Hq ? nullptr : kcache + (((int64_t)b * Hkv + (hh - Hq)) * Tmax + pos) * D;
+      if ((int)d0 < half) {
+        const Pack x1 = *reinterpret_cast<const Pack *>(hp + d0), x2 = *reinterpret_cast<const Pack *>(hp + d0 + half);
+        const T *ct = cos_t + (int64_t)pos * rot + d0, *st = sin_t + (int64_t)pos * rot + d0;
+        const Pack c1 = *reinterpret_cast<const Pack *>(ct), s1 = *reinterpret_cast<const Pack *>(st);
+        const Pack c2 = *reinterpret_cast<const Pack *>(ct + half), s2 = *reinterpret_cast<const Pack *>(st + half);
+        Pack o1, o2;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float v = (float)Scalar<T>::load(&x1.v[j]), v2 = (float)Scalar<T>::load(&x2.v[j]);
+          // the reference rounds x*cos, rot*sin and their sum separately (phi2.rs:75)
+          T a, bb;
+          Scalar<T>::store(&a, v * (float)Scalar<T>::load(&c1.v[j]));
+          Scalar<T>::store(&bb, -v2 * (float)Scalar<T>::load(&s1.v[j]));
+          Scalar<T>::store(&o1.v[j], (float)Scalar<T>::load(&a) + (float)Scalar<T>::load(&bb));
+          Scalar<T>::store(&a, v2 * (float)Scalar<T>::load(&c2.v[j]));
+          Scalar<T>::store(&bb, v * (float)Scalar<T>::load(&s2.v[j]));
+          Scalar<T>::store(&o2.v[j], (float)Scalar<T>::load(&a) + (float)Scalar<T>::load(&bb));
+        }
+        T *dst = kc ? kc : hp;
+        *reinterpret_cast<Pack *>(dst + d0) = o1;
+        *reinterpret_cast<Pack *>(dst + d0 + half) = o2;
+      } else if ((int)d0 >= rot && kc) {
+        *reinterpret_cast<Pack *>(kc + d0) = *reinterpret_cast<const Pack *>(hp + d0);
+      }
+    } else {
+      const uint32_t hv = hh - Hq - Hkv;
+      *reinterpret_cast<Pack *>(vcache + (((int64_t)b * Hkv + hv) * Tmax + pos) * D + d0) =
+          *reinterpret_cast<const Pack *>(row + QD + KD + hv * D + d0);
+    }
+  }
+}
+
 // Between two launches of the persistent decode kernel that no token selection separates.
 __global__ void k_next_epoch(DevState *st) { st->epoch += 1u; }
 
@@ -454,6 +508,14 @@ template <typename T> static void launch_embed(rai_hip_decoder *d, hipStream_t s
 template <typename T> static void launch_rope_append(rai_hip_decoder *d, hipStream_t st, int l, int B, int S) {
   const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
   int64_t total = (int64_t)B * S * (d->Hq + 2 * d->Hkv) * d->D;
+  constexpr int VEC = 16 / sizeof(T);
+  const int rot = d->cfg.rotary_dim;
+  if (d->D % VEC == 0 && (rot / 2) % VEC == 0 && (d->QD + 2 * d->KD) % VEC == 0 && total / VEC < ((int64_t)1 << 31)) {
+    hipLaunchKernelGGL((k_rope_append_vec<T>), dim3(grid1d(total / VEC)), dim3(256), 0, st, (T *)d->qkv,
+                       (T *)d->kcache + per_layer * l, (T *)d->vcache + per_layer * l, (const T *)d->cos_t,
+                       (const T *)d->sin_t, d->state, B, S, d->Hq, d->Hkv, d->D, rot, d->cfg.max_context);
+    return;
+  }
   hipLaunchKernelGGL((k_rope_append<T>), dim3(grid1d(total)), dim3(256), 0, st, (T *)d->qkv,
                      (T *)d->kcache + per_layer * l, (T *)d->vcache + per_layer * l, (const T *)d->cos_t,
                      (const T *)d->sin_t, d->state, B, S, d->Hq, d->Hkv, d->D, d->cfg.rotary_dim, d->cfg.max_context);
