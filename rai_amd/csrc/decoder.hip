@@ -707,8 +707,9 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   const int H = d->H, QD = d->QD, KD = d->KD, I = d->I;
   const int64_t M = (int64_t)B * S;
   const int ldq = QD + 2 * KD;
-  const bool fuse_norm = dt == RAI_BF16 && M <= 8;
   const int kind = d->cfg.arch == RAI_ARCH_GEMMA ? 2 : 1;
+  // the norm runs inside the Linear kernel for single rows and for the batched-decode row counts
+  const bool fuse_norm = dt == RAI_BF16 && (M <= 8 || linear_mfma_fuses_norm((int)M, H, kind));
   const int T_after = d->ctx_len + S;
   const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
 
@@ -809,7 +810,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   // last position -> final norm -> lm_head (qwen2.rs:355-357, gemma.rs:383-385)
   LinearArgs h = linear_args_default();
   char *last_rows = x + (size_t)(S - 1) * H * d->es;
-  if (dt == RAI_BF16 && B <= 8) {
+  if (dt == RAI_BF16 && (B <= 8 || linear_mfma_fuses_norm(B, H, kind))) {
     h.A = last_rows; h.lda = (int64_t)S * H;
     h.ln_kind = kind; h.ln_w = d->lnf_w; h.ln_eps = (float)d->cfg.norm_eps;
   } else {

@@ -60,6 +60,7 @@ int launch_linear_bf16(hipStream_t st, const LinearArgs &a);
 
 // f32 tile kernel for the same NT contraction, FMA in f32.
 int launch_linear_f32(hipStream_t st, const LinearArgs &a);
+bool linear_mfma_fuses_norm(int M, int K, int ln_kind);
 
 __device__ __forceinline__ float act_eval(int act, float x);
 // act(gate) * up with the reference's roundings of gate, act(gate) and up to bf16.

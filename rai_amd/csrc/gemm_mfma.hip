@@ -752,6 +752,45 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
         z = *reinterpret_cast<const bf16x8 *>((const uint16_t *)a.A + (int64_t)m * a.lda + k + lq * 8);
       xf[mt][ks] = z;
     }
+  // Optional RMSNorm of the activation rows (ln_kind 1: x * w / rms, 2: x * (1 + w) / rms), K not split
+  // over blocks: the sum of squares of a row is gathered from the four lanes and eight waves that hold
+  // its pieces, then every fragment is scaled and rounded to bf16 exactly as the stand-alone kernel does.
+  if (a.ln_kind > 0) {
+    float *rs = reinterpret_cast<float *>(lds);   // [8 waves][MT * 16 rows]; the accumulator area is not in use yet
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float ss = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { const float v = (float)xf[mt][ks][j]; ss = fmaf(v, v, ss); }
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      if (lq == 0) rs[wave * (MT * 16) + mt * 16 + lrow] = ss;
+    }
+    __syncthreads();
+    const uint16_t *lw = (const uint16_t *)a.ln_w;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) tot += rs[w * (MT * 16) + mt * 16 + lrow];
+      const float scale = 1.0f / sqrtf(tot / (float)a.K + a.ln_eps);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int k = k0 + ks * 32;
+        if (k < a.K) {
+          const bf16x8 wv = *reinterpret_cast<const bf16x8 *>(lw + k + lq * 8);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float wf = (float)wv[j];
+            xf[mt][ks][j] = (__bf16)((float)xf[mt][ks][j] * scale * (a.ln_kind == 2 ? 1.0f + wf : wf));
+          }
+        }
+      }
+    }
+    __syncthreads();   // the statistics have been read before the area is reused
+  }
   int koff[KS];   // K steps beyond K read column 0 (their activation fragments are zero)
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) koff[ks] = k0 + ks * 32 < a.K ? k0 + ks * 32 : 0;
@@ -886,12 +925,21 @@ template <int MT, int KS> static int launch_mfma_stream(hipStream_t st, const Li
   return launch_mfma_stream_cfg<MT, KS, 1>(st, a, splits);
 }
 
+// True when the small-M streaming kernel can apply the RMSNorm of the activation rows itself.
+bool linear_mfma_fuses_norm(int M, int K, int ln_kind) {
+  static const bool off = getenv("RAI_HIP_NO_MFMA_STREAM") != nullptr || getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr ||
+                          getenv("RAI_HIP_NO_FUSED_NORM") != nullptr;
+  if (off || (ln_kind != 1 && ln_kind != 2) || M <= 8 || M > 64 || K % 32) return false;
+  return K <= (M <= 32 ? 8 * 8 * 32 : 8 * 4 * 32);   // one block's K span: no split over blocks
+}
+
 int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
   RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
   RAI_REQUIRE(a.n_split >= 0 && a.n_split <= a.N && (a.n_split == a.N || a.out2), RAI_ERR_BAD_ARG,
               "linear: bad output split");
-  RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear: fused norm only on the skinny path");
+  RAI_REQUIRE(a.ln_kind < 0 || linear_mfma_fuses_norm(a.M, a.K, a.ln_kind), RAI_ERR_UNSUPPORTED,
+              "linear: fused norm needs M <= 8, or an RMS norm with M <= 64 and K within one block's span");
   if (a.glu) RAI_REQUIRE(a.N % 8 == 0 && !a.residual && a.n_split == a.N && a.act >= 0, RAI_ERR_BAD_ARG,
                          "linear mfma: bad gated-MLP arguments");
   RAI_REQUIRE(a.K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear mfma: K=%d must be a multiple of 32", a.K);
