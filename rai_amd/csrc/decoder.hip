@@ -861,6 +861,23 @@ static int check_fault(rai_hip_decoder *d) {
               b, iv[0], iv[1], iv[2], iv[3], iv[4], iv[5], iv[6]);
     }
   }
+  if (d->mega_prof && getenv("RAI_HIP_MEGA_PROF_SKEW")) {  // how late each block reaches the end of each phase, mean over layers
+    std::vector<unsigned long long> t((size_t)d->num_cu * d->L * 16);
+    RAI_HIP_TRY(hipMemcpy(t.data(), d->mega_prof, t.size() * 8, hipMemcpyDeviceToHost));
+    auto at = [&](int b, int l, int k) { return (double)t[((size_t)b * d->L + l) * 16 + k] * 0.01; };
+    const int stamps[3] = {1, 4, 6};
+    for (int k = 0; k < 3; ++k) {
+      std::vector<double> late(d->num_cu, 0.0);
+      for (int l = 0; l < d->L; ++l) {
+        double mn = 1e30;
+        for (int b = 0; b < d->num_cu; ++b) mn = at(b, l, stamps[k]) < mn ? at(b, l, stamps[k]) : mn;
+        for (int b = 0; b < d->num_cu; ++b) late[b] += (at(b, l, stamps[k]) - mn) / d->L;
+      }
+      fprintf(stderr, "mega skew phase %c:", "ABC"[k]);
+      for (int b = 0; b < d->num_cu; ++b) fprintf(stderr, " %.1f", late[b]);
+      fprintf(stderr, "\n");
+    }
+  }
   if (hs.fault == 0) return RAI_OK;
   hs.fault = 0;
   RAI_HIP_TRY(hipMemcpy(&d->state->fault, &hs.fault, sizeof(int), hipMemcpyHostToDevice));
