@@ -970,7 +970,7 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   }
   // Tile choice.  The LDS-DMA kernels stream K tiles straight into LDS; the 256x128 tile halves the
   // L2 -> LDS traffic per flop for one operand and is used once there are enough tiles of that size
-  // to give every CU at least one; smaller products keep the 128x128 tile (three blocks per CU).
+  // to give every CU two; smaller products keep the 128x128 tile (three blocks per CU).
   // RAI_HIP_GEMM_TILE = "128x128" | "256x128" | "256x256" | "classic" overrides (tuning aid).
   const char *knob = getenv("RAI_HIP_GEMM_TILE");
   if (knob) {
@@ -980,6 +980,10 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
   }
   const int big_tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
+  const int huge_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
+  // 256x256 (one block per CU, 4 LDS stages) once the tile count covers three rounds over the CUs and K is
+  // long enough to amortise its prologue and epilogue: 950-1040 TFLOP/s on 8k-class products against 830-900
+  if (splits == 1 && huge_tiles >= 3 * kNumCU && a.K >= 2048) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
   return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
 }
