@@ -27,7 +27,7 @@ struct MegaArgs {
   int L, H, I, QD, NA, n_qkv, Hq, rot, Tmax;
   uint16_t *x;              // [H] residual stream, updated in place
   // Vectors exchanged between blocks inside the launch, as 8-byte packets {two bf16 values, 32-bit tag}:
-  // a packet is valid for an exchange when its tag is epoch * 128 + exchange index + 1.
+  // a packet is valid for an exchange when its tag is epoch * 1024 + exchange index + 1.
   uint64_t *xp;             // [H / 2]      residual stream after a layer
   uint64_t *qkvp;           // [3 * QD / 2]
   uint64_t *actp;           // [I / 2]      gelu(fc1)
@@ -40,8 +40,11 @@ struct MegaArgs {
   int act;
   int rows_attn;            // rows of phases B/C given to each attention block
   unsigned long long *prof; // optional [blocks][L][16] time stamps (debugging aid), or null
+  unsigned spin_limit;      // polling rounds after which a wait gives up and raises DevState::fault
+  int mute_block;           // test hook: this block sends no phase-A packets, so its consumers time out; -1 = none
 };
 
+unsigned mega_default_spin_limit();
 bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why);
 int launch_phi2_decode_step(hipStream_t st, const MegaArgs &a, int D, int num_cu);
 

@@ -13,7 +13,7 @@
 // hides behind the 52 MB fc2 stream of phase B.
 //
 // There is no grid barrier.  The vectors that cross blocks (x, q|k|v, act, attn) are
-// written as 8-byte packets {two bf16 values, 32-bit tag}, tag = launch epoch * 128 +
+// written as 8-byte packets {two bf16 values, 32-bit tag}, tag = launch epoch * 1024 +
 // exchange index + 1, with device-scope write-through stores, and every consumer
 // polls exactly the packets it needs with device-scope loads until their tags match
 // (an 8-byte store is single-copy atomic, so a matching tag proves the payload).
@@ -41,6 +41,7 @@ constexpr int kMegaThreads = 512, kMegaWaves = 8;
 
 constexpr int kMegaStream = kMegaWaves - 1, kMegaService = kMegaWaves - 1;
 constexpr unsigned kMegaSpinLimit = 1u << 20;
+constexpr uint32_t kMegaTagsPerLaunch = 1024;   // more than the 3 exchanges per layer of any eligible model
 constexpr int kMegaRing = 16;
 constexpr int kMegaRowsAMax = 96;
 constexpr int kMegaRowsMax = 16;
@@ -231,7 +232,7 @@ __device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r)
 // payloads.  The wave leaves the loop together; the spin is bounded.
 template <int N>
 __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N], const bool (&on)[N], uint32_t tag,
-                                        uint32_t (&out)[N], int *fault) {
+                                        uint32_t (&out)[N], int *fault, unsigned spin_limit) {
   bool need[N];
 #pragma unroll
   for (int i = 0; i < N; ++i) { need[i] = on[i]; out[i] = 0u; }
@@ -250,7 +251,7 @@ __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N]
     }
     if (!__any(pending)) break;
     __builtin_amdgcn_s_sleep(1);   // a short pause between rounds: bounds the polling traffic
-    if (++spins > kMegaSpinLimit) {
+    if (++spins > spin_limit) {
       __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
@@ -334,7 +335,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   cur.ptr = a.Wa0;
   cur.done = !mg_seg_next(cur, sp);
   unsigned bar = 0;
-  const uint32_t tagbase = a.state->epoch * 128u;   // exchange tags of this launch: tagbase + index + 1
+  const uint32_t tagbase = a.state->epoch * kMegaTagsPerLaunch;   // exchange tags of this launch: tagbase + index + 1
   uint32_t tag_x = 0;                                // tag of the residual-stream packets of the previous layer
   const float att_scale = a.scale;
   unsigned long long *const prof = a.prof;
@@ -435,7 +436,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           uint32_t val[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < H / 2; }
-          mg_poll<4>(a.xp, idx, on, tag_x, val, fault);
+          mg_poll<4>(a.xp, idx, on, tag_x, val, fault, a.spin_limit);
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
@@ -506,8 +507,10 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         }
         uint64_t *dst = n < a.n_qkv ? a.qkvp + (n >> 1) : a.actp + ((n - a.n_qkv) >> 1);
         const uint64_t tg = (uint64_t)(tagbase + bar + 1u) << 32;
-        st_dev64(dst, tg | packed[0]);
-        st_dev64(dst + 1, tg | packed[1]);
+        if (wg != a.mute_block) {
+          st_dev64(dst, tg | packed[0]);
+          st_dev64(dst + 1, tg | packed[1]);
+        }
       }
       stamp(l, 1);
       ++bar;   // no barrier: phase B polls the packets it needs
@@ -535,7 +538,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         uint32_t val[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < I / 2; }
-        mg_poll<4>(a.actp, idx, on, tag_a, val, fault);
+        mg_poll<4>(a.actp, idx, on, tag_a, val, fault, a.spin_limit);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (on[i]) reinterpret_cast<uint32_t *>(xs)[idx[i]] = val[i];
@@ -548,7 +551,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           bool on[1] = {tid < 3 * D / 2};
           if (!on[0]) idx[0] = 0;
           uint32_t val[1];
-          mg_poll<1>(a.qkvp, idx, on, tag_a, val, fault);
+          mg_poll<1>(a.qkvp, idx, on, tag_a, val, fault, a.spin_limit);
           if (on[0]) {
             raw[which * D + 2 * pe] = __uint_as_float(val[0] << 16);
             raw[which * D + 2 * pe + 1] = __uint_as_float(val[0] & 0xffff0000u);
@@ -673,7 +676,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         uint32_t val[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < QD / 2; }
-        mg_poll<4>(a.attnp, idx, on, tag_b, val, fault);
+        mg_poll<4>(a.attnp, idx, on, tag_b, val, fault, a.spin_limit);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
@@ -721,6 +724,8 @@ size_t mega_lds_bytes(const MegaArgs &a, int D) {
   return (n + 15) & ~(size_t)15;
 }
 
+unsigned mega_default_spin_limit() { return kMegaSpinLimit; }
+
 bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
   auto no = [&](const char *w) { if (why) *why = w; return false; };
   if (a.H != 2560) return no("hidden size is not 2560");
@@ -729,6 +734,7 @@ bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
   if (a.Hq > num_cu || num_cu > 256) return no("more heads than CUs, or more than 256 CUs");
   if (a.n_qkv != 3 * a.QD || a.NA != a.n_qkv + a.I || a.n_qkv % 4 || a.NA % 4) return no("q|k|v layout");
   if (a.rot > D || (a.rot & 1)) return no("rotary_dim");
+  if (3 * a.L >= (int)kMegaTagsPerLaunch) return no("too many layers for the exchange tags of one launch");
 
   const int others = num_cu - a.Hq;
   const int ra = others > 0 ? a.rows_attn : (a.H + a.Hq - 1) / a.Hq;

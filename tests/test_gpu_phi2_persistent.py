@@ -1,5 +1,5 @@
 """The persistent per-token decode kernel (Phi-2 width, bf16, batch 1): every layer of
-a single-token step in one launch with grid barriers.  Checked against the CPU oracle
+a single-token step in one launch, blocks exchanging vectors as tagged packets.  Checked against the CPU oracle
 (rai-models/src/llm/phi2.rs restated) and against the launch-per-primitive path of the
 same library."""
 import numpy as np
@@ -7,6 +7,7 @@ import pytest
 
 from oracle import phi2
 from tests.test_gpu_phi2 import check_tokens, make
+from rai_amd._lib import RaiHipError
 from tests.util import assert_close
 
 pytestmark = pytest.mark.gpu
@@ -63,3 +64,30 @@ def test_persistent_generate_equals_per_primitive_path(hip, monkeypatch):
             break
     plain.close()
     mega.close()
+
+
+def test_lost_packet_times_out_and_reports(hip, monkeypatch):
+    """A block whose phase-A packets never arrive: the waves waiting for them give up after the spin
+    limit, every wave of the launch still runs to its end, the call returns an error, and the decoder
+    works again afterwards.  The condition is forced from the host (a test hook drops the packets and
+    the spin limit is made tiny); nothing faults on the device."""
+    cfg = wide_cfg()
+    dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
+    ids = np.random.Generator(np.random.PCG64(13)).integers(0, cfg.vocab_size, (1, 9)).astype(np.uint32)
+    one = np.array([[7]], np.uint32)
+    dec.forward(ids)
+    monkeypatch.setenv("RAI_HIP_MEGA_SPIN_LIMIT", "400")
+    monkeypatch.setenv("RAI_HIP_MEGA_TEST_MUTE_BLOCK", "40")
+    with pytest.raises(RaiHipError) as e:
+        dec.forward(one)
+    assert e.value.status == -5 and "timed out" in str(e.value)   # RAI_ERR_HIP
+    monkeypatch.delenv("RAI_HIP_MEGA_SPIN_LIMIT")
+    monkeypatch.delenv("RAI_HIP_MEGA_TEST_MUTE_BLOCK")
+    dec.clear_kv_cache()
+    logits, _ = dec.forward(ids)
+    assert_close(logits, ref.fwd(ids), "bf16", "prefill after the fault")
+    logits, tok = dec.forward(one)
+    want = ref.fwd(one)
+    assert_close(logits, want, "bf16", "persistent step after the fault")
+    check_tokens(tok, want, "bf16")
+    dec.close()
