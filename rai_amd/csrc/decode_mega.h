@@ -40,8 +40,9 @@ struct MegaArgs {
   int act;
   int rows_attn;            // rows of phases B/C given to each attention block
   unsigned long long *prof; // optional [blocks][L][16] time stamps (debugging aid), or null
+  // Failure-path test hooks, honoured only by the instrumented build of the kernel (prof != null):
   unsigned spin_limit;      // polling rounds after which a wait gives up and raises DevState::fault
-  int mute_block;           // test hook: this block sends no phase-A packets, so its consumers time out; -1 = none
+  int mute_block;           // this block sends no phase-A packets, so its consumers time out; -1 = none
 };
 
 unsigned mega_default_spin_limit();

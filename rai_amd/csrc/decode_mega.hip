@@ -229,8 +229,9 @@ __device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r)
 }
 
 // Reads N packets per lane (packet i at src[idx[i]] when on[i]) until each carries `tag`; returns the
-// payloads.  The wave leaves the loop together; the spin is bounded.
-template <int N>
+// payloads.  The wave leaves the loop together; the spin is bounded (by kMegaSpinLimit; the instrumented
+// build of the kernel, DBG, takes the bound from the launch arguments so that a test can make it tiny).
+template <int N, bool DBG>
 __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N], const bool (&on)[N], uint32_t tag,
                                         uint32_t (&out)[N], int *fault, unsigned spin_limit) {
   bool need[N];
@@ -251,7 +252,7 @@ __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N]
     }
     if (!__any(pending)) break;
     __builtin_amdgcn_s_sleep(1);   // a short pause between rounds: bounds the polling traffic
-    if (++spins > spin_limit) {
+    if (++spins > (DBG ? spin_limit : kMegaSpinLimit)) {
       __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
@@ -436,7 +437,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           uint32_t val[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < H / 2; }
-          mg_poll<4>(a.xp, idx, on, tag_x, val, fault, a.spin_limit);
+          mg_poll<4, PROF>(a.xp, idx, on, tag_x, val, fault, a.spin_limit);
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
@@ -507,7 +508,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         }
         uint64_t *dst = n < a.n_qkv ? a.qkvp + (n >> 1) : a.actp + ((n - a.n_qkv) >> 1);
         const uint64_t tg = (uint64_t)(tagbase + bar + 1u) << 32;
-        if (wg != a.mute_block) {
+        if (!PROF || wg != a.mute_block) {
           st_dev64(dst, tg | packed[0]);
           st_dev64(dst + 1, tg | packed[1]);
         }
@@ -538,7 +539,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         uint32_t val[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < I / 2; }
-        mg_poll<4>(a.actp, idx, on, tag_a, val, fault, a.spin_limit);
+        mg_poll<4, PROF>(a.actp, idx, on, tag_a, val, fault, a.spin_limit);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (on[i]) reinterpret_cast<uint32_t *>(xs)[idx[i]] = val[i];
@@ -551,7 +552,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           bool on[1] = {tid < 3 * D / 2};
           if (!on[0]) idx[0] = 0;
           uint32_t val[1];
-          mg_poll<1>(a.qkvp, idx, on, tag_a, val, fault, a.spin_limit);
+          mg_poll<1, PROF>(a.qkvp, idx, on, tag_a, val, fault, a.spin_limit);
           if (on[0]) {
             raw[which * D + 2 * pe] = __uint_as_float(val[0] << 16);
             raw[which * D + 2 * pe + 1] = __uint_as_float(val[0] & 0xffff0000u);
@@ -676,7 +677,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         uint32_t val[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < QD / 2; }
-        mg_poll<4>(a.attnp, idx, on, tag_b, val, fault, a.spin_limit);
+        mg_poll<4, PROF>(a.attnp, idx, on, tag_b, val, fault, a.spin_limit);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];

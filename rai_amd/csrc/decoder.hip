@@ -570,7 +570,7 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   static const int rows_attn = getenv("RAI_HIP_MEGA_ROWS_ATTN") ? atoi(getenv("RAI_HIP_MEGA_ROWS_ATTN")) : 0;
   m.rows_attn = rows_attn;
   m.prof = d->mega_prof;
-  // Failure-path test hooks, read on every launch that is not replayed from a graph.
+  // Failure-path test hooks (instrumented kernel only), read on every launch that is not replayed from a graph.
   const char *sl = getenv("RAI_HIP_MEGA_SPIN_LIMIT"), *mb = getenv("RAI_HIP_MEGA_TEST_MUTE_BLOCK");
   m.spin_limit = sl && atoi(sl) > 0 ? (unsigned)atoi(sl) : mega_default_spin_limit();
   m.mute_block = mb ? atoi(mb) : -1;

@@ -72,7 +72,9 @@ def test_lost_packet_times_out_and_reports(hip, monkeypatch):
     works again afterwards.  The condition is forced from the host (a test hook drops the packets and
     the spin limit is made tiny); nothing faults on the device."""
     cfg = wide_cfg()
+    monkeypatch.setenv("RAI_HIP_MEGA_PROF", "1")    # the instrumented build of the kernel honours the two hooks
     dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
+    monkeypatch.delenv("RAI_HIP_MEGA_PROF")
     ids = np.random.Generator(np.random.PCG64(13)).integers(0, cfg.vocab_size, (1, 9)).astype(np.uint32)
     one = np.array([[7]], np.uint32)
     dec.forward(ids)
