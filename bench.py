@@ -338,6 +338,9 @@ def main():
     dcd = float(np.mean(dec_ms))
     decode_tok_s = (NEW - 1) / (dcd / 1e3)     # the prefill produces token 0; NEW-1 single-token steps follow
     prefill_tok_s = PROMPT / (pre / 1e3)
+    # the same loop with the example's token choice (repeat penalty 1.10 over the last 64 tokens, last maximum)
+    dec.generate_sampled(prompt, NEW)
+    _, _, _, samp_ms = dec.generate_sampled(prompt, NEW)
 
     # dominant kernel: the persistent per-token kernel that runs all layers of a decode step (weights, biases,
     # norm parameters and the KV cache of the current context once per launch), timed live with one hipEvent
@@ -370,6 +373,7 @@ def main():
         "prefill_frac_of_bf16_mfma_peak": round(prefill_flops(cfg, PROMPT) / (pre / 1e3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "weights_load_s": round(load_s, 1),
         "first_tokens": [int(t) for t in toks[0, :8]],
+        "sampled_decode_tokens_per_s": round((NEW - 1) / (samp_ms / 1e3), 2),
         "roofline": {
             "kernel": "k_phi2_decode_step (persistent kernel: all 32 layers of one decode step, blocks exchange "
                       "tagged packets instead of grid barriers, weight ring prefetched across phases)",

@@ -338,6 +338,23 @@ int rai_hip_decoder_forward(rai_hip_decoder *dec, const uint32_t *ids_host, int3
  * decode_ms (nullable) are hipEvent times of the two phases. */
 int rai_hip_decoder_generate(rai_hip_decoder *dec, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
                              int32_t n_new, uint32_t *tokens_host, float *prefill_ms, float *decode_ms);
+/* The whole loop of examples/phi2/src/main.rs:72-95 on the device: as rai_hip_decoder_generate, but each
+ * token is chosen as the example does: the logits row as f32, apply_repeat_penalty (main.rs:39-50) over the
+ * distinct ids among the last repeat_last_n tokens of the sequence so far (prompt included; a logit >= 0 is
+ * divided by the penalty, any other multiplied; skipped when repeat_penalty < 1, main.rs:79), then
+ * sample_argmax (main.rs:29-37): the maximum under f32 total order, the LAST one on ties.  The example uses
+ * penalty 1.10 over 64 tokens.  The device loop always runs n_new steps; n_generated[batch] (nullable)
+ * receives for each row the count the example's loop would have stopped at (it stops after pushing
+ * eos_token, main.rs:83-86; pass a negative eos_token for "none"). */
+int rai_hip_decoder_generate_sampled(rai_hip_decoder *dec, const uint32_t *prompt_host, int32_t batch,
+                                     int32_t prompt_len, int32_t n_new, float repeat_penalty, int32_t repeat_last_n,
+                                     int64_t eos_token, uint32_t *tokens_host, int32_t *n_generated, float *prefill_ms,
+                                     float *decode_ms);
+/* apply_repeat_penalty + sample_argmax (examples/phi2/src/main.rs:29-50) as a primitive: logits [rows, vocab]
+ * f32 or bf16, context [rows, n] u32 (null: no penalty), out [rows] u32.  Context ids outside the vocabulary
+ * are ignored, as the reference's set lookup ignores them. */
+int rai_hip_sample_argmax(int dev, const rai_hip_tensor *logits, const rai_hip_tensor *context, float repeat_penalty,
+                          const rai_hip_tensor *out);
 /* Model::clear_kv_cache (phi2.rs:349-353). */
 int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *dec);
 /* Current cached context length. */

@@ -121,6 +121,10 @@ PROTOTYPES = {
     "rai_hip_decoder_forward": [_vp, C.POINTER(C.c_uint32), _i32, _i32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)],
     "rai_hip_decoder_generate": [_vp, C.POINTER(C.c_uint32), _i32, _i32, _i32, C.POINTER(C.c_uint32),
                                  C.POINTER(C.c_float), C.POINTER(C.c_float)],
+    "rai_hip_decoder_generate_sampled": [_vp, C.POINTER(C.c_uint32), _i32, _i32, _i32, C.c_float, _i32, _i64,
+                                         C.POINTER(C.c_uint32), C.POINTER(_i32), C.POINTER(C.c_float),
+                                         C.POINTER(C.c_float)],
+    "rai_hip_sample_argmax": [C.c_int, _TP, _TP, C.c_float, _TP],
     "rai_hip_decoder_time_decode_linear": [_vp, _i32, C.POINTER(C.c_float), C.POINTER(C.c_double)],
     "rai_hip_decoder_time_decode_step": [_vp, _i32, C.POINTER(C.c_float), C.POINTER(C.c_double)],
     "rai_hip_decoder_clear_kv_cache": [_vp],

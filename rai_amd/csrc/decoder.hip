@@ -80,6 +80,15 @@ struct rai_hip_decoder {
   hipGraphExec_t step_graph_n; // kGraphSteps consecutive single-token steps in one graph (same batch)
   int step_graph_batch;
   bool x_holds_next;          // d->x already holds the embedding of d->tokens
+  // token choice of the example loop (repeat penalty, last maximum wins) instead of plain greedy argmax
+  bool sample_on;
+  float sample_penalty;
+  int sample_last_n;
+  uint32_t *token_log;        // [max_batch][token_log_cap]: every token of each sequence so far, prompt first
+  int token_log_cap;
+  bool graph_sampled;         // what the cached step graphs were captured with
+  float graph_penalty;
+  int graph_last_n;
 };
 
 namespace rai {
@@ -226,6 +235,35 @@ __global__ void k_set_state(DevState *st, int pos, int step) {
   st->done = 0;
 }
 
+// Tail of the token-selection kernels (every thread of the block calls it with the block's chosen token):
+// the token's embedding row becomes the next step's input x[b], and the last block to finish advances the
+// device-side context length / step counters and the exchange epoch of the persistent decode kernel.
+template <typename T>
+__device__ __forceinline__ void publish_token(uint32_t chosen, int b, DevState *state, int B, int dpos, int dstep,
+                                              const T *embed, T *x_next, int H, float embed_scale) {
+  if (x_next) {
+    const T *row = embed + (int64_t)chosen * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+      if (embed_scale != 1.0f)
+        Scalar<T>::store(x_next + (int64_t)b * H + c, (typename Scalar<T>::compute)((float)Scalar<T>::load(row + c) * embed_scale));
+      else
+        x_next[(int64_t)b * H + c] = row[c];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // no fence: `step` was read (and used for an address) before this point, and what this block wrote is
+    // consumed by later kernels only
+    int prev = atomicAdd(&state->done, 1);
+    if (prev == B - 1) {  // every block has read `step` and written its outputs
+      state->epoch += 1u;   // the next launch of the decode kernel tags its packets differently
+      state->done = 0;
+      state->pos += dpos;
+      state->step += dstep;
+    }
+  }
+}
+
 // Greedy token selection for every sequence, one 1024-thread block per row of
 // logits: argmax (first maximum wins; NaN never wins except at index 0), the
 // token goes to tokens[b] and to history[step][b], the token's embedding row
@@ -297,27 +335,114 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
     chosen = bi;
   }
   __syncthreads();
-  if (x_next) {
-    const T *row = embed + (int64_t)chosen * H;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
-      if (embed_scale != 1.0f)
-        Scalar<T>::store(x_next + (int64_t)b * H + c, (typename Scalar<T>::compute)((float)Scalar<T>::load(row + c) * embed_scale));
-      else
-        x_next[(int64_t)b * H + c] = row[c];
+  publish_token<T>(chosen, b, state, B, dpos, dstep, embed, x_next, H, embed_scale);
+}
+
+// The token choice of the reference's example loop (examples/phi2/src/main.rs:29-50,76-87): the logits
+// row as f32, the repeat penalty applied once to every token id that occurs among the last `last_n`
+// tokens of the sequence so far (a logit >= 0 is divided by the penalty, any other is multiplied by it;
+// skipped when the penalty is below 1), then the maximum under f32 total order (-NaN < -inf < ... < -0 <
+// +0 < ... < +inf < +NaN) with the LAST maximum winning, as Iterator::max_by does.  The membership set is
+// a bitmap over the vocabulary in LDS (words = ceil(n / 32)).  Returns the chosen index to every thread.
+__device__ __forceinline__ uint32_t total_order_key(float v) {
+  const uint32_t u = __float_as_uint(v);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+template <typename T>
+__device__ uint32_t sample_row(const T *x, int64_t n, const uint32_t *window, int wn, float penalty, uint32_t *bitmap,
+                               unsigned long long *s_best) {
+  const int words = (int)((n + 31) / 32);
+  const bool use_pen = penalty >= 1.0f && wn > 0;
+  if (use_pen) {
+    for (int w = threadIdx.x; w < words; w += blockDim.x) bitmap[w] = 0u;
+    __syncthreads();
+    for (int j = threadIdx.x; j < wn; j += blockDim.x) {
+      const uint32_t t = window[j];
+      if ((int64_t)t < n) atomicOr(&bitmap[t >> 5], 1u << (t & 31u));
     }
+    __syncthreads();
   }
+  // (key << 32 | index): the maximum of this composite is the largest key and, among equals, the largest index
+  unsigned long long best = 0ull;
+  auto visit = [&](float v, uint32_t i) {
+    if (use_pen && ((bitmap[i >> 5] >> (i & 31u)) & 1u)) v = v >= 0.0f ? v / penalty : v * penalty;
+    const unsigned long long c = ((unsigned long long)total_order_key(v) << 32) | i;
+    best = c > best ? c : best;
+  };
+  constexpr int VEC = 16 / sizeof(T);
+  if (n % VEC == 0 && ((uintptr_t)x & 15) == 0) {
+    struct alignas(16) Pack { T v[VEC]; };
+    const Pack *xp = reinterpret_cast<const Pack *>(x);
+    const int64_t chunks = n / VEC;
+    for (int64_t c0 = threadIdx.x; c0 < chunks; c0 += (int64_t)blockDim.x * 4) {
+      Pack pk[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + (int64_t)u * blockDim.x;
+        if (c < chunks) pk[u] = xp[c];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t c = c0 + (int64_t)u * blockDim.x;
+        if (c < chunks) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) visit((float)Scalar<T>::load(&pk[u].v[j]), (uint32_t)(c * VEC + j));
+        }
+      }
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) visit((float)Scalar<T>::load(x + i), (uint32_t)i);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned long long other = (unsigned long long)__shfl_xor((long long)best, o, 64);
+    best = other > best ? other : best;
+  }
+  if ((threadIdx.x & 63) == 0) s_best[threadIdx.x >> 6] = best;
   __syncthreads();
   if (threadIdx.x == 0) {
-    // no fence: `step` was read (and used for an address) before this point, and what this block wrote is
-    // consumed by later kernels only
-    int prev = atomicAdd(&state->done, 1);
-    if (prev == B - 1) {  // every block has read `step` and written its outputs
-      state->epoch += 1u;   // the next launch of the decode kernel tags its packets differently
-      state->done = 0;
-      state->pos += dpos;
-      state->step += dstep;
-    }
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) best = s_best[w] > best ? s_best[w] : best;
+    s_best[0] = best;
   }
+  __syncthreads();
+  return (uint32_t)(s_best[0] & 0xffffffffull);
+}
+
+// The penalised choice as a primitive: one block per row of logits; context[b] holds n_context token ids.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+k_sample_rows(const T *logits, int64_t n, const uint32_t *context, int n_context, float penalty, uint32_t *out) {
+  extern __shared__ uint32_t samp_bitmap[];
+  __shared__ unsigned long long s_best[16];
+  const int b = blockIdx.x;
+  const uint32_t tok = sample_row<T>(logits + (int64_t)b * n, n, context + (int64_t)b * n_context, n_context, penalty,
+                                     samp_bitmap, s_best);
+  if (threadIdx.x == 0) out[b] = tok;
+}
+
+// k_select_token with the example loop's token choice.  log[b] (capacity log_cap) holds every token of
+// sequence b so far, prompt first; the sequence has state->pos + dpos tokens when this runs, and the chosen
+// token is appended behind them.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+k_sample_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
+               int dstep, const T *embed, T *x_next, int H, float embed_scale, uint32_t *log, int log_cap,
+               float penalty, int last_n) {
+  extern __shared__ uint32_t samp_bitmap[];
+  __shared__ unsigned long long s_best[16];
+  const int b = blockIdx.x;
+  const int step = state->step;
+  int n_tok = state->pos + dpos;
+  if (n_tok > log_cap - 1) n_tok = log_cap - 1;   // cannot happen for a call that passed the host's checks
+  const int wn = n_tok < last_n ? n_tok : last_n;
+  uint32_t *row = log + (int64_t)b * log_cap;
+  const uint32_t tok = sample_row<T>(logits + (int64_t)b * n, n, row + (n_tok - wn), wn, penalty, samp_bitmap, s_best);
+  if (threadIdx.x == 0) {
+    tokens[b] = tok;
+    if (history) history[(int64_t)step * B + b] = tok;
+    row[n_tok] = tok;
+  }
+  publish_token<T>(tok, b, state, B, dpos, dstep, embed, x_next, H, embed_scale);
 }
 
 template <typename T>
@@ -577,6 +702,38 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   return m;
 }
 
+constexpr int64_t kSampleMaxVocab = 15 * 1024 * 32;  // the membership bitmap of the penalised choice takes vocab / 8 bytes of LDS
+
+// Chooses the next token of every sequence from d->logits: plain greedy argmax, or the example loop's
+// choice when the decoder is in sampling mode.
+static int launch_token_choice(rai_hip_decoder *d, hipStream_t st, int B, int S, bool advance_step) {
+  const int dt = d->cfg.dtype;
+  uint32_t *hist = advance_step ? d->history : nullptr;
+  const int dstep = advance_step ? 1 : 0;
+  if (d->sample_on) {
+    const size_t lds = (size_t)((d->V + 31) / 32) * sizeof(uint32_t);
+    if (dt == RAI_BF16)
+      hipLaunchKernelGGL((k_sample_token<bf16_raw>), dim3(B), dim3(1024), lds, st, (const bf16_raw *)d->logits,
+                         (int64_t)d->V, d->tokens, hist, d->state, B, S, dstep, (const bf16_raw *)d->embed,
+                         (bf16_raw *)d->x, d->H, d->embed_scale, d->token_log, d->token_log_cap, d->sample_penalty,
+                         d->sample_last_n);
+    else
+      hipLaunchKernelGGL((k_sample_token<float>), dim3(B), dim3(1024), lds, st, (const float *)d->logits,
+                         (int64_t)d->V, d->tokens, hist, d->state, B, S, dstep, (const float *)d->embed, (float *)d->x,
+                         d->H, d->embed_scale, d->token_log, d->token_log_cap, d->sample_penalty, d->sample_last_n);
+    return launch_check("sample_token");
+  }
+  if (dt == RAI_BF16)
+    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
+                       (int64_t)d->V, d->tokens, hist, d->state, B, S, dstep, (const bf16_raw *)d->embed,
+                       (bf16_raw *)d->x, d->H, d->embed_scale);
+  else
+    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
+                       d->tokens, hist, d->state, B, S, dstep, (const float *)d->embed, (float *)d->x, d->H,
+                       d->embed_scale);
+  return launch_check("select_token");
+}
+
 // ids (B*S u32) are already in d->ids; device state holds the context length.
 // With from_tokens the input embeddings were already written to d->x by the
 // previous step's token selection (single-token steps only).
@@ -688,16 +845,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
   RAI_TRY(linear(d, st, h));
 
-  uint32_t *hist = advance_step ? d->history : nullptr;
-  if (dt == RAI_BF16)
-    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
-                       (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale);
-  else
-    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
-                       d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale);
-  RAI_TRY(launch_check("select_token"));
+  RAI_TRY(launch_token_choice(d, st, B, S, advance_step));
   d->ctx_len = T_after;
   return RAI_OK;
 }
@@ -826,16 +974,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
   RAI_TRY(linear(d, st, h));
 
-  uint32_t *hist = advance_step ? d->history : nullptr;
-  if (dt == RAI_BF16)
-    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
-                       (int64_t)d->V, d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, H, d->embed_scale);
-  else
-    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
-                       d->tokens, hist, d->state, B, S, advance_step ? 1 : 0, (const float *)d->embed, (float *)d->x, H,
-                       d->embed_scale);
-  RAI_TRY(launch_check("select_token"));
+  RAI_TRY(launch_token_choice(d, st, B, S, advance_step));
   d->ctx_len = T_after;
   return RAI_OK;
 }
@@ -935,6 +1074,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->step_graph_n = nullptr;
   d->step_graph_batch = 0;
   d->x_holds_next = false;
+  d->sample_on = false; d->sample_penalty = 0.f; d->sample_last_n = 0;
+  d->token_log = nullptr; d->token_log_cap = 0;
+  d->graph_sampled = false; d->graph_penalty = 0.f; d->graph_last_n = 0;
   const int vec = (int)(16 / d->es);
   int st = RAI_OK;
   auto bail = [&](int code) {
@@ -967,6 +1109,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->tokens = (uint32_t *)tmp;
   if ((st = dalloc(d, (size_t)d->history_cap * cfg->max_batch * sizeof(uint32_t), &tmp))) return bail(st);
   d->history = (uint32_t *)tmp;
+  d->token_log_cap = cfg->max_context + 1;
+  if ((st = dalloc(d, (size_t)d->token_log_cap * cfg->max_batch * sizeof(uint32_t), &tmp))) return bail(st);
+  d->token_log = (uint32_t *)tmp;
   if ((st = dalloc(d, sizeof(DevState), &tmp))) return bail(st);
   d->state = (DevState *)tmp;
   d->splitk_ws_bytes = (size_t)8 * d->max_rows * d->H * sizeof(float);
@@ -1109,8 +1254,9 @@ int rai_hip_decoder_forward(rai_hip_decoder *d, const uint32_t *ids_host, int32_
   return RAI_OK;
 }
 
-int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
-                             int32_t n_new, uint32_t *tokens_host, float *prefill_ms, float *decode_ms) {
+// The loop of both generate entry points; d->sample_on selects the token choice.
+static int generate_impl(rai_hip_decoder *d, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                         int32_t n_new, uint32_t *tokens_host, float *prefill_ms, float *decode_ms) {
   RAI_REQUIRE(prompt_host && tokens_host, RAI_ERR_BAD_ARG, "null argument");
   RAI_REQUIRE(n_new >= 1, RAI_ERR_BAD_ARG, "generate: n_new must be >= 1");
   RAI_TRY(rai_hip_decoder_clear_kv_cache(d));
@@ -1118,6 +1264,10 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
   RAI_REQUIRE(prompt_len + n_new - 1 <= d->cfg.max_context && n_new <= d->history_cap, RAI_ERR_BAD_SHAPE,
               "generate: %d + %d tokens exceed max_context %d", prompt_len, n_new, d->cfg.max_context);
   hipStream_t st = stream_of(d->dev);
+  if (d->sample_on)   // the token log starts as the prompt, one row per sequence
+    RAI_HIP_TRY(hipMemcpy2DAsync(d->token_log, (size_t)d->token_log_cap * sizeof(uint32_t), prompt_host,
+                                 (size_t)prompt_len * sizeof(uint32_t), (size_t)prompt_len * sizeof(uint32_t), batch,
+                                 hipMemcpyHostToDevice, st));
   hipEvent_t e0, e1, e2;
   RAI_HIP_TRY(hipEventCreate(&e0));
   RAI_HIP_TRY(hipEventCreate(&e1));
@@ -1156,10 +1306,14 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
     rc = forward_any(d, batch, 1, true, true);
     ++step;
   }
-  if (rc == RAI_OK && use_graph && d->step_graph_batch != batch) {
+  // the recorded launches bake in the batch and the token choice with its parameters
+  const bool same_choice = d->graph_sampled == d->sample_on &&
+                           (!d->sample_on || (d->graph_penalty == d->sample_penalty && d->graph_last_n == d->sample_last_n));
+  if (rc == RAI_OK && use_graph && (d->step_graph_batch != batch || !same_choice)) {
     if (d->step_graph) { (void)hipGraphExecDestroy(d->step_graph); d->step_graph = nullptr; }
     if (d->step_graph_n) { (void)hipGraphExecDestroy(d->step_graph_n); d->step_graph_n = nullptr; }
     d->step_graph_batch = batch;
+    d->graph_sampled = d->sample_on; d->graph_penalty = d->sample_penalty; d->graph_last_n = d->sample_last_n;
   }
   while (rc == RAI_OK && step < n_new) {
     const int left = n_new - step;
@@ -1202,6 +1356,74 @@ int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, in
     RAI_REQUIRE(bad == 0, RAI_ERR_INDEX, "decoder: %llu token ids outside the vocabulary", (unsigned long long)bad);
   }
   return rc;
+}
+
+int rai_hip_sample_argmax(int dev, const rai_hip_tensor *logits, const rai_hip_tensor *context, float repeat_penalty,
+                          const rai_hip_tensor *out) {
+  RAI_TRY(validate(logits, "logits"));
+  RAI_TRY(validate(out, "out"));
+  RAI_REQUIRE(logits->rank == 2 && is_contiguous(logits), RAI_ERR_BAD_SHAPE, "sample_argmax: logits must be contiguous [rows, vocab]");
+  RAI_REQUIRE(logits->dtype == RAI_F32 || logits->dtype == RAI_BF16, RAI_ERR_BAD_DTYPE, "sample_argmax: logits dtype %s",
+              dtype_name(logits->dtype));
+  const int64_t rows = logits->shape[0], V = logits->shape[1];
+  RAI_REQUIRE(V >= 1 && V <= kSampleMaxVocab, RAI_ERR_BAD_SHAPE, "sample_argmax: vocabulary %lld outside 1..%lld", (long long)V,
+              (long long)kSampleMaxVocab);
+  RAI_REQUIRE(out->dtype == RAI_U32 && out->rank == 1 && out->shape[0] == rows && is_contiguous(out), RAI_ERR_BAD_SHAPE,
+              "sample_argmax: out must be contiguous u32 [rows]");
+  RAI_REQUIRE(repeat_penalty == repeat_penalty, RAI_ERR_BAD_ARG, "sample_argmax: repeat_penalty is NaN");
+  int n_ctx = 0;
+  const uint32_t *ctx = nullptr;
+  if (context) {
+    RAI_TRY(validate(context, "context"));
+    RAI_REQUIRE(context->dtype == RAI_U32 && context->rank == 2 && context->shape[0] == rows && is_contiguous(context),
+                RAI_ERR_BAD_SHAPE, "sample_argmax: context must be contiguous u32 [rows, n]");
+    RAI_REQUIRE(context->shape[1] <= (1 << 20), RAI_ERR_BAD_SHAPE, "sample_argmax: context too long");
+    n_ctx = (int)context->shape[1];
+    ctx = (const uint32_t *)base_ptr(context);
+  }
+  if (rows == 0) return RAI_OK;
+  hipStream_t st = stream_of(dev);
+  if (!st) return RAI_ERR_HIP;
+  const size_t lds = (size_t)((V + 31) / 32) * sizeof(uint32_t);
+  if (logits->dtype == RAI_BF16)
+    hipLaunchKernelGGL((k_sample_rows<bf16_raw>), dim3((unsigned)rows), dim3(1024), lds, st, (const bf16_raw *)base_ptr(logits),
+                       V, ctx, n_ctx, repeat_penalty, (uint32_t *)base_ptr(out));
+  else
+    hipLaunchKernelGGL((k_sample_rows<float>), dim3((unsigned)rows), dim3(1024), lds, st, (const float *)base_ptr(logits), V,
+                       ctx, n_ctx, repeat_penalty, (uint32_t *)base_ptr(out));
+  return launch_check("sample_rows");
+}
+
+int rai_hip_decoder_generate(rai_hip_decoder *d, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                             int32_t n_new, uint32_t *tokens_host, float *prefill_ms, float *decode_ms) {
+  RAI_REQUIRE(d, RAI_ERR_BAD_ARG, "decoder is null");
+  d->sample_on = false;
+  return generate_impl(d, prompt_host, batch, prompt_len, n_new, tokens_host, prefill_ms, decode_ms);
+}
+
+int rai_hip_decoder_generate_sampled(rai_hip_decoder *d, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                                     int32_t n_new, float repeat_penalty, int32_t repeat_last_n, int64_t eos_token,
+                                     uint32_t *tokens_host, int32_t *n_generated, float *prefill_ms, float *decode_ms) {
+  RAI_REQUIRE(d, RAI_ERR_BAD_ARG, "decoder is null");
+  RAI_REQUIRE(repeat_last_n >= 0, RAI_ERR_BAD_ARG, "generate_sampled: repeat_last_n must be >= 0");
+  RAI_REQUIRE(repeat_penalty == repeat_penalty, RAI_ERR_BAD_ARG, "generate_sampled: repeat_penalty is NaN");
+  RAI_REQUIRE(d->V <= kSampleMaxVocab, RAI_ERR_UNSUPPORTED, "generate_sampled: vocabulary %d above %lld", d->V,
+              (long long)kSampleMaxVocab);
+  d->sample_on = true;
+  d->sample_penalty = repeat_penalty;
+  d->sample_last_n = repeat_last_n;
+  const int rc = generate_impl(d, prompt_host, batch, prompt_len, n_new, tokens_host, prefill_ms, decode_ms);
+  d->sample_on = false;
+  RAI_TRY(rc);
+  // the example loop stops after it has pushed the end-of-text token (main.rs:83-86): report how many tokens
+  // of each row it would have produced; the entries behind them are what a loop without the stop generates
+  for (int b = 0; n_generated && b < batch; ++b) {
+    int n = n_new;
+    for (int s = 0; eos_token >= 0 && s < n_new; ++s)
+      if ((int64_t)tokens_host[(size_t)b * n_new + s] == eos_token) { n = s + 1; break; }
+    n_generated[b] = n;
+  }
+  return RAI_OK;
 }
 
 int rai_hip_decoder_time_decode_step(rai_hip_decoder *d, int32_t sweeps, float *us_per_launch,

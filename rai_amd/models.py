@@ -100,6 +100,20 @@ class Decoder:
              toks.ctypes.data_as(C.POINTER(C.c_uint32)), C.byref(pm), C.byref(dm))
         return toks, pm.value, dm.value
 
+    def generate_sampled(self, prompt, n_new, repeat_penalty=1.10, repeat_last_n=64, eos_token=None):
+        """The example loop (examples/phi2/src/main.rs:72-95) with its repeat penalty and last-maximum
+        argmax: returns (tokens [B, n_new], n_generated [B], prefill_ms, decode_ms)."""
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        b, s = prompt.shape
+        toks = np.empty((b, n_new), np.uint32)
+        ngen = np.empty((b,), np.int32)
+        pm, dm = C.c_float(0), C.c_float(0)
+        call("rai_hip_decoder_generate_sampled", self._h, prompt.ctypes.data_as(C.POINTER(C.c_uint32)), b, s, n_new,
+             float(repeat_penalty), int(repeat_last_n), -1 if eos_token is None else int(eos_token),
+             toks.ctypes.data_as(C.POINTER(C.c_uint32)), ngen.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(pm),
+             C.byref(dm))
+        return toks, ngen, pm.value, dm.value
+
     def clear_kv_cache(self):
         call("rai_hip_decoder_clear_kv_cache", self._h)
 

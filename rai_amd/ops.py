@@ -123,6 +123,15 @@ def argmax(x, dim, keep_dim=False, _fn="rai_hip_argmax"):
     return out
 
 
+def sample_argmax(logits, context=None, repeat_penalty=1.10):
+    """apply_repeat_penalty + sample_argmax of examples/phi2/src/main.rs:29-50: logits [rows, vocab],
+    context [rows, n] u32 or None -> tokens [rows] u32."""
+    out = HipTensor.empty((logits.shape[0],), U32, logits.dev)
+    call("rai_hip_sample_argmax", logits.dev, _d(logits), None if context is None else _d(context),
+         float(repeat_penalty), _d(out))
+    return out
+
+
 def argmin(x, dim, keep_dim=False):
     return argmax(x, dim, keep_dim, "rai_hip_argmin")
 
