@@ -216,6 +216,23 @@ int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_
  * offending row is zero-filled. */
 int rai_hip_index_select(int dev, const rai_hip_tensor *in, const rai_hip_tensor *index, int32_t dim,
                          const rai_hip_tensor *out);
+/* Gather: candle.rs:838-849, ops/gather.rs:47-60.  x and index have equal rank and equal extents off `dim`;
+ * out has index's shape and x's dtype: out[.., j, ..] = x[.., index[.., j, ..], ..].  Contiguous operands
+ * (the reference makes the index contiguous itself, candle.rs:845).  Out-of-range indices as index_select. */
+int rai_hip_gather(int dev, const rai_hip_tensor *x, const rai_hip_tensor *index, int32_t dim, const rai_hip_tensor *out);
+/* IndexAdd: candle.rs:851-865, ops/index_add.rs:52-62 (the vjp of IndexSelect, ops/index_select.rs:40-48).
+ * index is rank 1 (u8/u32/i64), source has x's shape with extent len(index) on `dim`:
+ * out = x, then out[.., index[l], ..] += source[.., l, ..] for l = 0, 1, ... in that order, each sum rounded
+ * to the dtype.  x, source and out contiguous; out may alias x.  An out-of-range index contributes nothing
+ * and makes the next synchronising call fail with RAI_ERR_INDEX. */
+int rai_hip_index_add(int dev, const rai_hip_tensor *x, const rai_hip_tensor *index, const rai_hip_tensor *source,
+                      int32_t dim, const rai_hip_tensor *out);
+/* ScatterAdd: candle.rs:990-1004, ops/scatter_add.rs:52-60 (the vjp of Gather, ops/gather.rs:36-43).
+ * index and source share one shape with x's rank and x's extents off `dim`:
+ * out = x, then out[.., index[.., j, ..], ..] += source[.., j, ..] for j = 0, 1, ... in that order, each sum
+ * rounded to the dtype.  Contiguous operands; out-of-range indices as index_add. */
+int rai_hip_scatter_add(int dev, const rai_hip_tensor *x, const rai_hip_tensor *index, const rai_hip_tensor *source,
+                        int32_t dim, const rai_hip_tensor *out);
 /* Number of out-of-range indices seen by gathers since the last call (syncs). */
 int rai_hip_index_errors(int dev, uint64_t *count);
 

@@ -240,6 +240,69 @@ def index_select(x, dim, index):
     return np.take(x, index, axis=dim)
 
 
+def gather(x, dim, index):
+    """Gather: candle.rs:838-849, ops/gather.rs:47-60: out[.., j, ..] = x[.., index[.., j, ..], ..]; out has
+    index's shape.  Known answer rai-core/tests/ops.rs:156-161."""
+    x = np.asarray(x)
+    index = np.asarray(index).astype(np.int64)
+    d = dim % x.ndim
+    if x.ndim != index.ndim or any(i != d and x.shape[i] != index.shape[i] for i in range(x.ndim)):
+        raise ValueError("gather: shape mismatch")
+    if index.size and (index.min() < 0 or index.max() >= x.shape[d]):
+        raise IndexError("gather: index out of range")
+    return np.take_along_axis(x, index, axis=d)
+
+
+def _add_in_dtype(a, b, dt):
+    if dt in ("bf16", "f16", "f32", "f64"):
+        return rnd(a + b, dt)
+    with np.errstate(over="ignore"):      # integer dtypes wrap
+        return (np.asarray(a) + np.asarray(b)).astype(np.asarray(a).dtype)
+
+
+def index_add(x, dim, index, source, dt):
+    """IndexAdd: candle.rs:851-865, ops/index_add.rs:52-62: out = x; out[.., index[l], ..] += source[.., l, ..]
+    for l in order, every sum rounded to the storage dtype ([candle, unverified]: its Cpu loop adds in place
+    in the element type, source row by source row)."""
+    out = np.array(x, copy=True)
+    index = np.asarray(index).reshape(-1).astype(np.int64)
+    d = dim % out.ndim
+    source = np.asarray(source)
+    want = list(out.shape)
+    want[d] = index.size
+    if list(source.shape) != want:
+        raise ValueError("index_add: shape mismatch")
+    if index.size and (index.min() < 0 or index.max() >= out.shape[d]):
+        raise IndexError("index_add: index out of range")
+    o = np.moveaxis(out, d, 0)          # views: writes land in `out`
+    s = np.moveaxis(source, d, 0)
+    for l, r in enumerate(index):
+        o[r] = _add_in_dtype(o[r], s[l], dt)
+    return out
+
+
+def scatter_add(x, dim, index, source, dt):
+    """ScatterAdd: candle.rs:990-1004, ops/scatter_add.rs:52-60: out = x;
+    out[.., index[.., j, ..], ..] += source[.., j, ..] for j in order, every sum rounded to the storage dtype."""
+    out = np.array(x, copy=True)
+    index = np.asarray(index).astype(np.int64)
+    source = np.asarray(source)
+    d = dim % out.ndim
+    if index.shape != source.shape or index.ndim != out.ndim or any(
+            i != d and out.shape[i] != index.shape[i] for i in range(out.ndim)):
+        raise ValueError("scatter_add: shape mismatch")
+    if index.size and (index.min() < 0 or index.max() >= out.shape[d]):
+        raise IndexError("scatter_add: index out of range")
+    o = np.moveaxis(out, d, -1)         # [..., D] view
+    ix = np.moveaxis(index, d, -1)
+    sr = np.moveaxis(source, d, -1)
+    lead = np.indices(ix.shape[:-1]) if ix.ndim > 1 else ()
+    for j in range(ix.shape[-1]):
+        sel = tuple(lead) + (ix[..., j],)
+        o[sel] = _add_in_dtype(o[sel], sr[..., j], dt)
+    return out
+
+
 def narrow(x, dim, start, length):
     """Narrow: candle.rs:891-899."""
     sl = [slice(None)] * np.ndim(x)

@@ -102,6 +102,9 @@ PROTOTYPES = {
     "rai_hip_argmax": [C.c_int, _TP, _i32, _i32, _TP],
     "rai_hip_argmin": [C.c_int, _TP, _i32, _i32, _TP],
     "rai_hip_index_select": [C.c_int, _TP, _TP, _i32, _TP],
+    "rai_hip_gather": [C.c_int, _TP, _TP, _i32, _TP],
+    "rai_hip_index_add": [C.c_int, _TP, _TP, _TP, _i32, _TP],
+    "rai_hip_scatter_add": [C.c_int, _TP, _TP, _TP, _i32, _TP],
     "rai_hip_index_errors": [C.c_int, C.POINTER(C.c_uint64)],
     "rai_hip_matmul": [C.c_int, _TP, _TP, _TP],
     "rai_hip_linear": [C.c_int, _TP, _TP, _TP, _i32, _TP, _TP],

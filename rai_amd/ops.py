@@ -146,6 +146,30 @@ def index_select(x, dim, index):
     return out
 
 
+def gather(x, dim, index):
+    """Tensor::gather (ops/gather.rs:47-60): out has index's shape."""
+    d = dim % x.rank
+    out = HipTensor.empty(index.shape, x.dtype, x.dev)
+    call("rai_hip_gather", x.dev, _d(x), _d(index), d, _d(out))
+    return out
+
+
+def index_add(x, dim, index, source):
+    """Tensor::index_add (ops/index_add.rs:52-62)."""
+    d = dim % x.rank
+    out = HipTensor.empty(x.shape, x.dtype, x.dev)
+    call("rai_hip_index_add", x.dev, _d(x), _d(index), _d(source), d, _d(out))
+    return out
+
+
+def scatter_add(x, dim, index, source):
+    """Tensor::scatter_add (ops/scatter_add.rs:52-60)."""
+    d = dim % x.rank
+    out = HipTensor.empty(x.shape, x.dtype, x.dev)
+    call("rai_hip_scatter_add", x.dev, _d(x), _d(index), _d(source), d, _d(out))
+    return out
+
+
 def index_errors(dev=0):
     n = C.c_uint64(0)
     call("rai_hip_index_errors", dev, C.byref(n))
