@@ -271,7 +271,24 @@ def run_ops(args):
         lu, su = timed(lambda: ops.index_select(table, 0, ids), 50)
         rows.append(dict(op="index_select 4096 of [51200,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
                          achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
-        del table
+        # the gradient of that embedding lookup: cotangent rows added into the table at the ids
+        ct = rnd((4096, 2560), dt)
+        by = (2.0 * 51200 * 2560 + 4096 * 2560) * es      # table read + written once, cotangent read once
+        lu, su = timed(lambda: ops.index_add(table, 0, ids, ct), 20)
+        rows.append(dict(op="index_add 4096 rows into [51200,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
+                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        logits = rnd((64, 51200), dt)
+        tgt = HipTensor.from_storage(rng.integers(0, 51200, (64, 1)).astype(np.uint32), "u32")
+        by = 64.0 * (es + 4) + 64 * es
+        lu, su = timed(lambda: ops.gather(logits, 1, tgt), 50)
+        rows.append(dict(op="gather [64,51200] dim 1, one id per row", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
+                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        one = rnd((64, 1), dt)
+        by = 2.0 * 64 * 51200 * es
+        lu, su = timed(lambda: ops.scatter_add(logits, 1, tgt, one), 50)
+        rows.append(dict(op="scatter_add [64,1] into [64,51200] dim 1", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
+                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        del table, ct, logits
         x = rnd((64, 51200), dt)
         by = 1.0 * x.numel() * es
         lu, su = timed(lambda: ops.argmax(x, -1), 50)

@@ -53,6 +53,9 @@ typedef enum rai_op_kind {
   RAI_OP_BROADCAST = 19,
   RAI_OP_TO_CONTIGUOUS = 20,
   RAI_OP_ERR = 21,
+  RAI_OP_GATHER = 22,
+  RAI_OP_INDEX_ADD = 23,   /* inputs ordered [x, source, index] (ops/index_add.rs:57-59) */
+  RAI_OP_SCATTER_ADD = 24, /* inputs ordered [x, source, index] (ops/scatter_add.rs:57) */
   RAI_OP_COUNT_
 } rai_op_kind;
 
@@ -73,6 +76,11 @@ rai_tensor *rai_reduce(int32_t op, rai_tensor *x, const int32_t *dims, int32_t n
 rai_tensor *rai_argmax(rai_tensor *x, int32_t dim, int32_t keep_dim);
 rai_tensor *rai_argmin(rai_tensor *x, int32_t dim, int32_t keep_dim);
 rai_tensor *rai_index_select(rai_tensor *x, int32_t dim, rai_tensor *index);
+/* ops/gather.rs:47-60, ops/index_add.rs:52-62, ops/scatter_add.rs:52-60 (the primitives the vjp rules of
+ * index_select and gather evaluate); a shape the reference asserts on gives an error node. */
+rai_tensor *rai_gather(rai_tensor *x, int32_t dim, rai_tensor *index);
+rai_tensor *rai_index_add(rai_tensor *x, int32_t dim, rai_tensor *index, rai_tensor *source);
+rai_tensor *rai_scatter_add(rai_tensor *x, int32_t dim, rai_tensor *index, rai_tensor *source);
 rai_tensor *rai_narrow(rai_tensor *x, int32_t dim, int64_t start, int64_t len);
 rai_tensor *rai_concatenate(rai_tensor *const *xs, int32_t n, int32_t dim);
 rai_tensor *rai_where(rai_tensor *cond, rai_tensor *on_true, rai_tensor *on_false);

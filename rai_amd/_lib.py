@@ -157,6 +157,9 @@ GRAPH_PROTOTYPES = {
     "rai_argmax": (_T, [_T, _i32, _i32]),
     "rai_argmin": (_T, [_T, _i32, _i32]),
     "rai_index_select": (_T, [_T, _i32, _T]),
+    "rai_gather": (_T, [_T, _i32, _T]),
+    "rai_index_add": (_T, [_T, _i32, _T, _T]),
+    "rai_scatter_add": (_T, [_T, _i32, _T, _T]),
     "rai_narrow": (_T, [_T, _i32, _i64, _i64]),
     "rai_concatenate": (_T, [C.POINTER(_T), _i32, _i32]),
     "rai_where": (_T, [_T, _T, _T]),

@@ -209,6 +209,52 @@ int ev_index_select(rai_tensor *t) {
   ++g_stats.kernel_launches;
   return rai_hip_index_select(t->dev, &t->inputs[0]->view, &t->inputs[1]->view, (int32_t)t->ip[0], &t->view);
 }
+// A contiguous stand-in for an input view (the reference does the same with `.contiguous()`,
+// candle.rs:845,998-999); `tmp` owns the copy, if one was needed, until the rule returns.
+struct TempContiguous {
+  void *buf = nullptr;
+  rai_hip_tensor view;
+  int make(int dev, const rai_hip_tensor &src) {
+    view = src;
+    if (is_contiguous(&src)) return RAI_OK;
+    int64_t n = 1;
+    for (int i = 0; i < src.rank; ++i) n *= src.shape[i];
+    const size_t bytes = (size_t)n * dtype_size(src.dtype);
+    RAI_TRY(rai_hip_alloc(dev, bytes ? bytes : 1, &buf));
+    view.data = buf;
+    view.offset = 0;
+    int64_t st = 1;
+    for (int i = src.rank - 1; i >= 0; --i) { view.stride[i] = st; st *= src.shape[i]; }
+    ++g_stats.kernel_launches;
+    return rai_hip_copy(dev, &src, &view);
+  }
+  ~TempContiguous() { if (buf) (void)rai_hip_release(buf); }
+};
+int ev_gather(rai_tensor *t) {
+  RAI_TRY(alloc_output(t));
+  TempContiguous x, ix;
+  RAI_TRY(x.make(t->dev, t->inputs[0]->view));
+  RAI_TRY(ix.make(t->dev, t->inputs[1]->view));
+  ++g_stats.kernel_launches;
+  return rai_hip_gather(t->dev, &x.view, &ix.view, (int32_t)t->ip[0], &t->view);
+}
+int ev_index_add(rai_tensor *t) {  // inputs are ordered [x, source, index]
+  RAI_TRY(alloc_output(t));
+  TempContiguous x, src;
+  RAI_TRY(x.make(t->dev, t->inputs[0]->view));
+  RAI_TRY(src.make(t->dev, t->inputs[1]->view));
+  ++g_stats.kernel_launches;
+  return rai_hip_index_add(t->dev, &x.view, &t->inputs[2]->view, &src.view, (int32_t)t->ip[0], &t->view);
+}
+int ev_scatter_add(rai_tensor *t) {  // inputs are ordered [x, source, index]
+  RAI_TRY(alloc_output(t));
+  TempContiguous x, src, ix;
+  RAI_TRY(x.make(t->dev, t->inputs[0]->view));
+  RAI_TRY(src.make(t->dev, t->inputs[1]->view));
+  RAI_TRY(ix.make(t->dev, t->inputs[2]->view));
+  ++g_stats.kernel_launches;
+  return rai_hip_scatter_add(t->dev, &x.view, &ix.view, &src.view, (int32_t)t->ip[0], &t->view);
+}
 int ev_where(rai_tensor *t) {  // inputs are ordered [on_true, on_false, cond] (ops/where.rs:37-45)
   RAI_TRY(alloc_output(t));
   ++g_stats.kernel_launches;
@@ -309,7 +355,7 @@ int ev_reshape(rai_tensor *t) {
 const rule_fn kBuiltin[RAI_OP_COUNT_] = {
     ev_full, ev_arange, ev_from_array, ev_to_dtype, ev_unary, ev_binary, ev_matmul, ev_softmax, ev_log_softmax, ev_reduce,
     ev_argmax, ev_argmin, ev_index_select, ev_narrow, ev_concatenate, ev_where, ev_transpose, ev_reshape, ev_permute,
-    ev_broadcast, ev_to_contiguous, nullptr /* Err nodes never reach a rule */};
+    ev_broadcast, ev_to_contiguous, nullptr /* Err nodes never reach a rule */, ev_gather, ev_index_add, ev_scatter_add};
 rule_fn g_rules[RAI_OP_COUNT_];
 bool g_rules_init = false;
 void init_rules() {
@@ -322,7 +368,7 @@ const char *op_name(int op) {
   static const char *n[RAI_OP_COUNT_] = {"Full", "Arange", "FromArray", "ToDType", "Unary", "Binary", "MatMul", "Softmax",
                                          "LogSoftmax", "Reduce", "ArgMax", "ArgMin", "IndexSelect", "Narrow",
                                          "Concatenate", "Where", "Transpose", "Reshape", "Permute", "Broadcast",
-                                         "ToContiguous", "Err"};
+                                         "ToContiguous", "Err", "Gather", "IndexAdd", "ScatterAdd"};
   return op >= 0 && op < RAI_OP_COUNT_ ? n[op] : "?";
 }
 
@@ -673,6 +719,50 @@ rai_tensor *rai_index_select(rai_tensor *x, int32_t dim, rai_tensor *index) {
   std::vector<int64_t> shape = x->shape;
   shape[d] = numel_of(index->shape);
   rai_tensor *t = new_node(x->dev, x->dtype, shape, RAI_OP_INDEX_SELECT, {x, index});
+  t->ip = {d};
+  return t;
+}
+
+static bool index_dtype(int dt) { return dt == RAI_U8 || dt == RAI_U32 || dt == RAI_I64; }
+
+rai_tensor *rai_gather(rai_tensor *x, int32_t dim, rai_tensor *index) {
+  // ops/gather.rs:47-60: equal ranks, equal shapes once `dim` is removed; the output has index's shape
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank) return err_node(x->dev, x->dtype, {}, {x, index}, "dim out of range");
+  if (index->shape.size() != x->shape.size() || !index_dtype(index->dtype))
+    return err_node(x->dev, x->dtype, index->shape, {x, index}, incompatible(x, index));
+  for (int i = 0; i < rank; ++i)
+    if (i != d && index->shape[i] != x->shape[i]) return err_node(x->dev, x->dtype, index->shape, {x, index}, incompatible(x, index));
+  rai_tensor *t = new_node(x->dev, x->dtype, index->shape, RAI_OP_GATHER, {x, index});
+  t->ip = {d};
+  return t;
+}
+
+rai_tensor *rai_index_add(rai_tensor *x, int32_t dim, rai_tensor *index, rai_tensor *source) {
+  // ops/index_add.rs:52-62 (its asserts are a TODO there; the shapes candle's index_add requires are checked here)
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank) return err_node(x->dev, x->dtype, x->shape, {x, source, index}, "dim out of range");
+  bool ok = index->shape.size() == 1 && index_dtype(index->dtype) && source->shape.size() == x->shape.size() &&
+            source->dtype == x->dtype;
+  for (int i = 0; ok && i < rank; ++i) ok = source->shape[i] == (i == d ? index->shape[0] : x->shape[i]);
+  if (!ok) return err_node(x->dev, x->dtype, x->shape, {x, source, index}, incompatible(x, source));
+  rai_tensor *t = new_node(x->dev, x->dtype, x->shape, RAI_OP_INDEX_ADD, {x, source, index});
+  t->ip = {d};
+  return t;
+}
+
+rai_tensor *rai_scatter_add(rai_tensor *x, int32_t dim, rai_tensor *index, rai_tensor *source) {
+  // ops/scatter_add.rs:52-60
+  const int rank = (int)x->shape.size();
+  const int d = norm_dim(dim, rank);
+  if (d < 0 || d >= rank) return err_node(x->dev, x->dtype, x->shape, {x, source, index}, "dim out of range");
+  bool ok = index->shape == source->shape && index->shape.size() == x->shape.size() && index_dtype(index->dtype) &&
+            source->dtype == x->dtype;
+  for (int i = 0; ok && i < rank; ++i) ok = i == d || index->shape[i] == x->shape[i];
+  if (!ok) return err_node(x->dev, x->dtype, x->shape, {x, source, index}, incompatible(x, source));
+  rai_tensor *t = new_node(x->dev, x->dtype, x->shape, RAI_OP_SCATTER_ADD, {x, source, index});
   t->ip = {d};
   return t;
 }

@@ -7,6 +7,8 @@
 // collects its own contributions in increasing source order and rounds to the storage dtype after
 // each addition, so the result equals a sequential host loop bit for bit, duplicates included, and no
 // floating-point atomics (whose order varies from run to run) are used.
+#include <algorithm>
+
 #include "common.h"
 
 namespace rai {
@@ -38,53 +40,70 @@ k_gather(T *out, const T *x, const IT *index, int64_t outer, int64_t J, int64_t 
 }
 
 // x / out [outer, D, inner], source [outer, L, inner], index [L]: out[o, r, :] = x[o, r, :] + the rows
-// source[o, l, :] with index[l] == r, added in increasing l.  One block per output row (grid-stride);
-// the index list is scanned 256 entries at a time, the matches of a chunk are shared as ballot masks.
-constexpr int kIndexAddElems = 4;
-template <typename T, typename IT>
+// source[o, l, :] with index[l] == r, added in increasing l.  One wave per output row (grid-stride): it
+// scans the index list 64 entries at a time (one per lane, from an LDS copy when the list fits) and
+// walks the ballot mask of the matches in order.  A row is moved in units of U: 16-byte packs when the
+// row length and the addresses allow, single elements otherwise; kIndexAddUnits of them per lane and pass.
+constexpr int kIndexAddUnits = 8;
+constexpr int kIndexAddLdsEntries = 32768;   // 128 KB of staged indices
+template <typename T> struct alignas(16) Pack16 { T v[16 / sizeof(T)]; };
+template <typename T> __device__ __forceinline__ void add_unit(T &acc, const T &s) {
+  Scalar<T>::store(&acc, Scalar<T>::load(&acc) + Scalar<T>::load(&s));
+}
+template <typename T> __device__ __forceinline__ void add_unit(Pack16<T> &acc, const Pack16<T> &s) {
+#pragma unroll
+  for (int j = 0; j < (int)(16 / sizeof(T)); ++j) Scalar<T>::store(&acc.v[j], Scalar<T>::load(&acc.v[j]) + Scalar<T>::load(&s.v[j]));
+}
+template <typename U, typename IT>
 __global__ void __launch_bounds__(256)
-k_index_add(T *out, const T *x, const T *source, const IT *index, int64_t index_stride, int64_t outer, int64_t D,
-            int64_t L, int64_t inner, unsigned long long *errors) {
-  typedef typename Scalar<T>::compute CT;
-  __shared__ unsigned long long masks[4];
-  const int wave = threadIdx.x >> 6;
-  const int64_t rows = outer * D;
-  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+k_index_add(U *out, const U *x, const U *source, const IT *index, int64_t index_stride, int64_t outer, int64_t D,
+            int64_t L, int64_t units, int staged, unsigned long long *errors) {
+  extern __shared__ int32_t s_idx[];
+  if (staged) {   // ids outside [0, D) can match no row: stored as -1
+    for (int64_t l = threadIdx.x; l < L; l += blockDim.x) {
+      const int64_t id = (int64_t)index[l * index_stride];
+      const bool ok = id >= 0 && id < D;
+      s_idx[l] = ok ? (int32_t)id : -1;
+      if (!ok && blockIdx.x == 0) atomicAdd(errors, 1ull);
+    }
+    __syncthreads();
+  } else if (blockIdx.x == 0) {
+    for (int64_t l = threadIdx.x; l < L; l += blockDim.x) {
+      const int64_t id = (int64_t)index[l * index_stride];
+      if (id < 0 || id >= D) atomicAdd(errors, 1ull);
+    }
+  }
+  const int lane = threadIdx.x & 63;
+  const int64_t rows = outer * D, n_waves = (int64_t)gridDim.x * 4;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += n_waves) {
     const int64_t o = row / D, r = row - o * D;
-    for (int64_t i0 = 0; i0 < inner; i0 += 256 * kIndexAddElems) {
-      CT acc[kIndexAddElems];
+    for (int64_t i0 = 0; i0 < units; i0 += 64 * kIndexAddUnits) {
+      U acc[kIndexAddUnits];
 #pragma unroll
-      for (int u = 0; u < kIndexAddElems; ++u) {
-        const int64_t i = i0 + u * 256 + threadIdx.x;
-        acc[u] = i < inner ? Scalar<T>::load(x + row * inner + i) : CT(0);
+      for (int u = 0; u < kIndexAddUnits; ++u) {
+        const int64_t i = i0 + u * 64 + lane;
+        if (i < units) acc[u] = x[row * units + i];
       }
-      for (int64_t l0 = 0; l0 < L; l0 += 256) {
-        const int64_t l = l0 + threadIdx.x;
-        const int64_t id = l < L ? (int64_t)index[l * index_stride] : -1;
-        if (row == 0 && i0 == 0 && l < L && (id < 0 || id >= D)) atomicAdd(errors, 1ull);
-        const unsigned long long m = __ballot(id == r);
-        if ((threadIdx.x & 63) == 0) masks[wave] = m;
-        __syncthreads();
+      for (int64_t l0 = 0; l0 < L; l0 += 64) {
+        const int64_t l = l0 + lane;
+        int64_t id = -1;
+        if (l < L) id = staged ? (int64_t)s_idx[l] : (int64_t)index[l * index_stride];
+        unsigned long long m = __ballot(id == r);
+        while (m) {
+          const int b = __ffsll((long long)m) - 1;
+          m &= m - 1;
+          const U *srow = source + (o * L + l0 + b) * units;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          unsigned long long mm = masks[w];
-          while (mm) {
-            const int b = __ffsll((long long)mm) - 1;
-            mm &= mm - 1;
-            const int64_t ls = l0 + w * 64 + b;
-#pragma unroll
-            for (int u = 0; u < kIndexAddElems; ++u) {
-              const int64_t i = i0 + u * 256 + threadIdx.x;
-              if (i < inner) acc[u] = add_rounded<T>(acc[u], Scalar<T>::load(source + (o * L + ls) * inner + i));
-            }
+          for (int u = 0; u < kIndexAddUnits; ++u) {
+            const int64_t i = i0 + u * 64 + lane;
+            if (i < units) add_unit(acc[u], srow[i]);
           }
         }
-        __syncthreads();
       }
 #pragma unroll
-      for (int u = 0; u < kIndexAddElems; ++u) {
-        const int64_t i = i0 + u * 256 + threadIdx.x;
-        if (i < inner) Scalar<T>::store(out + row * inner + i, acc[u]);
+      for (int u = 0; u < kIndexAddUnits; ++u) {
+        const int64_t i = i0 + u * 64 + lane;
+        if (i < units) out[row * units + i] = acc[u];
       }
     }
   }
@@ -214,11 +233,29 @@ int rai_hip_index_add(int dev, const rai_hip_tensor *x, const rai_hip_tensor *in
   int64_t outer, inner;
   split_dims(x, d, &outer, &inner);
   unsigned long long *errs = index_error_counter(dev);
-  const int grid = grid_for(outer * D, 1);
+  const size_t es = dtype_size(x->dtype);
+  const bool packs = (inner * es) % 16 == 0 && (uintptr_t)base_ptr(x) % 16 == 0 && (uintptr_t)base_ptr(source) % 16 == 0 &&
+                     (uintptr_t)base_ptr(out) % 16 == 0;
+  const int64_t units = packs ? inner * (int64_t)es / 16 : inner;
+  const int staged = L <= kIndexAddLdsEntries && D <= 0x7fffffffLL ? 1 : 0;
+  const size_t lds = staged ? (size_t)(L > 0 ? L : 1) * sizeof(int32_t) : 0;
+  // one wave per row, four waves per block; few enough blocks that staging the index list stays cheap
+  const int grid = std::min(grid_for(outer * D, 4), kNumCU * 8);
   RAI_DISPATCH_ALL(x->dtype, T, {
     RAI_DISPATCH_INDEX(index->dtype, IT, {
-      hipLaunchKernelGGL((k_index_add<T, IT>), dim3(grid), dim3(256), 0, st, (T *)base_ptr(out), (const T *)base_ptr(x),
-                         (const T *)base_ptr(source), (const IT *)base_ptr(index), index->stride[0], outer, D, L, inner, errs);
+      if (packs) {
+        if (lds > 48 * 1024)
+          RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_index_add<Pack16<T>, IT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL((k_index_add<Pack16<T>, IT>), dim3(grid), dim3(256), lds, st, (Pack16<T> *)base_ptr(out),
+                           (const Pack16<T> *)base_ptr(x), (const Pack16<T> *)base_ptr(source), (const IT *)base_ptr(index),
+                           index->stride[0], outer, D, L, units, staged, errs);
+      } else {
+        if (lds > 48 * 1024)
+          RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_index_add<T, IT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL((k_index_add<T, IT>), dim3(grid), dim3(256), lds, st, (T *)base_ptr(out), (const T *)base_ptr(x),
+                           (const T *)base_ptr(source), (const IT *)base_ptr(index), index->stride[0], outer, D, L, units,
+                           staged, errs);
+      }
     });
   });
   return launch_check("index_add");

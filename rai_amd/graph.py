@@ -25,7 +25,7 @@ from ._lib import BF16, BINARY, DTYPE_BY_NAME, DTYPE_NAMES, DTYPE_SIZE, F16, F32
 
 OP_KINDS = ["Full", "Arange", "FromArray", "ToDType", "Unary", "Binary", "MatMul", "Softmax", "LogSoftmax", "Reduce",
             "ArgMax", "ArgMin", "IndexSelect", "Narrow", "Concatenate", "Where", "Transpose", "Reshape", "Permute",
-            "Broadcast", "ToContiguous", "Err"]
+            "Broadcast", "ToContiguous", "Err", "Gather", "IndexAdd", "ScatterAdd"]
 OP = {n: i for i, n in enumerate(OP_KINDS)}
 _NP = {U8: np.uint8, U32: np.uint32, I64: np.int64, F16: np.float16, BF16: np.uint16, F32: np.float32, F64: np.float64}
 
@@ -210,6 +210,15 @@ class Tensor:
 
     def index_select(self, dim, index):
         return Tensor(_lib.load().rai_index_select(self._h, dim, index._h))
+
+    def gather(self, dim, index):
+        return Tensor(_lib.load().rai_gather(self._h, dim, index._h))
+
+    def index_add(self, dim, index, source):
+        return Tensor(_lib.load().rai_index_add(self._h, dim, index._h, source._h))
+
+    def scatter_add(self, dim, index, source):
+        return Tensor(_lib.load().rai_scatter_add(self._h, dim, index._h, source._h))
 
     def narrow(self, dim, start, length):
         return Tensor(_lib.load().rai_narrow(self._h, dim, start, length))

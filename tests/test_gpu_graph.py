@@ -205,3 +205,27 @@ def test_phi2_through_the_graph_matches_oracle(hip, dt):
     # greedy ids through the graph: argmax node, u32, bit-exact against the oracle on the same logits
     tok = logits.argmax(-1).as_storage()[:, 0]
     assert tok.dtype == np.uint32 and np.array_equal(tok, np.argmax(got, -1))
+
+
+def test_gather_index_add_scatter_add_nodes(hip):
+    # the primitives the vjp rules of index_select and gather evaluate, on strided (transposed) inputs too
+    rng = np.random.default_rng(5)
+    x = rand(rng, (6, 9), "f32")
+    ix = rng.integers(0, 6, (4, 9)).astype(np.uint32)
+    got = dev(x, "f32").gather(0, Tensor.from_array(ix, "u32")).as_storage()
+    assert np.array_equal(got, oo.gather(x, 0, ix))
+    got = dev(x.T.copy(), "f32").t().gather(0, Tensor.from_array(ix, "u32")).as_storage()   # non-contiguous x
+    assert np.array_equal(got, oo.gather(x, 0, ix))
+    ids = rng.integers(0, 6, 13).astype(np.uint32)
+    src = rand(rng, (13, 9), "f32")
+    got = dev(x, "f32").index_add(0, Tensor.from_array(ids, "u32"), dev(src, "f32")).as_storage()
+    assert np.array_equal(got, oo.index_add(x, 0, ids, src, "f32"))
+    # adjoint pair as the reference's vjp builds it (ops/index_select.rs:40-48): zeros_like(x).index_add(dim, index, cotangent)
+    zero = Tensor.full(0.0, (6, 9), "f32")
+    got = zero.index_add(0, Tensor.from_array(ids, "u32"), dev(src.T.copy(), "f32").t()).as_storage()
+    assert np.array_equal(got, oo.index_add(np.zeros_like(x), 0, ids, src, "f32"))
+    upd = rand(rng, (4, 9), "f32")
+    got = dev(x, "f32").scatter_add(0, Tensor.from_array(ix, "u32"), dev(upd, "f32")).as_storage()
+    assert np.array_equal(got, oo.scatter_add(x, 0, ix, upd, "f32"))
+    with pytest.raises(Exception):
+        dev(x, "f32").gather(1, Tensor.from_array(ix, "u32")).as_storage()   # Err node surfaces at eval

@@ -53,6 +53,17 @@ def test_building_is_lazy_and_metadata_follows_the_reference():
     ids = Tensor.from_array(np.array([[1, 0], [2, 2]], np.uint32), "u32")
     assert a.index_select(1, ids).shape == (2, 4)   # index.elem_count() (index_select.rs:52-61)
     assert Tensor.arange(0, 10, 3).shape == (4,)
+    # gather takes the index's shape (gather.rs:47-60); index_add / scatter_add keep x's (index_add.rs:52-62)
+    gi = Tensor.from_array(np.zeros((5, 3), np.uint32), "u32")
+    assert a.gather(0, gi).shape == (5, 3) and a.gather(0, gi).op == "Gather" and a.gather(0, gi).num_inputs() == 2
+    one = Tensor.from_array(np.array([1, 1, 0, 0], np.uint8), "u8")
+    ia = a.index_add(0, one, Tensor.ones((4, 3), "f32"))
+    assert ia.shape == (2, 3) and ia.op == "IndexAdd" and ia.num_inputs() == 3
+    sa = a.scatter_add(0, gi, Tensor.ones((5, 3), "f32"))
+    assert sa.shape == (2, 3) and sa.op == "ScatterAdd"
+    assert a.gather(1, gi).op == "Err"                                  # extents off the dim differ
+    assert a.index_add(0, one, Tensor.ones((3, 3), "f32")).op == "Err"   # source extent != len(index)
+    assert a.scatter_add(0, gi, Tensor.ones((4, 3), "f32")).op == "Err"  # index and source shapes differ
 
 
 @pytest.mark.parametrize("lhs,rhs,out", [((2, 3), (3,), (2, 3)), ((1, 3), (2, 1), (2, 3)), ((4, 1, 5), (7, 1), (4, 7, 5)),
