@@ -289,7 +289,8 @@ int rai_hip_attention(int dev, const rai_hip_tensor *q, const rai_hip_tensor *k,
 typedef enum rai_hip_arch {
   RAI_ARCH_PHI2 = 0,  /* rai-models/src/llm/phi2.rs */
   RAI_ARCH_QWEN2 = 1, /* rai-models/src/llm/qwen2.rs */
-  RAI_ARCH_GEMMA = 2  /* rai-models/src/llm/gemma.rs */
+  RAI_ARCH_GEMMA = 2, /* rai-models/src/llm/gemma.rs */
+  RAI_ARCH_PHI3 = 3   /* rai-models/src/llm/phi3.rs: the Qwen2 block with fused qkv_proj / gate_up_proj, no biases */
 } rai_hip_arch;
 
 /* Union of the serde Config structs phi2.rs:9-24, qwen2.rs:8-24, gemma.rs:12-27. */

@@ -22,7 +22,7 @@ UNARY = {n: i for i, n in enumerate(
 BINARY = {n: i for i, n in enumerate(
     ["add", "sub", "mul", "div", "maximum", "minimum", "eq", "ne", "gt", "ge", "lt", "le"])}
 REDUCE = {"sum": 0, "max": 1, "min": 2}
-ARCH = {"phi2": 0, "qwen2": 1, "gemma": 2}
+ARCH = {"phi2": 0, "qwen2": 1, "gemma": 2, "phi3": 3}
 
 
 class RaiHipError(RuntimeError):

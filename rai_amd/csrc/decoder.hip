@@ -31,6 +31,10 @@ struct ParamSlot {
   char *dst;                // device address of element [0, 0]
   int64_t pitch;            // elements between consecutive rows at dst
   bool loaded;
+  // a parameter whose last rows2 rows go elsewhere (same pitch): Phi-3's gate_up_proj, whose gate rows and
+  // up rows interleave in the packed matrix
+  int64_t rows2;
+  char *dst2;
 };
 
 struct Layer {
@@ -469,7 +473,12 @@ static int dalloc(rai_hip_decoder *d, size_t bytes, char **out) {
 
 static void add_slot(rai_hip_decoder *d, const std::string &name, int64_t rows, int64_t cols, char *dst, int64_t pitch) {
   d->slot_by_name[name] = (int)d->slots.size();
-  d->slots.push_back(ParamSlot{name, rows, cols, dst, pitch, false});
+  d->slots.push_back(ParamSlot{name, rows, cols, dst, pitch, false, 0, nullptr});
+}
+static void add_split_slot(rai_hip_decoder *d, const std::string &name, int64_t rows, int64_t cols, char *dst, int64_t pitch,
+                           int64_t rows2, char *dst2) {
+  d->slot_by_name[name] = (int)d->slots.size();
+  d->slots.push_back(ParamSlot{name, rows, cols, dst, pitch, false, rows2, dst2});
 }
 
 // Rotary tables.  Reference chain (phi2.rs:44-64): inv_freq computed with f32
@@ -486,18 +495,37 @@ static float round_dt(float v, int dtype) {
   return v;
 }
 
+// f64 -> model dtype with a single rounding.  Going through f32 rounds twice, which differs exactly when
+// the f32 value lands on a bf16 tie: the part the first rounding dropped then decides the direction.
+static float round_dt_from_double(double v, int dtype) {
+  const float f = (float)v;
+  if (dtype != RAI_BF16) return f;
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) >= 0x7f800000u || (u & 0xffffu) != 0x8000u || (double)f == v) return round_dt(f, dtype);
+  const bool away = fabs(v) > fabs((double)f);   // the exact value lies beyond the tie
+  u = (u & 0xffff0000u) + (away ? 0x10000u : 0u);
+  float r;
+  memcpy(&r, &u, 4);
+  return r;
+}
+
 static int build_rope_tables(rai_hip_decoder *d) {
   const auto &c = d->cfg;
   const int rot = c.rotary_dim, half = rot / 2, P = c.max_position_embeddings;
   std::vector<float> cs((size_t)P * rot), sn((size_t)P * rot);
   for (int i = 0; i < half; ++i) {
-    float inv;
+    float inv, inv_dt;
     if (c.arch == RAI_ARCH_PHI2) inv = 1.0f / powf((float)c.rope_theta, (float)(2 * i) / (float)rot);
+    else if (c.arch == RAI_ARCH_PHI3) inv = (float)(1.0 / pow(c.rope_theta, (double)(2 * i) / (double)rot));
     else inv = 1.0f / (float)pow(c.rope_theta, (double)(2 * i) / (double)rot);
+    inv_dt = round_dt(inv, c.dtype);
+    if (c.arch == RAI_ARCH_PHI3)   // phi3.rs:45-51: an f64 tensor cast to the model dtype, one rounding from f64
+      inv_dt = round_dt_from_double(1.0 / pow(c.rope_theta, (double)(2 * i) / (double)rot), c.dtype);
     for (int p = 0; p < P; ++p) {
       float ang;
       if (c.rope_tables_f32) ang = (float)p * inv;
-      else ang = round_dt(round_dt((float)p, c.dtype) * round_dt(inv, c.dtype), c.dtype);
+      else ang = round_dt(round_dt((float)p, c.dtype) * inv_dt, c.dtype);
       float cv = round_dt(cosf(ang), c.dtype), sv = round_dt(sinf(ang), c.dtype);
       cs[(size_t)p * rot + i] = cs[(size_t)p * rot + i + half] = cv;
       sn[(size_t)p * rot + i] = sn[(size_t)p * rot + i + half] = sv;
@@ -580,7 +608,7 @@ static int create_phi2(rai_hip_decoder *d) {
 static int create_seq(rai_hip_decoder *d) {
   const size_t es = d->es;
   const int H = d->H, I = d->I, QD = d->QD, KD = d->KD, V = d->V;
-  const bool qwen = d->cfg.arch == RAI_ARCH_QWEN2;
+  const bool qwen = d->cfg.arch == RAI_ARCH_QWEN2, phi3 = d->cfg.arch == RAI_ARCH_PHI3;
   RAI_TRY(dalloc(d, (size_t)V * H * es, &d->embed));
   add_slot(d, "model.embed_tokens.weight", V, H, d->embed, H);
   d->layers.resize(d->L);
@@ -595,9 +623,13 @@ static int create_seq(rai_hip_decoder *d) {
     RAI_TRY(dalloc(d, (size_t)H * es, &ly.n1_w));
     RAI_TRY(dalloc(d, (size_t)H * es, &ly.n2_w));
     const std::string p = "model.layers." + std::to_string(l) + ".";
-    add_slot(d, p + "self_attn.q_proj.weight", QD, H, ly.Wqkv, H);
-    add_slot(d, p + "self_attn.k_proj.weight", KD, H, ly.Wqkv + (size_t)QD * H * es, H);
-    add_slot(d, p + "self_attn.v_proj.weight", KD, H, ly.Wqkv + (size_t)(QD + KD) * H * es, H);
+    if (phi3) {  // one projection whose rows are q | k | v (phi3.rs:131-132,166-176)
+      add_slot(d, p + "self_attn.qkv_proj.weight", NQ, H, ly.Wqkv, H);
+    } else {
+      add_slot(d, p + "self_attn.q_proj.weight", QD, H, ly.Wqkv, H);
+      add_slot(d, p + "self_attn.k_proj.weight", KD, H, ly.Wqkv + (size_t)QD * H * es, H);
+      add_slot(d, p + "self_attn.v_proj.weight", KD, H, ly.Wqkv + (size_t)(QD + KD) * H * es, H);
+    }
     if (qwen) {  // q/k/v carry a bias, o_proj does not (qwen2.rs:137-140)
       RAI_TRY(dalloc(d, (size_t)NQ * es, &ly.bqkv));
       add_slot(d, p + "self_attn.q_proj.bias", 1, QD, ly.bqkv, QD);
@@ -606,8 +638,12 @@ static int create_seq(rai_hip_decoder *d) {
     }
     add_slot(d, p + "self_attn.o_proj.weight", H, QD, ly.Wo, QD);
     // gate row n -> packed row 2n, up row n -> packed row 2n+1 (pitch of two rows)
-    add_slot(d, p + "mlp.gate_proj.weight", I, H, ly.Wgu, 2 * (int64_t)H);
-    add_slot(d, p + "mlp.up_proj.weight", I, H, ly.Wgu + (size_t)H * es, 2 * (int64_t)H);
+    if (phi3) {  // rows [0, I) are the gate, rows [I, 2I) the up projection (phi3.rs:97-101)
+      add_split_slot(d, p + "mlp.gate_up_proj.weight", 2 * (int64_t)I, H, ly.Wgu, 2 * (int64_t)H, I, ly.Wgu + (size_t)H * es);
+    } else {
+      add_slot(d, p + "mlp.gate_proj.weight", I, H, ly.Wgu, 2 * (int64_t)H);
+      add_slot(d, p + "mlp.up_proj.weight", I, H, ly.Wgu + (size_t)H * es, 2 * (int64_t)H);
+    }
     add_slot(d, p + "mlp.down_proj.weight", H, I, ly.Wdown, I);
     add_slot(d, p + "input_layernorm.weight", 1, H, ly.n1_w, H);
     add_slot(d, p + "post_attention_layernorm.weight", 1, H, ly.n2_w, H);
@@ -850,6 +886,13 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   return RAI_OK;
 }
 
+// Qwen2 / Gemma scale by an f64 1/sqrt(head_dim) cast to the model dtype (qwen2.rs:205, gemma.rs:238); Phi-3
+// computes the scalar in f32 (phi3.rs:202).
+static float seq_attn_scale(const rai_hip_decoder *d) {
+  if (d->cfg.arch == RAI_ARCH_PHI3) return 1.0f / sqrtf((float)d->D);
+  return (float)(1.0 / sqrt((double)d->D));
+}
+
 // Sequential pre-norm block of Qwen2 (qwen2.rs:253-266) and Gemma (gemma.rs:286-299):
 // x1 = x + o_proj(attn(norm1(x))); x = x1 + down(act(gate(norm2(x1))) * up(norm2(x1))).
 static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool from_tokens = false) {
@@ -901,7 +944,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
       t.cos_t = d->cos_t; t.sin_t = d->sin_t; t.rot = d->cfg.rotary_dim;
       t.pos_dev = &d->state->pos;
       t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.D = d->D; t.Tmax = d->cfg.max_context;
-      t.scale = (float)(1.0 / sqrt((double)d->D));
+      t.scale = seq_attn_scale(d);
       t.f32_scores = 0; t.dtype = dt;
       t.ws = (float *)d->attn_ws; t.counters = d->attn_counters;
       RAI_TRY(launch_attention_decode(st, t));
@@ -920,7 +963,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
       t.ks[2] = t.vs[2] = d->D;
       t.out_row_stride = QD;
       t.B = B; t.Hq = d->Hq; t.Hkv = d->Hkv; t.S = S; t.D = d->D;
-      t.scale = (float)(1.0 / sqrt((double)d->D));
+      t.scale = seq_attn_scale(d);
       t.causal = 1; t.f32_scores = 0; t.dtype = dt;
       t.T = T_after;
       RAI_TRY(launch_attention(st, t));
@@ -1046,7 +1089,8 @@ extern "C" {
 
 int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_decoder **out) {
   RAI_REQUIRE(cfg && out, RAI_ERR_BAD_ARG, "decoder_create: null argument");
-  RAI_REQUIRE(cfg->arch == RAI_ARCH_PHI2 || cfg->arch == RAI_ARCH_QWEN2 || cfg->arch == RAI_ARCH_GEMMA,
+  RAI_REQUIRE(cfg->arch == RAI_ARCH_PHI2 || cfg->arch == RAI_ARCH_QWEN2 || cfg->arch == RAI_ARCH_GEMMA ||
+                  cfg->arch == RAI_ARCH_PHI3,
               RAI_ERR_UNSUPPORTED, "decoder_create: architecture %d not available", cfg->arch);
   RAI_REQUIRE(cfg->dtype == RAI_BF16 || cfg->dtype == RAI_F32, RAI_ERR_BAD_DTYPE, "decoder_create: bf16 or f32");
   RAI_REQUIRE(cfg->hidden_size > 0 && cfg->num_attention_heads > 0 && cfg->num_key_value_heads > 0 &&
@@ -1198,8 +1242,11 @@ int rai_hip_decoder_load_param(rai_hip_decoder *d, const char *name, const void 
   RAI_REQUIRE(bytes == want, RAI_ERR_BAD_SHAPE, "decoder: parameter '%s' needs %zu bytes, got %zu", name, want, bytes);
   RAI_HIP_TRY(hipSetDevice(d->dev));
   RAI_HIP_TRY(hipStreamSynchronize(stream_of(d->dev)));
-  RAI_HIP_TRY(hipMemcpy2D(s.dst, (size_t)s.pitch * d->es, host_data, (size_t)s.cols * d->es, (size_t)s.cols * d->es,
-                          (size_t)s.rows, hipMemcpyHostToDevice));
+  const size_t row_bytes = (size_t)s.cols * d->es, rows1 = (size_t)(s.rows - s.rows2);
+  RAI_HIP_TRY(hipMemcpy2D(s.dst, (size_t)s.pitch * d->es, host_data, row_bytes, row_bytes, rows1, hipMemcpyHostToDevice));
+  if (s.rows2 > 0)
+    RAI_HIP_TRY(hipMemcpy2D(s.dst2, (size_t)s.pitch * d->es, (const char *)host_data + rows1 * row_bytes, row_bytes, row_bytes,
+                            (size_t)s.rows2, hipMemcpyHostToDevice));
   s.loaded = true;
   return RAI_OK;
 }
