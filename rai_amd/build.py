@@ -35,6 +35,14 @@ COMMON = [
 ]
 
 
+# Per-file additions.  attention.hip: its MFMA accumulators are rescaled by ordinary vector instructions every
+# key tile, so they must live in the registers those instructions can address; without this the compiler parks
+# them in the accumulation registers and copies them out and back around every rescale.
+EXTRA = {
+    "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def sources() -> list[Path]:
     return sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
 
@@ -51,7 +59,7 @@ def _compile(src: Path, force: bool) -> Path:
     headers = list(CSRC.glob("*.h")) + list((ROOT / "include").glob("*.h"))
     if not force and _newer(obj, [src] + headers):
         return obj
-    cmd = [HIPCC, *COMMON, "-x", "hip", "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *COMMON, *EXTRA.get(src.name, []), "-x", "hip", "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

@@ -838,7 +838,7 @@ typedef __attribute__((ext_vector_type(16))) float fa_f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t fa_u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t fa_u32x2;
 
-template <int NW, int D>
+template <int NW, int D, bool F32S>
 __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
   constexpr int KS = D / 16;            // K steps of the score product
   constexpr int DT = (D + 31) / 32;     // 32-row tiles of O^T
@@ -852,7 +852,8 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
   const int h = blockIdx.y, b = blockIdx.z;
   const int hk = h / (a.Hq / a.Hkv);
-  const int q0 = blockIdx.x * (NW * 32);
+  // the last query tiles see the most keys under a causal mask: they go first so that the short ones fill the tail
+  const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * (NW * 32);
   const int off = a.T - a.S;  // absolute position of query row 0
   const uint16_t *Kg = (const uint16_t *)a.k + b * a.ks[0] + hk * a.ks[1];
   const uint16_t *Vg = (const uint16_t *)a.v + b * a.vs[0] + hk * a.vs[1];
@@ -880,58 +881,90 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
   const float scale_r = round_to<bf16_raw>(a.scale);
 
   // K/V tiles go global -> registers -> LDS; with PF the loads of tile t+1 are issued before tile t is
-  // multiplied, so their latency hides behind the MFMAs (register budget allows it for D <= 128)
-  constexpr int CH = (64 * CPR + NT - 1) / NT;   // 16-byte chunks of K (and of V) per thread
+  // multiplied, so their latency hides behind the MFMAs (register budget allows it for D <= 128).
+  // K: 16-byte chunks, row-major into Ks.  V: each work item is one pair of head features (d, d+1) for 8
+  // consecutive keys: eight 4-byte loads (lanes run along d, so a wave reads whole rows), repacked in
+  // registers into the two 8-key rows of V^T, which are written with 8-byte stores.
+  constexpr int CH = (64 * CPR + NT - 1) / NT;   // 16-byte chunks of K per thread
+  constexpr int NP = D / 2;                      // feature pairs
+  constexpr int VI = (8 * NP + NT - 1) / NT;     // V work items per thread
   constexpr bool PF = D <= 128;
-  fa_u32x4 kreg[CH], vreg[CH];
+  fa_u32x4 kreg[CH];
+  uint32_t vx[PF ? VI : 1][8];
+  auto load_v = [&](int i, int k0, uint32_t (&x)[8]) {
+    const int c = tid + i * NT;
+    const int pr = c % NP, g = c / NP;
+    if (c < 8 * NP) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        int t = k0 + g * 8 + j;
+        t = t < a.T ? t : a.T - 1;   // rows past the context re-read its last row (masked below)
+        x[j] = *reinterpret_cast<const uint32_t *>(Vg + (int64_t)t * a.vs[2] + 2 * pr);
+      }
+    }
+  };
+  auto store_v = [&](int i, const uint32_t (&x)[8]) {
+    const int c = tid + i * NT;
+    const int pr = c % NP, g = c / NP;
+    if (c < 8 * NP) {
+      fa_u32x2 lo0, lo1, hi0, hi1;   // feature 2*pr: keys 0-3, 4-7; feature 2*pr+1: keys 0-3, 4-7
+      lo0.x = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
+      lo0.y = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
+      lo1.x = __builtin_amdgcn_perm(x[5], x[4], 0x05040100u);
+      lo1.y = __builtin_amdgcn_perm(x[7], x[6], 0x05040100u);
+      hi0.x = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
+      hi0.y = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
+      hi1.x = __builtin_amdgcn_perm(x[5], x[4], 0x07060302u);
+      hi1.y = __builtin_amdgcn_perm(x[7], x[6], 0x07060302u);
+      uint16_t *r0 = Vt + (2 * pr) * VP + g * 8, *r1 = r0 + VP;
+      *reinterpret_cast<fa_u32x2 *>(r0) = lo0;
+      *reinterpret_cast<fa_u32x2 *>(r0 + 4) = lo1;
+      *reinterpret_cast<fa_u32x2 *>(r1) = hi0;
+      *reinterpret_cast<fa_u32x2 *>(r1 + 4) = hi1;
+    }
+  };
   auto load_tile = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int c = tid + i * NT;
       const int key = c / CPR, dc = (c % CPR) * 8;
       int t = k0 + key;
-      t = t < a.T ? t : a.T - 1;   // rows past the context re-read its last row (masked below)
-      if (c < 64 * CPR) {
-        kreg[i] = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
-        vreg[i] = *reinterpret_cast<const fa_u32x4 *>(Vg + (int64_t)t * a.vs[2] + dc);
-      }
+      t = t < a.T ? t : a.T - 1;
+      if (c < 64 * CPR) kreg[i] = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
+    }
+    if constexpr (PF) {
+#pragma unroll
+      for (int i = 0; i < VI; ++i) load_v(i, k0, vx[i]);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + i * NT;
+      const int key = c / CPR, dc = (c % CPR) * 8;
+      if (c < 64 * CPR) *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kreg[i];
+    }
+    if constexpr (PF) {
+#pragma unroll
+      for (int i = 0; i < VI; ++i) store_v(i, vx[i]);
+    }
+  };
+  // without the prefetch registers the V items pass through one at a time
+  auto stage_v_direct = [&](int k0) {
+#pragma unroll 2
+    for (int i = 0; i < VI; ++i) {
+      uint32_t x[8];
+      load_v(i, k0, x);
+      store_v(i, x);
     }
   };
   if (PF && kv_end > 0) load_tile(0);
   for (int k0 = 0; k0 < kv_end; k0 += 64) {
     __syncthreads();
     // ---- stage K [64][D] and V^T [D][64]
-    if constexpr (PF) {
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const int c = tid + i * NT;
-        const int key = c / CPR, dc = (c % CPR) * 8;
-        if (c < 64 * CPR) {
-          *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kreg[i];
-          const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            Vt[(dc + 2 * e) * VP + key] = (uint16_t)(w[e] & 0xffffu);
-            Vt[(dc + 2 * e + 1) * VP + key] = (uint16_t)(w[e] >> 16);
-          }
-        }
-      }
-    } else {
-      for (int c = tid; c < 64 * CPR; c += NT) {
-        const int key = c / CPR, dc = (c % CPR) * 8;
-        int t = k0 + key;
-        t = t < a.T ? t : a.T - 1;
-        const fa_u32x4 kv = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
-        *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kv;
-        const fa_u32x4 vv = *reinterpret_cast<const fa_u32x4 *>(Vg + (int64_t)t * a.vs[2] + dc);
-        const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          Vt[(dc + 2 * e) * VP + key] = (uint16_t)(w[e] & 0xffffu);
-          Vt[(dc + 2 * e + 1) * VP + key] = (uint16_t)(w[e] >> 16);
-        }
-      }
-    }
+    if (!PF) load_tile(k0);
+    store_tile();
+    if (!PF) stage_v_direct(k0);
     __syncthreads();
     if (PF && k0 + 64 < kv_end) load_tile(k0 + 64);
     if (k0 > wave_last_key) continue;  // every key of this tile is masked for this wave (barriers stay uniform)
@@ -950,30 +983,59 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
     }
     // ---- scale, mask, online softmax (register r of sub-tile u is key k0 + 32u + 8*(r/4) + 4*half + r%4)
     const int q_abs = off + qrow;
+    // a tile wholly inside the context and (under a causal mask) wholly at or before this wave's first query
+    // needs no masking
+    const bool masked = k0 + 63 >= a.T || (a.causal && k0 + 63 > off + q0 + wave * 32);
+    if constexpr (F32S) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[u][r] *= a.scale;
+    } else {   // the product and its scaling are each rounded to bf16, two scores per conversion
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          uint32_t pk = pack_bf16x2(sc[u][r], sc[u][r + 1]);
+          pk = pack_bf16x2(__uint_as_float(pk << 16) * scale_r, __uint_as_float(pk & 0xffff0000u) * scale_r);
+          sc[u][r] = __uint_as_float(pk << 16);
+          sc[u][r + 1] = __uint_as_float(pk & 0xffff0000u);
+        }
+    }
+    if (masked) {
+      const int last_key = a.causal && q_abs < a.T - 1 ? q_abs : a.T - 1;   // newest key this lane's query may see
+      const int rel = last_key - k0 - 4 * half;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[u][r] = u * 32 + 8 * (r >> 2) + (r & 3) > rel ? -INFINITY : sc[u][r];
+    }
     float mx = -INFINITY;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = k0 + u * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        float v = a.f32_scores ? sc[u][r] * a.scale : round_to<bf16_raw>(round_to<bf16_raw>(sc[u][r]) * scale_r);
-        if (key >= a.T || (a.causal && key > q_abs)) v = -INFINITY;
-        sc[u][r] = v;
-        mx = fmaxf(mx, v);
-      }
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[u][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // fully masked so far: every p is exp(-inf) = 0
-    const float alpha = __expf(m_run - m_safe);
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float ml2 = m_safe * kLog2e;
+    const float alpha = __builtin_amdgcn_exp2f(m_run * kLog2e - ml2);
     float psum = 0.f;
     fa_bf16x8 pf[2][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __expf(sc[u][r] - m_safe);
-        psum += p;
-        pf[u][r >> 3][r & 7] = (__bf16)p;
+      for (int s2 = 0; s2 < 2; ++s2) {
+        fa_u32x4 w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[u][8 * s2 + 2 * j], kLog2e, -ml2));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[u][8 * s2 + 2 * j + 1], kLog2e, -ml2));
+          psum += p0 + p1;
+          w[j] = pack_bf16x2(p0, p1);
+        }
+        pf[u][s2] = __builtin_bit_cast(fa_bf16x8, w);
       }
     l_run = l_run * alpha + psum;
     m_run = m_new;
@@ -1019,9 +1081,12 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
 template <int D> static int launch_flash(hipStream_t st, const AttnArgs &a) {
   const int tiles4 = (a.S + 127) / 128;
   if ((int64_t)tiles4 * a.Hq * a.B >= kNumCU) {
-    hipLaunchKernelGGL((k_flash_prefill_bf16<4, D>), dim3(tiles4, a.Hq, a.B), dim3(256), 0, st, a);
+    if (a.f32_scores) hipLaunchKernelGGL((k_flash_prefill_bf16<4, D, true>), dim3(tiles4, a.Hq, a.B), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((k_flash_prefill_bf16<4, D, false>), dim3(tiles4, a.Hq, a.B), dim3(256), 0, st, a);
   } else {
-    hipLaunchKernelGGL((k_flash_prefill_bf16<2, D>), dim3((a.S + 63) / 64, a.Hq, a.B), dim3(128), 0, st, a);
+    const dim3 grid((a.S + 63) / 64, a.Hq, a.B);
+    if (a.f32_scores) hipLaunchKernelGGL((k_flash_prefill_bf16<2, D, true>), grid, dim3(128), 0, st, a);
+    else hipLaunchKernelGGL((k_flash_prefill_bf16<2, D, false>), grid, dim3(128), 0, st, a);
   }
   return launch_check("flash_prefill");
 }
