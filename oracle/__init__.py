@@ -17,8 +17,21 @@ Pinning status (see tests/test_oracle_*.py):
     answers readable from the reference's own tests (rai-core/tests/ops.rs,
     tests/eval.rs), brute force on tiny inputs, closed forms and independent
     library routines (torch CPU, scipy).
+  * gather, index_add, scatter_add: pinned against torch's routines (integer
+    dtypes and exactly representable floats, so the order of additions cannot
+    matter), the shapes of rai-core/tests/ops.rs:156-161 and
+    tests/check_grad.rs:117-169, and the adjoint identities their vjp rules
+    rely on.
+  * the example loop's token choice (oracle/sampling.py): pinned against a
+    pure-Python max_by over Rust's documented f32::total_cmp and hand-computed
+    penalty rows.
+  * the model files (phi2, qwen2/gemma, phi3): pinned against Hugging Face
+    transformers models built locally from in-memory configs with the oracle's
+    seeded weights.
   * Parity unpinned (only compiling candle could pin them): candle's exact f32
     summation order, its argmax NaN rule, its bf16 reduction accumulator width,
-    and whether candle's Cpu backend runs bf16 matmul at all.  The oracle uses
+    whether candle's Cpu backend runs bf16 matmul at all, and that its
+    index_add / scatter_add loops add source rows in index order in the element
+    type (one rounding per addition), which is what the oracle does.  The oracle uses
     f32 accumulation with one rounding to bf16 per primitive.
 """
