@@ -43,6 +43,8 @@ struct Layer {
   // Qwen2 / Gemma (sequential block): Wqkv [QD+2KD, H] (+bqkv), Wo [H, QD] (+bo),
   // Wgu [2I, H] with gate/up rows interleaved, Wdown [H, I], two RMSNorm weights
   char *Wqkv, *bqkv, *Wo, *bo, *Wgu, *Wdown, *n1_w, *n2_w;
+  // second copies in MFMA-fragment order for the batched-decode streaming kernel (built on first use)
+  char *Wa_f, *Wb_f, *Wqkv_f, *Wo_f, *Wgu_f, *Wdown_f;
 };
 
 }  // namespace rai
@@ -90,6 +92,8 @@ struct rai_hip_decoder {
   int sample_last_n;
   uint32_t *token_log;        // [max_batch][token_log_cap]: every token of each sequence so far, prompt first
   int token_log_cap;
+  char *head_f;               // fragment-order copy of the lm_head matrix
+  bool frag_ready;            // the fragment-order copies match the loaded parameters
   bool graph_sampled;         // what the cached step graphs were captured with
   float graph_penalty;
   int graph_last_n;
@@ -738,6 +742,38 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   return m;
 }
 
+// Batched decode (9..64 rows) streams every weight matrix once per step through the small-M MFMA kernel; that
+// kernel reads 1 KB per load instruction from a copy of the matrix in MFMA-fragment order.  The copies are made on
+// the first such step after the parameters changed (never under stream capture: generate runs its first
+// single-token step eagerly) and double the weight memory of the decoder.
+static bool wants_fragments(const rai_hip_decoder *d, int64_t M) {
+  static const bool off = getenv("RAI_HIP_NO_FRAG") != nullptr;
+  return !off && d->cfg.dtype == RAI_BF16 && M > 8 && M <= 64;
+}
+static int ensure_fragments(rai_hip_decoder *d, hipStream_t st) {
+  if (d->frag_ready) return RAI_OK;
+  auto one = [&](char *W, int64_t ldw, int N, int K, char **dst) -> int {
+    if (!W || K % 32) { *dst = nullptr; return RAI_OK; }
+    if (!*dst) RAI_TRY(dalloc(d, linear_fragment_elems(N, K) * d->es, dst));
+    return launch_linear_fragment_layout(st, W, ldw, N, K, *dst);
+  };
+  const int NQ = d->QD + 2 * d->KD;
+  for (Layer &ly : d->layers) {
+    if (d->cfg.arch == RAI_ARCH_PHI2) {
+      RAI_TRY(one(ly.Wa, d->H, d->NA, d->H, &ly.Wa_f));
+      RAI_TRY(one(ly.Wb, d->KB, d->H, d->KB, &ly.Wb_f));
+    } else {
+      RAI_TRY(one(ly.Wqkv, d->H, NQ, d->H, &ly.Wqkv_f));
+      RAI_TRY(one(ly.Wo, d->QD, d->H, d->QD, &ly.Wo_f));
+      RAI_TRY(one(ly.Wgu, d->H, 2 * d->I, d->H, &ly.Wgu_f));
+      RAI_TRY(one(ly.Wdown, d->I, d->H, d->I, &ly.Wdown_f));
+    }
+  }
+  RAI_TRY(one(d->head_w, d->H, d->V, d->H, &d->head_f));
+  d->frag_ready = true;
+  return RAI_OK;
+}
+
 constexpr int64_t kSampleMaxVocab = 15 * 1024 * 32;  // the membership bitmap of the penalised choice takes vocab / 8 bytes of LDS
 
 // Chooses the next token of every sequence from d->logits: plain greedy argmax, or the example loop's
@@ -782,6 +818,8 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   const int ldq = QD + 2 * KD;
   const bool fuse_ln = dt == RAI_BF16 && M <= 8;
   const int T_after = d->ctx_len + S;
+  const bool frag = wants_fragments(d, M);
+  if (frag) RAI_TRY(ensure_fragments(d, st));
 
   if (!from_tokens) {
     if (dt == RAI_BF16) launch_embed<bf16_raw>(d, st, M); else launch_embed<float>(d, st, M);
@@ -807,6 +845,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
       a.A = d->ln; a.lda = H;
     }
     a.W = ly.Wa; a.ldw = H; a.bias = ly.ba;
+    a.Wfrag = frag ? ly.Wa_f : nullptr;
     a.out1 = d->qkv; a.ld1 = ldq;
     a.out2 = d->cat + (size_t)QD * d->es; a.ld2 = d->KB;
     a.M = (int)M; a.N = d->NA; a.K = H; a.n_split = ldq;
@@ -854,6 +893,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
     LinearArgs b = linear_args_default();
     b.A = d->cat; b.lda = d->KB;
     b.W = ly.Wb; b.ldw = d->KB;
+    b.Wfrag = frag ? ly.Wb_f : nullptr;
     b.bias = ly.bd; b.bias2 = ly.bf;
     b.residual = x; b.ldr = H;
     b.out1 = xn; b.ld1 = H;
@@ -877,6 +917,10 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
     h.A = d->last; h.lda = H;
   }
   h.W = d->head_w; h.ldw = H; h.bias = d->head_b;
+  if (wants_fragments(d, B)) {
+    RAI_TRY(ensure_fragments(d, st));
+    h.Wfrag = d->head_f;
+  }
   h.out1 = d->logits; h.ld1 = d->V;
   h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
   RAI_TRY(linear(d, st, h));
@@ -907,6 +951,8 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
   const bool fuse_norm = dt == RAI_BF16 && (M <= 8 || linear_mfma_fuses_norm((int)M, H, kind));
   const int T_after = d->ctx_len + S;
   const size_t per_layer = (size_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
+  const bool frag = wants_fragments(d, M);
+  if (frag) RAI_TRY(ensure_fragments(d, st));
 
   if (!from_tokens) {
     if (dt == RAI_BF16) launch_embed<bf16_raw>(d, st, M); else launch_embed<float>(d, st, M);
@@ -928,6 +974,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
       a.A = d->ln; a.lda = H;
     }
     a.W = ly.Wqkv; a.ldw = H; a.bias = ly.bqkv;
+    a.Wfrag = frag ? ly.Wqkv_f : nullptr;
     a.out1 = d->qkv; a.ld1 = ldq;
     a.M = (int)M; a.N = ldq; a.K = H; a.n_split = ldq;
     a.splitk_ws = d->splitk_ws; a.splitk_ws_bytes = d->splitk_ws_bytes;
@@ -972,6 +1019,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     LinearArgs o = linear_args_default();
     o.A = d->attn; o.lda = QD;
     o.W = ly.Wo; o.ldw = QD; o.bias = ly.bo;
+    o.Wfrag = frag ? ly.Wo_f : nullptr;
     o.residual = x; o.ldr = H;
     o.out1 = x1; o.ld1 = H;
     o.M = (int)M; o.N = H; o.K = QD; o.n_split = H;
@@ -987,6 +1035,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
       g.A = d->ln; g.lda = H;
     }
     g.W = ly.Wgu; g.ldw = H;
+    g.Wfrag = frag ? ly.Wgu_f : nullptr;
     g.out1 = d->glu; g.ld1 = I;
     g.M = (int)M; g.N = 2 * I; g.K = H; g.n_split = 2 * I;
     g.act = d->cfg.hidden_act; g.act_from = 0; g.glu = 1;
@@ -995,6 +1044,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     LinearArgs dn = linear_args_default();
     dn.A = d->glu; dn.lda = I;
     dn.W = ly.Wdown; dn.ldw = I;
+    dn.Wfrag = frag ? ly.Wdown_f : nullptr;
     dn.residual = x1; dn.ldr = H;
     dn.out1 = x; dn.ld1 = H;
     dn.M = (int)M; dn.N = H; dn.K = I; dn.n_split = H;
@@ -1013,6 +1063,10 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     h.A = d->last; h.lda = H;
   }
   h.W = d->head_w; h.ldw = H;
+  if (wants_fragments(d, B)) {
+    RAI_TRY(ensure_fragments(d, st));
+    h.Wfrag = d->head_f;
+  }
   h.out1 = d->logits; h.ld1 = d->V;
   h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
   RAI_TRY(linear(d, st, h));
@@ -1121,6 +1175,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->sample_on = false; d->sample_penalty = 0.f; d->sample_last_n = 0;
   d->token_log = nullptr; d->token_log_cap = 0;
   d->graph_sampled = false; d->graph_penalty = 0.f; d->graph_last_n = 0;
+  d->head_f = nullptr; d->frag_ready = false;
   const int vec = (int)(16 / d->es);
   int st = RAI_OK;
   auto bail = [&](int code) {
@@ -1248,6 +1303,7 @@ int rai_hip_decoder_load_param(rai_hip_decoder *d, const char *name, const void 
     RAI_HIP_TRY(hipMemcpy2D(s.dst2, (size_t)s.pitch * d->es, (const char *)host_data + rows1 * row_bytes, row_bytes, row_bytes,
                             (size_t)s.rows2, hipMemcpyHostToDevice));
   s.loaded = true;
+  d->frag_ready = false;   // the fragment-order copies are rebuilt on the next batched decode step
   return RAI_OK;
 }
 

@@ -42,6 +42,10 @@ struct LinearArgs {
   // yields too few tiles to fill the GPU (tile kernel only).
   void *splitk_ws;
   size_t splitk_ws_bytes;
+  // Optional second copy of W in MFMA-fragment order for the small-M streaming kernel (9 <= M <= 64): the
+  // 16 rows x 32 columns that one wave loads with one instruction are 1 KB of consecutive memory
+  // ([N / 16 row tiles][K / 32 steps][64 lanes][8 elements], see linear_fragment_layout); null: read W itself.
+  const void *Wfrag;
 };
 inline LinearArgs linear_args_default() {
   LinearArgs a;
@@ -50,6 +54,11 @@ inline LinearArgs linear_args_default() {
   a.ln_kind = -1;
   return a;
 }
+
+// Elements of the fragment-major copy of a [N, K] bf16 matrix (K % 32 == 0; N is padded to a multiple of 16 with
+// zero rows), and the kernel that writes it.
+size_t linear_fragment_elems(int N, int K);
+int launch_linear_fragment_layout(hipStream_t st, const void *W, int64_t ldw, int N, int K, void *Wfrag);
 
 // bf16 MFMA tile kernel (M >= 1; efficient for M >= 64).
 int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a);

@@ -730,7 +730,32 @@ template <int MT> static int launch_mfma_skinny(hipStream_t st, const LinearArgs
 // output are summed through LDS and the Linear epilogue is applied.  A K span of
 // 256*KS covers K = 2048 (M <= 32) without splitting K over blocks, so the qkv / dense
 // shapes of a batched decode step need neither a partial-sum buffer nor a second kernel.
-template <int MT, int KS, int G>
+// Fragment-major copy of W: element j of lane l of (row tile t, K step s) is W[16 t + l % 16][32 s + 8 (l / 16) + j].
+__global__ void __launch_bounds__(256) k_linear_fragment_layout(bf16x8 *out, const uint16_t *W, int64_t ldw, int N, int ksteps,
+                                                                int64_t total) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(i & 63);
+    const int64_t ts = i >> 6;
+    const int s = (int)(ts % ksteps);
+    const int64_t t = ts / ksteps;
+    const int64_t n = t * 16 + (lane & 15);
+    bf16x8 v = {};
+    if (n < N) v = *reinterpret_cast<const bf16x8 *>(W + n * ldw + s * 32 + (lane >> 4) * 8);
+    out[i] = v;
+  }
+}
+size_t linear_fragment_elems(int N, int K) { return (size_t)((N + 15) / 16) * 16 * (size_t)K; }
+int launch_linear_fragment_layout(hipStream_t st, const void *W, int64_t ldw, int N, int K, void *Wfrag) {
+  RAI_REQUIRE(K % 32 == 0 && ldw % 8 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)Wfrag % 16 == 0, RAI_ERR_BAD_STRIDE,
+              "fragment layout: K must be a multiple of 32 and the operands 16-byte aligned");
+  const int64_t total = (int64_t)((N + 15) / 16) * (K / 32) * 64;
+  const int64_t blocks = (total + 255) / 256;
+  hipLaunchKernelGGL(k_linear_fragment_layout, dim3((unsigned)(blocks < 65535 ? blocks : 65535)), dim3(256), 0, st,
+                     (bf16x8 *)Wfrag, (const uint16_t *)W, ldw, N, K / 32, total);
+  return launch_check("linear_fragment_layout");
+}
+
+template <int MT, int KS, int G, bool FRAG>
 __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, int tiles, float *partial) {
   constexpr int NW = 8;
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
@@ -795,15 +820,23 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) koff[ks] = k0 + ks * 32 < a.K ? k0 + ks * 32 : 0;
   const uint16_t *wbase = (const uint16_t *)a.W + lq * 8;
+  const bf16x8 *fbase = reinterpret_cast<const bf16x8 *>(a.Wfrag) + lane;
+  const int ksteps = a.K / 32;
 
   bf16x8 wa[KS], wb[KS];
   auto load_tile = [&](bf16x8 (&w)[KS], int tile) {
     tile = tile < tiles ? tile : tiles - 1;
-    int n = tile * 16 + lrow;
-    n = n < a.N ? n : a.N - 1;
-    const uint16_t *p = wbase + (int64_t)n * a.ldw;
+    if constexpr (FRAG) {   // one instruction reads 1 KB of consecutive memory
+      const bf16x8 *p = fbase + (int64_t)tile * ksteps * 64;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) w[ks] = *reinterpret_cast<const bf16x8 *>(p + koff[ks]);
+      for (int ks = 0; ks < KS; ++ks) w[ks] = p[(koff[ks] >> 5) * 64];
+    } else {
+      int n = tile * 16 + lrow;
+      n = n < a.N ? n : a.N - 1;
+      const uint16_t *p = wbase + (int64_t)n * a.ldw;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) w[ks] = *reinterpret_cast<const bf16x8 *>(p + koff[ks]);
+    }
     // keep the whole tile's loads together and ahead of the multiplies that follow: left alone,
     // the scheduler sinks each load to just before its use and the prefetch distance collapses
     __builtin_amdgcn_sched_barrier(0);
@@ -884,7 +917,11 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
   }
 }
 
-template <int MT, int KS, int G> static int launch_mfma_stream_cfg(hipStream_t st, const LinearArgs &a, int splits) {
+template <int MT, int KS, int G, bool FRAG = false>
+static int launch_mfma_stream_cfg(hipStream_t st, const LinearArgs &a, int splits) {
+  if constexpr (!FRAG) {
+    if (a.Wfrag) return launch_mfma_stream_cfg<MT, KS, G, true>(st, a, splits);
+  }
   const int tiles = (a.N + 15) / 16;
   const int groups = (tiles + G - 1) / G;
   int blocks_x = kNumCU / splits;
@@ -893,12 +930,12 @@ template <int MT, int KS, int G> static int launch_mfma_stream_cfg(hipStream_t s
   const size_t lds = (size_t)8 * G * MT * 64 * sizeof(f32x4);
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma_stream<MT, KS, G>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma_stream<MT, KS, G, FRAG>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
   float *partial = splits > 1 ? (float *)a.splitk_ws : nullptr;
-  hipLaunchKernelGGL((k_linear_bf16_mfma_stream<MT, KS, G>), dim3(blocks_x, splits), dim3(512), lds, st, a, tiles,
+  hipLaunchKernelGGL((k_linear_bf16_mfma_stream<MT, KS, G, FRAG>), dim3(blocks_x, splits), dim3(512), lds, st, a, tiles,
                      partial);
   RAI_TRY(launch_check("linear_bf16_mfma_stream"));
   if (splits > 1) {
