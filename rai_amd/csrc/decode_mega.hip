@@ -137,9 +137,9 @@ template <int R> __device__ __forceinline__ void mg_rotate(mg_u32x4 (&ring)[kMeg
 struct MgSplit {
   const uint16_t *Wa0, *Wb0;
   int64_t wa_stride, wb_stride;
-  int L, H, KB, QD, KTA, KTB, KTC;
-  int nA0, n0;
-  int tA0, tA1, tB0, tB1, tC0, tC1;
+  int L, H, KB, QD, KTA, KTBC;
+  int nA0, nA2, n0;                  // first Wa row of segment A1 (q|k|v rows) and of A2 (fc1 rows); first Wb row
+  int tA0, tA1, tA2_0, tA2_1, tB0, tB1;
 };
 
 struct MgCursor {
@@ -152,24 +152,29 @@ struct MgCursor {
 __device__ __forceinline__ bool mg_seg_next(MgCursor &c, const MgSplit &sp) {
   int layer = c.layer, seg = c.seg;
 
-  const int tA0 = sp.tA0, tA1 = sp.tA1, tB0 = sp.tB0, tB1 = sp.tB1, tC0 = sp.tC0, tC1 = sp.tC1;
-  const int KTA = sp.KTA, KTB = sp.KTB, KTC = sp.KTC;
+  // segments of a layer, in streaming order: A1 (q|k|v rows of Wa), A2 (fc1 rows of Wa), BC (whole rows of Wb:
+  // dense columns, then fc2 columns)
+  // (the fields are copied into values first: selecting between struct members by `seg` directly makes the
+  // compiler keep the struct in scratch memory and select addresses)
+  const int tA0 = sp.tA0, tA1 = sp.tA1, tA2_0 = sp.tA2_0, tA2_1 = sp.tA2_1, tB0 = sp.tB0, tB1 = sp.tB1;
+  const int KTA = sp.KTA, KTBC = sp.KTBC, nA0 = sp.nA0, nA2 = sp.nA2;
   for (;;) {
     if (++seg == 3) { seg = 0; ++layer; }
     if (layer >= sp.L) return false;
-    const int t0 = seg == 0 ? tA0 : seg == 1 ? tB0 : tC0;
-    const int t1 = seg == 0 ? tA1 : seg == 1 ? tB1 : tC1;
+    const int t0 = seg == 0 ? tA0 : seg == 1 ? tA2_0 : tB0;
+    const int t1 = seg == 0 ? tA1 : seg == 1 ? tA2_1 : tB1;
     if (t1 <= t0) continue;
-    const int KT = seg == 0 ? KTA : seg == 1 ? KTB : KTC;
+    const int KT = seg <= 1 ? KTA : KTBC;
     const int row = t0 / KT;
     c.layer = layer; c.seg = seg; c.KT = KT; c.t = t0; c.t1 = t1;
     c.kc = t0 - row * KT;
-    if (seg == 0) {
+    if (seg <= 1) {
+      const int first = seg == 0 ? nA0 : nA2;
       c.ld = sp.H;
-      c.ptr = sp.Wa0 + layer * sp.wa_stride + (int64_t)(sp.nA0 + row) * sp.H;
+      c.ptr = sp.Wa0 + layer * sp.wa_stride + (int64_t)(first + row) * sp.H;
     } else {
       c.ld = sp.KB;
-      c.ptr = sp.Wb0 + layer * sp.wb_stride + (int64_t)(sp.n0 + row) * sp.KB + (seg == 1 ? sp.QD : 0);
+      c.ptr = sp.Wb0 + layer * sp.wb_stride + (int64_t)(sp.n0 + row) * sp.KB;
     }
     return true;
   }
@@ -188,14 +193,27 @@ __device__ __forceinline__ mg_u32x4 mg_next_load(MgCursor &c, const MgSplit &sp,
   }
   return v;
 }
-// Consumes tiles [t0, t1) of a [rows][KT] tile grid from the ring (entry 0 first),
-// multiplying them with the activation vector in LDS; leaves one partial sum per
-// (row, wave).  Returns how many entries the ring must be rotated afterwards.
+// Consumes tiles [t0, t1) of a [rows][KT] tile grid from the ring (entry 0 first), then tiles [u0, u1) of a
+// second grid with the same KT and the same activation vector, without a pause between the two; multiplies
+// them with the activation vector in LDS and leaves one partial sum per (row, wave) in `part` / `part2`.
+// When the first range is done (also when it is empty) lane 0 adds one to *done1, after its partial sums are in
+// LDS.  Returns how many entries the ring must be rotated afterwards.
 __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCursor &c, const MgSplit &sp, int t0, int t1,
-                                            int KT, const uint16_t *xv, float *part, int lane, int wave) {
+                                            int u0, int u1, int KT, const uint16_t *xv, float *part, float *part2,
+                                            uint32_t *done1, int lane, int wave) {
   float acc = 0.f;
-  int t = t0, row = t0 / KT;
+  const int n1 = t1 > t0 ? t1 - t0 : 0, n2 = u1 > u0 ? u1 - u0 : 0;
+  const int total = n1 + n2;
+  int left = total;
+  int to_switch = n1;            // steps until the first range is exhausted (0: already in the second)
+  int t = t0, te = t1, row = t0 / KT;
   int kc = t0 - row * KT;
+#define MG_TO_SECOND                                                                                              \
+  {                                                                                                               \
+    if (done1 && lane == 0) __hip_atomic_fetch_add(done1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);     \
+    t = u0; te = u1; row = u0 / KT; kc = u0 - row * KT; part = part2;                                             \
+  }
+  if (n1 == 0) MG_TO_SECOND
 #define MG_STEP(r)                                                                         \
   {                                                                                        \
     const mg_u32x4 x4 = *reinterpret_cast<const mg_u32x4 *>(xv + kc * 512 + lane * 8);     \
@@ -203,22 +221,26 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
     r = mg_next_load(c, sp, lane);                                                         \
     ++t;                                                                                   \
     ++kc;                                                                                  \
-    if (kc == KT || t == t1) {                                                             \
-      const float total = mg_wave_sum(acc);                                                \
-      if (lane == 0) part[row * kMegaWaves + wave] = total;                                \
+    if (kc == KT || t == te) {                                                             \
+      const float total_ = mg_wave_sum(acc);                                               \
+      if (lane == 0) part[row * kMegaWaves + wave] = total_;                               \
       acc = 0.f;                                                                           \
       if (kc == KT) { kc = 0; ++row; }                                                     \
+      if (to_switch == 1) MG_TO_SECOND                                                     \
     }                                                                                      \
+    --to_switch;                                                                           \
   }
-  while (t + kMegaRing <= t1) {
+  while (left >= kMegaRing) {
 #pragma unroll
     for (int p = 0; p < kMegaRing; ++p) MG_STEP(ring[p])
+    left -= kMegaRing;
   }
 #pragma unroll
   for (int p = 0; p < kMegaRing; ++p)
-    if (t < t1) MG_STEP(ring[p])
+    if (p < left) MG_STEP(ring[p])
 #undef MG_STEP
-  return t1 > t0 ? (t1 - t0) % kMegaRing : 0;
+#undef MG_TO_SECOND
+  return total % kMegaRing;
 }
 __device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r) {
   static_assert((kMegaRing & (kMegaRing - 1)) == 0 && kMegaRing <= 16, "rotation is composed from powers of two");
@@ -259,21 +281,55 @@ __device__ __forceinline__ void mg_poll(const uint64_t *src, const int (&idx)[N]
     if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
   }
 }
+// mg_poll over one list drawn from two packet arrays: entries below n0 come from src0 (tag0), the others from
+// src1 at index - n0 (tag1).
+template <int N, bool DBG>
+__device__ __forceinline__ void mg_poll2(const uint64_t *src0, uint32_t tag0, int n0, const uint64_t *src1, uint32_t tag1,
+                                         const int (&idx)[N], const bool (&on)[N], uint32_t (&out)[N], int *fault,
+                                         unsigned spin_limit) {
+  bool need[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) { need[i] = on[i]; out[i] = 0u; }
+  unsigned spins = 0;
+  for (;;) {
+    uint64_t pk[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      pk[i] = need[i] ? ld_dev64(idx[i] < n0 ? src0 + idx[i] : src1 + (idx[i] - n0)) : 0ull;
+    bool pending = false;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (need[i]) {
+        if ((uint32_t)(pk[i] >> 32) == (idx[i] < n0 ? tag0 : tag1)) { out[i] = (uint32_t)pk[i]; need[i] = false; }
+        else pending = true;
+      }
+    }
+    if (!__any(pending)) break;
+    __builtin_amdgcn_s_sleep(1);
+    if (++spins > (DBG ? spin_limit : kMegaSpinLimit)) {
+      __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+  }
+}
 template <int KTA, int D, bool PROF>
 __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   constexpr int NCOL = D / 8;
   constexpr int NG_V = kMegaThreads / NCOL;
   extern __shared__ __attribute__((aligned(16))) unsigned char mg_smem[];
   const int H = KTA * 512, I = a.I, QD = a.QD, KB = QD + I;
-  const int KTB = I / 512, KTC = QD / 512;
+  const int KTBC = KB / 512;
 
-  uint16_t *xs = reinterpret_cast<uint16_t *>(mg_smem);
-  uint16_t *xa = xs + I;
-  uint16_t *xn = xa + QD;
+  // xa (attention output, QD values) and xs (activations, I values) are adjacent: together they are the input
+  // vector of a whole row of Wb (dense columns | fc2 columns).  xa also stages the residual stream for LayerNorm.
+  uint16_t *xa = reinterpret_cast<uint16_t *>(mg_smem);
+  uint16_t *xs = xa + QD;
+  uint16_t *xn = xs + I;
   float *partA = reinterpret_cast<float *>(xn + H);
   float *partB = partA + kMegaRowsAMax * kMegaWaves;
-  float *partC = partB + kMegaRowsMax * kMegaWaves;
-  float *qf = partC + kMegaRowsMax * kMegaWaves;
+  uint32_t *a1_done = reinterpret_cast<uint32_t *>(partB + kMegaRowsMax * kMegaWaves);   // stream waves past segment A1
+  float *qf = partB + 2 * kMegaRowsMax * kMegaWaves;
   float *raw = qf + D;
   float *knew = raw + 3 * D;
   float *vnew = knew + D;
@@ -296,11 +352,29 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     rope_s = bf16_bits_to_f32(a.sin_t[(int64_t)pos * a.rot + tid0]);
   }
 
-  const int nA0 = 4 * (int)((int64_t)(a.NA / 4) * wg / G), nA1 = 4 * (int)((int64_t)(a.NA / 4) * (wg + 1) / G);
+  // Phase A rows.  Every block takes a share of the q|k|v rows and streams them first (segment A1), so that the
+  // attention blocks can start while the fc1 rows (segment A2) are still being streamed; the fc1 rows go to the
+  // blocks that run no attention head (to all blocks when every block runs one).
+  const bool is_attn = wg < a.Hq;
+  const int nA0 = 4 * (int)((int64_t)(a.n_qkv / 4) * wg / G), nA1 = 4 * (int)((int64_t)(a.n_qkv / 4) * (wg + 1) / G);
   const int rowsA = nA1 - nA0;
+  int fA0 = 0, fA1 = 0;
+  {
+    const int n_attn_blocks = a.Hq < G ? a.Hq : G;
+    const int others = G - n_attn_blocks;
+    if (others == 0) {
+      fA0 = 4 * (int)((int64_t)(I / 4) * wg / G);
+      fA1 = 4 * (int)((int64_t)(I / 4) * (wg + 1) / G);
+    } else if (!is_attn) {
+      const int o = wg - n_attn_blocks;
+      fA0 = 4 * (int)((int64_t)(I / 4) * o / others);
+      fA1 = 4 * (int)((int64_t)(I / 4) * (o + 1) / others);
+    }
+  }
+  const int rowsA2 = fA1 - fA0;
+  const int nA2 = a.n_qkv + fA0;
 
   int n0, n1;
-  const bool is_attn = wg < a.Hq;
   {
     const int n_attn_blocks = a.Hq < G ? a.Hq : G;
     const int others = G - n_attn_blocks;
@@ -318,24 +392,25 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   }
   const int nrows = n1 - n0;
 
-  const int ttA = rowsA * KTA, ttB = nrows * KTB, ttC = nrows * KTC;
+  const int ttA = rowsA * KTA, ttA2 = rowsA2 * KTA, ttB = nrows * KTBC;
   const bool streams = wave < kMegaStream;
   const int tA0 = streams ? ttA * wave / kMegaStream : 0, tA1 = streams ? ttA * (wave + 1) / kMegaStream : 0;
+  const int tA2_0 = streams ? ttA2 * wave / kMegaStream : 0, tA2_1 = streams ? ttA2 * (wave + 1) / kMegaStream : 0;
   const int tB0 = streams ? ttB * wave / kMegaStream : 0, tB1 = streams ? ttB * (wave + 1) / kMegaStream : 0;
-  const int tC0 = streams ? ttC * wave / kMegaStream : 0, tC1 = streams ? ttC * (wave + 1) / kMegaStream : 0;
 
   mg_u32x4 ring[kMegaRing];
   mg_u32x4 kreg[kMegaUK], vreg[kMegaUV];
 
   MgSplit sp;
-  sp.Wa0 = a.Wa0; sp.Wb0 = a.Wb0; sp.wa_stride = a.wa_stride; sp.wb_stride = a.wb_stride; sp.L = a.L; sp.H = H; sp.KB = KB; sp.QD = QD; sp.KTA = KTA; sp.KTB = KTB; sp.KTC = KTC;
-  sp.nA0 = nA0; sp.n0 = n0;
-  sp.tA0 = tA0; sp.tA1 = tA1; sp.tB0 = tB0; sp.tB1 = tB1; sp.tC0 = tC0; sp.tC1 = tC1;
+  sp.Wa0 = a.Wa0; sp.Wb0 = a.Wb0; sp.wa_stride = a.wa_stride; sp.wb_stride = a.wb_stride; sp.L = a.L; sp.H = H; sp.KB = KB; sp.QD = QD; sp.KTA = KTA; sp.KTBC = KTBC;
+  sp.nA0 = nA0; sp.nA2 = nA2; sp.n0 = n0;
+  sp.tA0 = tA0; sp.tA1 = tA1; sp.tA2_0 = tA2_0; sp.tA2_1 = tA2_1; sp.tB0 = tB0; sp.tB1 = tB1;
   MgCursor cur;
   cur.layer = 0; cur.seg = -1; cur.kc = 0; cur.KT = 1; cur.t = 0; cur.t1 = 0; cur.ld = 0;
   cur.ptr = a.Wa0;
   cur.done = !mg_seg_next(cur, sp);
   unsigned bar = 0;
+  int pending_rot = 0;
   const uint32_t tagbase = a.state->epoch * kMegaTagsPerLaunch;   // exchange tags of this launch: tagbase + index + 1
   uint32_t tag_x = 0;                                // tag of the residual-stream packets of the previous layer
   const float att_scale = a.scale;
@@ -400,6 +475,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   };
 
   for (int e = tid0; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
+  if (tid0 == 0) *a1_done = 0u;
 
   {
     const int lane = tid0 & 63;
@@ -422,10 +498,20 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     {
       const int tid = mg_opaque(tid0), lane = tid & 63;
       const bool service = wave == kMegaService;
+      // An attention block requests the cached keys and values of its head first: they do not depend on this
+      // layer's inputs, one CU can only keep so many cache lines in flight (the ~200 KB take several memory
+      // round trips), and the block would otherwise just wait for the residual stream.
+      if (is_attn) {
+        const int col = tid % NCOL, grp = tid / NCOL;
+        k_load(Kc, tid);
+        v_load(Vc, grp, col, grp < NG_V);
+      }
 
-      uint64_t bias_a = 0;
+      uint64_t bias_a = 0, bias_a2 = 0;
       if (service && lane * 4 < rowsA) bias_a = *reinterpret_cast<const uint64_t *>(ly.ba + nA0 + lane * 4);
-      if (tid < 2 * kMegaRowsMax * kMegaWaves) partB[tid] = 0.f;
+      if (service && lane * 4 < rowsA2) bias_a2 = *reinterpret_cast<const uint64_t *>(ly.ba + nA2 + lane * 4);
+      if (tid < kMegaRowsMax * kMegaWaves) partB[tid] = 0.f;
+      if (tid == 0) *a1_done = 0u;
       // the residual stream into LDS (xa is free until phase C): the plain vector for layer 0 (written
       // before this launch), else the packets of the previous layer's last phase, polled by all threads
       if (l == 0) {
@@ -486,42 +572,57 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         *reinterpret_cast<mg_u32x4 *>(xn + wave * 512 + lane * 8) = mg_u32x4{o[0], o[1], o[2], o[3]};
       }
       wg_sync();
-      const int rot = mg_run_phase(ring, cur, sp, tA0, tA1, KTA, xn, partA, lane, wave);
-      wg_sync();
-
-      if (service && lane * 4 < rowsA) {
-        const int n = nA0 + lane * 4;
-        uint32_t packed[2];
+      // The service wave turns the partial sums of a finished segment into packets (bias; activation for the
+      // fc1 rows).  It does so for the q|k|v rows as soon as every stream wave has left segment A1, while those
+      // waves stream the fc1 rows: the attention blocks get their inputs a whole segment early.
+      auto publish_a = [&](int n_first, int rows, const float *part, uint64_t bias, bool is_fc1) __attribute__((always_inline)) {
+        if (service && lane * 4 < rows) {
+          const int n = n_first + lane * 4;
+          uint32_t packed[2];
 #pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
-          float v[2];
+          for (int h2 = 0; h2 < 2; ++h2) {
+            float v[2];
 #pragma unroll
-          for (int k = 0; k < 2; ++k) {
-            const int e = lane * 4 + h2 * 2 + k;
-            float s4 = __uint_as_float((uint32_t)((bias_a >> (16 * (h2 * 2 + k))) & 0xffffu) << 16);
+            for (int k = 0; k < 2; ++k) {
+              const int e = lane * 4 + h2 * 2 + k;
+              float s4 = __uint_as_float((uint32_t)((bias >> (16 * (h2 * 2 + k))) & 0xffffu) << 16);
 #pragma unroll
-            for (int w = 0; w < kMegaStream; ++w) s4 += partA[e * kMegaWaves + w];
-            if (n >= a.n_qkv) s4 = act_eval(a.act, s4);
-            v[k] = s4;
+              for (int w = 0; w < kMegaStream; ++w) s4 += part[e * kMegaWaves + w];
+              if (is_fc1) s4 = act_eval(a.act, s4);
+              v[k] = s4;
+            }
+            packed[h2] = pack_bf16x2(v[0], v[1]);
           }
-          packed[h2] = pack_bf16x2(v[0], v[1]);
+          uint64_t *dst = is_fc1 ? a.actp + ((n - a.n_qkv) >> 1) : a.qkvp + (n >> 1);
+          const uint64_t tg = (uint64_t)(tagbase + bar + 1u) << 32;
+          if (!PROF || wg != a.mute_block) {
+            st_dev64(dst, tg | packed[0]);
+            st_dev64(dst + 1, tg | packed[1]);
+          }
         }
-        uint64_t *dst = n < a.n_qkv ? a.qkvp + (n >> 1) : a.actp + ((n - a.n_qkv) >> 1);
-        const uint64_t tg = (uint64_t)(tagbase + bar + 1u) << 32;
-        if (!PROF || wg != a.mute_block) {
-          st_dev64(dst, tg | packed[0]);
-          st_dev64(dst + 1, tg | packed[1]);
+      };
+      // the ring is rotated only now, just before it is consumed again: a rotation moves registers that loads
+      // are still writing, i.e. it waits for the newest of them, and by now those have had a whole exchange to land
+      mg_rotate_by(ring, pending_rot);
+      pending_rot = mg_run_phase(ring, cur, sp, tA0, tA1, tA2_0, tA2_1, KTA, xn, partA, partA + rowsA * kMegaWaves,
+                                 a1_done, lane, wave);
+      if (service) {   // its own ranges are empty: it arrives here at once and waits for the seven others
+        unsigned spins = 0;
+        while (__hip_atomic_load(a1_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)kMegaWaves) {
+          __builtin_amdgcn_s_sleep(1);
+          if (++spins > kMegaSpinLimit) {
+            __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
         }
+        publish_a(nA0, rowsA, partA, bias_a, false);
       }
+      wg_sync();
+      publish_a(nA2, rowsA2, partA + rowsA * kMegaWaves, bias_a2, true);
       stamp(l, 1);
       ++bar;   // no barrier: phase B polls the packets it needs
       stamp(l, 8);
-      mg_rotate_by(ring, rot);
-      if (is_attn) {
-        const int col = tid % NCOL, grp = tid / NCOL;
-        k_load(Kc, tid);
-        v_load(Vc, grp, col, grp < NG_V);
-      }
+      stamp(l, 9);
       wg_sync();
       stamp(l, 2);
     }
@@ -531,19 +632,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       for (int e = tid; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
 
       const uint32_t tag_a = tagbase + bar;   // bar was advanced past the A -> B exchange: its tag is index + 1
-      // a block without fc2 rows (an attention block, by default) does not wait for the activations:
-      // its attention starts as soon as the few blocks that produce its head's q, k and v are done
-      for (int base = 0; nrows > 0 && base < I / 2; base += kMegaThreads * 4) {
-        int idx[4];
-        bool on[4];
-        uint32_t val[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < I / 2; }
-        mg_poll<4, PROF>(a.actp, idx, on, tag_a, val, fault, a.spin_limit);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (on[i]) reinterpret_cast<uint32_t *>(xs)[idx[i]] = val[i];
-      }
+      // (a block with rows of Wb polls the activations together with the attention output, further down)
       if (is_attn) {
         const int h = wg;
         {
@@ -558,6 +647,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
             raw[which * D + 2 * pe + 1] = __uint_as_float(val[0] & 0xffff0000u);
           }
         }
+        stamp(l, 10);
         wg_sync();
         if (tid < D) {
           qf[tid] = mg_rope(raw, tid, a.rot, rope_c, rope_s);
@@ -577,6 +667,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
             k_partials(qb + tid);
           }
         }
+        stamp(l, 11);
         wg_sync();
         for (int t = tid; t < pos; t += kMegaThreads) {
           float sc = 0.f;
@@ -612,6 +703,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         sum = 0.f;
 #pragma unroll
         for (int w = 0; w < kMegaWaves; ++w) sum += sh[kMegaWaves + w];
+        stamp(l, 12);
 
         {
           const int col = tid % NCOL, grp = tid / NCOL;
@@ -648,21 +740,10 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           }
           st_dev64(a.attnp + (h * D) / 2 + lane, ((uint64_t)(tagbase + bar + 1u) << 32) | pack_bf16x2(o[0], o[1]));
         }
+        stamp(l, 13);
       }
-      wg_sync();
-      stamp(l, 3);
-      const int rot = mg_run_phase(ring, cur, sp, tB0, tB1, KTB, xs, partB, lane, wave);
-      stamp(l, 4);
-      // no barrier here: the consumers of the attention output poll its packets
-      mg_rotate_by(ring, rot);
-      wg_sync();
-      stamp(l, 5);
-    }
-
-    {
-      const int tid = mg_opaque(tid0), lane = tid & 63;
+      // ---- rows of Wb: [attention output | activations] . [dense columns | fc2 columns], one stream
       const bool service = wave == kMegaService;
-
       uint64_t res4 = 0, bd4 = 0, bf4 = 0;
       if (service && lane * 4 < nrows) {
         res4 = ld_dev64(a.x + n0 + lane * 4);
@@ -671,20 +752,27 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       }
       const uint32_t tag_b = tagbase + bar + 1u;
       ++bar;
-      for (int base = 0; base < QD / 2; base += kMegaThreads * 4) {
-        int idx[4];
-        bool on[4];
-        uint32_t val[4];
+      // one list of packets: QD / 2 of the attention output, then I / 2 activations; they land in xa | xs, which
+      // are adjacent.  Seven packets per thread and round, so the list takes two round trips instead of four.
+      const int n_attn_pk = QD / 2, n_pk = (QD + I) / 2;
+      for (int base = 0; nrows > 0 && base < n_pk; base += kMegaThreads * 7) {
+        int idx[7];
+        bool on[7];
+        uint32_t val[7];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < QD / 2; }
-        mg_poll<4, PROF>(a.attnp, idx, on, tag_b, val, fault, a.spin_limit);
+        for (int i = 0; i < 7; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < n_pk; }
+        mg_poll2<7, PROF>(a.attnp, tag_b, n_attn_pk, a.actp, tag_a, idx, on, val, fault, a.spin_limit);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 7; ++i)
           if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
       }
       wg_sync();
-      const int rot = mg_run_phase(ring, cur, sp, tC0, tC1, KTC, xa, partC, lane, wave);
+      stamp(l, 3);
+      mg_rotate_by(ring, pending_rot);
+      pending_rot = mg_run_phase(ring, cur, sp, tB0, tB1, 0, 0, KTBC, xa, partB, partB, nullptr, lane, wave);
+      stamp(l, 4);
       wg_sync();
+      stamp(l, 5);
 
       if (service && lane * 4 < nrows) {
         auto elem = [](uint64_t v, int k) { return __uint_as_float((uint32_t)((v >> (16 * k)) & 0xffffu) << 16); };
@@ -695,8 +783,6 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           float sacc = 0.f;
 #pragma unroll
           for (int w = 0; w < kMegaStream; ++w) sacc += partB[e * kMegaWaves + w];
-#pragma unroll
-          for (int w = 0; w < kMegaStream; ++w) sacc += partC[e * kMegaWaves + w];
           v[k] = sacc + (elem(bd4, k) + elem(bf4, k)) + elem(res4, k);
         }
         const uint32_t lo = pack_bf16x2(v[0], v[1]), hi = pack_bf16x2(v[2], v[3]);
@@ -708,10 +794,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       tag_x = tagbase + bar + 1u;
       ++bar;
       stamp(l, 6);
-      if (l + 1 < a.L) {   // no barrier: the next layer's LayerNorm polls the packets
-        mg_rotate_by(ring, rot);
-        wg_sync();
-      }
+      if (l + 1 < a.L) wg_sync();   // no grid barrier: the next layer's LayerNorm polls the packets
       stamp(l, 7);
     }
   }
@@ -744,7 +827,10 @@ bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
     const int rem = a.H - a.Hq * ra;
     if (rem < 0 || rem / others + 4 > kMegaRowsMax) return no("too many rows per block");
   }
-  if (a.NA / num_cu + 4 > kMegaRowsAMax) return no("too many phase A rows per block");
+  {
+    const int fc1_blocks = others > 0 ? others : num_cu;
+    if (a.n_qkv / num_cu + 4 + a.I / fc1_blocks + 4 > kMegaRowsAMax) return no("too many phase A rows per block");
+  }
   if (mega_lds_bytes(a, D) > 150 * 1024) return no("context too long for the LDS score buffer");
   return true;
 }
