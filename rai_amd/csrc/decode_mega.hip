@@ -45,7 +45,7 @@ constexpr uint32_t kMegaTagsPerLaunch = 1024;   // more than the 3 exchanges per
 constexpr int kMegaRing = 16;
 constexpr int kMegaRowsAMax = 96;
 constexpr int kMegaRowsMax = 16;
-constexpr int kMegaUK = 13, kMegaUV = 13;
+constexpr int kMegaUK = 13, kMegaUV = 12;
 
 __device__ __forceinline__ float mg_dot2(uint32_t a, uint32_t b, float c) {
   mg_bf16x2 p, q;
@@ -336,6 +336,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   float *red = vnew + D;
   float *sh = red + NG_V * D;
   float *red2 = sh + 2 * kMegaWaves;
+  uint32_t *qh = reinterpret_cast<uint32_t *>(red2);   // q of the current head as packed bf16 (red2 is used after the scores)
   float *scores = red2 + 4 * D;
   float *pd = scores + a.Tmax + 1;
 
@@ -431,17 +432,10 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       const int q = q0 + kMegaThreads * u;
       if (q < pos * NCOL) {
         const int c = q % NCOL;
-        const float4 qa = *reinterpret_cast<const float4 *>(qf + c * 8);
-        const float4 qb = *reinterpret_cast<const float4 *>(qf + c * 8 + 4);
-        const uint32_t w4[4] = {kreg[u].x, kreg[u].y, kreg[u].z, kreg[u].w};
-        float acc = qa.x * __uint_as_float(w4[0] << 16);
-        acc = fmaf(qa.y, __uint_as_float(w4[0] & 0xffff0000u), acc);
-        acc = fmaf(qa.z, __uint_as_float(w4[1] << 16), acc);
-        acc = fmaf(qa.w, __uint_as_float(w4[1] & 0xffff0000u), acc);
-        acc = fmaf(qb.x, __uint_as_float(w4[2] << 16), acc);
-        acc = fmaf(qb.y, __uint_as_float(w4[2] & 0xffff0000u), acc);
-        acc = fmaf(qb.z, __uint_as_float(w4[3] << 16), acc);
-        acc = fmaf(qb.w, __uint_as_float(w4[3] & 0xffff0000u), acc);
+        // q after the rotary embedding is exactly representable in bf16 (the reference rounds it to the model
+        // dtype before the upcast, phi2.rs:244-247), so the products equal the f32 ones
+        const mg_u32x4 q4 = *reinterpret_cast<const mg_u32x4 *>(qh + c * 4);
+        const float acc = mg_dot8(kreg[u], q4, 0.f);
         pd[q] = acc;
       }
     }
@@ -650,9 +644,11 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         stamp(l, 10);
         wg_sync();
         if (tid < D) {
-          qf[tid] = mg_rope(raw, tid, a.rot, rope_c, rope_s);
+          const float qr = mg_rope(raw, tid, a.rot, rope_c, rope_s);
           const float kr = mg_rope(raw + D, tid, a.rot, rope_c, rope_s);
           const float vr = raw[2 * D + tid];
+          qf[tid] = qr;
+          reinterpret_cast<uint16_t *>(qh)[tid] = f32_to_bf16_bits(qr);   // exact: qr carries bf16 precision
           knew[tid] = kr;
           vnew[tid] = vr;
           Kc[(int64_t)pos * D + tid] = f32_to_bf16_bits(kr);
