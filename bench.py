@@ -393,7 +393,8 @@ def main():
         "sampled_decode_tokens_per_s": round((NEW - 1) / (samp_ms / 1e3), 2),
         "roofline": {
             "kernel": "k_phi2_decode_step (persistent kernel: all 32 layers of one decode step, blocks exchange "
-                      "tagged packets instead of grid barriers, weight ring prefetched across phases)",
+                      "tagged packets instead of grid barriers, weight ring prefetched across segments, "
+                      "attention inputs published ahead of the fc1 stream)",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,

@@ -3,14 +3,16 @@
 // parallel attention + MLP block) for batch 1, bf16.
 //
 // One 512-thread block per CU stays resident for the whole token.  A layer is
-// three weight-streaming phases:
-//   A  LayerNorm(x) . Wa^T + bias   -> q | k | v | gelu(fc1)      (rows split over blocks)
-//   B  head h attention on block h  ||  fc2 partial products on the other blocks
-//   C  dense(attn) partial + fc2 partial + biases + residual -> x (same rows as B)
+// three weight-streaming segments:
+//   A1  LayerNorm(x) . Wa[q|k|v rows]^T + bias -> q | k | v   (rows split over all blocks, streamed first)
+//   A2  LayerNorm(x) . Wa[fc1 rows]^T + bias   -> gelu(fc1)   (rows split over the blocks without an attention head)
+//       head h attention on block h, started as soon as the A1 packets arrive, i.e. while A2 streams
+//   BC  [attn | act] . Wb^T + biases + residual -> x          (whole rows of Wb = dense | fc2 columns)
 // Weights do not depend on activations: every wave keeps a ring of weight tiles
-// in flight that runs ahead across the phase boundaries, so HBM keeps streaming
-// while a block waits for its inputs.  Attention (latency bound, 0.2 MB per head)
-// hides behind the 52 MB fc2 stream of phase B.
+// in flight that runs ahead across the segment boundaries, so HBM keeps streaming
+// while a block waits for its inputs.  A1 runs into A2 without a pause: each stream wave
+// bumps a counter in LDS when it leaves A1, and the service wave publishes the q|k|v
+// packets when all have.
 //
 // There is no grid barrier.  The vectors that cross blocks (x, q|k|v, act, attn) are
 // written as 8-byte packets {two bf16 values, 32-bit tag}, tag = launch epoch * 1024 +
