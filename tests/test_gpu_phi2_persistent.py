@@ -93,3 +93,24 @@ def test_lost_packet_times_out_and_reports(hip, monkeypatch):
     assert_close(logits, want, "bf16", "persistent step after the fault")
     check_tokens(tok, want, "bf16")
     dec.close()
+
+
+def test_persistent_step_long_context_takes_several_prefetch_passes(hip):
+    """Beyond ~612 cached positions one head's values, and beyond ~665 its keys, no longer fit the registers the
+    attention blocks prefetch them into, so the kernel fetches them in several passes; the benchmark's last
+    tokens run there."""
+    cfg = wide_cfg(max_position_embeddings=768)
+    dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=704)
+    ids = np.random.Generator(np.random.PCG64(14)).integers(0, cfg.vocab_size, (1, 660)).astype(np.uint32)
+    logits, _ = dec.forward(ids)
+    want = ref.fwd(ids)
+    assert_close(logits, want, "bf16", "prefill logits")
+    nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
+    for step in range(10):                   # context 660..669: two passes over the values, from 666 on also over the keys
+        logits, tok = dec.forward(nxt)
+        want = ref.fwd(nxt)
+        assert_close(logits, want, "bf16", f"decode step at context {660 + step}")
+        check_tokens(tok, want, "bf16")
+        nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
+    assert dec.context_len() == 670
+    dec.close()
