@@ -6,6 +6,8 @@
 
 namespace rai {
 
+constexpr int kMegaActPackets = 256 * 16;   // slots of the activation packets: 16 for each of up to 256 producer blocks
+
 struct DevState {
   int pos;    // tokens already in the KV cache
   int step;   // greedy steps taken by the current generate call
@@ -30,8 +32,8 @@ struct MegaArgs {
   // a packet is valid for an exchange when its tag is epoch * 1024 + exchange index + 1.
   uint64_t *xp;             // [H / 2]      residual stream after a layer
   uint64_t *qkvp;           // [3 * QD / 2]
-  uint64_t *actp;           // [I / 2]      gelu(fc1)
-  uint64_t *attnp;          // [QD / 2]
+  uint64_t *actp;           // [kMegaActPackets] gelu(fc1), three values to a packet, 16 packets per producer block
+  uint64_t *attnp;          // [Hq * ceil(D / 3)] attention output, three values to a packet
   uint16_t *kcache, *vcache;
   int64_t kv_layer_stride;  // elements between consecutive layers of the cache
   const uint16_t *cos_t, *sin_t;

@@ -341,6 +341,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   uint32_t *qh = reinterpret_cast<uint32_t *>(red2);   // q of the current head as packed bf16 (red2 is used after the scores)
   float *scores = red2 + 4 * D;
   float *pd = scores + a.Tmax + 1;
+  uint32_t *pkmeta = reinterpret_cast<uint32_t *>(pd + (size_t)a.Tmax * NCOL);   // [9][512]
 
   const int tid0 = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid0 >> 6);
@@ -376,6 +377,30 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   }
   const int rowsA2 = fA1 - fA0;
   const int nA2 = a.n_qkv + fA0;
+  // The activations and the attention output travel three values to a packet ({3 bf16, 16-bit tag}), in slots
+  // that belong to their producer: block o of the fc1 producers owns 16 slots (it has at most 48 rows), head h owns
+  // kPkHead = ceil(D / 3).  A consumer wants both vectors whole, and 9 packets per thread cover them in one poll.
+  constexpr int kPkFc1 = 16, kPkHead = (D + 2) / 3, kPkPoll = 9;
+  const int fc1_first = (a.Hq < G ? a.Hq : G) < G ? (a.Hq < G ? a.Hq : G) : 0;   // index of the first fc1 producer
+  const int fc1_blocks = G - fc1_first;
+  const int fc1_me = wg - fc1_first;
+  const int n_attn_pk = a.Hq * kPkHead;
+  for (int i = 0; i < kPkPoll; ++i) {   // this thread's packets of the combined poll (the same in every layer)
+    const int idx = i * kMegaThreads + tid0;
+    int first = 0, count = 0;
+    if (idx < n_attn_pk) {
+      const int h = idx / kPkHead, p3 = (idx - h * kPkHead) * 3;
+      first = h * D + p3;
+      count = D - p3;
+    } else if (idx < n_attn_pk + fc1_blocks * kPkFc1) {
+      const int s2 = idx - n_attn_pk, o = s2 / kPkFc1, p3 = (s2 - o * kPkFc1) * 3;
+      const int r0 = 4 * (int)((int64_t)(I / 4) * o / fc1_blocks), r1 = 4 * (int)((int64_t)(I / 4) * (o + 1) / fc1_blocks);
+      first = QD + r0 + p3;
+      count = r1 - r0 - p3;
+    }
+    count = count < 0 ? 0 : count > 3 ? 3 : count;
+    pkmeta[idx] = (uint32_t)first | ((uint32_t)count << 16);
+  }
 
   int n0, n1;
   {
@@ -505,7 +530,11 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
 
       uint64_t bias_a = 0, bias_a2 = 0;
       if (service && lane * 4 < rowsA) bias_a = *reinterpret_cast<const uint64_t *>(ly.ba + nA0 + lane * 4);
-      if (service && lane * 4 < rowsA2) bias_a2 = *reinterpret_cast<const uint64_t *>(ly.ba + nA2 + lane * 4);
+      if (service) {   // rows 3 lane .. 3 lane + 2 of this block's fc1 share
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (lane * 3 + j < rowsA2) bias_a2 |= (uint64_t)ly.ba[nA2 + lane * 3 + j] << (16 * j);
+      }
       if (tid < kMegaRowsMax * kMegaWaves) partB[tid] = 0.f;
       if (tid == 0) *a1_done = 0u;
       // the residual stream into LDS (xa is free until phase C): the plain vector for layer 0 (written
@@ -614,7 +643,23 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         publish_a(nA0, rowsA, partA, bias_a, false);
       }
       wg_sync();
-      publish_a(nA2, rowsA2, partA + rowsA * kMegaWaves, bias_a2, true);
+      if (service && lane * 3 < rowsA2) {   // gelu(fc1) of this block's rows, three to a packet
+        const float *part = partA + rowsA * kMegaWaves;
+        uint32_t hv[3] = {0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          const int e = lane * 3 + j;
+          if (e < rowsA2) {
+            float s4 = __uint_as_float((uint32_t)((bias_a2 >> (16 * j)) & 0xffffu) << 16);
+#pragma unroll
+            for (int w = 0; w < kMegaStream; ++w) s4 += part[e * kMegaWaves + w];
+            hv[j] = f32_to_bf16_bits(act_eval(a.act, s4));
+          }
+        }
+        const uint64_t tg = (uint64_t)((tagbase + bar + 1u) & 0xffffu) << 48;
+        if (!PROF || wg != a.mute_block)
+          st_dev64(a.actp + fc1_me * kPkFc1 + lane, tg | ((uint64_t)hv[2] << 32) | ((uint64_t)hv[1] << 16) | hv[0]);
+      }
       stamp(l, 1);
       ++bar;   // no barrier: phase B polls the packets it needs
       stamp(l, 8);
@@ -728,15 +773,17 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           red2[tid] = r;
         }
         wg_sync();
-        if (wave == kMegaService && lane < D / 2) {
+        if (wave == kMegaService && lane < kPkHead) {
           const float inv = 1.0f / sum, p_new = scores[pos];
-          float o[2];
+          uint32_t hv[3] = {0u, 0u, 0u};
 #pragma unroll
-          for (int k = 0; k < 2; ++k) {
-            const int d = 2 * lane + k;
-            o[k] = (p_new * vnew[d] + red2[d] + red2[D + d] + red2[2 * D + d] + red2[3 * D + d]) * inv;
+          for (int k = 0; k < 3; ++k) {
+            const int d = 3 * lane + k;
+            if (d < D)
+              hv[k] = f32_to_bf16_bits((p_new * vnew[d] + red2[d] + red2[D + d] + red2[2 * D + d] + red2[3 * D + d]) * inv);
           }
-          st_dev64(a.attnp + (h * D) / 2 + lane, ((uint64_t)(tagbase + bar + 1u) << 32) | pack_bf16x2(o[0], o[1]));
+          const uint64_t tg = (uint64_t)((tagbase + bar + 1u) & 0xffffu) << 48;
+          st_dev64(a.attnp + h * kPkHead + lane, tg | ((uint64_t)hv[2] << 32) | ((uint64_t)hv[1] << 16) | hv[0]);
         }
         stamp(l, 13);
       }
@@ -750,19 +797,46 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       }
       const uint32_t tag_b = tagbase + bar + 1u;
       ++bar;
-      // one list of packets: QD / 2 of the attention output, then I / 2 activations; they land in xa | xs, which
-      // are adjacent.  Seven packets per thread and round, so the list takes two round trips instead of four.
-      const int n_attn_pk = QD / 2, n_pk = (QD + I) / 2;
-      for (int base = 0; nrows > 0 && base < n_pk; base += kMegaThreads * 7) {
-        int idx[7];
-        bool on[7];
-        uint32_t val[7];
+      // one list of packets: Hq * kPkHead of the attention output, then fc1_blocks * kPkFc1 of the activations;
+      // nine per thread cover it in one poll, i.e. one memory round trip when everything has arrived.  Where a
+      // packet's values go in [xa | xs] and how many of its three are real sits in pkmeta (filled at kernel start).
+      if (nrows > 0) {
+        uint64_t pk[kPkPoll];
+        uint32_t need = 0u;
 #pragma unroll
-        for (int i = 0; i < 7; ++i) { idx[i] = base + i * kMegaThreads + tid; on[i] = idx[i] < n_pk; }
-        mg_poll2<7, PROF>(a.attnp, tag_b, n_attn_pk, a.actp, tag_a, idx, on, val, fault, a.spin_limit);
+        for (int i = 0; i < kPkPoll; ++i) {
+          pk[i] = 0ull;
+          if ((pkmeta[i * kMegaThreads + tid] >> 16) != 0u) need |= 1u << i;
+        }
+        const uint32_t t16a = tag_b & 0xffffu, t16f = tag_a & 0xffffu;
+        unsigned spins = 0;
+        for (;;) {
 #pragma unroll
-        for (int i = 0; i < 7; ++i)
-          if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
+          for (int i = 0; i < kPkPoll; ++i) {
+            const int idx = i * kMegaThreads + tid;
+            if (need & (1u << i)) pk[i] = ld_dev64(idx < n_attn_pk ? a.attnp + idx : a.actp + (idx - n_attn_pk));
+          }
+#pragma unroll
+          for (int i = 0; i < kPkPoll; ++i) {
+            const int idx = i * kMegaThreads + tid;
+            if ((need & (1u << i)) && (uint32_t)(pk[i] >> 48) == (idx < n_attn_pk ? t16a : t16f)) need &= ~(1u << i);
+          }
+          if (!__any(need != 0u)) break;
+          __builtin_amdgcn_s_sleep(1);
+          if (++spins > (PROF ? a.spin_limit : kMegaSpinLimit)) {
+            __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          if ((spins & 255u) == 0 && __hip_atomic_load(fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+        }
+#pragma unroll
+        for (int i = 0; i < kPkPoll; ++i) {
+          const uint32_t meta = pkmeta[i * kMegaThreads + tid];
+          const uint32_t first = meta & 0xffffu, count = meta >> 16;
+          if (count > 0) xa[first] = (uint16_t)(pk[i] & 0xffffu);
+          if (count > 1) xa[first + 1] = (uint16_t)((pk[i] >> 16) & 0xffffu);
+          if (count > 2) xa[first + 2] = (uint16_t)((pk[i] >> 32) & 0xffffu);
+        }
       }
       wg_sync();
       stamp(l, 3);
@@ -802,7 +876,7 @@ size_t mega_lds_bytes(const MegaArgs &a, int D) {
   const int NG_V = kMegaThreads / (D / 8);
   size_t n = (size_t)(a.I + a.QD + a.H) * 2;
   n += sizeof(float) * ((kMegaRowsAMax + 2 * kMegaRowsMax) * kMegaWaves + 6 * (size_t)D + (size_t)NG_V * D +
-                        2 * kMegaWaves + 4 * (size_t)D + (size_t)a.Tmax + 1 + (size_t)a.Tmax * (D / 8));
+                        2 * kMegaWaves + 4 * (size_t)D + (size_t)a.Tmax + 1 + (size_t)a.Tmax * (D / 8) + 9 * kMegaThreads);
   return (n + 15) & ~(size_t)15;
 }
 
@@ -828,6 +902,9 @@ bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
   {
     const int fc1_blocks = others > 0 ? others : num_cu;
     if (a.n_qkv / num_cu + 4 + a.I / fc1_blocks + 4 > kMegaRowsAMax) return no("too many phase A rows per block");
+    // three-value packets: 16 slots per fc1 producer, ceil(D / 3) per head, inside the packet arrays of I / 2 and QD / 2
+    if (4 * ((a.I / 4 + fc1_blocks - 1) / fc1_blocks) > 48 || fc1_blocks * 16 > kMegaActPackets)
+      return no("activation packets do not fit their slots");
   }
   if (mega_lds_bytes(a, D) > 150 * 1024) return no("context too long for the LDS score buffer");
   return true;

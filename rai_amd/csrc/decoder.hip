@@ -725,7 +725,7 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   m.xp = d->mega_xchg;
   m.qkvp = m.xp + d->H / 2;
   m.actp = m.qkvp + (d->QD + 2 * d->KD) / 2;
-  m.attnp = m.actp + d->I / 2;
+  m.attnp = m.actp + kMegaActPackets;
   m.kcache = (uint16_t *)d->kcache; m.vcache = (uint16_t *)d->vcache;
   m.kv_layer_stride = (int64_t)d->cfg.max_batch * d->Hkv * d->cfg.max_context * d->D;
   m.cos_t = (const uint16_t *)d->cos_t; m.sin_t = (const uint16_t *)d->sin_t;
@@ -1237,7 +1237,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->mega_xchg = nullptr;
   if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_NO_MEGA") == nullptr) {
     {  // zeroed: tag 0 is never a valid exchange tag
-      const size_t packets = (size_t)(d->H + d->QD + 2 * d->KD + d->I + d->QD) / 2 + 8;
+      // x and q|k|v: two values to a packet; activations: 16 packets for each of up to 256 producers;
+      // attention output: ceil(D / 3) packets per head
+      const size_t packets = (size_t)(d->H + d->QD + 2 * d->KD) / 2 + kMegaActPackets + (size_t)d->Hq * ((d->D + 2) / 3) + 8;
       if ((st = dalloc(d, packets * sizeof(uint64_t), &tmp))) return bail(st);
       d->mega_xchg = (uint64_t *)tmp;
       if (hipMemset(d->mega_xchg, 0, packets * sizeof(uint64_t)) != hipSuccess)
