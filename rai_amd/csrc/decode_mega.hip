@@ -15,10 +15,13 @@
 // packets when all have.
 //
 // There is no grid barrier.  The vectors that cross blocks (x, q|k|v, act, attn) are
-// written as 8-byte packets {two bf16 values, 32-bit tag}, tag = launch epoch * 1024 +
-// exchange index + 1, with device-scope write-through stores, and every consumer
-// polls exactly the packets it needs with device-scope loads until their tags match
-// (an 8-byte store is single-copy atomic, so a matching tag proves the payload).
+// written as 8-byte packets, tag = launch epoch * 1024 + exchange index + 1, with
+// device-scope write-through stores, and every consumer polls exactly the packets it
+// needs with device-scope loads until their tags match (an 8-byte store is single-copy
+// atomic, so a matching tag proves the payload).  x and q|k|v use {two bf16 values,
+// 32-bit tag} at the vector's own index; act and attn, which every Wb block needs whole,
+// use {three bf16 values, low 16 bits of the tag} in producer-owned slots (16 per fc1
+// block, ceil(D / 3) per head), so that nine packets per thread, one poll, fetch both.
 // Data and notification are therefore one memory trip, not a store, its
 // acknowledgement, a flag and a second read; a buffer is safe to overwrite two
 // exchanges later because receiving a block's packets proves that block has left the
