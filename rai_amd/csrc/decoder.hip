@@ -1218,7 +1218,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->token_log = (uint32_t *)tmp;
   if ((st = dalloc(d, sizeof(DevState), &tmp))) return bail(st);
   d->state = (DevState *)tmp;
-  d->splitk_ws_bytes = (size_t)8 * d->max_rows * d->H * sizeof(float);
+  d->splitk_ws_bytes = (size_t)12 * d->max_rows * d->H * sizeof(float);
   if (d->splitk_ws_bytes > ((size_t)256 << 20)) d->splitk_ws_bytes = (size_t)256 << 20;
   if ((st = dalloc(d, d->splitk_ws_bytes, &d->splitk_ws))) return bail(st);
   if ((st = dalloc(d, attention_decode_ws_bytes(cfg->max_batch, d->Hq, d->D), &d->attn_ws))) return bail(st);

@@ -1002,8 +1002,25 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   const int tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
   int splits = 1;
   if (a.splitk_ws && tiles < kNumCU) {
-    while (splits < 8 && tiles * splits * 2 <= 2 * kNumCU && a.K / (splits * 2) >= 512) splits *= 2;
-    while (splits > 1 && (size_t)splits * a.M * a.N * sizeof(float) > a.splitk_ws_bytes) splits /= 2;
+    // Cost model in units of one K tile of one block: blocks go round-robin over the CUs, a CU holds up to three,
+    // n co-resident blocks share a CU at a combined rate of 0.5 / 0.85 / 1 (one block alone cannot hide its own
+    // barriers and memory latency), each block pays ~8 units of prologue + epilogue, and every split adds a pass over
+    // the f32 partial sums (~7 units at 512 x 2560).  Measured at 512 x 2560 x 12800: 3, 4, 6, 9, 12 splits give
+    // 6.69, 6.64, 6.28, 6.44, 6.79 ms per 32-layer prefill, the order this model predicts.
+    const int kt = a.K / 32;
+    float best = 0.f;
+    for (int s = 1; s <= 12; ++s) {
+      if (s > 1 && (kt / s < 8 || (size_t)s * a.M * a.N * sizeof(float) > a.splitk_ws_bytes)) break;
+      const float per_block = (float)((kt + s - 1) / s) + 8.f;
+      int left = (tiles * s + kNumCU - 1) / kNumCU;   // blocks on the busiest CU
+      float cost = (s > 1 ? 7.f * s : 0.f) * ((float)a.M * a.N / (512.f * 2560.f));
+      while (left > 0) {
+        const int n = left < 3 ? left : 3;
+        cost += n * per_block / (n == 1 ? 0.5f : n == 2 ? 0.85f : 1.f);
+        left -= n;
+      }
+      if (s == 1 || cost < best) { best = cost; splits = s; }
+    }
   }
   // Tile choice.  The LDS-DMA kernels stream K tiles straight into LDS; the 256x128 tile halves the
   // L2 -> LDS traffic per flop for one operand and is used once there are enough tiles of that size
