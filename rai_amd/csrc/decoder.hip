@@ -832,6 +832,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
     MegaArgs m = mega_args(d);
     RAI_TRY(launch_phi2_decode_step(st, m, d->D, d->num_cu));
   }
+  bool ln_ready = false;   // d->ln already holds this layer's LayerNorm(x): the previous layer's last Linear wrote it
   for (int l = 0; l < (use_mega ? 0 : d->L); ++l) {
     const Layer &ly = d->layers[l];
     LinearArgs a = linear_args_default();
@@ -839,11 +840,14 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
       a.A = x; a.lda = H;
       a.ln_kind = 0; a.ln_w = ly.ln_w; a.ln_b = ly.ln_b; a.ln_eps = (float)d->cfg.norm_eps;
     } else {
-      rai_hip_tensor tx = desc2(x, dt, M, H, H), tw = desc1(ly.ln_w, dt, H), tb = desc1(ly.ln_b, dt, H),
-                     to = desc2(d->ln, dt, M, H, H);
-      RAI_TRY(rai_hip_layer_norm(d->dev, &tx, &tw, &tb, d->cfg.norm_eps, &to));
+      if (!ln_ready) {
+        rai_hip_tensor tx = desc2(x, dt, M, H, H), tw = desc1(ly.ln_w, dt, H), tb = desc1(ly.ln_b, dt, H),
+                       to = desc2(d->ln, dt, M, H, H);
+        RAI_TRY(rai_hip_layer_norm(d->dev, &tx, &tw, &tb, d->cfg.norm_eps, &to));
+      }
       a.A = d->ln; a.lda = H;
     }
+    ln_ready = false;
     a.W = ly.Wa; a.ldw = H; a.bias = ly.ba;
     a.Wfrag = frag ? ly.Wa_f : nullptr;
     a.out1 = d->qkv; a.ld1 = ldq;
@@ -899,6 +903,13 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
     b.out1 = xn; b.ld1 = H;
     b.M = (int)M; b.N = H; b.K = d->KB; b.n_split = H;
     b.splitk_ws = d->splitk_ws; b.splitk_ws_bytes = d->splitk_ws_bytes;
+    if (!fuse_ln && dt == RAI_BF16 && l + 1 < d->L) {
+      // the next layer's input LayerNorm rides on the pass that sums this product's split-K partial sums
+      const Layer &nx = d->layers[l + 1];
+      b.post_ln_out = d->ln; b.post_ln_w = nx.ln_w; b.post_ln_b = nx.ln_b; b.post_ln_eps = (float)d->cfg.norm_eps;
+      ln_ready = linear_fuses_post_norm(b);
+      if (!ln_ready) b.post_ln_out = nullptr;
+    }
     RAI_TRY(linear(d, st, b));
     char *tmp = x; x = xn; xn = tmp;
   }

@@ -46,7 +46,17 @@ struct LinearArgs {
   // 16 rows x 32 columns that one wave loads with one instruction are 1 KB of consecutive memory
   // ([N / 16 row tiles][K / 32 steps][64 lanes][8 elements], see linear_fragment_layout); null: read W itself.
   const void *Wfrag;
+  // Optional LayerNorm of the finished output rows, written to post_ln_out ([M, N], dense) next to out1: the pass
+  // that sums the split-K partial products has the whole row at hand, so the norm that consumes the output (the next
+  // block's input LayerNorm) costs no launch of its own.  Only that pass offers it: ask linear_fuses_post_norm()
+  // first and run the norm separately when it says no.
+  void *post_ln_out;
+  const void *post_ln_w;
+  const void *post_ln_b;
+  float post_ln_eps;
 };
+// True when launch_linear_bf16 with these arguments will also write post_ln_out.
+bool linear_fuses_post_norm(const LinearArgs &a);
 inline LinearArgs linear_args_default() {
   LinearArgs a;
   memset(&a, 0, sizeof(a));

@@ -516,6 +516,136 @@ __global__ void __launch_bounds__(256) k_splitk_epilogue(LinearArgs a, int split
   }
 }
 
+// The same pass for a Linear whose output rows are normalised next: a wave owns a row (N <= 512 * ITEMS columns, 8
+// per lane and item), sums the partial products, applies bias / activation / residual, stores the bf16 row, and then
+// runs LayerNorm on the stored (rounded) values with the arithmetic of the stand-alone norm kernel -- same
+// per-lane order, same wave reductions -- so fusing changes no bit (rai-nn/src/layer_norm.rs:32-42).
+template <int ITEMS>
+__global__ void __launch_bounds__(128) k_splitk_epilogue_ln(LinearArgs a, int splits, const float *partial) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 2 + (threadIdx.x >> 6);
+  if (row >= a.M) return;
+  const int packs = a.N / 8;
+  const int64_t total = (int64_t)a.M * a.N;
+  const uint16_t *bias = (const uint16_t *)a.bias, *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+  float v[ITEMS][8];
+  float s = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int p = lane + it * 64;
+    if (p < packs) {
+      const int n = p * 8;
+      float x[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = 0.f;
+      const float *pp = partial + (int64_t)row * a.N + n;
+      // six splits' loads are issued together (a wave has a whole row to itself and little else to overlap with);
+      // the additions stay in split order
+      for (int s0 = 0; s0 < splits; s0 += 6) {
+        f32x4 p0[6], p1[6];
+#pragma unroll
+        for (int u = 0; u < 6; ++u) {
+          const int sp = s0 + u < splits ? s0 + u : splits - 1;
+          p0[u] = *reinterpret_cast<const f32x4 *>(pp + (int64_t)sp * total);
+          p1[u] = *reinterpret_cast<const f32x4 *>(pp + (int64_t)sp * total + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 6; ++u) {
+          if (s0 + u < splits) {
+            x[0] += p0[u].x; x[1] += p0[u].y; x[2] += p0[u].z; x[3] += p0[u].w;
+            x[4] += p1[u].x; x[5] += p1[u].y; x[6] += p1[u].z; x[7] += p1[u].w;
+          }
+        }
+      }
+      float b1[8], b2[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) b1[e] = b2[e] = 0.f;
+      if (bias) unpack8(*reinterpret_cast<const u32x4 *>(bias + n), b1);
+      if (bias2) unpack8(*reinterpret_cast<const u32x4 *>(bias2 + n), b2);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] += b1[e] + b2[e];
+      if (a.act >= 0) act8(a.act, x, n, a.act_from);
+      if (res) {
+        float rv[8];
+        unpack8(*reinterpret_cast<const u32x4 *>(res + (int64_t)row * a.ldr + n), rv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] += rv[e];
+      }
+      u32x4 o;
+      o.x = (uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
+      o.y = (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
+      o.z = (uint32_t)f32_to_bf16_bits(x[4]) | ((uint32_t)f32_to_bf16_bits(x[5]) << 16);
+      o.w = (uint32_t)f32_to_bf16_bits(x[6]) | ((uint32_t)f32_to_bf16_bits(x[7]) << 16);
+      *reinterpret_cast<u32x4 *>((uint16_t *)a.out1 + (int64_t)row * a.ld1 + n) = o;
+      unpack8(o, v[it]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += v[it][e];
+    }
+  }
+  s = wave_sum(s);
+  const float mean = s / (float)a.N;
+  float q = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int p = lane + it * 64;
+    if (p < packs) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = v[it][e] - mean;
+        q += d * d;
+      }
+    }
+  }
+  q = wave_sum(q);
+  const float scale = 1.0f / sqrtf(q / (float)a.N + a.post_ln_eps);
+  const uint16_t *lw = (const uint16_t *)a.post_ln_w, *lb = (const uint16_t *)a.post_ln_b;
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int p = lane + it * 64;
+    if (p < packs) {
+      const int n = p * 8;
+      float wv[8], bv[8];
+      if (lw) unpack8(*reinterpret_cast<const u32x4 *>(lw + n), wv);
+      if (lb) unpack8(*reinterpret_cast<const u32x4 *>(lb + n), bv);
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float y = (v[it][e] - mean) * scale;
+        if (lw) y *= wv[e];
+        if (lb) y += bv[e];
+        h[e] = f32_to_bf16_bits(y);
+      }
+      u32x4 o = {h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+      *reinterpret_cast<u32x4 *>((uint16_t *)a.post_ln_out + (int64_t)row * a.N + n) = o;
+    }
+  }
+}
+
+// Whether the pass over the partial sums can also normalise the rows: one ungated output, whole 16-byte packs.
+static bool post_norm_fits(const LinearArgs &a) {
+  auto al16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+  return a.post_ln_out && !a.glu && a.n_split >= a.N && a.N % 8 == 0 && a.N <= 4096 && a.ld1 % 8 == 0 && al16(a.out1) &&
+         al16(a.post_ln_out) && (!a.bias || al16(a.bias)) && (!a.bias2 || al16(a.bias2)) &&
+         (!a.residual || (a.ldr % 8 == 0 && al16(a.residual))) && (!a.post_ln_w || al16(a.post_ln_w)) &&
+         (!a.post_ln_b || al16(a.post_ln_b)) && a.splitk_ws && ((uintptr_t)a.splitk_ws & 15) == 0;
+}
+// Sums the partial products of a tile GEMM that split K (and normalises the rows when asked to and possible).
+static int launch_splitk_epilogue(hipStream_t st, const LinearArgs &a, int splits, const float *partial) {
+  if (post_norm_fits(a)) {
+    const int items = (a.N / 8 + 63) / 64;
+    const dim3 grid((a.M + 1) / 2), block(128);
+    if (items <= 2) hipLaunchKernelGGL(k_splitk_epilogue_ln<2>, grid, block, 0, st, a, splits, partial);
+    else if (items <= 5) hipLaunchKernelGGL(k_splitk_epilogue_ln<5>, grid, block, 0, st, a, splits, partial);
+    else hipLaunchKernelGGL(k_splitk_epilogue_ln<8>, grid, block, 0, st, a, splits, partial);
+    return launch_check("splitk_epilogue_ln");
+  }
+  const int64_t total = (int64_t)a.M * a.N;
+  const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+  hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, partial);
+  return launch_check("splitk_epilogue");
+}
+
 template <int BM, int BN, int BK, int SH = 0> static int launch_cfg(hipStream_t st, const LinearArgs &a, int splits) {
   constexpr size_t lds = gemm_lds_bytes<BM, BN, (SH ? BK : BK + 8)>();
   static bool attr_set = false;
@@ -537,12 +667,7 @@ template <int BM, int BN, int BK, int SH = 0> static int launch_cfg(hipStream_t 
   hipLaunchKernelGGL((k_gemm_bf16_mfma<BM, BN, BK, SH>), dim3(grid_x, splits), dim3(256), lds, st, a, splits, k_per_split,
                      partial);
   RAI_TRY(launch_check("gemm_bf16_mfma"));
-  if (splits > 1) {
-    int64_t total = (int64_t)a.M * a.N;
-    int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-    hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);
-    RAI_TRY(launch_check("splitk_epilogue"));
-  }
+  if (splits > 1) RAI_TRY(launch_splitk_epilogue(st, a, splits, (const float *)partial));
   return RAI_OK;
 }
 
@@ -567,12 +692,7 @@ template <int BM, int BN, int NS, int SH> static int launch_cfg_dma(hipStream_t 
   hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH>), dim3(grid_x, splits), dim3(256), lds, st, a, splits,
                      k_per_split, partial);
   RAI_TRY(launch_check("gemm_bf16_mfma_dma"));
-  if (splits > 1) {
-    int64_t total = (int64_t)a.M * a.N;
-    int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-    hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);
-    RAI_TRY(launch_check("splitk_epilogue"));
-  }
+  if (splits > 1) RAI_TRY(launch_splitk_epilogue(st, a, splits, (const float *)partial));
   return RAI_OK;
 }
 
@@ -970,6 +1090,41 @@ bool linear_mfma_fuses_norm(int M, int K, int ln_kind) {
   return K <= (M <= 32 ? 8 * 8 * 32 : 8 * 4 * 32);   // one block's K span: no split over blocks
 }
 
+// Split K when the tile count alone cannot fill the GPU and a workspace was provided.
+static int tile_splits(const LinearArgs &a) {
+  const int tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
+  int splits = 1;
+  if (a.splitk_ws && tiles < kNumCU) {
+    // Cost model in units of one K tile of one block: blocks go round-robin over the CUs, a CU holds up to three,
+    // n co-resident blocks share a CU at a combined rate of 0.5 / 0.85 / 1 (one block alone cannot hide its own
+    // barriers and memory latency), each block pays ~8 units of prologue + epilogue, and every split adds a pass over
+    // the f32 partial sums (~7 units at 512 x 2560).  Measured at 512 x 2560 x 12800: 3, 4, 6, 9, 12 splits give
+    // 6.69, 6.64, 6.28, 6.44, 6.79 ms per 32-layer prefill, the order this model predicts.
+    const int kt = a.K / 32;
+    float best = 0.f;
+    for (int s = 1; s <= 12; ++s) {
+      if (s > 1 && (kt / s < 8 || (size_t)s * a.M * a.N * sizeof(float) > a.splitk_ws_bytes)) break;
+      const float per_block = (float)((kt + s - 1) / s) + 8.f;
+      int left = (tiles * s + kNumCU - 1) / kNumCU;   // blocks on the busiest CU
+      float cost = (s > 1 ? 7.f * s : 0.f) * ((float)a.M * a.N / (512.f * 2560.f));
+      while (left > 0) {
+        const int n = left < 3 ? left : 3;
+        cost += n * per_block / (n == 1 ? 0.5f : n == 2 ? 0.85f : 1.f);
+        left -= n;
+      }
+      if (s == 1 || cost < best) { best = cost; splits = s; }
+    }
+  }
+  return splits;
+}
+
+bool linear_fuses_post_norm(const LinearArgs &a) {
+  // the tile kernels serve more than 64 rows; their split-K pass is the one that can normalise
+  // (RAI_HIP_NO_POST_NORM: run the norm as its own launch, for comparison)
+  if (getenv("RAI_HIP_NO_POST_NORM")) return false;
+  return a.M > 64 && post_norm_fits(a) && tile_splits(a) > 1;
+}
+
 int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
   RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
@@ -998,30 +1153,8 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (mt == 3) return launch_mfma_skinny<3>(st, a);
     return launch_mfma_skinny<4>(st, a);
   }
-  // Split K when the tile count alone cannot fill the GPU and a workspace was provided.
   const int tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
-  int splits = 1;
-  if (a.splitk_ws && tiles < kNumCU) {
-    // Cost model in units of one K tile of one block: blocks go round-robin over the CUs, a CU holds up to three,
-    // n co-resident blocks share a CU at a combined rate of 0.5 / 0.85 / 1 (one block alone cannot hide its own
-    // barriers and memory latency), each block pays ~8 units of prologue + epilogue, and every split adds a pass over
-    // the f32 partial sums (~7 units at 512 x 2560).  Measured at 512 x 2560 x 12800: 3, 4, 6, 9, 12 splits give
-    // 6.69, 6.64, 6.28, 6.44, 6.79 ms per 32-layer prefill, the order this model predicts.
-    const int kt = a.K / 32;
-    float best = 0.f;
-    for (int s = 1; s <= 12; ++s) {
-      if (s > 1 && (kt / s < 8 || (size_t)s * a.M * a.N * sizeof(float) > a.splitk_ws_bytes)) break;
-      const float per_block = (float)((kt + s - 1) / s) + 8.f;
-      int left = (tiles * s + kNumCU - 1) / kNumCU;   // blocks on the busiest CU
-      float cost = (s > 1 ? 7.f * s : 0.f) * ((float)a.M * a.N / (512.f * 2560.f));
-      while (left > 0) {
-        const int n = left < 3 ? left : 3;
-        cost += n * per_block / (n == 1 ? 0.5f : n == 2 ? 0.85f : 1.f);
-        left -= n;
-      }
-      if (s == 1 || cost < best) { best = cost; splits = s; }
-    }
-  }
+  const int splits = tile_splits(a);
   // Tile choice.  The LDS-DMA kernels stream K tiles straight into LDS; the 256x128 tile halves the
   // L2 -> LDS traffic per flop for one operand and is used once there are enough tiles of that size
   // to give every CU two; smaller products keep the 128x128 tile (three blocks per CU).

@@ -127,6 +127,25 @@ def test_graph_replay_equals_eager_steps(hip, monkeypatch):
     dec.close()
 
 
+def test_prefill_norm_fused_into_split_k_pass_changes_no_bit(hip, monkeypatch):
+    """A 96-token prefill goes through the tile GEMM; its dense|fc2 product splits K and the pass over the
+    partial sums also writes the next layer's LayerNorm.  Same logits, bit for bit, as with the norm as its own
+    launch, and both match the oracle."""
+    cfg = small_cfg(num_hidden_layers=3, max_position_embeddings=128)
+    ids = np.random.Generator(np.random.PCG64(5)).integers(0, cfg.vocab_size, (1, 96)).astype(np.uint32)
+    dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=128)
+    fused, tok = dec.forward(ids)
+    monkeypatch.setenv("RAI_HIP_NO_POST_NORM", "1")
+    dec2, _ = make(cfg, "bf16", hip, max_batch=1, max_context=128)
+    plain, tok2 = dec2.forward(ids)
+    monkeypatch.delenv("RAI_HIP_NO_POST_NORM")
+    np.testing.assert_array_equal(np.asarray(fused), np.asarray(plain))
+    np.testing.assert_array_equal(tok, tok2)
+    want = ref.fwd(ids)
+    assert_close(fused, want, "bf16", "prefill logits, fused norm")
+    check_tokens(tok, want, "bf16")
+
+
 def test_gqa_and_tied_head(hip):
     # num_key_value_heads < heads (repeat_kv phi2.rs:190-200) and tie_word_embeddings
     cfg = small_cfg(num_key_value_heads=2, tie_word_embeddings=True)
