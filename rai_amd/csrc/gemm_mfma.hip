@@ -55,11 +55,22 @@ template <int BM, int BN, int PITCH> constexpr int gemm_lds_bytes() {
 
 // Applies activation `act` to the elements of x[8] whose column n + e is >= from.  The switch on the
 // (block-uniform) activation sits outside the element loop, so only one activation's code runs.
+// The results are rounded to bf16 (relative step 2^-8), so tanh-GELU and SiLU are evaluated through the hardware
+// exponential and reciprocal (relative error ~1e-6) instead of the library tanhf / expf and a division:
+// 0.5 x (1 + tanh u) = x / (1 + exp(-2u)).  The f32 Linear keeps the library functions (act_eval).
+__device__ __forceinline__ float act_eval_bf16_out(int act, float x) {
+  if (act == RAI_UN_NEW_GELU) {
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.0f * 1.4426950408889634f * u));
+  }
+  if (act == RAI_UN_SILU) return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+  return act_eval(act, x);
+}
 __device__ __forceinline__ void act8(int act, float (&x)[8], int n, int from) {
 #define RAI_ACT_CASE(K)                                     \
   case K:                                                   \
     _Pragma("unroll") for (int e = 0; e < 8; ++e)           \
-      if (n + e >= from) x[e] = act_eval(K, x[e]);          \
+      if (n + e >= from) x[e] = act_eval_bf16_out(K, x[e]); \
     break;
   switch (act) {
     RAI_ACT_CASE(RAI_UN_GELU)
