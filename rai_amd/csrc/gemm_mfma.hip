@@ -1132,7 +1132,8 @@ static int tile_splits(const LinearArgs &a) {
 bool linear_fuses_post_norm(const LinearArgs &a) {
   // the tile kernels serve more than 64 rows; their split-K pass is the one that can normalise
   // (RAI_HIP_NO_POST_NORM: run the norm as its own launch, for comparison)
-  if (getenv("RAI_HIP_NO_POST_NORM")) return false;
+  const char *off = getenv("RAI_HIP_NO_POST_NORM");   // read per call: the test switches it within one process
+  if (off && *off) return false;
   return a.M > 64 && post_norm_fits(a) && tile_splits(a) > 1;
 }
 
