@@ -146,6 +146,33 @@ def test_prefill_norm_fused_into_split_k_pass_changes_no_bit(hip, monkeypatch):
     check_tokens(tok, want, "bf16")
 
 
+@pytest.mark.parametrize("hidden,heads,inter", [(2560, 32, 10240), (4096, 32, 4096)])
+def test_prefill_norm_fused_at_wide_rows(hip, monkeypatch, hidden, heads, inter):
+    """The fused summation + LayerNorm pass at 5 and 8 column groups per lane (rows of 2560 and 4096): bit-identical
+    logits to the path with the stand-alone norm."""
+    cfg = small_cfg(hidden_size=hidden, num_attention_heads=heads, intermediate_size=inter, num_hidden_layers=2,
+                    max_position_embeddings=128, vocab_size=512, partial_rotary_factor=0.25)   # an even rotary_dim
+    ids = np.random.Generator(np.random.PCG64(6)).integers(0, cfg.vocab_size, (1, 80)).astype(np.uint32)
+
+    def with_random_vectors(dec):
+        # biases and norm parameters away from the 0 / 1 of random_params, so that a dropped one would show
+        rng = np.random.Generator(np.random.PCG64(7))
+        for name, size in sorted(dec.param_names().items()):
+            if name.endswith(".bias") or name.endswith("layernorm.weight"):
+                dec.load_param(name, to_storage((0.5 + rng.random(size, dtype=np.float32)) * np.float32(0.1), "bf16"))
+        return dec
+
+    dec = with_random_vectors(make(cfg, "bf16", hip, max_batch=1, max_context=128)[0])
+    fused, tok = dec.forward(ids)
+    del dec
+    monkeypatch.setenv("RAI_HIP_NO_POST_NORM", "1")
+    dec2 = with_random_vectors(make(cfg, "bf16", hip, max_batch=1, max_context=128)[0])
+    plain, tok2 = dec2.forward(ids)
+    np.testing.assert_array_equal(np.asarray(fused), np.asarray(plain))
+    np.testing.assert_array_equal(tok, tok2)
+    assert np.isfinite(np.asarray(fused, dtype=np.float32)).all()
+
+
 def test_gqa_and_tied_head(hip):
     # num_key_value_heads < heads (repeat_kv phi2.rs:190-200) and tie_word_embeddings
     cfg = small_cfg(num_key_value_heads=2, tie_word_embeddings=True)
