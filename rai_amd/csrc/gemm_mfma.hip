@@ -48,8 +48,8 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
 }
 
 // LDS a tile kernel needs: two stages of A and B tiles, or the epilogue staging area if that is larger.
-template <int BM, int BN, int PITCH> constexpr int gemm_lds_bytes() {
-  constexpr int tiles = 2 * (BM + BN) * PITCH * 2, staging = 4 * 32 * (BN / 2 + 4) * 4;
+template <int BM, int BN, int PITCH, int WGN = 2> constexpr int gemm_lds_bytes() {
+  constexpr int tiles = 2 * (BM + BN) * PITCH * 2, staging = 2 * WGN * 32 * (BN / WGN + 4) * 4;
   return tiles > staging ? tiles : staging;
 }
 
@@ -90,16 +90,18 @@ __device__ __forceinline__ void unpack8(const u32x4 &p, float (&f)[8]) {
 // Tile epilogue shared by the tile kernels: every wave stages 32 x WN accumulators at a time in
 // LDS (the tile buffers are free by then) and writes 16-byte rows with bias / activation /
 // residual applied, or raw f32 partial sums when K is split over several blocks.
-template <int BM, int BN, int LDS_BYTES>
-__device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (&acc)[BM / 64][BN / 64], uint16_t *lds,
-                                                   int m0, int n0, int wave, int lane, int split, float *partial) {
-  constexpr int WM = BM / 2, WN = BN / 2;
+// (WGN = waves along N: the block is a 2 x WGN grid of waves.)
+template <int BM, int BN, int LDS_BYTES, int WGN = 2>
+__device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (&acc)[BM / 64][BN / (32 * WGN)],
+                                                   uint16_t *lds, int m0, int n0, int wave, int lane, int split,
+                                                   float *partial) {
+  constexpr int WM = BM / 2, WN = BN / WGN;
   constexpr int MT = WM / 32, NT = WN / 32;
   constexpr int EP = WN + 4;                // epilogue staging pitch (floats)
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   // ---- epilogue: stage 32 x WN accumulators per wave in LDS, write 8 columns per lane
   float *stage = reinterpret_cast<float *>(lds) + wave * 32 * EP;
-  static_assert(4 * 32 * EP * 4 <= LDS_BYTES, "epilogue staging does not fit the tile buffers");
+  static_assert(2 * WGN * 32 * EP * 4 <= LDS_BYTES, "epilogue staging does not fit the tile buffers");
   constexpr int CG = WN / 8;                 // 8-column groups per staged row
   constexpr int ITEMS = 32 * CG / 64;        // per lane
   const uint16_t *bias = (const uint16_t *)a.bias;
@@ -350,17 +352,19 @@ __global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits
 //     bare s_barrier make tile t+1 visible to the block (and retire stage t-1 for refilling) with one
 //     barrier per K tile.  The barrier carries no fence: a fence would wait for every outstanding
 //     LDS load, i.e. drain the pipeline.
-template <int BM, int BN, int NS, int SH>
-__global__ void __launch_bounds__(256) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
+template <int BM, int BN, int NS, int SH, int WGN = 2>
+__global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
+  // block = 2 x WGN waves.  WGN = 4 (eight waves, wave tile (BM/2) x (BN/4)) keeps two waves on every SIMD: one
+  // multiplies while the other sits in its wait for the next tile, and twice as many waves issue loads.
   constexpr int BK = 32, PITCH = BK;
-  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int WM = BM / 2, WN = BN / WGN;
   constexpr int MT = WM / 32, NT = WN / 32;
-  constexpr int LA = BM / 64, LB = BN / 64;          // loads per wave per K tile (16 rows each)
+  constexpr int LA = BM / (32 * WGN), LB = BN / (32 * WGN);   // loads per wave per K tile (16 rows each)
   constexpr int STAGE = (BM + BN) * BK;              // elements per stage: A rows then B rows
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
   const int tile = xcd_remap(blockIdx.x, total);
@@ -497,7 +501,8 @@ __global__ void __launch_bounds__(256) k_gemm_bf16_mfma_dma(LinearArgs a, int sp
   // the refetches issued past the end must land before the stages are reused for the epilogue
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  gemm_tile_epilogue<BM, BN, gemm_lds_bytes<BM, BN, PITCH * NS / 2>()>(a, acc, lds, m0, n0, wave, lane, split, partial);
+  gemm_tile_epilogue<BM, BN, gemm_lds_bytes<BM, BN, PITCH * NS / 2, WGN>(), WGN>(a, acc, lds, m0, n0, wave, lane, split,
+                                                                                 partial);
 }
 
 // Sums the per-split partial products and applies the Linear epilogue.
@@ -682,11 +687,12 @@ template <int BM, int BN, int BK, int SH = 0> static int launch_cfg(hipStream_t 
   return RAI_OK;
 }
 
-template <int BM, int BN, int NS, int SH> static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
-  constexpr size_t lds = gemm_lds_bytes<BM, BN, 32 * NS / 2>();
+template <int BM, int BN, int NS, int SH, int WGN = 2>
+static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
+  constexpr size_t lds = gemm_lds_bytes<BM, BN, 32 * NS / 2, WGN>();
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma<BM, BN, NS, SH>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
@@ -700,7 +706,7 @@ template <int BM, int BN, int NS, int SH> static int launch_cfg_dma(hipStream_t 
     k_per_split = per * 32;
     partial = (float *)a.splitk_ws;
   }
-  hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH>), dim3(grid_x, splits), dim3(256), lds, st, a, splits,
+  hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN>), dim3(grid_x, splits), dim3(128 * WGN), lds, st, a, splits,
                      k_per_split, partial);
   RAI_TRY(launch_check("gemm_bf16_mfma_dma"));
   if (splits > 1) RAI_TRY(launch_splitk_epilogue(st, a, splits, (const float *)partial));
@@ -1177,12 +1183,15 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (!strcmp(knob, "256x128")) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
     if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
+    if (!strcmp(knob, "256x256x8w")) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   }
   const int big_tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
   const int huge_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-  // 256x256 (one block per CU, 4 LDS stages) once the tile count covers three rounds over the CUs and K is
-  // long enough to amortise its prologue and epilogue: 950-1040 TFLOP/s on 8k-class products against 830-900
-  if (splits == 1 && huge_tiles >= 3 * kNumCU && a.K >= 2048) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
+  // 256x256 in its eight-wave form (one block per CU, 4 LDS stages, two waves per SIMD) once there are 1.5 tiles per
+  // CU: the tile with the most flops per byte drawn from L2, which is what bounds these kernels.  Measured against
+  // the previous choices: 16384 x 8960 x 1536 845 against 736 TFLOP/s, 16384 x 2048 x 1536 983 against 834,
+  // 4096 x 10240 x 2560 896 against 789, 8192^3 1024 either way; the four-wave 256x256 form is 3-9 % behind it.
+  if (splits == 1 && 2 * huge_tiles >= 3 * kNumCU) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
   return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
 }
