@@ -1187,11 +1187,13 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   }
   const int big_tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
   const int huge_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-  // 256x256 in its eight-wave form (one block per CU, 4 LDS stages, two waves per SIMD) once there are 1.5 tiles per
-  // CU: the tile with the most flops per byte drawn from L2, which is what bounds these kernels.  Measured against
-  // the previous choices: 16384 x 8960 x 1536 845 against 736 TFLOP/s, 16384 x 2048 x 1536 983 against 834,
-  // 4096 x 10240 x 2560 896 against 789, 8192^3 1024 either way; the four-wave 256x256 form is 3-9 % behind it.
-  if (splits == 1 && 2 * huge_tiles >= 3 * kNumCU) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
+  // 256x256 in its eight-wave form (one block per CU, 4 LDS stages, two waves per SIMD) once its tiles cover a good
+  // half of the CUs: the tile with the most flops per byte drawn from L2, which is what bounds these kernels.
+  // Measured against the smaller tiles: 16384 x 8960 x 1536 845 against 736 TFLOP/s, 16384 x 2048 x 1536 983 against
+  // 834, 4096 x 10240 x 2560 896 against 789, 4096 x 2560 x 10240 (160 tiles) 837 against 650, 512 x 17920 x 2560
+  // (140 tiles) 689 against 621; with 128 tiles or fewer the smaller tiles win (4096 x 2048 x 2048: 618 against 760).
+  // The four-wave 256x256 form is 3-9 % behind the eight-wave one everywhere.
+  if (splits == 1 && 32 * huge_tiles >= 17 * kNumCU) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
   return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
 }
