@@ -1176,7 +1176,7 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   // Tile choice.  The LDS-DMA kernels stream K tiles straight into LDS; the 256x128 tile halves the
   // L2 -> LDS traffic per flop for one operand and is used once there are enough tiles of that size
   // to give every CU two; smaller products keep the 128x128 tile (three blocks per CU).
-  // RAI_HIP_GEMM_TILE = "128x128" | "256x128" | "256x256" | "classic" overrides (tuning aid).
+  // RAI_HIP_GEMM_TILE = "128x128" | "256x128" | "256x256" | "256x256x8w" | "classic" overrides (tuning aid).
   const char *knob = getenv("RAI_HIP_GEMM_TILE");
   if (knob) {
     if (!strcmp(knob, "128x128")) return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
