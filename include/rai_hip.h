@@ -201,8 +201,14 @@ int rai_hip_reduce(int dev, int op, const rai_hip_tensor *in, const int32_t *dim
 int rai_hip_softmax(int dev, const rai_hip_tensor *in, int32_t dim, const rai_hip_tensor *out);
 int rai_hip_log_softmax(int dev, const rai_hip_tensor *in, int32_t dim, const rai_hip_tensor *out);
 
-/* ArgMax/ArgMin along `dim`: candle.rs:917-944, ops/argmax.rs:48-61.  Output U32,
- * first index wins ties; NaN never wins.  `out` has `dim` removed or kept as 1. */
+/* ArgMax/ArgMin along `dim`: candle.rs:917-944, ops/argmax.rs:48-61.  Output U32.
+ * The result is that of a sequential scan from element 0 which replaces its running
+ * best only on a strict comparison (`>` for argmax, `<` for argmin): the first index
+ * wins ties, -0.0 and +0.0 tie, and because every comparison with NaN is false a NaN
+ * is never taken over a number while a NaN at element 0 is never replaced (NaN wins
+ * from index 0 only; an all-NaN axis yields 0).  That NaN rule restates how candle's
+ * CPU loop is believed to behave; nothing in the reference's tests pins it.
+ * `out` has `dim` removed or kept as 1. */
 int rai_hip_argmax(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
                    const rai_hip_tensor *out);
 int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
@@ -252,6 +258,21 @@ int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, co
  * K-contiguous. */
 int rai_hip_linear(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, const rai_hip_tensor *bias,
                    int32_t act, const rai_hip_tensor *residual, const rai_hip_tensor *out);
+
+/* Several Linear layers that read the same input, evaluated as ONE contraction over
+ * their concatenated weight rows -- the form the decoders use for q|k|v|fc1
+ * (rai-models/src/llm/phi2.rs:99-101,202-206), for dense|fc2 with the two biases
+ * (phi2.rs:293-299) and for the gated MLP act(gate(x)) * up(x) (qwen2.rs:100-104).
+ * bf16 only.  x [M,K], w [N,K] (K-contiguous rows), bias / bias2 nullable [N] (both
+ * added in f32), act (or -1) applied to columns n >= act_from, residual nullable [M,N].
+ *   glu == 0: columns [0, n1) go to out1 [M,n1], columns [n1, N) to out2 [M,N-n1]
+ *             (n1 = out1's width; n1 == N: out2 null; a residual needs n1 == N).
+ *   glu != 0: w's rows are interleaved gate_0, up_0, gate_1, ...; out1 [M,N/2] gets
+ *             act(gate) * up with the reference's roundings of gate, act(gate), up.
+ * k_splits: 0 = automatic; > 0 asks the tile kernel (M > 64) for that many K splits. */
+int rai_hip_linear_packed(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, const rai_hip_tensor *bias,
+                          const rai_hip_tensor *bias2, int32_t act, int32_t act_from, const rai_hip_tensor *residual,
+                          int32_t glu, int32_t k_splits, const rai_hip_tensor *out1, const rai_hip_tensor *out2);
 
 /* LayerNorm::fwd rai-nn/src/layer_norm.rs:32-42 over the last dim (population
  * variance, eps inside the square root); w, b nullable together. */

@@ -108,6 +108,7 @@ PROTOTYPES = {
     "rai_hip_index_errors": [C.c_int, C.POINTER(C.c_uint64)],
     "rai_hip_matmul": [C.c_int, _TP, _TP, _TP],
     "rai_hip_linear": [C.c_int, _TP, _TP, _TP, _i32, _TP, _TP],
+    "rai_hip_linear_packed": [C.c_int, _TP, _TP, _TP, _TP, _i32, _i32, _TP, _i32, _i32, _TP, _TP],
     "rai_hip_layer_norm": [C.c_int, _TP, _TP, _TP, _dbl, _TP],
     "rai_hip_rms_norm": [C.c_int, _TP, _TP, _dbl, _i32, _TP],
     "rai_hip_rope": [C.c_int, _TP, _TP, _TP, _i32, _i64, _TP],

@@ -42,6 +42,9 @@ struct LinearArgs {
   // yields too few tiles to fill the GPU (tile kernel only).
   void *splitk_ws;
   size_t splitk_ws_bytes;
+  // > 0: the tile kernel cuts K into this many splits (when the workspace holds them) instead of asking its cost
+  // model; 0: automatic.
+  int force_splits;
   // Optional second copy of W in MFMA-fragment order for the small-M streaming kernel (9 <= M <= 64): the
   // 16 rows x 32 columns that one wave loads with one instruction are 1 KB of consecutive memory
   // ([N / 16 row tiles][K / 32 steps][64 lanes][8 elements], see linear_fragment_layout); null: read W itself.

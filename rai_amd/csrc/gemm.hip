@@ -856,4 +856,83 @@ int rai_hip_linear(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, co
   return x->dtype == RAI_BF16 ? launch_linear_bf16(st, la) : launch_linear_f32(st, la);
 }
 
+int rai_hip_linear_packed(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, const rai_hip_tensor *bias,
+                          const rai_hip_tensor *bias2, int32_t act, int32_t act_from, const rai_hip_tensor *residual,
+                          int32_t glu, int32_t k_splits, const rai_hip_tensor *out1, const rai_hip_tensor *out2) {
+  RAI_TRY(validate(x, "x"));
+  RAI_TRY(validate(w, "w"));
+  RAI_TRY(validate(out1, "out1"));
+  RAI_REQUIRE(x->dtype == RAI_BF16, RAI_ERR_BAD_DTYPE, "linear_packed: bf16 required");
+  RAI_REQUIRE(w->dtype == x->dtype && out1->dtype == x->dtype, RAI_ERR_BAD_DTYPE, "linear_packed: dtype mismatch");
+  RAI_REQUIRE(w->rank == 2 && x->rank == 2 && out1->rank == 2, RAI_ERR_BAD_SHAPE, "linear_packed: x, w, out1 must be rank 2");
+  const int64_t M = x->shape[0], N = w->shape[0], K = w->shape[1];
+  RAI_REQUIRE(x->shape[1] == K && out1->shape[0] == M, RAI_ERR_BAD_SHAPE, "linear_packed: x[%lld,%lld] w[%lld,%lld] out1[%lld,..]",
+              (long long)M, (long long)x->shape[1], (long long)N, (long long)K, (long long)out1->shape[0]);
+  RAI_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1LL << 31) && N < (1LL << 31), RAI_ERR_BAD_SHAPE, "linear_packed: bad problem size");
+  RAI_REQUIRE(x->stride[1] == 1 && w->stride[1] == 1 && is_contiguous(out1), RAI_ERR_BAD_STRIDE,
+              "linear_packed: x and w must be K-contiguous, outputs contiguous");
+  RAI_REQUIRE(act == -1 || act == RAI_UN_GELU || act == RAI_UN_NEW_GELU || act == RAI_UN_SILU || act == RAI_UN_RELU ||
+                  act == RAI_UN_TANH,
+              RAI_ERR_BAD_ARG, "linear_packed: unsupported activation %d", act);
+  RAI_REQUIRE(act_from >= 0 && act_from <= N && k_splits >= 0, RAI_ERR_BAD_ARG, "linear_packed: bad act_from / k_splits");
+  const int64_t n1 = out1->shape[1];
+  LinearArgs la = linear_args_default();
+  if (glu) {
+    RAI_REQUIRE(N % 2 == 0 && n1 == N / 2 && !out2 && !residual && !bias2 && act >= 0 && act_from == 0, RAI_ERR_BAD_ARG,
+                "linear_packed: a gated product writes N/2 columns to out1 and takes an activation, no residual, "
+                "no second bias and no second output");
+    la.n_split = (int)N;
+  } else {
+    RAI_REQUIRE(n1 >= 1 && n1 <= N, RAI_ERR_BAD_SHAPE, "linear_packed: out1 has %lld of %lld columns", (long long)n1, (long long)N);
+    la.n_split = (int)n1;
+    if (n1 < N) {
+      RAI_REQUIRE(out2, RAI_ERR_BAD_ARG, "linear_packed: out2 missing for columns [%lld, %lld)", (long long)n1, (long long)N);
+      RAI_TRY(validate(out2, "out2"));
+      RAI_REQUIRE(out2->dtype == x->dtype && out2->rank == 2 && out2->shape[0] == M && out2->shape[1] == N - n1 &&
+                      is_contiguous(out2),
+                  RAI_ERR_BAD_SHAPE, "linear_packed: out2 must be a contiguous [%lld,%lld]", (long long)M, (long long)(N - n1));
+      RAI_REQUIRE(!residual, RAI_ERR_BAD_ARG, "linear_packed: a residual needs a single output");
+      la.out2 = base_ptr(out2);
+      la.ld2 = N - n1;
+    } else {
+      RAI_REQUIRE(!out2, RAI_ERR_BAD_ARG, "linear_packed: out1 takes every column, out2 must be null");
+    }
+  }
+  la.A = base_ptr(x);
+  la.lda = M == 1 ? K : x->stride[0];
+  la.W = base_ptr(w);
+  la.ldw = N == 1 ? K : w->stride[0];
+  const rai_hip_tensor *bs[2] = {bias, bias2};
+  for (int i = 0; i < 2; ++i) {
+    if (!bs[i]) continue;
+    RAI_TRY(validate(bs[i], "bias"));
+    RAI_REQUIRE(bs[i]->dtype == x->dtype && bs[i]->rank == 1 && bs[i]->shape[0] == N && (bs[i]->stride[0] == 1 || N == 1),
+                RAI_ERR_BAD_SHAPE, "linear_packed: a bias must be a contiguous [%lld] vector of x's dtype", (long long)N);
+    (i ? la.bias2 : la.bias) = base_ptr(bs[i]);
+  }
+  if (residual) {
+    RAI_TRY(validate(residual, "residual"));
+    RAI_REQUIRE(residual->dtype == x->dtype && same_shape(residual, out1) && is_contiguous(residual), RAI_ERR_BAD_SHAPE,
+                "linear_packed: residual must be contiguous with the output's shape");
+    la.residual = base_ptr(residual);
+    la.ldr = N;
+  }
+  la.out1 = base_ptr(out1);
+  la.ld1 = n1;
+  la.M = (int)M;
+  la.N = (int)N;
+  la.K = (int)K;
+  la.act = act;
+  la.act_from = act_from;
+  la.glu = glu ? 1 : 0;
+  la.force_splits = k_splits;
+  hipStream_t st = stream_of(dev);
+  if (!st) return RAI_ERR_HIP;
+  if (la.M > 8) {
+    RAI_REQUIRE(K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear_packed: M > 8 needs K %% 32 == 0 (K=%lld)", (long long)K);
+    RAI_TRY(splitk_workspace(dev, &la));
+  }
+  return launch_linear_bf16(st, la);
+}
+
 }  // extern "C"

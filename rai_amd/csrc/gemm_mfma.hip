@@ -1111,6 +1111,12 @@ bool linear_mfma_fuses_norm(int M, int K, int ln_kind) {
 static int tile_splits(const LinearArgs &a) {
   const int tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
   int splits = 1;
+  if (a.force_splits > 0) {
+    const int kt = a.K / 32;
+    int s = a.force_splits < kt ? a.force_splits : kt;
+    while (s > 1 && (!a.splitk_ws || (size_t)s * a.M * a.N * sizeof(float) > a.splitk_ws_bytes)) --s;
+    return s < 1 ? 1 : s;
+  }
   if (a.splitk_ws && tiles < kNumCU) {
     // Cost model in units of one K tile of one block: blocks go round-robin over the CUs, a CU holds up to three,
     // n co-resident blocks share a CU at a combined rate of 0.5 / 0.85 / 1 (one block alone cannot hide its own

@@ -140,8 +140,18 @@ struct RopeArgs {
   int64_t tab_row_stride;
 };
 
+// A value rounded to storage type T and widened again: the rounding every node of the reference's rotary chain
+// (x * cos, rotate_half(x) * sin, their sum: rai-models/src/llm/phi2.rs:66-77) applies to its result.
+template <typename T> __device__ __forceinline__ float rope_round(float v) {
+  T tmp;
+  Scalar<T>::store(&tmp, (typename Scalar<T>::compute)v);
+  return (float)Scalar<T>::load(&tmp);
+}
+
 template <typename T, typename TT>
 __global__ void __launch_bounds__(256) k_rope(T *out, const T *x, const TT *cos_t, const TT *sin_t, RopeArgs a) {
+#pragma clang fp contract(off)   // two products and a sum, each rounded on its own: no fused multiply-add
+
   const int64_t total = a.B * a.H * a.S * a.D;
   for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
     int64_t d = e % a.D;
@@ -159,7 +169,7 @@ __global__ void __launch_bounds__(256) k_rope(T *out, const T *x, const TT *cos_
       // rotate_half = cat(-x2, x1)
       float other = d < a.half ? -(float)Scalar<T>::load(xp + (d + a.half) * a.xs[3])
                                : (float)Scalar<T>::load(xp + (d - a.half) * a.xs[3]);
-      v = v * c + other * sn;
+      v = rope_round<T>(v * c) + rope_round<T>(other * sn);
     }
     Scalar<T>::store(out + e, v);
   }
@@ -171,6 +181,7 @@ __global__ void __launch_bounds__(256) k_rope(T *out, const T *x, const TT *cos_
 // divisions).
 template <typename T, typename TT>
 __global__ void __launch_bounds__(256) k_rope_vec(T *out, const T *x, const TT *cos_t, const TT *sin_t, RopeArgs a) {
+#pragma clang fp contract(off)
   constexpr int VEC = 16 / sizeof(T);
   struct alignas(16) Pack { T v[VEC]; };
   const uint32_t cpr = (uint32_t)(a.D / VEC), S = (uint32_t)a.S, H = (uint32_t)a.H;
@@ -188,7 +199,8 @@ __global__ void __launch_bounds__(256) k_rope_vec(T *out, const T *x, const TT *
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         const float c = (float)Scalar<TT>::load(cos_t + trow + j), sn = (float)Scalar<TT>::load(sin_t + trow + j);
-        const float r = (float)Scalar<T>::load(&v.v[j]) * c + sign * (float)Scalar<T>::load(&o.v[j]) * sn;
+        const float r = rope_round<T>((float)Scalar<T>::load(&v.v[j]) * c) +
+                        rope_round<T>(sign * (float)Scalar<T>::load(&o.v[j]) * sn);
         Scalar<T>::store(&v.v[j], (typename Scalar<T>::compute)r);
       }
     }

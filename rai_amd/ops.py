@@ -210,6 +210,18 @@ def linear(x, w, bias=None, act=None, residual=None):
     return out
 
 
+def linear_packed(x, w, bias=None, bias2=None, act=None, act_from=0, residual=None, glu=False, n1=None, k_splits=0):
+    """rai_hip_linear_packed: several Linears over one input as one contraction.  Returns out1, or
+    (out1, out2) when n1 < N splits the columns over two outputs."""
+    m, n = x.shape[0], w.shape[0]
+    n1 = n // 2 if glu else (n if n1 is None else n1)
+    out1 = HipTensor.empty((m, n1), x.dtype, x.dev)
+    out2 = None if glu or n1 == n else HipTensor.empty((m, n - n1), x.dtype, x.dev)
+    call("rai_hip_linear_packed", x.dev, _d(x), _d(w), _d(bias), _d(bias2), -1 if act is None else UNARY[act],
+         int(act_from), _d(residual), int(glu), int(k_splits), _d(out1), _d(out2))
+    return out1 if out2 is None else (out1, out2)
+
+
 def layer_norm(x, w, b, eps):
     out = HipTensor.empty(x.shape, x.dtype, x.dev)
     call("rai_hip_layer_norm", x.dev, _d(x), _d(w), _d(b), float(eps), _d(out))

@@ -1,0 +1,97 @@
+"""Qwen2-1.5B and Gemma-2B at their full widths (two layers of each, so that the CPU oracle stays affordable):
+
+* Qwen2-1.5B architecture, bf16: batched prefill of 16 x 1024 tokens with the causal mask: hidden 1536,
+  12 query / 2 KV heads of 128, SwiGLU 8960, RMSNorm eps 1e-6, RoPE theta 1e6, vocabulary 151936.
+* Gemma-2B architecture, bf16: decode at batch 32 on a 2048-token context per sequence: hidden 2048, 8 query /
+  1 KV head of 256, GeGLU 16384, RMSNorm with (1 + w), embedding scaled by sqrt(2048), tied 256000-way head.
+
+The device runs the whole batch; sequences are independent of each other through every operator, so the oracle
+(rai-models/src/llm/qwen2.rs, gemma.rs restated) is run on a few of the sequences and compared row by row.
+"""
+import numpy as np
+import pytest
+
+from oracle import qwen2
+from oracle.dtypes import rnd, to_storage
+from tests.test_gpu_phi2 import check_tokens
+from tests.util import assert_close, assert_logits_close, progress, synthetic_params
+
+pytestmark = pytest.mark.gpu
+
+
+def build(cfg, max_batch, max_context, request):
+    from rai_amd.models import Decoder
+    dt = "bf16"
+    progress(request, "generating seeded weights")
+    params = synthetic_params(qwen2.param_shapes(cfg), dt, seed=0, norm_weight=0.0 if cfg.arch == "gemma" else 1.0)
+    g = np.random.Generator(np.random.PCG64(77))
+    for k in params:   # biases and norm weights away from their trivial values
+        if k.endswith(".bias"):
+            params[k] = rnd(0.02 * g.standard_normal(params[k].shape).astype(np.float32), dt)
+        elif k.endswith("norm.weight"):
+            params[k] = rnd(params[k] + 0.1 * g.standard_normal(params[k].shape).astype(np.float32), dt)
+    dec = Decoder(cfg.arch, dt, vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
+                  intermediate_size=cfg.intermediate_size, num_hidden_layers=cfg.num_hidden_layers,
+                  num_attention_heads=cfg.num_attention_heads, num_key_value_heads=cfg.num_key_value_heads,
+                  head_dim=cfg.head_dim, rotary_dim=cfg.head_dim, max_position_embeddings=cfg.max_position_embeddings,
+                  hidden_act=cfg.hidden_act, tie_word_embeddings=cfg.arch == "gemma", rope_theta=cfg.rope_theta,
+                  norm_eps=cfg.rms_norm_eps, max_batch=max_batch, max_context=max_context)
+    names = dec.param_names()
+    assert set(names) == set(params)
+    for n in names:
+        dec.load_param(n, to_storage(params[n], dt))
+    return dec, params
+
+
+def test_qwen2_1p5b_widths_prefill_16x1024(hip, request):
+    cfg = qwen2.Config("qwen2", 151936, 1536, 8960, 2, 12, 2, "silu", max_position_embeddings=2048, rope_theta=1e6,
+                       head_dim=128)
+    dec, params = build(cfg, 16, 1024 + 8, request)
+    ids = np.random.Generator(np.random.PCG64(31)).integers(0, cfg.vocab_size, (16, 1024)).astype(np.uint32)
+    logits, tok = dec.forward(ids)                 # 16384 rows: eight-wave 256x256 tiles, GQA flash attention
+    assert logits.shape == (16, cfg.vocab_size)
+    rows = [0, 6, 15]
+    progress(request, f"oracle prefill of sequences {rows}")
+    ref = qwen2.Model(cfg, params, "bf16")
+    # the same stored weights and the same (bf16) rotary tables, f32 arithmetic without intermediate rounding: at
+    # this width and length the bf16 node-by-node chain is ~2 % (of the largest logit) away from it by itself
+    exact = qwen2.Model(cfg, params, "f32")
+    exact.sin, exact.cos = ref.sin, ref.cos
+    want = ref.fwd(ids[rows])
+    errs = assert_logits_close(logits[rows], want, exact.fwd(ids[rows]), "bf16", "Qwen2-1.5B widths, prefill 16 x 1024")
+    progress(request, "relative errors: device vs unrounded %.4f, chain vs unrounded %.4f, device vs chain %.4f" % errs)
+    check_tokens(tok[rows], want, "bf16")
+    # one decode step on top of the 1024-token cache for all 16 sequences
+    nxt = tok.copy().reshape(16, 1)
+    nxt[rows, 0] = np.argmax(want, -1).astype(np.uint32)
+    logits, tok = dec.forward(nxt)
+    want = ref.fwd(nxt[rows])
+    assert_logits_close(logits[rows], want, exact.fwd(nxt[rows]), "bf16", "decode step at context 1024")
+    check_tokens(tok[rows], want, "bf16")
+    dec.close()
+
+
+def test_gemma_2b_widths_decode_batch32_context2048(hip, request):
+    cfg = qwen2.Config("gemma", 256000, 2048, 16384, 2, 8, 1, "gelu", max_position_embeddings=4096, head_dim=256)
+    B, CTX = 32, 2048
+    dec, params = build(cfg, B, CTX + 8, request)
+    ids = np.random.Generator(np.random.PCG64(32)).integers(0, cfg.vocab_size, (B, CTX)).astype(np.uint32)
+    progress(request, "device prefill 32 x 2048")
+    logits, tok = dec.forward(ids)
+    rows = [0, 13, 31]
+    progress(request, f"oracle prefill of sequences {rows}")
+    ref = qwen2.Model(cfg, params, "bf16")
+    want = ref.fwd(ids[rows])
+    assert_close(logits[rows], want, "bf16", "Gemma-2B widths, prefill 32 x 2048: logits")
+    check_tokens(tok[rows], want, "bf16")
+    for step in range(4):                          # batch-32 decode: weight-streaming MFMA Linears, MQA decode attention,
+        nxt = tok.copy().reshape(B, 1)             # 256000-row tied head, device argmax
+        nxt[rows, 0] = np.argmax(want, -1).astype(np.uint32)
+        logits, tok = dec.forward(nxt)
+        want = ref.fwd(nxt[rows])
+        assert_close(logits[rows], want, "bf16", f"decode step {step} at context {CTX + step}")
+        check_tokens(tok[rows], want, "bf16")
+        # every row's token is the argmax of that row's own logits (first maximum), bit-exactly
+        assert np.array_equal(tok, np.argmax(logits, -1).astype(np.uint32))
+    assert dec.context_len() == CTX + 4
+    dec.close()

@@ -40,3 +40,83 @@ def assert_close(got, want, dt, what="", scale=None):
     err = np.abs(got[fin] - want[fin])
     bad = err > tol
     assert not bad.any(), f"{what}: max err {err.max():.3e} > tol {tol:.3e} ({bad.sum()} of {err.size} elements)"
+
+
+# Per-element bound for elementwise work (unary, binary, cast, activations, RoPE): relative to each element's own
+# magnitude, with an absolute floor far below the values in play, so that an error on a small element cannot hide
+# behind the largest one of the tensor.
+ELEM_RTOL = {"f32": 1e-4, "f64": 1e-9, "bf16": 2e-2, "f16": 4e-3}
+
+
+def assert_close_elem(got, want, dt, what="", atol=None):
+    """|got - want| <= rtol * |want| + atol for every element (atol defaults to rtol * 1e-3 * max|want|)."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, f"{what}: shape {got.shape} vs {want.shape}"
+    if want.size == 0:
+        return
+    fin = np.isfinite(want)
+    assert np.array_equal(np.isfinite(got), fin), f"{what}: non-finite pattern differs"
+    assert np.array_equal(np.isnan(got), np.isnan(want)), f"{what}: NaN pattern differs"
+    assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)]), f"{what}: infinities differ"
+    if not fin.any():
+        return
+    rtol = ELEM_RTOL[dt]
+    if atol is None:
+        atol = rtol * 1e-3 * float(np.max(np.abs(want[fin])))
+    err = np.abs(got[fin] - want[fin])
+    bound = rtol * np.abs(want[fin]) + atol
+    bad = err > bound
+    if bad.any():
+        i = int(np.argmax(err - bound))
+        raise AssertionError(f"{what}: {bad.sum()} of {err.size} elements off; worst: got {got[fin][i]!r} want "
+                             f"{want[fin][i]!r} (err {err[i]:.3e} > {bound[i]:.3e})")
+
+
+def progress(request, msg):
+    """One line on the real stdout, past pytest's capture: long tests show they are alive."""
+    cap = request.config.pluginmanager.getplugin("capturemanager")
+    if cap is None:
+        print(msg, flush=True)
+        return
+    with cap.global_and_fixture_disabled():
+        print(f"\n[{request.node.name}] {msg}", end="", flush=True)
+
+
+def synthetic_params(shapes, dt, seed=0, std=0.02, norm_weight=1.0, workers=8):
+    """The benchmark's seeded weights (rai_amd.synthetic: N(0, std) per tensor from PCG64(seed, crc32(name)), zero
+    biases, constant norm weights) as a dict name -> carrier array already rounded to dt, generated in threads."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    from rai_amd import synthetic
+
+    def make(item):
+        name, shape = item
+        n = int(np.prod(shape))
+        if name.endswith("norm.weight"):
+            a = np.full(n, norm_weight, np.float32)
+        else:
+            a = synthetic.tensor(name, n, seed, std)
+        return name, rnd(a, dt).reshape(shape)
+
+    with ThreadPoolExecutor(max_workers=workers) as ex:
+        return dict(ex.map(make, shapes.items()))
+
+
+def assert_logits_close(got, chain, exact, dt, what=""):
+    """For whole-model logits at full width, where the reference's node-by-node evaluation in bf16 (`chain`: every
+    primitive's result rounded to the storage dtype) is itself a few per cent away from the same computation without
+    intermediate rounding (`exact`: the same stored weights, rotary tables and inputs, f32 arithmetic): the device,
+    which rounds less often than the chain, is held to the dtype's relative tolerance against `exact`, and may not
+    be farther from `chain` than that tolerance plus the chain's own measured rounding noise.  Errors are relative
+    to the largest magnitude of the expected logits, as in assert_close."""
+    got, chain, exact = (np.asarray(a, dtype=np.float64) for a in (got, chain, exact))
+    assert got.shape == chain.shape == exact.shape, f"{what}: shapes {got.shape} {chain.shape} {exact.shape}"
+    assert np.isfinite(got).all(), f"{what}: non-finite logits"
+    scale = float(np.max(np.abs(exact)))
+    tol = RTOL[dt] * scale
+    e_dev, e_chain, e_dc = (float(np.max(np.abs(a - b))) for a, b in ((got, exact), (chain, exact), (got, chain)))
+    assert e_dev <= tol, f"{what}: device vs unrounded reference arithmetic {e_dev:.3e} > {tol:.3e}"
+    assert e_dc <= tol + e_chain, (f"{what}: device vs node-by-node chain {e_dc:.3e} > {tol:.3e} + chain noise "
+                                   f"{e_chain:.3e}")
+    return e_dev / scale, e_chain / scale, e_dc / scale
