@@ -214,6 +214,20 @@ int rai_hip_argmax(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_
 int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
                    const rai_hip_tensor *out);
 
+/* rai_hip_argmax for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and same result as rai_hip_argmax, but the per-(row, split)
+ * partial results of the long-axis kernel live in a fixed array in device memory
+ * instead of the grown-on-demand workspace, and the call performs no hipMalloc /
+ * hipFree: rai_hip_init(dev) must have succeeded before (otherwise RAI_ERR_HIP).
+ * Limit: rows x splits <= 65536 partial results (the axis is only split while that
+ * product stays below 1024, so in effect: at most 65536 rows; more returns
+ * RAI_ERR_UNSUPPORTED).  All calls
+ * on one GPU share that GPU's array: calls that overlap on one device (different
+ * streams or threads) race; calls on the library's stream are ordered and safe. */
+int rai_hip_argmax_static(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
+                          const rai_hip_tensor *out);
+
 /* ---------------------------------------------------------------- indexing */
 
 /* IndexSelect: candle.rs:867-878, ops/index_select.rs:52-61.  index is a rank-1

@@ -101,6 +101,7 @@ PROTOTYPES = {
     "rai_hip_log_softmax": [C.c_int, _TP, _i32, _TP],
     "rai_hip_argmax": [C.c_int, _TP, _i32, _i32, _TP],
     "rai_hip_argmin": [C.c_int, _TP, _i32, _i32, _TP],
+    "rai_hip_argmax_static": [C.c_int, _TP, _i32, _i32, _TP],
     "rai_hip_index_select": [C.c_int, _TP, _TP, _i32, _TP],
     "rai_hip_gather": [C.c_int, _TP, _TP, _i32, _TP],
     "rai_hip_index_add": [C.c_int, _TP, _TP, _TP, _i32, _TP],

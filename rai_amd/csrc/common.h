@@ -41,6 +41,11 @@ struct DeviceCtx;
 // Returns nullptr (and sets the error) when dev is out of range or init fails.
 DeviceCtx *ctx(int dev);
 hipStream_t stream_of(int dev);
+// The stream of an already initialised device; never creates a context (no allocation): nullptr + error otherwise.
+hipStream_t stream_if_ready(int dev);
+// Looks up this device's address of the fixed scratch array of the allocation-free argmax (reduce.hip); called once
+// per device, with that device current, while its context is created.
+int arg_static_scratch_init(int dev);
 // Workspace that lives as long as the device context (grown on demand, never
 // shrinks); used by kernels that need partial results.  Stream-ordered reuse.
 int workspace(int dev, size_t bytes, void **out);

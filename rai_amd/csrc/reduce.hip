@@ -466,8 +466,25 @@ template <bool LOG> static int softmax_impl(int dev, const rai_hip_tensor *in, i
   return launch_check("softmax");
 }
 
+// Partial results of the allocation-free argmax: a fixed array in device memory instead of the grown-on-demand
+// workspace.  Every GPU holds its own copy at its own address; the address is looked up once per device when the
+// device context is created (arg_static_scratch_init) and only that pointer is ever handed to kernels.
+static constexpr size_t kArgStaticParts = 65536;   // (row, split) partial results one call may produce
+static constexpr size_t kArgStaticBytes = kArgStaticParts * (sizeof(double) + sizeof(uint32_t)) + 64;
+static __device__ __align__(256) unsigned char scratch[kArgStaticBytes];
+static void *g_scratch_ptr[16] = {nullptr};
+
+int arg_static_scratch_init(int dev) {
+  if (dev < 0 || dev >= 16) return fail(RAI_ERR_BAD_ARG, "device index %d out of range", dev);
+  void *p = nullptr;
+  RAI_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  g_scratch_ptr[dev] = p;
+  return RAI_OK;
+}
+
 template <bool IS_MAX>
-static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim, const rai_hip_tensor *out) {
+static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim, const rai_hip_tensor *out,
+                    bool no_alloc = false) {
   RAI_TRY(validate(in, "in"));
   RAI_TRY(validate(out, "out"));
   RAI_REQUIRE(out->dtype == RAI_U32, RAI_ERR_BAD_DTYPE, "argmax: output must be u32");
@@ -478,7 +495,8 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
   bool reduced[RAI_HIP_MAX_RANK] = {false};
   reduced[d] = true;
   RAI_TRY(check_reduced_shape(in, reduced, keep_dim, out, "argmax"));
-  hipStream_t st = stream_of(dev);
+  // the allocation-free form must not create a device context either (that allocates): rai_hip_init comes first
+  hipStream_t st = no_alloc ? stream_if_ready(dev) : stream_of(dev);
   if (!st) return RAI_ERR_HIP;
   if (numel(out) == 0) return RAI_OK;
   ReduceSpace s;
@@ -494,7 +512,15 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
     while (rows * splits < 2 * kNumCU && n / (splits * 2) >= 2048) splits *= 2;
     void *ws = nullptr;
     size_t nparts = (size_t)rows * splits;
-    RAI_TRY(workspace(dev, nparts * (sizeof(double) + sizeof(uint32_t)) + 64, &ws));
+    if (no_alloc) {
+      RAI_REQUIRE(nparts <= kArgStaticParts, RAI_ERR_UNSUPPORTED,
+                  "argmax_static: %lld rows x %d splits = %zu partial results, the static scratch holds %zu",
+                  (long long)rows, splits, nparts, kArgStaticParts);
+      ws = g_scratch_ptr[dev];
+      RAI_REQUIRE(ws, RAI_ERR_HIP, "argmax_static: scratch address of device %d unknown (rai_hip_init failed?)", dev);
+    } else {
+      RAI_TRY(workspace(dev, nparts * (sizeof(double) + sizeof(uint32_t)) + 64, &ws));
+    }
     double *pd = (double *)ws;
     float *pf = (float *)ws;
     uint32_t *pi = (uint32_t *)((char *)ws + nparts * sizeof(double));
@@ -580,6 +606,9 @@ int rai_hip_argmax(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_
 }
 int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim, const rai_hip_tensor *out) {
   return arg_impl<false>(dev, in, dim, keep_dim, out);
+}
+int rai_hip_argmax_static(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim, const rai_hip_tensor *out) {
+  return arg_impl<true>(dev, in, dim, keep_dim, out, true);
 }
 
 }  // extern "C"

@@ -77,9 +77,19 @@ DeviceCtx *ctx(int dev) {
     set_error("device %d init failed: %s", dev, hipGetErrorString(e));
     return nullptr;
   }
+  // per-device addresses of the library's fixed device arrays (this device is current here)
+  if (arg_static_scratch_init(dev) != RAI_OK) return nullptr;
   c->dev = dev;
   c->ready = true;
   return c;
+}
+
+hipStream_t stream_if_ready(int dev) {
+  if (dev < 0 || dev >= kMaxDev || !g_ctx[dev].ready) {
+    set_error("device %d is not initialised: call rai_hip_init(%d) first", dev, dev);
+    return nullptr;
+  }
+  return g_ctx[dev].stream;
 }
 
 hipStream_t stream_of(int dev) {

@@ -136,6 +136,12 @@ def argmin(x, dim, keep_dim=False):
     return argmax(x, dim, keep_dim, "rai_hip_argmin")
 
 
+def argmax_static(x, dim, out, keep_dim=False):
+    """rai_hip_argmax_static: argmax into the caller's `out`, with no allocation inside the library."""
+    call("rai_hip_argmax_static", x.dev, _d(x), dim % x.rank, int(keep_dim), _d(out))
+    return out
+
+
 # ---------------------------------------------------------------- indexing
 def index_select(x, dim, index):
     d = dim % x.rank
