@@ -57,13 +57,38 @@ def prefill_flops(cfg, s):
     return lin + attn + 2.0 * v * h
 
 
+def check_first_tokens(tokens):
+    """The greedy tokens of this workload against the CPU oracle's (tests/golden/phi2_bench_first_tokens.json, written
+    by tests/golden/make_phi2_bench_tokens.py from the oracle alone; tests/test_gpu_config2_phi2_full.py checks the
+    fixture itself).  A token may differ only where the oracle's own two best logits are a near tie at the bf16
+    tolerance; the sequences may part ways after that.  Anything else ends the run: a fast wrong answer is no result."""
+    path = os.path.join(ROOT, "tests", "golden", "phi2_bench_first_tokens.json")
+    with open(path) as f:
+        gold = json.load(f)
+    for s, want in enumerate(gold["tokens"]):
+        if int(tokens[s]) != want:
+            if gold["top2_gap"][s] <= 2e-2 * gold["max_abs_logit"][s]:
+                return f"identical for {s} tokens, then a near tie of the oracle's logits (gap {gold['top2_gap'][s]:.4f})"
+            sys.exit(f"bench.py: greedy token {s} is {int(tokens[s])}, the CPU oracle says {want} "
+                     f"(top-2 gap {gold['top2_gap'][s]:.4f}): refusing to report a throughput")
+    return f"identical for all {len(gold['tokens'])} checked tokens"
+
+
 def cpu_baseline(steps_decode=2, layers=2):
     """The oracle (a NumPy port of rai's Cpu evaluation, bf16 storage with f32
     math) timed on this host on a bounded sample: the first `layers` decoder
     layers plus embedding and lm_head, 512-token prefill, then `steps_decode`
     decode tokens; the per-layer times are scaled to 32 layers."""
     from oracle import phi2
-    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    # threads = physical cores of this host, capped by the share the environment grants (OMP_NUM_THREADS); the BLAS
+    # pool NumPy's matmul runs on is set to that count and the count it reports back is what goes into the line
+    import psutil
+    from threadpoolctl import threadpool_info, threadpool_limits
+    want = min(psutil.cpu_count(logical=False) or os.cpu_count() or 1,
+               int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    threadpool_limits(limits=want)
+    pools = [p["num_threads"] for p in threadpool_info() if p.get("user_api") == "blas"]
+    threads = max(pools) if pools else want
     cfg = phi2.Config(num_hidden_layers=layers)
     params = phi2.random_params(cfg, "bf16", seed=0)
     model = phi2.Model(cfg, params, "bf16")
@@ -199,12 +224,18 @@ def run_gemma_decode(args):
 
 
 def run_ops(args):
-    """Primitive sweep, bf16 and f32: each op timed over a batched loop (hipEvents) and as a single launch."""
+    """Primitive sweep, bf16 and f32.  Every op is launched through the C ABI into an output allocated beforehand,
+    with the tensor descriptors built once, so the timed loop holds launches only: `loop_us` is the hipEvent time of
+    a back-to-back loop divided by its length (launch rate or kernel time, whichever is longer), `single_us` one
+    launch between two events.  The kernels' own durations are in the rocprofv3 kernel trace of this same command
+    (profiles/op_sweep_kernel_trace.md)."""
     import ctypes as C
 
     from rai_amd import _lib, ops
+    from rai_amd._lib import REDUCE, UNARY  # noqa: F401
     from rai_amd.hip import HipTensor, sync
     _lib.call("rai_hip_init", 0)
+    lib = _lib.load()
     rng = np.random.default_rng(0)
 
     def rnd(shape, dt, scale=1.0):
@@ -212,6 +243,19 @@ def run_ops(args):
         if dt == "bf16":
             return HipTensor.from_storage((a.view(np.uint32) >> 16).astype(np.uint16), "bf16")
         return HipTensor.from_storage(a, "f32")
+
+    def launcher(name, *args):
+        """A zero-argument callable that performs exactly one C-ABI call with everything prepared."""
+        fn = getattr(lib, name)
+        keep = [a.desc() if isinstance(a, HipTensor) else a for a in args]
+        cargs = [C.byref(k) if isinstance(k, _lib.TensorDesc) else k for k in keep]
+
+        def go():
+            st = fn(*cargs)
+            if st != 0:
+                _lib.check(st)
+        go.keep = (keep, args)
+        return go
 
     def timed(fn, iters):
         t = C.c_void_p()
@@ -225,6 +269,7 @@ def run_ops(args):
         ms = C.c_float()
         _lib.call("rai_hip_timer_elapsed_ms", t, C.byref(ms))
         loop_us = ms.value * 1e3 / iters
+        sync()
         _lib.call("rai_hip_timer_start", t)
         fn()
         _lib.call("rai_hip_timer_stop", t)
@@ -233,67 +278,53 @@ def run_ops(args):
         return loop_us, ms.value * 1e3
 
     rows = []
+
+    def hbm(op, dt, by, fn, iters=100):
+        lu, su = timed(fn, iters)
+        rows.append(dict(op=op, dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3, unit="GB/s",
+                         frac=by / lu / 1e3 / HBM_PEAK_GBS, bytes=int(by)))
+
     for dt, es in (("bf16", 2), ("f32", 4)):
         a, b = rnd((4096, 2560), dt), rnd((2560, 10240), dt)
-        lu, su = timed(lambda: ops.matmul(a, b), 10)
+        out = HipTensor.empty((4096, 10240), dt)
         fl = 2.0 * 4096 * 2560 * 10240
         peak = MFMA_BF16_PEAK_TFLOPS if dt == "bf16" else 157.3
+        lu, su = timed(launcher("rai_hip_matmul", 0, a, b, out), 10)
         rows.append(dict(op="matmul [4096,2560]x[2560,10240]", dtype=dt, loop_us=lu, single_us=su, bound="mfma",
                          achieved=fl / lu / 1e6, unit="TFLOP/s", frac=fl / lu / 1e6 / peak))
         w = rnd((10240, 2560), dt)
-        lu, su = timed(lambda: ops.linear(a, w), 10)
+        lu, su = timed(launcher("rai_hip_linear", 0, a, w, None, -1, None, out), 10)
         rows.append(dict(op="linear x[4096,2560] . W[10240,2560]^T", dtype=dt, loop_us=lu, single_us=su, bound="mfma",
                          achieved=fl / lu / 1e6, unit="TFLOP/s", frac=fl / lu / 1e6 / peak))
-        del a, b, w
+        del a, b, w, out
         x = rnd((32, 128, 2048), dt, 3.0)
-        lu, su = timed(lambda: ops.softmax(x, -1), 50)
-        by = 2.0 * x.numel() * es
-        rows.append(dict(op="softmax [32,128,2048]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
-                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        out = HipTensor.empty(x.shape, dt)
+        hbm("softmax [32,128,2048]", dt, 2.0 * x.numel() * es, launcher("rai_hip_softmax", 0, x, 2, out))
         x = rnd((4096, 2560), dt)
+        out = HipTensor.empty(x.shape, dt)
         w1, b1 = rnd((2560,), dt), rnd((2560,), dt)
         by = 2.0 * x.numel() * es
-        lu, su = timed(lambda: ops.layer_norm(x, w1, b1, 1e-5), 50)
-        rows.append(dict(op="layer_norm [4096,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
-                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
-        lu, su = timed(lambda: ops.rms_norm(x, w1, 1e-6), 50)
-        rows.append(dict(op="rms_norm [4096,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
-                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        hbm("layer_norm [4096,2560]", dt, by, launcher("rai_hip_layer_norm", 0, x, w1, b1, 1e-5, out))
+        hbm("rms_norm [4096,2560]", dt, by, launcher("rai_hip_rms_norm", 0, x, w1, 1e-6, 0, out))
         x = rnd((1, 32, 2048, 80), dt)
+        out = HipTensor.empty(x.shape, dt)
         cos, sin = ops.rope_tables(2048, 32, 10000.0, dt)
-        by = 2.0 * x.numel() * es
-        lu, su = timed(lambda: ops.rope(x, cos, sin, 32, 0), 50)
-        rows.append(dict(op="rope [1,32,2048,80] rot 32", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
-                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        hbm("rope [1,32,2048,80] rot 32", dt, 2.0 * x.numel() * es, launcher("rai_hip_rope", 0, x, cos, sin, 32, 0, out))
         table = rnd((51200, 2560), dt)
         ids = HipTensor.from_storage(rng.integers(0, 51200, 4096).astype(np.uint32), "u32")
-        by = 2.0 * 4096 * 2560 * es
-        lu, su = timed(lambda: ops.index_select(table, 0, ids), 50)
-        rows.append(dict(op="index_select 4096 of [51200,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
-                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        out = HipTensor.empty((4096, 2560), dt)
+        hbm("index_select 4096 of [51200,2560]", dt, 2.0 * 4096 * 2560 * es + 4096 * 4,
+            launcher("rai_hip_index_select", 0, table, ids, 0, out))
         # the gradient of that embedding lookup: cotangent rows added into the table at the ids
         ct = rnd((4096, 2560), dt)
-        by = (2.0 * 51200 * 2560 + 4096 * 2560) * es      # table read + written once, cotangent read once
-        lu, su = timed(lambda: ops.index_add(table, 0, ids, ct), 20)
-        rows.append(dict(op="index_add 4096 rows into [51200,2560]", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
-                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
-        logits = rnd((64, 51200), dt)
-        tgt = HipTensor.from_storage(rng.integers(0, 51200, (64, 1)).astype(np.uint32), "u32")
-        by = 64.0 * (es + 4) + 64 * es
-        lu, su = timed(lambda: ops.gather(logits, 1, tgt), 50)
-        rows.append(dict(op="gather [64,51200] dim 1, one id per row", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
-                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
-        one = rnd((64, 1), dt)
-        by = 2.0 * 64 * 51200 * es
-        lu, su = timed(lambda: ops.scatter_add(logits, 1, tgt, one), 50)
-        rows.append(dict(op="scatter_add [64,1] into [64,51200] dim 1", dtype=dt, loop_us=lu, single_us=su, bound="hbm",
-                         achieved=by / lu / 1e3, unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
-        del table, ct, logits
+        out = HipTensor.empty(table.shape, dt)
+        hbm("index_add 4096 rows into [51200,2560]", dt, (2.0 * 51200 * 2560 + 4096 * 2560) * es,
+            launcher("rai_hip_index_add", 0, table, ids, ct, 0, out), 20)
+        del table, ct, out
         x = rnd((64, 51200), dt)
-        by = 1.0 * x.numel() * es
-        lu, su = timed(lambda: ops.argmax(x, -1), 50)
-        rows.append(dict(op="argmax [64,51200]", dtype=dt, loop_us=lu, single_us=su, bound="hbm", achieved=by / lu / 1e3,
-                         unit="GB/s", frac=by / lu / 1e3 / HBM_PEAK_GBS))
+        out = HipTensor.empty((64,), "u32")
+        hbm("argmax [64,51200]", dt, 1.0 * x.numel() * es, launcher("rai_hip_argmax", 0, x, 1, 0, out))
+        hbm("argmax_static [64,51200]", dt, 1.0 * x.numel() * es, launcher("rai_hip_argmax_static", 0, x, 1, 0, out))
     sync()
     for r in rows:
         r.update(loop_us=round(r["loop_us"], 2), single_us=round(r["single_us"], 2), achieved=round(r["achieved"], 1),
@@ -389,7 +420,7 @@ def main():
         "prefill_ms": round(pre, 3),
         "prefill_frac_of_bf16_mfma_peak": round(prefill_flops(cfg, PROMPT) / (pre / 1e3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "weights_load_s": round(load_s, 1),
-        "first_tokens": [int(t) for t in toks[0, :8]],
+        "first_tokens": [int(t) for t in toks[0, :17]],
         "sampled_decode_tokens_per_s": round((NEW - 1) / (samp_ms / 1e3), 2),
         "roofline": {
             "kernel": "k_phi2_decode_step (persistent kernel: all 32 layers of one decode step, blocks exchange "
@@ -408,6 +439,8 @@ def main():
                                 "GB_per_s": round(gemv_bytes / (gemv_us * 1e-6) / 1e9, 1)},
     }
     dec.close()
+    if args.layers == PHI2["num_hidden_layers"]:
+        out["tokens_match_oracle"] = check_first_tokens(toks[0])
     if args.pmc_calibrate:
         import ctypes as C
 

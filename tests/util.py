@@ -1,6 +1,9 @@
 """Helpers shared by the parity tests: upload/download in storage dtypes and the
 tolerances of the correctness bar (f32: 1e-4 relative, bf16: 2e-2 relative,
-integers and indices: bit-exact)."""
+integers and indices: bit-exact).  Two forms: assert_close bounds the error by the
+largest magnitude of the expected tensor (contractions, reductions, norms, logits);
+assert_close_elem bounds every element by its own magnitude (unary, binary, cast,
+activations, RoPE)."""
 import numpy as np
 
 from oracle.dtypes import from_storage, rnd, to_storage
