@@ -56,6 +56,7 @@ typedef enum rai_op_kind {
   RAI_OP_GATHER = 22,
   RAI_OP_INDEX_ADD = 23,   /* inputs ordered [x, source, index] (ops/index_add.rs:57-59) */
   RAI_OP_SCATTER_ADD = 24, /* inputs ordered [x, source, index] (ops/scatter_add.rs:57) */
+  RAI_OP_TO_DEVICE = 25,   /* ToDevice<Hip>: ops/to_device.rs, registered per device at dispatch.rs:117-121 */
   RAI_OP_COUNT_
 } rai_op_kind;
 
@@ -89,6 +90,9 @@ rai_tensor *rai_reshape(rai_tensor *x, const int64_t *shape, int32_t rank);   /*
 rai_tensor *rai_permute(rai_tensor *x, const int32_t *dims, int32_t rank);
 rai_tensor *rai_broadcast_to(rai_tensor *x, const int64_t *shape, int32_t rank);
 rai_tensor *rai_to_contiguous(rai_tensor *x);
+/* Tensor::to_device (ops/to_device.rs:48-59): x itself (a new reference) when it already lives on Hip(dev),
+ * else a ToDevice node on the target device whose rule copies across devices (rai_hip_to_device). */
+rai_tensor *rai_to_device(rai_tensor *x, int32_t dev);
 
 /* ---- handles and metadata (tensor.rs) */
 void rai_tensor_retain(rai_tensor *t);

@@ -148,6 +148,15 @@ int rai_hip_h2d(int dev, void *dst_dev, const void *src_host, size_t bytes);
 int rai_hip_d2h(int dev, void *dst_host, const void *src_dev, size_t bytes);
 int rai_hip_d2d(int dev, void *dst_dev, const void *src_dev, size_t bytes);
 
+/* ToDevice<Hip>: rai-core/src/ops/to_device.rs:48-59, evaluated at backend/candle.rs:776-790.
+ * Copies the strided tensor `in`, resident on HIP device src_dev, into the contiguous
+ * tensor `out` on HIP device dst_dev (same dtype and shape).  src_dev == dst_dev is a
+ * plain strided copy on that device's stream; across devices the source is made
+ * contiguous on its own device and moved with a peer copy ordered after the source
+ * stream's work.  (Host -> device is rai_hip_h2d into a fresh buffer, device -> host is
+ * rai_hip_d2h of a contiguous copy: the two other directions of the reference's op.) */
+int rai_hip_to_device(int src_dev, const rai_hip_tensor *in, int dst_dev, const rai_hip_tensor *out);
+
 /* hipEvent timers on the device's stream (measurement only). */
 int rai_hip_timer_create(int dev, void **timer);
 int rai_hip_timer_start(void *timer);

@@ -84,6 +84,7 @@ PROTOTYPES = {
     "rai_hip_h2d": [C.c_int, _vp, _vp, C.c_size_t],
     "rai_hip_d2h": [C.c_int, _vp, _vp, C.c_size_t],
     "rai_hip_d2d": [C.c_int, _vp, _vp, C.c_size_t],
+    "rai_hip_to_device": [C.c_int, _TP, C.c_int, _TP],
     "rai_hip_timer_create": [C.c_int, C.POINTER(_vp)],
     "rai_hip_timer_start": [_vp],
     "rai_hip_timer_stop": [_vp],
@@ -170,6 +171,7 @@ GRAPH_PROTOTYPES = {
     "rai_permute": (_T, [_T, _I32P, _i32]),
     "rai_broadcast_to": (_T, [_T, _I64P, _i32]),
     "rai_to_contiguous": (_T, [_T]),
+    "rai_to_device": (_T, [_T, _i32]),
     "rai_tensor_retain": (None, [_T]),
     "rai_tensor_release": (None, [_T]),
     "rai_tensor_rank": (_i32, [_T]),

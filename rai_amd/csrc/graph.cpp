@@ -265,6 +265,11 @@ int ev_to_contiguous(rai_tensor *t) {
   ++g_stats.kernel_launches;
   return rai_hip_copy(t->dev, &t->inputs[0]->view, &t->view);
 }
+int ev_to_device(rai_tensor *t) {  // ops/to_device.rs: the node lives on the target device, its input on the source
+  RAI_TRY(alloc_output(t));
+  ++g_stats.kernel_launches;
+  return rai_hip_to_device(t->inputs[0]->dev, &t->inputs[0]->view, t->dev, &t->view);
+}
 int ev_concatenate(rai_tensor *t) {
   RAI_TRY(alloc_output(t));
   const int dim = (int)t->ip[0];
@@ -355,7 +360,8 @@ int ev_reshape(rai_tensor *t) {
 const rule_fn kBuiltin[RAI_OP_COUNT_] = {
     ev_full, ev_arange, ev_from_array, ev_to_dtype, ev_unary, ev_binary, ev_matmul, ev_softmax, ev_log_softmax, ev_reduce,
     ev_argmax, ev_argmin, ev_index_select, ev_narrow, ev_concatenate, ev_where, ev_transpose, ev_reshape, ev_permute,
-    ev_broadcast, ev_to_contiguous, nullptr /* Err nodes never reach a rule */, ev_gather, ev_index_add, ev_scatter_add};
+    ev_broadcast, ev_to_contiguous, nullptr /* Err nodes never reach a rule */, ev_gather, ev_index_add, ev_scatter_add,
+    ev_to_device};
 rule_fn g_rules[RAI_OP_COUNT_];
 bool g_rules_init = false;
 void init_rules() {
@@ -368,7 +374,7 @@ const char *op_name(int op) {
   static const char *n[RAI_OP_COUNT_] = {"Full", "Arange", "FromArray", "ToDType", "Unary", "Binary", "MatMul", "Softmax",
                                          "LogSoftmax", "Reduce", "ArgMax", "ArgMin", "IndexSelect", "Narrow",
                                          "Concatenate", "Where", "Transpose", "Reshape", "Permute", "Broadcast",
-                                         "ToContiguous", "Err", "Gather", "IndexAdd", "ScatterAdd"};
+                                         "ToContiguous", "Err", "Gather", "IndexAdd", "ScatterAdd", "ToDevice"};
   return op >= 0 && op < RAI_OP_COUNT_ ? n[op] : "?";
 }
 
@@ -860,6 +866,13 @@ rai_tensor *rai_broadcast_to(rai_tensor *x, const int64_t *shape, int32_t rank) 
   return new_node(x->dev, x->dtype, s, RAI_OP_BROADCAST, {x});
 }
 
+rai_tensor *rai_to_device(rai_tensor *x, int32_t dev) {
+  if (x->dev == dev) {   // ops/to_device.rs:49-52: already there, the same tensor
+    ++x->refs;
+    return x;
+  }
+  return new_node(dev, x->dtype, x->shape, RAI_OP_TO_DEVICE, {x});
+}
 rai_tensor *rai_to_contiguous(rai_tensor *x) { return new_node(x->dev, x->dtype, x->shape, RAI_OP_TO_CONTIGUOUS, {x}); }
 
 // ------------------------------------------------------------------ handles and metadata

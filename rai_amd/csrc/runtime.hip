@@ -337,6 +337,42 @@ int rai_hip_d2d(int dev, void *dst_dev, const void *src_dev, size_t bytes) {
   return RAI_OK;
 }
 
+int rai_hip_to_device(int src_dev, const rai_hip_tensor *in, int dst_dev, const rai_hip_tensor *out) {
+  RAI_TRY(validate(in, "in"));
+  RAI_TRY(validate(out, "out"));
+  RAI_REQUIRE(in->dtype == out->dtype, RAI_ERR_BAD_DTYPE, "to_device: dtype %s vs %s", dtype_name(in->dtype),
+              dtype_name(out->dtype));
+  RAI_REQUIRE(same_shape(in, out), RAI_ERR_BAD_SHAPE, "to_device: shapes differ");
+  RAI_REQUIRE(is_contiguous(out), RAI_ERR_BAD_STRIDE, "to_device: output must be contiguous");
+  if (src_dev == dst_dev) return rai_hip_copy(dst_dev, in, out);
+  DeviceCtx *cs = ctx(src_dev), *cd = ctx(dst_dev);
+  if (!cs || !cd) return RAI_ERR_HIP;
+  const size_t bytes = (size_t)numel(in) * dtype_size(in->dtype);
+  if (bytes == 0) return RAI_OK;
+  // a contiguous image of the source on its own device (the tensor itself when it already is one)
+  void *tmp = nullptr;
+  const void *src = (const char *)in->data + in->offset * (int64_t)dtype_size(in->dtype);
+  if (!is_contiguous(in)) {
+    RAI_TRY(rai_hip_alloc(src_dev, bytes, &tmp));
+    rai_hip_tensor t = *out;
+    t.data = tmp;
+    t.offset = 0;
+    int rc = rai_hip_copy(src_dev, in, &t);
+    if (rc != RAI_OK) { (void)rai_hip_release(tmp); return rc; }
+    src = tmp;
+  }
+  // the peer copy runs on the destination's stream, after everything queued on the source's stream so far
+  hipError_t e = hipStreamSynchronize(cs->stream);
+  if (e == hipSuccess) e = hipSetDevice(dst_dev);
+  if (e == hipSuccess)
+    e = hipMemcpyPeerAsync((char *)out->data + out->offset * (int64_t)dtype_size(out->dtype), dst_dev, src, src_dev, bytes,
+                           cd->stream);
+  if (e == hipSuccess && tmp) e = hipStreamSynchronize(cd->stream);   // tmp goes back to the source's pool below
+  if (tmp) (void)rai_hip_release(tmp);
+  if (e != hipSuccess) return fail(RAI_ERR_HIP, "to_device %d -> %d: %s", src_dev, dst_dev, hipGetErrorString(e));
+  return RAI_OK;
+}
+
 struct Timer {
   int dev;
   hipEvent_t a, b;

@@ -25,7 +25,7 @@ from ._lib import BF16, BINARY, DTYPE_BY_NAME, DTYPE_NAMES, DTYPE_SIZE, F16, F32
 
 OP_KINDS = ["Full", "Arange", "FromArray", "ToDType", "Unary", "Binary", "MatMul", "Softmax", "LogSoftmax", "Reduce",
             "ArgMax", "ArgMin", "IndexSelect", "Narrow", "Concatenate", "Where", "Transpose", "Reshape", "Permute",
-            "Broadcast", "ToContiguous", "Err", "Gather", "IndexAdd", "ScatterAdd"]
+            "Broadcast", "ToContiguous", "Err", "Gather", "IndexAdd", "ScatterAdd", "ToDevice"]
 OP = {n: i for i, n in enumerate(OP_KINDS)}
 _NP = {U8: np.uint8, U32: np.uint32, I64: np.int64, F16: np.float16, BF16: np.uint16, F32: np.float32, F64: np.float64}
 
@@ -90,6 +90,10 @@ class Tensor:
     @property
     def dtype(self):
         return DTYPE_NAMES[_lib.load().rai_tensor_dtype(self._h)]
+
+    @property
+    def device(self):
+        return int(_lib.load().rai_tensor_device(self._h))
 
     @property
     def op(self):
@@ -246,6 +250,10 @@ class Tensor:
 
     def to_contiguous(self):
         return Tensor(_lib.load().rai_to_contiguous(self._h))
+
+    def to_device(self, dev):
+        """Tensor::to_device (ops/to_device.rs:48-59): the same tensor when it already lives on Hip(dev)."""
+        return Tensor(_lib.load().rai_to_device(self._h, int(dev)))
 
     # ------------------------------------------------------------ high-level ops (the reference's decompositions)
     def flatten(self):

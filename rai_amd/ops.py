@@ -42,6 +42,13 @@ def from_array(arr, dtype, dev=0):
     return HipTensor.from_storage(arr, dtype, dev)
 
 
+def to_device(x, dev):
+    """ToDevice<Hip> (backend/candle.rs:776-790): a contiguous copy of x on HIP device `dev`."""
+    out = HipTensor.empty(x.shape, x.dtype, dev)
+    call("rai_hip_to_device", x.dev, _d(x), int(dev), _d(out))
+    return out
+
+
 def to_dtype(x, dtype):
     dt = _dt(dtype)
     if dt == x.dtype:

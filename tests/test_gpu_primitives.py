@@ -226,6 +226,15 @@ def test_contiguous_of_views_and_concat(R, dt):
               np.concatenate([a[..., 4:], a[..., :4]], -1))
 
 
+def test_to_device_copies_a_strided_view(R):
+    # ToDevice<Hip> (backend/candle.rs:776-790): this box has one GPU, so source and target are the same device
+    a = rand(rng(140), (6, 10, 16), "bf16")
+    x = up(a, "bf16").transpose(0, 2).narrow(1, 2, 5)
+    y = R.to_device(x, 0)
+    assert y.is_contiguous() and y.buf.ptr != x.buf.ptr
+    assert np.array_equal(down(y), np.swapaxes(a, 0, 2)[:, 2:7])
+
+
 # ------------------------------------------------------------------ reductions
 @pytest.mark.parametrize("dt", FLOATS)
 @pytest.mark.parametrize("dims,keep", [((-1,), True), ((-1,), False), ((0,), False), ((1,), True), ((0, 2), False),

@@ -125,3 +125,13 @@ def test_dispatcher_table():
     finally:
         g.dispatch_register_builtin("Softmax")
     assert g.dispatch_has_rule("Softmax")
+
+
+def test_to_device_on_the_same_device_is_the_same_tensor():
+    # ops/to_device.rs:49-52: x.to_device(x.device()) returns x itself, no node is added
+    x = Tensor.ones((2, 3), "f32", dev=0)
+    y = x.to_device(0)
+    assert y.id == x.id and y.device == 0
+    z = x.neg().to_device(1)        # another device: a ToDevice node on the target device, same shape and dtype
+    assert z.device == 1 and z.shape == (2, 3) and z.op == "ToDevice" and z.dtype == "f32"
+    assert g.dispatch_has_rule("ToDevice")
