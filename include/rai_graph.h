@@ -127,13 +127,23 @@ int rai_dispatch_unregister(int32_t op_kind);
 int rai_dispatch_register_builtin(int32_t op_kind);
 int32_t rai_dispatch_has_rule(int32_t op_kind);
 
-/* ---- fusion pass control and counters */
+/* ---- fusion passes: control and counters */
+/* Elementwise pass: chains of elementwise primitives as one launch, bit-identical with node-by-node evaluation. */
 int rai_graph_set_fusion(int32_t enabled);
+/* Composition pass: the compositions rai's modules are made of -- Linear with bias (rai-nn/src/linear.rs:59-69),
+ * LayerNorm (layer_norm.rs:32-42), RmsNorm (rms_norm.rs:18-22), the rotary embedding and the attention block of
+ * rai-models/src/llm/phi2.rs:66-77,244-262 -- are recognised by structure in the recorded graph and evaluated by
+ * their fused launcher (rai_hip_linear / layer_norm / rms_norm / rope / attention).  Taken only when no interior
+ * node is observable from outside.  Results agree with node-by-node evaluation within the dtype's tolerance (the
+ * fused launchers round less often), not bit for bit. */
+int rai_graph_set_compose(int32_t enabled);
 typedef struct rai_graph_stats {
   uint64_t nodes_evaluated;   /* nodes that received data */
   uint64_t kernel_launches;   /* device launches issued by eval (views launch nothing) */
   uint64_t fused_regions;     /* multi-node elementwise regions evaluated by one launch */
   uint64_t fused_nodes;       /* nodes folded into those regions */
+  uint64_t composed_regions;  /* compositions evaluated by one fused launcher */
+  uint64_t composed_nodes;    /* nodes folded into those compositions */
 } rai_graph_stats;
 int rai_graph_get_stats(rai_graph_stats *out, int32_t reset);
 

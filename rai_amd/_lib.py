@@ -139,7 +139,7 @@ PROTOTYPES = {
 
 class GraphStats(C.Structure):
     _fields_ = [("nodes_evaluated", C.c_uint64), ("kernel_launches", C.c_uint64), ("fused_regions", C.c_uint64),
-                ("fused_nodes", C.c_uint64)]
+                ("fused_nodes", C.c_uint64), ("composed_regions", C.c_uint64), ("composed_nodes", C.c_uint64)]
 
 
 _T = C.c_void_p  # rai_tensor *
@@ -191,6 +191,7 @@ GRAPH_PROTOTYPES = {
     "rai_dispatch_register_builtin": (C.c_int, [_i32]),
     "rai_dispatch_has_rule": (_i32, [_i32]),
     "rai_graph_set_fusion": (C.c_int, [_i32]),
+    "rai_graph_set_compose": (C.c_int, [_i32]),
     "rai_graph_get_stats": (C.c_int, [C.POINTER(GraphStats), _i32]),
 }
 

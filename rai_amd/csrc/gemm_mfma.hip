@@ -434,6 +434,8 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, 
     if constexpr ((n) == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                   \
     else if constexpr ((n) == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");              \
     else if constexpr ((n) == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");              \
+    else if constexpr ((n) == 7) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");              \
+    else if constexpr ((n) == 14) asm volatile("s_waitcnt vmcnt(14)" ::: "memory");            \
     else if constexpr ((n) == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");              \
     else if constexpr ((n) == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");            \
     else if constexpr ((n) == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");            \
@@ -1187,6 +1189,7 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   if (knob) {
     if (!strcmp(knob, "128x128")) return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
     if (!strcmp(knob, "256x128")) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
+    if (!strcmp(knob, "256x192")) return launch_cfg_dma<256, 192, 4, 2>(st, a, splits);
     if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
     if (!strcmp(knob, "256x256x8w")) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);

@@ -40,7 +40,8 @@ namespace {
 
 uint64_t g_next_id = 1;
 bool g_fusion = true;
-rai_graph_stats g_stats = {0, 0, 0, 0};
+bool g_compose = true;
+rai_graph_stats g_stats = {0, 0, 0, 0, 0, 0};
 
 int64_t numel_of(const std::vector<int64_t> &s) {
   int64_t n = 1;
@@ -422,7 +423,8 @@ struct FusionPlan {
 // A node is folded into its consumer when it is elementwise, exactly one edge of
 // the tape uses it, that user is elementwise too, it is not a requested output,
 // and no handle outside the tape refers to it (refs == that one edge).
-void plan_fusion(const std::vector<rai_tensor *> &tape, rai_tensor *const *outputs, int n_out, FusionPlan *plan) {
+void plan_fusion(const std::vector<rai_tensor *> &tape, rai_tensor *const *outputs, int n_out, FusionPlan *plan,
+                 const std::unordered_set<uint64_t> &composed) {
   std::unordered_map<uint64_t, int> uses;
   std::unordered_map<uint64_t, const rai_tensor *> user;
   for (const rai_tensor *t : tape)
@@ -434,10 +436,11 @@ void plan_fusion(const std::vector<rai_tensor *> &tape, rai_tensor *const *outpu
   for (int i = 0; i < n_out; ++i) is_output.insert(outputs[i]->id);
   for (const rai_tensor *t : tape) {
     if (!elementwise(t) || is_output.count(t->id) || !g_rules[t->op]) continue;  // fusion never hides a missing rule
+    if (composed.count(t->id)) continue;                                         // root or interior of a composition
     auto u = uses.find(t->id);
     if (u == uses.end() || u->second != 1 || t->refs != 1) continue;
     const rai_tensor *c = user[t->id];
-    if (!elementwise(c) || numel_of(c->shape) != numel_of(t->shape) || c->shape != t->shape) continue;
+    if (!elementwise(c) || composed.count(c->id) || numel_of(c->shape) != numel_of(t->shape) || c->shape != t->shape) continue;
     plan->inlined.insert(t->id);
   }
 }
@@ -554,6 +557,344 @@ int eval_plain(rai_tensor *t, const FusionPlan &plan) {
   RAI_TRY(rule(t));
   t->evaluated = true;
   ++g_stats.nodes_evaluated;
+  return RAI_OK;
+}
+
+// ------------------------------------------------------------------ composition pass
+// rai's modules are compositions of primitives (rai-nn/src/{linear,layer_norm,rms_norm}.rs, the rotary embedding and
+// the attention block of rai-models/src/llm/phi2.rs); recorded node by node they are 10-20 launches each.  This pass
+// recognises those compositions in the tape, by structure, and evaluates each with the one fused launcher that
+// exists for it.  A composition is taken only when every interior node is invisible from outside it: unevaluated, not
+// a requested output, no handle outside the tape, every consumer inside the composition.  The fused launchers keep
+// f32 between the steps the reference rounds after, so a composed result agrees with the node-by-node one within
+// the dtype's tolerance, not bit for bit (the elementwise pass above is the bit-exact one).
+enum CompKind { COMP_LINEAR = 0, COMP_LAYER_NORM, COMP_RMS_NORM, COMP_ROPE, COMP_ATTENTION };
+struct Composite {
+  int kind;
+  rai_tensor *in[5];   // operands: evaluated before the root is reached (they precede it in the tape)
+  double f0;           // eps / scale
+  int64_t i0, i1;      // rotary dim and offset / causal flag
+  std::vector<rai_tensor *> interior;
+};
+struct ComposePlan {
+  std::unordered_map<uint64_t, Composite> roots;
+  std::unordered_set<uint64_t> absorbed;
+};
+struct UseInfo {
+  std::unordered_map<uint64_t, std::vector<const rai_tensor *>> users;   // edges from nodes of the tape
+};
+
+struct Matcher {
+  std::vector<rai_tensor *> interior;
+  bool ok = true;
+  // descends into an unevaluated node of kind `op`; records it as interior
+  rai_tensor *node(rai_tensor *t, int op) {
+    if (!ok || !t || t->evaluated || t->op != op) { ok = false; return nullptr; }
+    interior.push_back(t);
+    return t;
+  }
+  bool bin(rai_tensor *t, int sub, rai_tensor **a, rai_tensor **b) {
+    rai_tensor *n = node(t, RAI_OP_BINARY);
+    if (!n || n->sub != sub) { ok = false; return false; }
+    *a = n->inputs[0];
+    *b = n->inputs[1];
+    return true;
+  }
+  rai_tensor *un(rai_tensor *t, int sub) {
+    rai_tensor *n = node(t, RAI_OP_UNARY);
+    if (!n || n->sub != sub) { ok = false; return nullptr; }
+    return n->inputs[0];
+  }
+  // the operand behind an optional Broadcast view
+  rai_tensor *strip_bc(rai_tensor *t) {
+    if (ok && t && !t->evaluated && t->op == RAI_OP_BROADCAST) { interior.push_back(t); return t->inputs[0]; }
+    return t;
+  }
+  // the operand behind an optional cast to `dtype` (ToDType of an equal dtype never makes a node)
+  rai_tensor *strip_cast(rai_tensor *t, int dtype) {
+    if (ok && t && !t->evaluated && t->op == RAI_OP_TO_DTYPE && t->dtype == dtype) { interior.push_back(t); return t->inputs[0]; }
+    return t;
+  }
+  // a scalar constant: Full, or Full cast to the tensor's dtype (ops/full.rs:85-92)
+  bool konst(rai_tensor *t, double *v) {
+    if (!ok || !t) return ok = false;
+    if (t->op == RAI_OP_FULL) { if (!t->evaluated) interior.push_back(t); *v = t->p0; return true; }
+    if (!t->evaluated && t->op == RAI_OP_TO_DTYPE && t->inputs[0]->op == RAI_OP_FULL) {
+      interior.push_back(t);
+      if (!t->inputs[0]->evaluated) interior.push_back(t->inputs[0]);
+      *v = t->inputs[0]->p0;
+      return true;
+    }
+    return ok = false;
+  }
+  // sum over the last dim, keep_dim
+  rai_tensor *sum_last_keep(rai_tensor *t) {
+    rai_tensor *n = node(t, RAI_OP_REDUCE);
+    if (!n) return nullptr;
+    const int rank = (int)n->inputs[0]->shape.size();
+    if (n->sub != RAI_RED_SUM || n->ip.size() != 2 || n->ip[0] != 1 || n->ip[1] != rank - 1) { ok = false; return nullptr; }
+    return n->inputs[0];
+  }
+  rai_tensor *narrow(rai_tensor *t, int64_t dim, int64_t *start, int64_t *len) {
+    rai_tensor *n = node(t, RAI_OP_NARROW);
+    if (!n || n->ip[0] != dim) { ok = false; return nullptr; }
+    *start = n->ip[1];
+    *len = n->ip[2];
+    return n->inputs[0];
+  }
+  // hlops/mean.rs:4-7 over the last dim, keep_dim: sum / n
+  bool mean_of(rai_tensor *t, rai_tensor *x) {
+    rai_tensor *s, *nc;
+    double n = 0;
+    if (!bin(t, RAI_BIN_DIV, &s, &nc) || !konst(nc, &n)) return false;
+    if (sum_last_keep(s) != x || !ok || n != (double)x->shape.back()) return ok = false;
+    return true;
+  }
+};
+
+std::unordered_map<uint64_t, bool> g_causal_masks;   // mask node id -> "is the causal mask"; cleared per eval
+
+bool vec_param(const rai_tensor *p, int64_t n, int dtype) { return p && p->shape.size() == 1 && p->shape[0] == n && p->dtype == dtype; }
+bool norm_dtype(int dt) { return dt == RAI_F32 || dt == RAI_BF16 || dt == RAI_F16; }
+
+// rai-nn/src/layer_norm.rs:32-42: w * ((x - mean) * rsqrt(var + eps)) + b, var = sum((x - mean)^2) / n (hlops/var.rs:33-38)
+bool match_layer_norm(rai_tensor *t, Composite *c) {
+  Matcher m;
+  rai_tensor *y, *bb, *wb, *xs, *d, *rb, *x, *mb, *ve, *var, *epsc, *s, *nc, *x2, *mb2;
+  if (!norm_dtype(t->dtype) || t->shape.empty() || !m.bin(t, RAI_BIN_ADD, &y, &bb)) return false;
+  rai_tensor *bias = m.strip_bc(bb);
+  if (!m.bin(y, RAI_BIN_MUL, &wb, &xs)) return false;
+  rai_tensor *w = m.strip_bc(wb);
+  const int64_t n = t->shape.back();
+  if (!vec_param(w, n, t->dtype) || !vec_param(bias, n, t->dtype)) return false;
+  if (!m.bin(xs, RAI_BIN_MUL, &d, &rb) || !m.bin(d, RAI_BIN_SUB, &x, &mb) || x->shape != t->shape) return false;
+  if (!m.mean_of(m.strip_bc(mb), x)) return false;
+  ve = m.un(m.strip_bc(rb), RAI_UN_RSQRT);
+  double eps = 0, nn = 0;
+  if (!ve || !m.bin(ve, RAI_BIN_ADD, &var, &epsc) || !m.konst(epsc, &eps)) return false;
+  if (!m.bin(var, RAI_BIN_DIV, &s, &nc) || !m.konst(nc, &nn) || nn != (double)n) return false;
+  rai_tensor *sq = m.sum_last_keep(s);
+  rai_tensor *d2 = sq ? m.un(sq, RAI_UN_SQUARE) : nullptr;
+  if (!d2 || !m.bin(d2, RAI_BIN_SUB, &x2, &mb2) || x2 != x || !m.mean_of(m.strip_bc(mb2), x) || !m.ok) return false;
+  c->kind = COMP_LAYER_NORM;
+  c->in[0] = x; c->in[1] = w; c->in[2] = bias;
+  c->f0 = eps;
+  c->interior = m.interior;
+  return true;
+}
+
+// rai-nn/src/rms_norm.rs:18-22: w * x * rsqrt(sum((x / sqrt(n))^2) + eps)
+bool match_rms_norm(rai_tensor *t, Composite *c) {
+  Matcher m;
+  rai_tensor *wx, *rb, *wb, *x, *ve, *s, *epsc, *x2, *cc;
+  if (!norm_dtype(t->dtype) || t->shape.empty() || !m.bin(t, RAI_BIN_MUL, &wx, &rb) || !m.bin(wx, RAI_BIN_MUL, &wb, &x)) return false;
+  rai_tensor *w = m.strip_bc(wb);
+  const int64_t n = t->shape.back();
+  if (!vec_param(w, n, t->dtype) || x->shape != t->shape) return false;
+  ve = m.un(m.strip_bc(rb), RAI_UN_RSQRT);
+  double eps = 0, div = 0;
+  if (!ve || !m.bin(ve, RAI_BIN_ADD, &s, &epsc) || !m.konst(epsc, &eps)) return false;
+  rai_tensor *sq = m.sum_last_keep(s);
+  rai_tensor *xd = sq ? m.un(sq, RAI_UN_SQUARE) : nullptr;
+  if (!xd || !m.bin(xd, RAI_BIN_DIV, &x2, &cc) || x2 != x || !m.konst(cc, &div) || !m.ok) return false;
+  if (fabs(div * div - (double)n) > 1e-3 * (double)n) return false;
+  c->kind = COMP_RMS_NORM;
+  c->in[0] = x; c->in[1] = w;
+  c->f0 = eps;
+  c->interior = m.interior;
+  return true;
+}
+
+// rai-nn/src/linear.rs:59-69 with a bias: x @ broadcast_left(W).t() + b
+bool match_linear(rai_tensor *t, Composite *c) {
+  Matcher m;
+  rai_tensor *mm, *bb;
+  if ((t->dtype != RAI_BF16 && t->dtype != RAI_F32) || t->shape.size() < 2 || !m.bin(t, RAI_BIN_ADD, &mm, &bb)) return false;
+  rai_tensor *bias = m.strip_bc(bb);
+  rai_tensor *mn = m.node(mm, RAI_OP_MATMUL);
+  if (!mn || !vec_param(bias, t->shape.back(), t->dtype)) return false;
+  rai_tensor *x = mn->inputs[0];
+  rai_tensor *wt = m.node(mn->inputs[1], RAI_OP_TRANSPOSE);
+  if (!wt) return false;
+  const int r = (int)wt->shape.size();
+  if (!((wt->ip[0] == r - 2 && wt->ip[1] == r - 1) || (wt->ip[0] == r - 1 && wt->ip[1] == r - 2))) return false;
+  rai_tensor *w = m.strip_bc(wt->inputs[0]);
+  if (!m.ok || w->shape.size() != 2 || w->dtype != t->dtype || x->dtype != t->dtype || x->shape.size() != t->shape.size()) return false;
+  if (w->shape[0] != t->shape.back() || w->shape[1] != x->shape.back()) return false;
+  c->kind = COMP_LINEAR;
+  c->in[0] = x; c->in[1] = w; c->in[2] = bias;
+  c->interior = m.interior;
+  return true;
+}
+
+// rai-models/src/llm/phi2.rs:66-77: cat([xs_rot * cos + cat([-x2, x1]) * sin, xs_pass]) on [B, H, S, D], tables narrowed to
+// rows [offset, offset + S)
+bool match_rope(rai_tensor *t, Composite *c) {
+  Matcher m;
+  if (!norm_dtype(t->dtype) || t->shape.size() != 4) return false;
+  rai_tensor *cat = m.node(t, RAI_OP_CONCATENATE);
+  if (!cat || cat->ip[0] != 3 || cat->inputs.size() != 2) return false;
+  int64_t st = 0, len = 0, rd = 0, off_c = 0, off_s = 0, sl = 0;
+  rai_tensor *xs = m.narrow(cat->inputs[1], 3, &st, &len);          // xs_pass
+  if (!xs || xs->shape != t->shape) return false;
+  rd = st;
+  if (rd <= 0 || rd % 2 || st + len != t->shape[3]) return false;
+  rai_tensor *p1, *p2, *xr, *cb, *rh, *sb;
+  if (!m.bin(cat->inputs[0], RAI_BIN_ADD, &p1, &p2) || !m.bin(p1, RAI_BIN_MUL, &xr, &cb) || !m.bin(p2, RAI_BIN_MUL, &rh, &sb)) return false;
+  if (m.narrow(xr, 3, &st, &len) != xs || st != 0 || len != rd) return false;       // xs_rot (recorded once more below: same node)
+  rai_tensor *cosn = m.strip_bc(cb), *sinn = m.strip_bc(sb);
+  rai_tensor *cos_t = m.narrow(cosn, 0, &off_c, &sl);
+  if (!cos_t || sl != t->shape[2]) return false;
+  rai_tensor *sin_t = m.narrow(sinn, 0, &off_s, &sl);
+  if (!sin_t || sl != t->shape[2] || off_s != off_c) return false;
+  rai_tensor *rhc = m.node(rh, RAI_OP_CONCATENATE);
+  if (!rhc || rhc->ip[0] != 3 || rhc->inputs.size() != 2) return false;
+  rai_tensor *x2 = m.un(rhc->inputs[0], RAI_UN_NEG);
+  if (!x2) return false;
+  rai_tensor *a = m.narrow(x2, 3, &st, &len);
+  if (a != xr || st != rd / 2 || len != rd / 2) return false;
+  rai_tensor *b = m.narrow(rhc->inputs[1], 3, &st, &len);
+  if (b != xr || st != 0 || len != rd / 2 || !m.ok) return false;
+  if (cos_t->shape.size() != 2 || cos_t->shape[1] != rd || sin_t->shape != cos_t->shape || cos_t->dtype != t->dtype ||
+      sin_t->dtype != t->dtype)
+    return false;
+  c->kind = COMP_ROPE;
+  c->in[0] = xs; c->in[1] = cos_t; c->in[2] = sin_t;
+  c->i0 = rd; c->i1 = off_c;
+  c->interior = m.interior;
+  return true;
+}
+
+// rai-models/src/llm/phi2.rs:244-262: softmax(where(mask, -inf, q.f32 @ (k.f32.t() * scale))).to_dtype(v) @ v, then
+// transpose(1, 2) and reshape to [B, S, H * D].  The mask, when present, must be the causal one of phi2.rs:104-109.
+bool match_attention(rai_tensor *t, Composite *c) {
+  Matcher m;
+  if ((t->dtype != RAI_BF16 && t->dtype != RAI_F32 && t->dtype != RAI_F16) || t->shape.size() != 3) return false;
+  rai_tensor *rs = m.node(t, RAI_OP_RESHAPE);
+  rai_tensor *tr = rs ? m.node(rs->inputs[0], RAI_OP_TRANSPOSE) : nullptr;
+  if (!tr || tr->shape.size() != 4 || !((tr->ip[0] == 1 && tr->ip[1] == 2) || (tr->ip[0] == 2 && tr->ip[1] == 1))) return false;
+  rai_tensor *pv = m.node(tr->inputs[0], RAI_OP_MATMUL);
+  if (!pv) return false;
+  rai_tensor *v = pv->inputs[1];
+  rai_tensor *sm = m.node(m.strip_cast(pv->inputs[0], t->dtype), RAI_OP_SOFTMAX);
+  if (!sm || sm->dtype != RAI_F32 || sm->ip[0] != 3) return false;
+  rai_tensor *w = sm->inputs[0];
+  rai_tensor *mask = nullptr;
+  if (!w->evaluated && w->op == RAI_OP_WHERE) {   // inputs [on_true, on_false, cond]
+    m.interior.push_back(w);
+    double fill = 0;
+    if (!m.konst(w->inputs[0], &fill) || !(fill < 0 && std::isinf(fill))) return false;
+    mask = m.strip_bc(w->inputs[2]);
+    w = w->inputs[1];
+  }
+  rai_tensor *qk = m.node(w, RAI_OP_MATMUL);
+  if (!qk) return false;
+  rai_tensor *q = m.strip_cast(qk->inputs[0], RAI_F32);
+  rai_tensor *kt, *sc;
+  double scale = 0;
+  if (!m.bin(qk->inputs[1], RAI_BIN_MUL, &kt, &sc) || !m.konst(sc, &scale)) return false;
+  rai_tensor *ktn = m.node(kt, RAI_OP_TRANSPOSE);
+  if (!ktn || !((ktn->ip[0] == 2 && ktn->ip[1] == 3) || (ktn->ip[0] == 3 && ktn->ip[1] == 2))) return false;
+  rai_tensor *k = m.strip_cast(ktn->inputs[0], RAI_F32);
+  if (!m.ok || q->shape.size() != 4 || k->shape.size() != 4 || v->shape != k->shape) return false;
+  if (q->dtype != t->dtype || k->dtype != t->dtype || v->dtype != t->dtype) return false;
+  const int64_t B = q->shape[0], H = q->shape[1], S = q->shape[2], D = q->shape[3], T = k->shape[2];
+  if (k->shape[0] != B || k->shape[1] != H || k->shape[3] != D || t->shape[0] != B || t->shape[1] != S || t->shape[2] != H * D)
+    return false;
+  int causal = 0;
+  if (mask) {   // u8 [S, T] uploaded from the host: 1 exactly where key j lies after query i
+    if (mask->op != RAI_OP_FROM_ARRAY || mask->dtype != RAI_U8 || mask->shape.size() != 2 || mask->shape[0] != S ||
+        mask->shape[1] != T || (int64_t)mask->host.size() != S * T || S > T)
+      return false;
+    auto seen = g_causal_masks.find(mask->id);   // one mask node serves every layer: check its bytes once per eval
+    if (seen == g_causal_masks.end()) {
+      bool is_causal = true;
+      for (int64_t i = 0; i < S && is_causal; ++i)
+        for (int64_t j = 0; j < T; ++j)
+          if ((mask->host[i * T + j] != 0) != (j > i + (T - S))) { is_causal = false; break; }
+      seen = g_causal_masks.emplace(mask->id, is_causal).first;
+    }
+    if (!seen->second) return false;
+    causal = 1;
+  }
+  c->kind = COMP_ATTENTION;
+  c->in[0] = q; c->in[1] = k; c->in[2] = v;
+  c->f0 = scale;
+  c->i0 = causal;
+  c->interior = m.interior;
+  return true;
+}
+
+void plan_compositions(const std::vector<rai_tensor *> &tape, const UseInfo &ui, ComposePlan *plan) {
+  typedef bool (*match_fn)(rai_tensor *, Composite *);
+  static const match_fn kMatchers[] = {match_layer_norm, match_rms_norm, match_linear, match_rope, match_attention};
+  std::unordered_set<uint64_t> in_tape;
+  for (const rai_tensor *t : tape) in_tape.insert(t->id);
+  g_causal_masks.clear();
+  for (rai_tensor *t : tape) {
+    if (plan->absorbed.count(t->id)) continue;
+    for (match_fn f : kMatchers) {
+      Composite c = {};
+      if (!f(t, &c)) continue;
+      // interior = everything the matcher walked through except the root itself (the same node may have been
+      // reached twice)
+      std::unordered_set<uint64_t> inside;
+      std::vector<rai_tensor *> interior;
+      for (rai_tensor *n : c.interior)
+        if (n != t && inside.insert(n->id).second) interior.push_back(n);
+      bool sealed = true;
+      for (rai_tensor *n : interior) {
+        auto u = ui.users.find(n->id);
+        const size_t n_users = u == ui.users.end() ? 0 : u->second.size();
+        // evaluated constants are operands, not interior; everything else must be pending, claimed by nobody else,
+        // have a rule (fusing never hides a missing rule), and be referenced only by edges from inside
+        if (n->evaluated || !in_tape.count(n->id) || plan->absorbed.count(n->id) || plan->roots.count(n->id) ||
+            !g_rules[n->op] || (size_t)n->refs != n_users) { sealed = false; break; }
+        for (const rai_tensor *usr : u->second)
+          if (usr != t && !inside.count(usr->id)) { sealed = false; break; }
+        if (!sealed) break;
+      }
+      for (int i = 0; i < 5 && sealed; ++i)
+        if (c.in[i] && inside.count(c.in[i]->id)) sealed = false;   // an operand must be materialised
+      if (!sealed || !g_rules[t->op]) continue;
+      c.interior = interior;
+      for (rai_tensor *n : interior) plan->absorbed.insert(n->id);
+      plan->roots[t->id] = c;
+      break;
+    }
+  }
+}
+
+int run_composite(rai_tensor *t, const Composite &c) {
+  RAI_TRY(alloc_output(t));
+  switch (c.kind) {
+    case COMP_LINEAR:
+      return rai_hip_linear(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, -1, nullptr, &t->view);
+    case COMP_LAYER_NORM:
+      return rai_hip_layer_norm(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, c.f0, &t->view);
+    case COMP_RMS_NORM:
+      return rai_hip_rms_norm(t->dev, &c.in[0]->view, &c.in[1]->view, c.f0, 0, &t->view);
+    case COMP_ROPE:
+      return rai_hip_rope(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, (int32_t)c.i0, c.i1, &t->view);
+    case COMP_ATTENTION:
+      return rai_hip_attention(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, c.f0, (int32_t)c.i0, 1, &t->view);
+    default:
+      return fail(RAI_ERR_BAD_ARG, "unknown composition %d", c.kind);
+  }
+}
+
+// Node-by-node evaluation of a composition's interior (when the fused launcher declines the operands' layout).
+int eval_pending_inputs(rai_tensor *t) {
+  for (rai_tensor *in : t->inputs) {
+    if (in->evaluated) continue;
+    RAI_TRY(eval_pending_inputs(in));
+    rule_fn rule = g_rules[in->op];
+    RAI_REQUIRE(rule, RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(in->op));
+    int st = rule(in);
+    if (st != RAI_OK) { drop_storage(in); return st; }
+    in->evaluated = true;
+    ++g_stats.nodes_evaluated;
+  }
   return RAI_OK;
 }
 
@@ -929,14 +1270,37 @@ int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
   init_rules();
   std::vector<rai_tensor *> tape;
   RAI_TRY(topo_sort(outputs, n, &tape));
+  ComposePlan comp;
+  std::unordered_set<uint64_t> composed;   // roots and interiors: the elementwise pass leaves them alone
+  if (g_compose) {
+    UseInfo ui;
+    for (const rai_tensor *t : tape)
+      for (const rai_tensor *in : t->inputs) ui.users[in->id].push_back(t);
+    plan_compositions(tape, ui, &comp);
+    composed = comp.absorbed;
+    for (const auto &r : comp.roots) composed.insert(r.first);
+  }
   FusionPlan plan;
-  if (g_fusion) plan_fusion(tape, outputs, n, &plan);
+  if (g_fusion) plan_fusion(tape, outputs, n, &plan, composed);
   for (rai_tensor *t : tape) {
-    if (t->evaluated || plan.inlined.count(t->id)) continue;
+    if (t->evaluated || plan.inlined.count(t->id) || comp.absorbed.count(t->id)) continue;
     rule_fn rule = g_rules[t->op];
     RAI_REQUIRE(rule, RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op));
     int st = RAI_ERR_UNSUPPORTED;
-    if (elementwise(t) && has_inlined_input(t, plan)) {
+    auto cr = comp.roots.find(t->id);
+    if (cr != comp.roots.end()) {
+      st = run_composite(t, cr->second);
+      if (st == RAI_OK) {
+        ++g_stats.kernel_launches;
+        ++g_stats.composed_regions;
+        g_stats.composed_nodes += cr->second.interior.size() + 1;
+      } else if (st == RAI_ERR_BAD_STRIDE || st == RAI_ERR_UNSUPPORTED || st == RAI_ERR_BAD_SHAPE || st == RAI_ERR_BAD_DTYPE) {
+        // the fused launcher declines these operands: evaluate the recorded nodes one by one instead
+        drop_storage(t);
+        st = eval_pending_inputs(t);
+        if (st == RAI_OK) st = rule(t);
+      }
+    } else if (elementwise(t) && has_inlined_input(t, plan)) {
       // the rules of the inlined members must exist too: fusion never hides a missing rule
       st = eval_region(t, plan);
       if (st == RAI_ERR_UNSUPPORTED) {  // region too large for one program: evaluate its members one by one
@@ -1009,6 +1373,10 @@ int32_t rai_dispatch_has_rule(int32_t op_kind) {
 }
 
 // ------------------------------------------------------------------ fusion control and counters
+int rai_graph_set_compose(int32_t enabled) {
+  g_compose = enabled != 0;
+  return RAI_OK;
+}
 int rai_graph_set_fusion(int32_t enabled) {
   g_fusion = enabled != 0;
   return RAI_OK;

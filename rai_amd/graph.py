@@ -320,11 +320,18 @@ def set_fusion(enabled):
     check(_lib.load().rai_graph_set_fusion(int(bool(enabled))))
 
 
+def set_compose(enabled):
+    """Composition pass on / off: Linear + bias, LayerNorm, RmsNorm, rotary embedding and the attention block as one
+    fused launch each (tolerance-level agreement with node-by-node evaluation)."""
+    check(_lib.load().rai_graph_set_compose(int(bool(enabled))))
+
+
 def stats(reset=False):
     s = GraphStats()
     check(_lib.load().rai_graph_get_stats(C.byref(s), int(reset)))
     return {"nodes_evaluated": s.nodes_evaluated, "kernel_launches": s.kernel_launches,
-            "fused_regions": s.fused_regions, "fused_nodes": s.fused_nodes}
+            "fused_regions": s.fused_regions, "fused_nodes": s.fused_nodes,
+            "composed_regions": s.composed_regions, "composed_nodes": s.composed_nodes}
 
 
 def dispatch_unregister(op):

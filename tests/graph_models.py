@@ -13,8 +13,8 @@ import math
 
 import numpy as np
 
-from . import graph as g
-from .graph import Tensor, cat
+from rai_amd import graph as g
+from rai_amd.graph import Tensor, cat
 
 
 class Phi2Graph:

@@ -22,13 +22,17 @@ def rand(rng, shape, dt, scale=1.0):
     return rnd(rng.standard_normal(shape).astype(np.float32) * scale, dt)
 
 
-def run(build, fusion):
+def run(build, fusion, compose=False):
+    """Builds and evaluates with the elementwise pass on/off; the composition pass is off unless asked for, so that
+    the bit-identity checks of the elementwise pass compare like with like."""
     g.set_fusion(fusion)
+    g.set_compose(compose)
     g.stats(reset=True)
     out = build()
     storage = out.as_storage()
     st = g.stats()
     g.set_fusion(True)
+    g.set_compose(True)
     return storage, st, out
 
 
@@ -186,7 +190,7 @@ def test_phi2_through_the_graph_matches_oracle(hip, dt):
     # the model code of phi2.rs recorded as a lazy graph and evaluated node by node on the
     # device (the reference's own execution scheme), prefill then two cached decode steps
     from oracle import phi2
-    from rai_amd.graph_models import Phi2Graph
+    from tests.graph_models import Phi2Graph
     cfg = phi2.Config(vocab_size=300, hidden_size=128, intermediate_size=256, num_hidden_layers=2,
                       num_attention_heads=4, max_position_embeddings=64)
     params = phi2.random_params(cfg, dt, seed=0)
@@ -201,6 +205,9 @@ def test_phi2_through_the_graph_matches_oracle(hip, dt):
         assert_close(got, want, dt, f"graph phi2 step {step}")
         st = g.stats()
         assert st["fused_regions"] > 0 and st["kernel_launches"] < st["nodes_evaluated"]
+        # the composition pass (on by default) takes every module of the two layers and the head: per layer one
+        # LayerNorm, six Linears with bias, two rotary embeddings and one attention block
+        assert st["composed_regions"] == 2 * 10 + 2, st
         ids = np.argmax(want, -1).astype(np.uint32).reshape(2, 1)
     # greedy ids through the graph: argmax node, u32, bit-exact against the oracle on the same logits
     tok = logits.argmax(-1).as_storage()[:, 0]
@@ -229,3 +236,91 @@ def test_gather_index_add_scatter_add_nodes(hip):
     assert np.array_equal(got, oo.scatter_add(x, 0, ix, upd, "f32"))
     with pytest.raises(Exception):
         dev(x, "f32").gather(1, Tensor.from_array(ix, "u32")).as_storage()   # Err node surfaces at eval
+
+
+# ------------------------------------------------------------------ composition pass
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_compositions_are_taken_by_one_launch_each(hip, dt):
+    rng = np.random.default_rng(7)
+    x, w, b = rand(rng, (4, 21, 96), dt), rand(rng, (96,), dt), rand(rng, (96,), dt)
+    wl, bl = rand(rng, (40, 96), dt, 0.2), rand(rng, (40,), dt)
+    cases = {
+        "layer_norm": (lambda: g.layer_norm(dev(x, dt), dev(w, dt), dev(b, dt), 1e-5), onn.layer_norm(x, w, b, 1e-5, dt)),
+        "rms_norm": (lambda: g.rms_norm(dev(x, dt), dev(w, dt), 1e-6), onn.rms_norm(x, w, 1e-6, dt)),
+        "linear": (lambda: g.linear(dev(x, dt), dev(wl, dt), dev(bl, dt)), onn.linear(x, wl, bl, dt)),
+    }
+    for name, (build, want) in cases.items():
+        composed, st_c, _ = run(build, True, compose=True)
+        plain, st_p, _ = run(build, True, compose=False)
+        assert st_c["composed_regions"] == 1 and st_c["kernel_launches"] == 1, (name, st_c)
+        assert st_p["composed_regions"] == 0 and st_p["kernel_launches"] > 1, (name, st_p)
+        assert_close(from_storage(composed, dt), want, dt, f"{name} composed")
+        assert_close(from_storage(plain, dt), want, dt, f"{name} node by node")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_rotary_and_attention_compositions(hip, dt):
+    from oracle import phi2
+    from tests.graph_models import Phi2Graph
+    cfg = phi2.Config(vocab_size=50, hidden_size=160, intermediate_size=64, num_hidden_layers=1, num_attention_heads=2,
+                      max_position_embeddings=64)
+    model = Phi2Graph(cfg, {}, dt)
+    rng = np.random.default_rng(8)
+    xs = rand(rng, (2, 2, 9, 80), dt)
+    sin, cos = phi2.rotary_tables(cfg, dt)
+    g.eval_all([model.sin, model.cos])          # the tables are shared state of the model, built once
+    for offset in (0, 13):
+        build = lambda: model._rotary(dev(xs, dt), offset)
+        composed, st_c, _ = run(build, True, compose=True)
+        plain, st_p, _ = run(build, True, compose=False)
+        assert st_c["composed_regions"] == 1 and st_p["composed_regions"] == 0
+        assert st_c["kernel_launches"] < st_p["kernel_launches"]
+        want = phi2.rotary(xs, sin, cos, cfg.rotary_dim, offset, dt)
+        assert_close(from_storage(composed, dt), want, dt, "rotary composed")
+        assert np.array_equal(composed, plain), "the rotary launcher rounds where the node chain rounds"
+    # the attention block of phi2.rs:244-262 with the causal mask, and without one on a longer key range (decode)
+    B, H, D = 2, 3, 80
+    for S, T, causal in ((9, 9, True), (1, 30, False)):
+        q, k, v = rand(rng, (B, H, S, D), dt), rand(rng, (B, H, T, D), dt), rand(rng, (B, H, T, D), dt)
+
+        def build():
+            w = dev(q, dt).to_dtype("f32").matmul(dev(k, dt).to_dtype("f32").t() * (1.0 / np.sqrt(D)))
+            if causal:
+                m = Tensor.from_array(np.triu(np.ones((S, T), np.uint8), 1), "u8").broadcast_to(w.shape)
+                w = m.where_cond(w.full_like(float("-inf")), w)
+            return w.softmax(-1).to_dtype(dt).matmul(dev(v, dt)).transpose(1, 2).reshape((B, S, H * D))
+
+        composed, st_c, _ = run(build, True, compose=True)
+        plain, st_p, _ = run(build, True, compose=False)
+        assert st_c["composed_regions"] == 1 and st_c["kernel_launches"] == 1, st_c
+        assert st_p["kernel_launches"] >= 4
+        assert_close(from_storage(composed, dt), from_storage(plain, dt), dt, "attention composed vs node by node")
+    # a mask that is not the causal one must not be taken for it
+    S = T = 9
+    q, k, v = (rand(rng, (B, H, S, D), dt) for _ in range(3))
+    odd = np.triu(np.ones((S, T), np.uint8), 2)
+
+    def build_odd():
+        w = dev(q, dt).to_dtype("f32").matmul(dev(k, dt).to_dtype("f32").t() * 0.1)
+        w = Tensor.from_array(odd, "u8").broadcast_to(w.shape).where_cond(w.full_like(float("-inf")), w)
+        return w.softmax(-1).to_dtype(dt).matmul(dev(v, dt)).transpose(1, 2).reshape((B, S, H * D))
+
+    _, st, _ = run(build_odd, True, compose=True)
+    assert st["composed_regions"] == 0
+
+
+def test_composition_is_not_taken_when_an_interior_node_is_observable(hip):
+    rng = np.random.default_rng(9)
+    x, w, b = rand(rng, (5, 64), "f32"), rand(rng, (64,), "f32"), rand(rng, (64,), "f32")
+    xd = dev(x, "f32")
+    mean = xd.mean(-1, True)                       # the caller keeps the mean: LayerNorm below recomputes its own,
+    var = xd.var(-1, True)                         # but this variance node is the one the norm uses
+    xs = (xd - mean) * (var + 1e-5).rsqrt()
+    y = dev(w, "f32") * xs + dev(b, "f32")
+    g.set_compose(True)
+    g.stats(reset=True)
+    got = y.as_storage()
+    st = g.stats()
+    assert st["composed_regions"] == 0             # `mean`, `var`, `xs` are held outside the graph
+    assert_close(got, onn.layer_norm(x, w, b, 1e-5, "f32"), "f32")
+    assert_close(var.as_storage(), onn.var(x, -1, True, "f32"), "f32", "the held node is still evaluated")
