@@ -335,6 +335,57 @@ def run_ops(args):
           {"ops": rows})
 
 
+def run_phi2_graph(args, n_new=16):
+    """The drop-in path: Phi-2 recorded node for node through the lazy-graph API the way rai-models/src/llm/phi2.rs
+    builds it (tests/graph_models.py, KV cache by concatenation) and evaluated by the C++ evaluator with its
+    composition and elementwise passes.  Greedy decode, batch 1, 512-token prompt; the time per token includes
+    recording the graph from Python (ctypes), which a Rust front end would do far faster."""
+    from oracle.phi2 import Config, param_shapes
+    from rai_amd import graph as g, synthetic
+    from rai_amd.graph import Tensor
+    from tests.graph_models import Phi2Graph
+    cfg = Config(num_hidden_layers=args.layers)
+    params = {}
+    for name, shape in param_shapes(cfg).items():
+        a = synthetic.to_storage(synthetic.tensor(name, int(np.prod(shape)), 0, 0.02), "bf16").reshape(shape)
+        params[name] = Tensor.from_array(a, "bf16")
+    g.eval_all(list(params.values()))
+    model = Phi2Graph(cfg, params, "bf16")
+    prompt = synthetic.prompt(cfg.vocab_size, 1, PROMPT, seed=1)
+    out = {}
+    for label, compose in (("composed", True), ("node_by_node", False)):
+        g.set_compose(compose)
+        model.clear_kv_cache()
+        ids = prompt
+        toks, t_rec, t_eval, launches, nodes = [], 0.0, 0.0, 0, 0
+        steps = n_new if compose else min(n_new, 4)
+        for step in range(steps + 1):
+            g.stats(reset=True)
+            t0 = time.perf_counter()
+            nxt = model.fwd(Tensor.from_array(ids, "u32")).argmax(-1)
+            t1 = time.perf_counter()
+            tok = nxt.as_storage().reshape(-1)
+            t2 = time.perf_counter()
+            st = g.stats()
+            if step == 0:
+                out[f"{label}_prefill_ms"] = round((t2 - t0) * 1e3, 2)
+            else:
+                t_rec += t1 - t0
+                t_eval += t2 - t1
+                launches += st["kernel_launches"]
+                nodes += st["nodes_evaluated"] + st["fused_nodes"] + st["composed_nodes"]
+            toks.append(int(tok[0]))
+            ids = tok.reshape(1, 1).astype(np.uint32)
+        out[f"{label}_decode_tokens_per_s"] = round(steps / (t_rec + t_eval), 2)
+        out[f"{label}_record_ms_per_token"] = round(t_rec / steps * 1e3, 3)
+        out[f"{label}_eval_ms_per_token"] = round(t_eval / steps * 1e3, 3)
+        out[f"{label}_launches_per_token"] = round(launches / steps, 1)
+        out[f"{label}_first_tokens"] = toks[:8]
+    g.set_compose(True)
+    out["recorded_nodes_per_token"] = round(nodes / steps, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -346,6 +397,8 @@ def main():
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     ap.add_argument("--layers", type=int, default=PHI2["num_hidden_layers"],
                     help="debug only: fewer layers (the JSON line then says so and is not the headline workload)")
+    ap.add_argument("--graph-tokens", type=int, default=16,
+                    help="tokens decoded through the lazy-graph path for the graph_decode_* fields (0: skip)")
     ap.add_argument("--workload", default="phi2-decode", choices=["phi2-decode", "qwen2-prefill", "gemma-decode", "ops"],
                     help="phi2-decode is the headline line; the others are the remaining configurations of the path")
     args = ap.parse_args()
@@ -451,6 +504,9 @@ def main():
         for _ in range(3):
             _lib.call("rai_hip_copy", 0, C.byref(src.desc()), C.byref(dst.desc()))
         sync()
+    if args.graph_tokens > 0:
+        out["graph_path"] = run_phi2_graph(args, args.graph_tokens)
+        out["graph_decode_tokens_per_s"] = out["graph_path"]["composed_decode_tokens_per_s"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)

@@ -358,6 +358,11 @@ typedef struct rai_hip_decoder_config {
    * (phi2.rs:53-57: positions and pos*inv_freq rounded to bf16 for a bf16
    * model); 1: angles computed in f32 and rounded once. */
   int32_t rope_tables_f32;
+  /* Phi-2's optional LayerNorm of the query / key projections (phi2.rs:207-216).  The reference applies a
+   * LayerNorm over head_dim elements to the un-split [.., heads * head_dim] projection, a graph that is only
+   * well-formed for a single head; the drivers do not implement it: non-zero -> RAI_ERR_UNSUPPORTED.  (The lazy-graph
+   * evaluator of rai_graph.h runs such a model node by node, Err node included, as the reference would.) */
+  int32_t qk_layernorm;
   double rope_theta;
   double norm_eps;
 } rai_hip_decoder_config;
@@ -388,6 +393,9 @@ int rai_hip_decoder_dtype(rai_hip_decoder *dec, int32_t *dtype);
 /* Number of parameter names the architecture expects / i-th name (for loaders). */
 int rai_hip_decoder_param_count(rai_hip_decoder *dec, int32_t *count);
 int rai_hip_decoder_param_name(rai_hip_decoder *dec, int32_t i, char *buf, size_t buflen, int64_t *numel);
+/* The logical shape of parameter i: a matrix [rows, cols] as the reference's module holds it (Linear: [out, in]),
+ * a vector as rows == 1.  The safetensors loader requires the file's tensor to have exactly this shape. */
+int rai_hip_decoder_param_shape(rai_hip_decoder *dec, int32_t i, int64_t *rows, int64_t *cols);
 /* Model::fwd (phi2.rs:334-347): ids_host[batch*seq] u32 are appended after the
  * cached context; returns last-position logits [batch, vocab] as f32 in
  * logits_host (nullable) and greedy tokens (device argmax, first-max) in

@@ -114,6 +114,13 @@ impl Decoder {
             .collect()
     }
 
+    /// `[rows, cols]` of parameter `i` (a vector has one row).
+    pub fn param_shape(&self, i: i32) -> (i64, i64) {
+        let (mut r, mut c) = (0i64, 0i64);
+        check(unsafe { rai_hip_decoder_param_shape(self.h, i, &mut r, &mut c) });
+        (r, c)
+    }
+
     /// One parameter from host bytes in the model dtype's storage form, e.g. in a loop over
     /// `model.named_params()` with `safetensors::View::data(&tensor)`.
     pub fn load_param(&self, name: &str, bytes: &[u8]) {

@@ -56,6 +56,10 @@ def param_shapes(cfg):
         out[p + "self_attn.v_proj.bias"] = (kv,)
         out[p + "self_attn.dense.weight"] = (h, h)
         out[p + "self_attn.dense.bias"] = (h,)
+        if cfg.qk_layernorm:   # phi2.rs:163-169: LayerNorm::new(head_dim, ..)
+            for n in ("q_layernorm", "k_layernorm"):
+                out[p + f"self_attn.{n}.weight"] = (cfg.head_dim,)
+                out[p + f"self_attn.{n}.bias"] = (cfg.head_dim,)
         out[p + "mlp.fc1.weight"] = (i, h)
         out[p + "mlp.fc1.bias"] = (i,)
         out[p + "mlp.fc2.weight"] = (h, i)
@@ -123,6 +127,14 @@ class Model:
         q = nn.linear(xs, p[pre + "q_proj.weight"], p[pre + "q_proj.bias"], dt)
         k = nn.linear(xs, p[pre + "k_proj.weight"], p[pre + "k_proj.bias"], dt)
         v = nn.linear(xs, p[pre + "v_proj.weight"], p[pre + "v_proj.bias"], dt)
+        if cfg.qk_layernorm:
+            # phi2.rs:207-216 applies the LayerNorm (parameters of head_dim elements) to the projections BEFORE they
+            # are split into heads, i.e. over a last dim of heads * head_dim: broadcasting the [head_dim] weight against
+            # it is an IncompatibleShape error node unless there is a single head.  Restated as is.
+            if nh * hd != hd or nkv * hd != hd:
+                raise ValueError(f"IncompatibleShape {{ lhs: [{hd}], rhs: [{b}, {s}, {nh * hd}] }}")
+            q = nn.layer_norm(q, p[pre + "q_layernorm.weight"], p[pre + "q_layernorm.bias"], cfg.layer_norm_eps, dt)
+            k = nn.layer_norm(k, p[pre + "k_layernorm.weight"], p[pre + "k_layernorm.bias"], cfg.layer_norm_eps, dt)
         q = q.reshape(b, s, nh, hd).transpose(0, 2, 1, 3)
         k = k.reshape(b, s, nkv, hd).transpose(0, 2, 1, 3)
         v = v.reshape(b, s, nkv, hd).transpose(0, 2, 1, 3)

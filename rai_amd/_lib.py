@@ -60,6 +60,7 @@ class DecoderConfig(C.Structure):
         ("max_batch", C.c_int32),
         ("max_context", C.c_int32),
         ("rope_tables_f32", C.c_int32),
+        ("qk_layernorm", C.c_int32),
         ("rope_theta", C.c_double),
         ("norm_eps", C.c_double),
     ]
@@ -124,6 +125,7 @@ PROTOTYPES = {
     "rai_hip_decoder_dtype": [_vp, C.POINTER(_i32)],
     "rai_hip_decoder_param_count": [_vp, C.POINTER(_i32)],
     "rai_hip_decoder_param_name": [_vp, _i32, C.c_char_p, C.c_size_t, C.POINTER(_i64)],
+    "rai_hip_decoder_param_shape": [_vp, _i32, C.POINTER(_i64), C.POINTER(_i64)],
     "rai_hip_decoder_forward": [_vp, C.POINTER(C.c_uint32), _i32, _i32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)],
     "rai_hip_decoder_generate": [_vp, C.POINTER(C.c_uint32), _i32, _i32, _i32, C.POINTER(C.c_uint32),
                                  C.POINTER(C.c_float), C.POINTER(C.c_float)],

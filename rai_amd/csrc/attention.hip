@@ -742,7 +742,7 @@ template <int D> static int launch_decode_mfma(hipStream_t st, const AttnDecodeA
 // The MFMA kernel serves bf16 grouped-query shapes whose longest context fits
 // kDecodeMaxSplits blocks of kMfmaDecodeKeysMax keys.
 static bool decode_mfma_eligible(const AttnDecodeArgs &a) {
-  static const bool off = getenv("RAI_HIP_NO_MFMA_DECODE") != nullptr;
+  const bool off = getenv("RAI_HIP_NO_MFMA_DECODE") != nullptr;   // per call: a test compares both kernels in one process
   const int rep = a.Hq / a.Hkv;
   return !off && a.dtype == RAI_BF16 && rep >= 4 && rep <= 16 && (a.D == 64 || a.D == 128 || a.D == 256) &&
          (a.Tmax + kMfmaDecodeKeysMax - 1) / kMfmaDecodeKeysMax <= kDecodeMaxSplits;

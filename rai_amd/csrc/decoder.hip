@@ -1173,6 +1173,8 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   RAI_REQUIRE(cfg->hidden_act == RAI_UN_NEW_GELU || cfg->hidden_act == RAI_UN_GELU || cfg->hidden_act == RAI_UN_SILU ||
                   cfg->hidden_act == RAI_UN_RELU,
               RAI_ERR_BAD_ARG, "decoder_create: hidden_act %d", cfg->hidden_act);
+  RAI_REQUIRE(!cfg->qk_layernorm, RAI_ERR_UNSUPPORTED,
+              "decoder_create: qk_layernorm (rai-models/src/llm/phi2.rs:207-216) is not implemented by the decoder drivers");
   if (!ctx(dev)) return RAI_ERR_HIP;
   rai_hip_decoder *d = new rai_hip_decoder();
   d->dev = dev;
@@ -1303,6 +1305,14 @@ int rai_hip_decoder_param_name(rai_hip_decoder *d, int32_t i, char *buf, size_t 
   RAI_REQUIRE(i >= 0 && i < (int32_t)d->slots.size(), RAI_ERR_BAD_ARG, "parameter index %d out of range", i);
   snprintf(buf, buflen, "%s", d->slots[i].name.c_str());
   if (numel) *numel = d->slots[i].rows * d->slots[i].cols;
+  return RAI_OK;
+}
+
+int rai_hip_decoder_param_shape(rai_hip_decoder *d, int32_t i, int64_t *rows, int64_t *cols) {
+  RAI_REQUIRE(d && rows && cols, RAI_ERR_BAD_ARG, "null argument");
+  RAI_REQUIRE(i >= 0 && i < (int32_t)d->slots.size(), RAI_ERR_BAD_ARG, "parameter index %d out of range", i);
+  *rows = d->slots[i].rows;
+  *cols = d->slots[i].cols;
   return RAI_OK;
 }
 

@@ -1103,8 +1103,9 @@ template <int MT, int KS> static int launch_mfma_stream(hipStream_t st, const Li
 
 // True when the small-M streaming kernel can apply the RMSNorm of the activation rows itself.
 bool linear_mfma_fuses_norm(int M, int K, int ln_kind) {
-  static const bool off = getenv("RAI_HIP_NO_MFMA_STREAM") != nullptr || getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr ||
-                          getenv("RAI_HIP_NO_FUSED_NORM") != nullptr;
+  // read per call (three getenv are nothing next to a launch): tests force the fallback kernels within one process
+  const bool off = getenv("RAI_HIP_NO_MFMA_STREAM") != nullptr || getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr ||
+                   getenv("RAI_HIP_NO_FUSED_NORM") != nullptr;
   if (off || (ln_kind != 1 && ln_kind != 2) || M <= 8 || M > 64 || K % 32) return false;
   return K <= (M <= 32 ? 8 * 8 * 32 : 8 * 4 * 32);   // one block's K span: no split over blocks
 }
@@ -1163,8 +1164,8 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.K % 32 == 0, RAI_ERR_UNSUPPORTED, "linear mfma: K=%d must be a multiple of 32", a.K);
   RAI_REQUIRE(a.lda % 8 == 0 && a.ldw % 8 == 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0,
               RAI_ERR_BAD_STRIDE, "linear mfma: operands must be 16-byte aligned with row strides multiple of 8");
-  static const bool no_skinny = getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr;
-  static const bool no_stream = getenv("RAI_HIP_NO_MFMA_STREAM") != nullptr;
+  const bool no_skinny = getenv("RAI_HIP_NO_MFMA_SKINNY") != nullptr;
+  const bool no_stream = getenv("RAI_HIP_NO_MFMA_STREAM") != nullptr;
   if (a.M <= 64 && !no_skinny && !no_stream) {
     int splits = 1;
     if (a.M <= 16 && mfma_stream_fits<1, 8>(a, &splits)) return launch_mfma_stream<1, 8>(st, a, splits);

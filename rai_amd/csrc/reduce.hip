@@ -235,7 +235,7 @@ template <typename C, bool IS_MAX> __device__ __forceinline__ bool better(C bv, 
 template <typename T, bool IS_MAX>
 __global__ void __launch_bounds__(256)
 k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int64_t axis_stride, int splits,
-                  float *pval_f, double *pval_d, uint32_t *pidx) {
+                  float *pval_f, double *pval_d, uint32_t *pidx, uint32_t *counters, uint32_t *out) {
   typedef typename Scalar<T>::compute C;
   __shared__ C shv[4];
   __shared__ uint32_t shi[4];
@@ -299,8 +299,36 @@ k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int6
   if (threadIdx.x == 0) {
     for (int w = 1; w < 4; ++w)
       if (better<C, IS_MAX>(shv[w], shi[w], bv, bi)) { bv = shv[w]; bi = shi[w]; }
-    if (sizeof(C) == 8) pval_d[blockIdx.x] = (double)bv; else pval_f[blockIdx.x] = (float)bv;
-    pidx[blockIdx.x] = bi;
+    if (!out) {   // two-launch form: k_arg_row_final merges
+      if (sizeof(C) == 8) pval_d[blockIdx.x] = (double)bv; else pval_f[blockIdx.x] = (float)bv;
+      pidx[blockIdx.x] = bi;
+      return;
+    }
+    // One-launch form: the block of a row that arrives last merges the row's partial results.  They cross blocks
+    // (and XCDs, whose L2s are not coherent for ordinary accesses) as device-scope relaxed atomics, which write
+    // through / read around the L2; the arrival counter is bumped only after this block's stores have completed,
+    // and the last block sets it back to zero for the next call.
+    if (splits > 1) {
+      if (sizeof(C) == 8) __hip_atomic_store(&pval_d[blockIdx.x], (double)bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_store(&pval_f[blockIdx.x], (float)bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&pidx[blockIdx.x], bi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (atomicAdd(&counters[row], 1u) != (uint32_t)splits - 1u) return;
+      const int64_t base = row * splits;
+      for (int sp = 0; sp < splits; ++sp) {
+        C v;
+        if (sizeof(C) == 8) v = (C)__hip_atomic_load(&pval_d[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else v = (C)__hip_atomic_load(&pval_f[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t i = __hip_atomic_load(&pidx[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (sp == 0) { bv = v; bi = i; }
+        else if (better<C, IS_MAX>(v, i, bv, bi)) { bv = v; bi = i; }
+      }
+      __hip_atomic_store(&counters[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // all-NaN row: every candidate is NaN and index 0 wins already; a NaN at element 0 wins in the reference's
+    // sequential scan even with finite values elsewhere
+    const C first = Scalar<T>::load(x);
+    out[row] = (bi == 0xffffffffu || first != first) ? 0u : bi;
   }
 }
 
@@ -470,7 +498,9 @@ template <bool LOG> static int softmax_impl(int dev, const rai_hip_tensor *in, i
 // workspace.  Every GPU holds its own copy at its own address; the address is looked up once per device when the
 // device context is created (arg_static_scratch_init) and only that pointer is ever handed to kernels.
 static constexpr size_t kArgStaticParts = 65536;   // (row, split) partial results one call may produce
-static constexpr size_t kArgStaticBytes = kArgStaticParts * (sizeof(double) + sizeof(uint32_t)) + 64;
+// values (8 bytes, f64 rows), indices and one arrival counter per row; the counters start at zero (the array is
+// zero-initialised when the code object is loaded) and every call leaves them at zero
+static constexpr size_t kArgStaticBytes = kArgStaticParts * (sizeof(double) + 2 * sizeof(uint32_t));
 static __device__ __align__(256) unsigned char scratch[kArgStaticBytes];
 static void *g_scratch_ptr[16] = {nullptr};
 
@@ -512,21 +542,31 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
     while (rows * splits < 2 * kNumCU && n / (splits * 2) >= 2048) splits *= 2;
     void *ws = nullptr;
     size_t nparts = (size_t)rows * splits;
-    if (no_alloc) {
+    if (no_alloc)
       RAI_REQUIRE(nparts <= kArgStaticParts, RAI_ERR_UNSUPPORTED,
                   "argmax_static: %lld rows x %d splits = %zu partial results, the static scratch holds %zu",
                   (long long)rows, splits, nparts, kArgStaticParts);
+    if (nparts <= kArgStaticParts && dev >= 0 && dev < 16 && g_scratch_ptr[dev]) {
+      // one launch: partial results and arrival counters in the fixed device array, the last block of a row merges
       ws = g_scratch_ptr[dev];
-      RAI_REQUIRE(ws, RAI_ERR_HIP, "argmax_static: scratch address of device %d unknown (rai_hip_init failed?)", dev);
-    } else {
-      RAI_TRY(workspace(dev, nparts * (sizeof(double) + sizeof(uint32_t)) + 64, &ws));
+      double *pd = (double *)ws;
+      uint32_t *pi = (uint32_t *)((char *)ws + kArgStaticParts * sizeof(double));
+      uint32_t *cnt = pi + kArgStaticParts;
+      RAI_DISPATCH_FLOAT(in->dtype, T,
+                         hipLaunchKernelGGL((k_arg_row_partial<T, IS_MAX>), dim3((unsigned)nparts), dim3(256), 0, st,
+                                            (const T *)base_ptr(in), rows, n, row_stride, ax, splits, (float *)ws, pd, pi,
+                                            cnt, o));
+      return launch_check("arg_row");
     }
+    RAI_REQUIRE(!no_alloc, RAI_ERR_HIP, "argmax_static: scratch address of device %d unknown (rai_hip_init failed?)", dev);
+    RAI_TRY(workspace(dev, nparts * (sizeof(double) + sizeof(uint32_t)) + 64, &ws));
     double *pd = (double *)ws;
     float *pf = (float *)ws;
     uint32_t *pi = (uint32_t *)((char *)ws + nparts * sizeof(double));
     RAI_DISPATCH_FLOAT(in->dtype, T,
                        hipLaunchKernelGGL((k_arg_row_partial<T, IS_MAX>), dim3((unsigned)nparts), dim3(256), 0, st,
-                                          (const T *)base_ptr(in), rows, n, row_stride, ax, splits, pf, pd, pi));
+                                          (const T *)base_ptr(in), rows, n, row_stride, ax, splits, pf, pd, pi,
+                                          (uint32_t *)nullptr, (uint32_t *)nullptr));
     RAI_TRY(launch_check("arg_partial"));
     int fgrid = (int)((rows + 63) / 64);
     if (in->dtype == RAI_F64)

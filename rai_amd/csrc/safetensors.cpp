@@ -224,6 +224,7 @@ int map_file(const char *path, MappedFile *f) {
 
 struct StTensor {
   std::string dtype;
+  std::vector<int64_t> shape;
   int64_t numel = 0;
   const uint8_t *bytes = nullptr;
   size_t nbytes = 0;
@@ -261,9 +262,16 @@ int index_file(const char *path, const MappedFile &f, std::map<std::string, StTe
     st.dtype = dt->str;
     st.numel = 1;
     for (auto &d : sh->arr) {
-      RAI_REQUIRE(d.kind == JsonValue::Number && d.num >= 0 && d.num == std::floor(d.num), RAI_ERR_IO,
-                  "safetensors: '%s': bad shape for tensor '%s'", path, kv.first.c_str());
-      st.numel *= (int64_t)d.num;
+      // an untrusted header: every extent must be an integer a double holds exactly, and the element count must
+      // stay inside the file (which also keeps the product far from overflow)
+      RAI_REQUIRE(d.kind == JsonValue::Number && d.num >= 0 && d.num == std::floor(d.num) && d.num <= 9007199254740992.0,
+                  RAI_ERR_IO, "safetensors: '%s': bad shape for tensor '%s'", path, kv.first.c_str());
+      const int64_t ext = (int64_t)d.num;
+      RAI_REQUIRE(ext == 0 || st.numel <= (int64_t)f.size / ext, RAI_ERR_IO,
+                  "safetensors: '%s': shape of tensor '%s' describes more elements than the file has bytes", path,
+                  kv.first.c_str());
+      st.numel *= ext;
+      st.shape.push_back(ext);
     }
     const double b = off->arr[0].num, e = off->arr[1].num;
     RAI_REQUIRE(off->arr[0].kind == JsonValue::Number && off->arr[1].kind == JsonValue::Number && b >= 0 && e >= b &&
@@ -374,6 +382,14 @@ int rai_hip_decoder_load_safetensors(rai_hip_decoder *dec, const char *const *pa
     const StTensor &t = it->second;
     RAI_REQUIRE(t.numel == numel, RAI_ERR_BAD_SHAPE, "load_safetensors: parameter '%s' has %lld elements, '%s' holds %lld",
                 name, (long long)numel, t.file.c_str(), (long long)t.numel);
+    // the same element count is not enough: a transposed or flattened matrix would load and give wrong logits
+    int64_t rows = 0, cols = 0;
+    RAI_TRY(rai_hip_decoder_param_shape(dec, i, &rows, &cols));
+    const bool vec_ok = rows == 1 && t.shape.size() == 1 && t.shape[0] == cols;
+    const bool mat_ok = t.shape.size() == 2 && t.shape[0] == rows && t.shape[1] == cols;
+    RAI_REQUIRE(vec_ok || mat_ok, RAI_ERR_BAD_SHAPE, "load_safetensors: parameter '%s' is [%lld, %lld], '%s' holds rank %zu [%lld%s",
+                name, (long long)rows, (long long)cols, t.file.c_str(), t.shape.size(),
+                (long long)(t.shape.empty() ? 0 : t.shape[0]), t.shape.size() > 1 ? ", ..]" : "]");
     const bool same = (dtype == RAI_BF16 && t.dtype == "BF16") || (dtype == RAI_F32 && t.dtype == "F32");
     if (same) {
       RAI_TRY(rai_hip_decoder_load_param(dec, name, t.bytes, t.nbytes));

@@ -20,7 +20,8 @@ class Decoder:
     def __init__(self, arch, dtype, *, vocab_size, hidden_size, intermediate_size, num_hidden_layers,
                  num_attention_heads, num_key_value_heads=None, head_dim=None, rotary_dim=None,
                  max_position_embeddings=2048, hidden_act="gelu_new", tie_word_embeddings=False, rope_theta=10000.0,
-                 norm_eps=1e-5, max_batch=1, max_context=None, rope_tables_f32=False, dev=0):
+                 norm_eps=1e-5, max_batch=1, max_context=None, rope_tables_f32=False, qk_layernorm=False,
+                 dev=0):
         head_dim = head_dim or hidden_size // num_attention_heads
         cfg = DecoderConfig()
         cfg.arch = ARCH[arch]
@@ -39,6 +40,7 @@ class Decoder:
         cfg.max_batch = max_batch
         cfg.max_context = max_context or max_position_embeddings
         cfg.rope_tables_f32 = int(rope_tables_f32)
+        cfg.qk_layernorm = int(qk_layernorm)
         cfg.rope_theta = rope_theta
         cfg.norm_eps = norm_eps
         self.cfg, self.dtype, self.dev = cfg, dtype, dev

@@ -56,8 +56,12 @@ class Phi2Graph:
         pre = f"model.layers.{l}.self_attn."
         b, s, _ = xs.shape
         nh, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
-        q = self._linear(xs, pre + "q_proj").reshape((b, s, nh, hd)).transpose(1, 2)
-        k = self._linear(xs, pre + "k_proj").reshape((b, s, nkv, hd)).transpose(1, 2)
+        q, k = self._linear(xs, pre + "q_proj"), self._linear(xs, pre + "k_proj")
+        if getattr(cfg, "qk_layernorm", False):   # phi2.rs:207-216: on the un-split projections
+            q = g.layer_norm(q, self.p[pre + "q_layernorm.weight"], self.p[pre + "q_layernorm.bias"], cfg.layer_norm_eps)
+            k = g.layer_norm(k, self.p[pre + "k_layernorm.weight"], self.p[pre + "k_layernorm.bias"], cfg.layer_norm_eps)
+        q = q.reshape((b, s, nh, hd)).transpose(1, 2)
+        k = k.reshape((b, s, nkv, hd)).transpose(1, 2)
         v = self._linear(xs, pre + "v_proj").reshape((b, s, nkv, hd)).transpose(1, 2)
         offset = 0 if self.kv[l] is None else self.kv[l][0].shape[2]
         q, k = self._rotary(q, offset), self._rotary(k, offset)

@@ -324,3 +324,38 @@ def test_composition_is_not_taken_when_an_interior_node_is_observable(hip):
     assert st["composed_regions"] == 0             # `mean`, `var`, `xs` are held outside the graph
     assert_close(got, onn.layer_norm(x, w, b, 1e-5, "f32"), "f32")
     assert_close(var.as_storage(), onn.var(x, -1, True, "f32"), "f32", "the held node is still evaluated")
+
+
+def test_phi2_qk_layernorm_through_the_graph(hip):
+    # phi2.rs:207-216: one head is the only well-formed case (the parameters have head_dim elements, the projection
+    # heads * head_dim); with more heads the recorded graph holds the reference's IncompatibleShape error node
+    from oracle import phi2
+    from rai_amd._lib import RaiHipError
+    from rai_amd.models import Decoder
+    from tests.graph_models import Phi2Graph
+    dt = "f32"
+    cfg = phi2.Config(vocab_size=200, hidden_size=80, intermediate_size=160, num_hidden_layers=2, num_attention_heads=1,
+                      max_position_embeddings=48, qk_layernorm=True)
+    params = phi2.random_params(cfg, dt, seed=2, std=0.1)
+    rng = np.random.default_rng(12)
+    for k in params:
+        if "layernorm" in k:
+            params[k] = rnd(params[k] + 0.1 * rng.standard_normal(params[k].shape).astype(np.float32), dt)
+    ref = phi2.Model(cfg, params, dt)
+    model = Phi2Graph(cfg, {k: dev(v, dt) for k, v in params.items()}, dt)
+    ids = rng.integers(0, cfg.vocab_size, (2, 9)).astype(np.uint32)
+    for _ in range(2):
+        got = from_storage(model.fwd(Tensor.from_array(ids, "u32")).as_storage(), dt)[:, 0, :]
+        want = ref.fwd(ids)
+        assert_close(got, want, dt, "phi2 with qk_layernorm through the graph")
+        ids = np.argmax(want, -1).astype(np.uint32).reshape(2, 1)
+    many = phi2.Config(vocab_size=200, hidden_size=160, intermediate_size=160, num_hidden_layers=1,
+                       num_attention_heads=2, max_position_embeddings=48, qk_layernorm=True)
+    pm = phi2.random_params(many, dt, seed=2)
+    bad = Phi2Graph(many, {k: dev(v, dt) for k, v in pm.items()}, dt).fwd(Tensor.from_array(ids[:, :1], "u32"))
+    with pytest.raises(RaiHipError, match="IncompatibleShape"):
+        bad.as_storage()
+    with pytest.raises(RaiHipError) as e:          # the decoder drivers decline the option
+        Decoder("phi2", dt, vocab_size=200, hidden_size=80, intermediate_size=160, num_hidden_layers=1,
+                num_attention_heads=1, rotary_dim=32, qk_layernorm=True)
+    assert e.value.status == -7

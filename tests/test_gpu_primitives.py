@@ -407,9 +407,16 @@ def test_fused_linear_bias_act_residual(R, dt, m):
     assert_close(down(R.linear(up(x, dt), up(w, dt))), onn.linear(x, w, None, dt), dt, "linear plain")
 
 
+@pytest.mark.parametrize("kernel", ["stream", "skinny", "tile"])
 @pytest.mark.parametrize("m", [9, 16, 31, 64])
 @pytest.mark.parametrize("k,n", [(4096, 200), (1056, 2048), (16384, 64), (96, 50)])
-def test_linear_small_batch_deep_k(R, m, k, n):
+def test_linear_small_batch_deep_k(R, monkeypatch, m, k, n, kernel):
+    # 9..64 rows: the weight-streaming MFMA kernel by default; its two fallbacks (activations in LDS with K split over
+    # blocks, and the tile kernel) are forced through the switches the library reads at every call
+    if kernel != "stream":
+        monkeypatch.setenv("RAI_HIP_NO_MFMA_STREAM", "1")
+    if kernel == "tile":
+        monkeypatch.setenv("RAI_HIP_NO_MFMA_SKINNY", "1")
     # batched-decode shapes: 9..64 activation rows against a weight matrix read once; K deep enough
     # to be split over blocks and staged in several chunks, N not a multiple of the 16-row tile
     g = rng(125)

@@ -141,6 +141,26 @@ def test_load_safetensors_errors(hip, tmp_path):
     with pytest.raises(RaiHipError) as e:
         dec.load_safetensors(tmp_path / "b.safetensors")
     assert e.value.status == -2 and "model.final_layernorm.weight" in str(e.value)
+    # right element count, wrong shape: a transposed matrix must not load
+    bad = dict(master)
+    name = "model.layers.0.mlp.fc1.weight"
+    bad[name] = np.ascontiguousarray(master[name].T)
+    write_safetensors(tmp_path / "b2.safetensors", bad, "F32")
+    with pytest.raises(RaiHipError) as e:
+        dec.load_safetensors(tmp_path / "b2.safetensors")
+    assert e.value.status == -2 and name in str(e.value)
+    # a header whose shape describes far more elements than the file holds
+    blob = (tmp_path / "a.safetensors").read_bytes()
+    hlen = struct.unpack("<Q", blob[:8])[0]
+    import json as _json
+    hdr = _json.loads(blob[8:8 + hlen])
+    first = next(k for k in hdr if k != "__metadata__")
+    hdr[first]["shape"] = [2 ** 40, 2 ** 40]
+    h2 = _json.dumps(hdr).encode()
+    (tmp_path / "b3.safetensors").write_bytes(struct.pack("<Q", len(h2)) + h2 + blob[8 + hlen:])
+    with pytest.raises(RaiHipError) as e:
+        dec.load_safetensors(tmp_path / "b3.safetensors")
+    assert e.value.status == -10
     # integer tensor where a floating parameter is expected
     write_safetensors(tmp_path / "c.safetensors", master, {k: ("I64" if k == "model.final_layernorm.bias" else "F32") for k in master})
     with pytest.raises(RaiHipError) as e:

@@ -9,14 +9,14 @@ import torch
 from oracle import phi2
 
 
-def hf_model(cfg, params):
+def hf_model(cfg, params, qk_layernorm=False):
     from transformers import PhiConfig, PhiForCausalLM
     hc = PhiConfig(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size,
                    num_hidden_layers=cfg.num_hidden_layers, num_attention_heads=cfg.num_attention_heads,
                    num_key_value_heads=cfg.num_key_value_heads, max_position_embeddings=cfg.max_position_embeddings,
                    partial_rotary_factor=cfg.partial_rotary_factor, hidden_act="gelu_new",
                    layer_norm_eps=cfg.layer_norm_eps, rope_theta=cfg.rope_theta, tie_word_embeddings=False,
-                   resid_pdrop=0.0, embd_pdrop=0.0, attention_dropout=0.0, qk_layernorm=False)
+                   resid_pdrop=0.0, embd_pdrop=0.0, attention_dropout=0.0, qk_layernorm=qk_layernorm)
     hc._attn_implementation = "eager"
     m = PhiForCausalLM(hc).eval()
     sd = {k: torch.from_numpy(np.asarray(v, np.float32)) for k, v in params.items()}
@@ -80,3 +80,28 @@ def test_bf16_model_close_to_f32_model_and_param_names():
     lb = phi2.Model(cfg, pb, "bf16").fwd(ids)
     lf = phi2.Model(cfg, pb, "f32").fwd(ids)      # same (bf16-representable) weights, f32 arithmetic
     assert np.max(np.abs(lb - lf)) <= 2e-2 * np.max(np.abs(lf))
+
+
+def test_qk_layernorm_single_head_matches_hf_and_many_heads_is_the_references_shape_error():
+    # phi2.rs:207-216 normalises the un-split projections with head_dim-sized parameters: well-formed for one head
+    # only, where it coincides with transformers' per-head q/k LayerNorm
+    cfg = phi2.Config(vocab_size=300, hidden_size=80, intermediate_size=160, num_hidden_layers=2, num_attention_heads=1,
+                      max_position_embeddings=48, qk_layernorm=True)
+    params = phi2.random_params(cfg, "f32", seed=4, std=0.1)
+    g = np.random.Generator(np.random.PCG64(10))
+    for k in params:
+        if k.endswith(".bias"):
+            params[k] = (0.05 * g.standard_normal(params[k].shape)).astype(np.float32)
+        elif k.endswith("layernorm.weight"):
+            params[k] = (1 + 0.1 * g.standard_normal(params[k].shape)).astype(np.float32)
+    assert params["model.layers.0.self_attn.q_layernorm.weight"].shape == (80,)
+    ids = g.integers(0, cfg.vocab_size, (2, 11)).astype(np.uint32)
+    hf = hf_model(cfg, params, qk_layernorm=True)
+    with torch.no_grad():
+        want = hf(torch.from_numpy(ids.astype(np.int64))).logits[:, -1, :].numpy()
+    got = phi2.Model(cfg, params, "f32").fwd(ids)
+    assert np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want))
+    many = phi2.Config(vocab_size=300, hidden_size=160, intermediate_size=160, num_hidden_layers=1,
+                       num_attention_heads=2, max_position_embeddings=48, qk_layernorm=True)
+    with pytest.raises(ValueError, match="IncompatibleShape"):
+        phi2.Model(many, phi2.random_params(many, "f32", seed=4), "f32").fwd(ids)
