@@ -434,8 +434,6 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, 
     if constexpr ((n) == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                   \
     else if constexpr ((n) == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");              \
     else if constexpr ((n) == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");              \
-    else if constexpr ((n) == 7) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");              \
-    else if constexpr ((n) == 14) asm volatile("s_waitcnt vmcnt(14)" ::: "memory");            \
     else if constexpr ((n) == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");              \
     else if constexpr ((n) == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");            \
     else if constexpr ((n) == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");            \
@@ -549,33 +547,52 @@ __global__ void __launch_bounds__(128) k_splitk_epilogue_ln(LinearArgs a, int sp
   const uint16_t *res = (const uint16_t *)a.residual;
   float v[ITEMS][8];
   float s = 0.f;
+  // Sum of the partial products first, for two column groups of the lane at a time: the loads of six splits of both
+  // groups (24 x 16 bytes per lane) are in flight together -- a wave has a whole row to itself and nothing else to
+  // overlap its memory round trips with -- while every element's additions stay in split order.
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[it][e] = 0.f;
+#pragma unroll
+  for (int it0 = 0; it0 < ITEMS; it0 += 2) {
+    const float *pp[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int p = lane + (it0 + j < ITEMS ? it0 + j : it0) * 64;
+      pp[j] = partial + (int64_t)row * a.N + (p < packs ? p : lane % packs) * 8;   // clamped groups are never used
+    }
+    for (int s0 = 0; s0 < splits; s0 += 6) {
+      f32x4 p0[2][6], p1[2][6];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int u = 0; u < 6; ++u) {
+          const int sp = s0 + u < splits ? s0 + u : splits - 1;
+          p0[j][u] = *reinterpret_cast<const f32x4 *>(pp[j] + (int64_t)sp * total);
+          p1[j][u] = *reinterpret_cast<const f32x4 *>(pp[j] + (int64_t)sp * total + 4);
+        }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (it0 + j < ITEMS) {
+          float *x = v[it0 + j];
+#pragma unroll
+          for (int u = 0; u < 6; ++u) {
+            if (s0 + u < splits) {
+              x[0] += p0[j][u].x; x[1] += p0[j][u].y; x[2] += p0[j][u].z; x[3] += p0[j][u].w;
+              x[4] += p1[j][u].x; x[5] += p1[j][u].y; x[6] += p1[j][u].z; x[7] += p1[j][u].w;
+            }
+          }
+        }
+      }
+    }
+  }
 #pragma unroll
   for (int it = 0; it < ITEMS; ++it) {
     const int p = lane + it * 64;
     if (p < packs) {
       const int n = p * 8;
-      float x[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = 0.f;
-      const float *pp = partial + (int64_t)row * a.N + n;
-      // six splits' loads are issued together (a wave has a whole row to itself and little else to overlap with);
-      // the additions stay in split order
-      for (int s0 = 0; s0 < splits; s0 += 6) {
-        f32x4 p0[6], p1[6];
-#pragma unroll
-        for (int u = 0; u < 6; ++u) {
-          const int sp = s0 + u < splits ? s0 + u : splits - 1;
-          p0[u] = *reinterpret_cast<const f32x4 *>(pp + (int64_t)sp * total);
-          p1[u] = *reinterpret_cast<const f32x4 *>(pp + (int64_t)sp * total + 4);
-        }
-#pragma unroll
-        for (int u = 0; u < 6; ++u) {
-          if (s0 + u < splits) {
-            x[0] += p0[u].x; x[1] += p0[u].y; x[2] += p0[u].z; x[3] += p0[u].w;
-            x[4] += p1[u].x; x[5] += p1[u].y; x[6] += p1[u].z; x[7] += p1[u].w;
-          }
-        }
-      }
+      float (&x)[8] = v[it];
       float b1[8], b2[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) b1[e] = b2[e] = 0.f;
@@ -1190,7 +1207,6 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   if (knob) {
     if (!strcmp(knob, "128x128")) return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
     if (!strcmp(knob, "256x128")) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
-    if (!strcmp(knob, "256x192")) return launch_cfg_dma<256, 192, 4, 2>(st, a, splits);
     if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
     if (!strcmp(knob, "256x256x8w")) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
