@@ -652,6 +652,48 @@ __global__ void __launch_bounds__(256) k_transpose_2d(T *dst, const T *src, int 
   }
 }
 
+// The same transposition with 16-byte accesses on both sides (N, K multiples of 16 / sizeof(T), 16-byte aligned
+// operands): a 64 x 64 tile is read as rows of 16-byte chunks, and every thread then gathers the 16 bytes of one
+// output chunk (consecutive k for one n) from LDS.  The odd pitch in 32-bit words keeps the column gathers off a
+// single bank.
+template <typename T>
+__global__ void __launch_bounds__(256) k_transpose_2d_vec(T *dst, const T *src, int K, int N) {
+  constexpr int V = 16 / sizeof(T), CPR = 64 / V;      // elements per chunk, chunks per tile row
+  constexpr int PITCH = sizeof(T) == 2 ? 66 : 65;      // 33 resp. 65 words per row
+  struct alignas(16) Pack { T v[V]; };
+  __shared__ T tile[64][PITCH];
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
+    const int i = c / CPR, j = (c % CPR) * V;
+    const int k = k0 + i, n = n0 + j;
+    if (k < K && n < N) {
+      const Pack p = *reinterpret_cast<const Pack *>(src + (int64_t)k * N + n);
+#pragma unroll
+      for (int e = 0; e < V; ++e) tile[i][j + e] = p.v[e];
+    }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
+    const int i = c / CPR, j = (c % CPR) * V;            // output row n0 + i, k chunk at k0 + j
+    const int n = n0 + i, k = k0 + j;
+    if (n < N && k < K) {
+      Pack p;
+#pragma unroll
+      for (int e = 0; e < V; ++e) p.v[e] = tile[j + e][i];
+      *reinterpret_cast<Pack *>(dst + (int64_t)n * K + k) = p;
+    }
+  }
+}
+
+template <typename T> static void launch_transpose_2d(hipStream_t st, T *dst, const T *src, int K, int N) {
+  const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
+  constexpr int V = 16 / sizeof(T);
+  if (N % V == 0 && K % V == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0)
+    hipLaunchKernelGGL(k_transpose_2d_vec<T>, grid, dim3(256), 0, st, dst, src, K, N);
+  else
+    hipLaunchKernelGGL(k_transpose_2d<T>, grid, dim3(256), 0, st, dst, src, K, N);
+}
+
 int launch_linear_f32(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem");
   RAI_REQUIRE(a.ln_kind < 0, RAI_ERR_UNSUPPORTED, "linear f32: no fused norm");
@@ -752,13 +794,10 @@ int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, co
       void *tmp = nullptr;
       RAI_TRY(rai_hip_alloc(dev, (size_t)N * K * dtype_size(b->dtype), &tmp));
       hipStream_t tst = stream_of(dev);
-      const dim3 tgrid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
       if (b->dtype == RAI_BF16)
-        hipLaunchKernelGGL(k_transpose_2d<uint16_t>, tgrid, dim3(256), 0, tst, (uint16_t *)tmp,
-                           (const uint16_t *)base_ptr(b), (int)K, (int)N);
+        launch_transpose_2d<uint16_t>(tst, (uint16_t *)tmp, (const uint16_t *)base_ptr(b), (int)K, (int)N);
       else
-        hipLaunchKernelGGL(k_transpose_2d<float>, tgrid, dim3(256), 0, tst, (float *)tmp, (const float *)base_ptr(b),
-                           (int)K, (int)N);
+        launch_transpose_2d<float>(tst, (float *)tmp, (const float *)base_ptr(b), (int)K, (int)N);
       int rc = launch_check("transpose_2d");
       if (rc == RAI_OK) {
         rai_hip_tensor b2 = *b;  // [.., K, N] view of the transposed copy: strides (1, K), batch strides 0

@@ -296,35 +296,53 @@ k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int6
   }
   if ((threadIdx.x & 63) == 0) { shv[threadIdx.x >> 6] = bv; shi[threadIdx.x >> 6] = bi; }
   __syncthreads();
+  if (threadIdx.x >= 64) return;   // wave 0 finishes the block
   if (threadIdx.x == 0) {
     for (int w = 1; w < 4; ++w)
       if (better<C, IS_MAX>(shv[w], shi[w], bv, bi)) { bv = shv[w]; bi = shi[w]; }
-    if (!out) {   // two-launch form: k_arg_row_final merges
+  }
+  if (!out) {   // two-launch form: k_arg_row_final merges
+    if (threadIdx.x == 0) {
       if (sizeof(C) == 8) pval_d[blockIdx.x] = (double)bv; else pval_f[blockIdx.x] = (float)bv;
       pidx[blockIdx.x] = bi;
-      return;
     }
-    // One-launch form: the block of a row that arrives last merges the row's partial results.  They cross blocks
-    // (and XCDs, whose L2s are not coherent for ordinary accesses) as device-scope relaxed atomics, which write
-    // through / read around the L2; the arrival counter is bumped only after this block's stores have completed,
-    // and the last block sets it back to zero for the next call.
-    if (splits > 1) {
+    return;
+  }
+  // One-launch form: the block of a row that arrives last merges the row's partial results.  They cross blocks
+  // (and XCDs, whose L2s are not coherent for ordinary accesses) as device-scope relaxed atomics, which write
+  // through / read around the L2; the arrival counter is bumped only after this block's stores have completed,
+  // and the last block sets it back to zero for the next call.  The merge is one memory round trip: every lane of
+  // the wave fetches one split's result, then the lanes are reduced with the same ordering.
+  if (splits > 1) {
+    int last = 0;
+    if (threadIdx.x == 0) {
       if (sizeof(C) == 8) __hip_atomic_store(&pval_d[blockIdx.x], (double)bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else __hip_atomic_store(&pval_f[blockIdx.x], (float)bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(&pidx[blockIdx.x], bi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (atomicAdd(&counters[row], 1u) != (uint32_t)splits - 1u) return;
-      const int64_t base = row * splits;
-      for (int sp = 0; sp < splits; ++sp) {
-        C v;
-        if (sizeof(C) == 8) v = (C)__hip_atomic_load(&pval_d[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else v = (C)__hip_atomic_load(&pval_f[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t i = __hip_atomic_load(&pidx[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (sp == 0) { bv = v; bi = i; }
-        else if (better<C, IS_MAX>(v, i, bv, bi)) { bv = v; bi = i; }
-      }
-      __hip_atomic_store(&counters[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      last = atomicAdd(&counters[row], 1u) == (uint32_t)splits - 1u;
     }
+    if (!__shfl(last, 0, 64)) return;
+    const int64_t base = row * splits;
+    bool got = false;
+    bv = C(NAN);
+    bi = 0xffffffffu;
+    for (int sp = threadIdx.x; sp < splits; sp += 64) {
+      C v;
+      if (sizeof(C) == 8) v = (C)__hip_atomic_load(&pval_d[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else v = (C)__hip_atomic_load(&pval_f[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t i = __hip_atomic_load(&pidx[base + sp], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (!got || better<C, IS_MAX>(v, i, bv, bi)) { bv = v; bi = i; got = true; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      C ov = shfl_xor_c<C>(bv, o);
+      uint32_t oi = (uint32_t)__shfl_xor((int)bi, o, 64);
+      if (better<C, IS_MAX>(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (threadIdx.x == 0) {
     // all-NaN row: every candidate is NaN and index 0 wins already; a NaN at element 0 wins in the reference's
     // sequential scan even with finite values elsewhere
     const C first = Scalar<T>::load(x);
