@@ -335,6 +335,68 @@ def run_ops(args):
           {"ops": rows})
 
 
+def run_gemm_tiles(args):
+    """The bf16 tile GEMM on the Phi-2 prefill shapes (and the op-sweep shape), every tile shape forced in turn
+    through RAI_HIP_GEMM_TILE, Linear with bias and gelu_new as the q|k|v|fc1 product has them: shows what tile
+    quantisation at M = 512 costs and that no tile shape escapes it."""
+    import ctypes as C
+
+    from rai_amd import _lib
+    from rai_amd._lib import UNARY
+    from rai_amd.hip import HipTensor, sync
+    _lib.call("rai_hip_init", 0)
+    lib = _lib.load()
+    rng = np.random.default_rng(0)
+
+    def rnd(shape):
+        a = rng.standard_normal(shape, dtype=np.float32)
+        return HipTensor.from_storage((a.view(np.uint32) >> 16).astype(np.uint16), "bf16")
+
+    shapes = [(512, 17920, 2560), (512, 10240, 2560), (512, 7680, 2560), (512, 2560, 12800), (4096, 10240, 2560)]
+    tiles = ["128x128", "256x128", "256x256", "256x256x8w", None]
+    rows = []
+    for m, n, k in shapes:
+        x, b, out = rnd((m, k)), rnd((n,)), HipTensor.empty((m, n), "bf16")
+        # "cold": the launches rotate over enough copies of the weight (> 600 MB together) that none is still in the
+        # 256 MB memory-side cache when its turn comes, as inside a model; "warm": one weight, resident after warm-up
+        w0 = rnd((n, k))
+        copies = [w0] + ([rnd((n, k)) for _ in range(-(-600_000_000 // (2 * n * k)) - 1)] if args.cold else [])
+        dx, db, do = x.desc(), b.desc(), out.desc()
+        dws = [c.desc() for c in copies]
+        for tile in tiles:
+            if tile is None:
+                os.environ.pop("RAI_HIP_GEMM_TILE", None)
+            else:
+                os.environ["RAI_HIP_GEMM_TILE"] = tile
+
+            turn = [0]
+
+            def go():
+                dw = dws[turn[0] % len(dws)]
+                turn[0] += 1
+                _lib.check(lib.rai_hip_linear(0, C.byref(dx), C.byref(dw), C.byref(db), UNARY["new_gelu"], None, C.byref(do)))
+            t = C.c_void_p()
+            _lib.call("rai_hip_timer_create", 0, C.byref(t))
+            for _ in range(10):
+                go()
+            _lib.call("rai_hip_timer_start", t)
+            for _ in range(50):
+                go()
+            _lib.call("rai_hip_timer_stop", t)
+            ms = C.c_float()
+            _lib.call("rai_hip_timer_elapsed_ms", t, C.byref(ms))
+            _lib.call("rai_hip_timer_destroy", t)
+            us = ms.value * 1e3 / 50
+            rows.append({"shape": f"{m}x{n}x{k}", "tile": tile or "auto", "us": round(us, 1),
+                         "tflops": round(2.0 * m * n * k / us / 1e6, 1)})
+    os.environ.pop("RAI_HIP_GEMM_TILE", None)
+    sync()
+    best = max(r["tflops"] for r in rows if r["shape"] == "512x17920x2560")
+    _line("bf16 Linear 512x17920x2560 (+bias, gelu_new) TFLOP/s on 1 MI355X", best, "TFLOP/s", 50, 10, 0.0,
+          "tile GEMM, every tile shape forced in turn on the Phi-2 prefill shapes",
+          {"weights": "cold (rotating copies)" if args.cold else "warm (one copy)", "tiles": rows})
+
+
 def run_phi2_graph(args, n_new=16):
     """The drop-in path: Phi-2 recorded node for node through the lazy-graph API the way rai-models/src/llm/phi2.rs
     builds it (tests/graph_models.py, KV cache by concatenation) and evaluated by the C++ evaluator with its
@@ -399,7 +461,9 @@ def main():
                     help="debug only: fewer layers (the JSON line then says so and is not the headline workload)")
     ap.add_argument("--graph-tokens", type=int, default=16,
                     help="tokens decoded through the lazy-graph path for the graph_decode_* fields (0: skip)")
-    ap.add_argument("--workload", default="phi2-decode", choices=["phi2-decode", "qwen2-prefill", "gemma-decode", "ops"],
+    ap.add_argument("--cold", action="store_true",
+                    help="gemm-tiles: rotate over weight copies so every launch reads its weight from HBM, as in a model")
+    ap.add_argument("--workload", default="phi2-decode", choices=["phi2-decode", "qwen2-prefill", "gemma-decode", "ops", "gemm-tiles"],
                     help="phi2-decode is the headline line; the others are the remaining configurations of the path")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -410,6 +474,8 @@ def main():
         return run_gemma_decode(args)
     if args.workload == "ops":
         return run_ops(args)
+    if args.workload == "gemm-tiles":
+        return run_gemm_tiles(args)
 
     from rai_amd import synthetic
     from rai_amd.hip import sync
