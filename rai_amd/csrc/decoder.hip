@@ -836,6 +836,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   for (int l = 0; l < (use_mega ? 0 : d->L); ++l) {
     const Layer &ly = d->layers[l];
     LinearArgs a = linear_args_default();
+    a.splitk_ws = d->splitk_ws; a.splitk_ws_bytes = d->splitk_ws_bytes;
     if (fuse_ln) {
       a.A = x; a.lda = H;
       a.ln_kind = 0; a.ln_w = ly.ln_w; a.ln_b = ly.ln_b; a.ln_eps = (float)d->cfg.norm_eps;
@@ -1038,6 +1039,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     RAI_TRY(linear(d, st, o));
 
     LinearArgs g = linear_args_default();
+    g.splitk_ws = d->splitk_ws; g.splitk_ws_bytes = d->splitk_ws_bytes;
     if (fuse_norm) {
       g.A = x1; g.lda = H;
       g.ln_kind = kind; g.ln_w = ly.n2_w; g.ln_eps = (float)d->cfg.norm_eps;
@@ -1233,6 +1235,9 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->state = (DevState *)tmp;
   d->splitk_ws_bytes = (size_t)12 * d->max_rows * d->H * sizeof(float);
   if (d->splitk_ws_bytes > ((size_t)256 << 20)) d->splitk_ws_bytes = (size_t)256 << 20;
+  // the stream-K form of the tile kernel (prefill products of 136 tiles and more) parks partial tiles here
+  if (cfg->dtype == RAI_BF16 && d->max_rows >= 256 && d->splitk_ws_bytes < ((size_t)192 << 20))
+    d->splitk_ws_bytes = (size_t)192 << 20;
   if ((st = dalloc(d, d->splitk_ws_bytes, &d->splitk_ws))) return bail(st);
   if ((st = dalloc(d, attention_decode_ws_bytes(cfg->max_batch, d->Hq, d->D), &d->attn_ws))) return bail(st);
   if ((st = dalloc(d, attention_decode_counter_bytes(cfg->max_batch, d->Hq), &tmp))) return bail(st);

@@ -60,6 +60,9 @@ struct LinearArgs {
 };
 // True when launch_linear_bf16 with these arguments will also write post_ln_out.
 bool linear_fuses_post_norm(const LinearArgs &a);
+// Workspace (LinearArgs::splitk_ws) the stream-K form of the bf16 tile kernel needs for an M x N x K Linear; 0 when
+// that form does not apply to the shape.  At most 192 MB.
+size_t linear_streamk_workspace_bytes(int M, int N, int K);
 inline LinearArgs linear_args_default() {
   LinearArgs a;
   memset(&a, 0, sizeof(a));

@@ -110,6 +110,35 @@ __device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (
   const bool vec_out = (a.ld1 % 8 == 0) && (a.n_split % 8 == 0) && (a.n_split == a.N || a.ld2 % 8 == 0) &&
                        ((uintptr_t)a.out1 % 16 == 0) && (a.n_split == a.N || (uintptr_t)a.out2 % 16 == 0) &&
                        (!res || (a.ldr % 8 == 0 && (uintptr_t)res % 16 == 0)) && a.N % 8 == 0;
+  // A lane serves the same 8 columns in every pass (64 lanes are a multiple of the CG column groups of a staged row):
+  // their bias values are fetched once, ahead of the passes, not inside each of them, where the load's latency
+  // (about a microsecond under load) sat between the LDS read and the store of every pass.
+  static_assert(64 % CG == 0, "a lane must keep its column group from pass to pass");
+  const int n = n0 + wn * WN + (lane % CG) * 8;
+  const bool whole = n + 8 <= a.N;
+  float bv[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bv[e] = 0.f;
+  if (bias && !partial && n < a.N) {
+    if (whole && ((uintptr_t)(bias + n) & 15) == 0) unpack8(*reinterpret_cast<const u32x4 *>(bias + n), bv);
+    else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (n + e < a.N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+    }
+  }
+  if (bias2 && !partial && n < a.N) {
+    float b2[8];
+    if (whole && ((uintptr_t)(bias2 + n) & 15) == 0) {
+      unpack8(*reinterpret_cast<const u32x4 *>(bias2 + n), b2);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bv[e] += b2[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (n + e < a.N) bv[e] += bf16_bits_to_f32(bias2[n + e]);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     // accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32]
@@ -124,7 +153,6 @@ __device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (
       const int item = lane + it * 64;
       const int row = item / CG, cg = item % CG;
       const int m = m0 + wm * WM + i * 32 + row;
-      const int n = n0 + wn * WN + cg * 8;
       if (m >= a.M || n >= a.N) continue;
       const f32x4 v0 = *reinterpret_cast<const f32x4 *>(stage + row * EP + cg * 8);
       const f32x4 v1 = *reinterpret_cast<const f32x4 *>(stage + row * EP + cg * 8 + 4);
@@ -140,31 +168,6 @@ __device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (
             if (n + e < a.N) p[e] = v[e];
         }
         continue;
-      }
-      // bias values of the 8 columns: one 16-byte load when the row of columns is whole and aligned
-      const bool whole = n + 8 <= a.N;
-      float bv[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) bv[e] = 0.f;
-      if (bias) {
-        if (whole && ((uintptr_t)(bias + n) & 15) == 0) unpack8(*reinterpret_cast<const u32x4 *>(bias + n), bv);
-        else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n + e < a.N) bv[e] = bf16_bits_to_f32(bias[n + e]);
-        }
-      }
-      if (bias2) {
-        float b2[8];
-        if (whole && ((uintptr_t)(bias2 + n) & 15) == 0) {
-          unpack8(*reinterpret_cast<const u32x4 *>(bias2 + n), b2);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) bv[e] += b2[e];
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n + e < a.N) bv[e] += bf16_bits_to_f32(bias2[n + e]);
-        }
       }
       if (a.glu) {  // columns n..n+7 are four (gate, up) pairs -> four outputs at column n/2
         uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
@@ -352,31 +355,18 @@ __global__ void __launch_bounds__(256) k_gemm_bf16_mfma(LinearArgs a, int splits
 //     bare s_barrier make tile t+1 visible to the block (and retire stage t-1 for refilling) with one
 //     barrier per K tile.  The barrier carries no fence: a fence would wait for every outstanding
 //     LDS load, i.e. drain the pipeline.
-template <int BM, int BN, int NS, int SH, int WGN = 2>
-__global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
-  // block = 2 x WGN waves.  WGN = 4 (eight waves, wave tile (BM/2) x (BN/4)) keeps two waves on every SIMD: one
-  // multiplies while the other sits in its wait for the next tile, and twice as many waves issue loads.
+// K loop of the LDS-DMA tile kernels: acc = A[m0.., k_begin..] . W[n0.., k_begin..]^T over KT tiles of 32, with the
+// software pipeline described above.  Ends with every load landed and the block synchronised, so the caller may reuse
+// the LDS stages.
+template <int BM, int BN, int NS, int SH, int WGN>
+__device__ __forceinline__ void dma_tile_mainloop(const LinearArgs &a, uint16_t *lds, int m0, int n0, int k_begin, int KT,
+                                                  int wave, int lane, f32x16 (&acc)[BM / 64][BN / (32 * WGN)]) {
   constexpr int BK = 32, PITCH = BK;
   constexpr int WM = BM / 2, WN = BN / WGN;
   constexpr int MT = WM / 32, NT = WN / 32;
   constexpr int LA = BM / (32 * WGN), LB = BN / (32 * WGN);   // loads per wave per K tile (16 rows each)
   constexpr int STAGE = (BM + BN) * BK;              // elements per stage: A rows then B rows
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
-  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
-  const int total = tiles_m * tiles_n;
-  const int tile = xcd_remap(blockIdx.x, total);
-  if (tile >= total) return;
-  int tile_m, tile_n;
-  tile_coords(tile, tiles_m, tiles_n, &tile_m, &tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int split = blockIdx.y;
-  const int k_begin = split * k_per_split;
-  const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
-  const int KT = (k_end - k_begin) / BK;
-
   // lane -> (row within the 16-row group, swizzled chunk)
   const int lrow = lane >> 2;
   const uint16_t *gpa[LA], *gpb[LB];
@@ -407,7 +397,6 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, 
       __builtin_amdgcn_global_load_lds((const void *)(gpb[j] + kt * BK), (lds_ptr)(sb + j * 16 * BK), 16, 0, 0);
   };
 
-  f32x16 acc[MT][NT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -501,8 +490,168 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, 
   // the refetches issued past the end must land before the stages are reused for the epilogue
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+}
+
+template <int BM, int BN, int NS, int SH, int WGN = 2>
+__global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
+  // block = 2 x WGN waves.  WGN = 4 (eight waves, wave tile (BM/2) x (BN/4)) keeps two waves on every SIMD: one
+  // multiplies while the other sits in its wait for the next tile, and twice as many waves issue loads.
+  constexpr int BK = 32, PITCH = BK;
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int tile = xcd_remap(blockIdx.x, total);
+  if (tile >= total) return;
+  int tile_m, tile_n;
+  tile_coords(tile, tiles_m, tiles_n, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int split = blockIdx.y;
+  const int k_begin = split * k_per_split;
+  const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
+  const int KT = (k_end - k_begin) / BK;
+
+  f32x16 acc[BM / 64][BN / (32 * WGN)];
+  dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, k_begin, KT, wave, lane, acc);
   gemm_tile_epilogue<BM, BN, gemm_lds_bytes<BM, BN, PITCH * NS / 2, WGN>(), WGN>(a, acc, lds, m0, n0, wave, lane, split,
                                                                                  partial);
+}
+
+// ---- stream-K form of the eight-wave 256x256 tile kernel ---------------------------------------------------------
+// One block per CU.  When the tile count is not a multiple of the CU count, the last partial round would leave CUs
+// idle for a whole tile time (140 tiles on 256 CUs: 45 % of the machine).  Here the K tiles of those `sk_tiles` tiles
+// are dealt out evenly instead: block p (in XCD order, so neighbours share an L2) takes units [start(p), start(p+1))
+// of the sk_tiles * KT (tile, K tile) units, i.e. the tail of one tile and the head of the next.  A tile is then the
+// work of two or three blocks: each stores its f32 accumulators to its slot of the workspace in register order
+// with device-scope stores and counts itself in; the block that arrives
+// last adds the slots in slot order (so the sum does not depend on who was last) and runs the epilogue.  Nobody
+// waits for anybody.  The remaining tiles follow in whole rounds, one tile per block as before.
+struct StreamKArgs {
+  int sk_tiles;   // tiles 0 .. sk_tiles-1 are shared out by K tile; the rest run whole
+  int q, rem;     // units per block: blocks 0 .. rem-1 take q + 1, the others q
+  int max_parts;  // slots per tile in the workspace
+  float *ws;      // [sk_tiles][max_parts][BM * BN] f32
+  int *counters;  // [sk_tiles][2] (tickets, stored shares), zero between launches
+};
+
+__device__ __forceinline__ int sk_start(const StreamKArgs &k, int p) { return p * k.q + (p < k.rem ? p : k.rem); }
+__device__ __forceinline__ int sk_block_of(const StreamKArgs &k, int u) {
+  const int big = k.rem * (k.q + 1);
+  return u < big ? u / (k.q + 1) : k.rem + (u - big) / k.q;
+}
+
+template <int BM, int BN, int NS, int SH, int WGN>
+__global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma_streamk(LinearArgs a, StreamKArgs sk) {
+  constexpr int BK = 32, PITCH = BK;
+  constexpr int MT = BM / 64, NT = BN / (32 * WGN);
+  constexpr int LDS_BYTES = gemm_lds_bytes<BM, BN, PITCH * NS / 2, WGN>();
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  __shared__ int s_ticket;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int KT = a.K / BK;
+  const int P = gridDim.x;
+  const int p = xcd_remap(blockIdx.x, P);   // P is a multiple of the XCD count
+  f32x16 acc[MT][NT];
+
+  // one loop over this block's segments (shares of tiles first, then whole tiles), so that the K loop and the
+  // epilogue are instantiated once
+  int u = sk_start(sk, p);
+  const int u_end = sk_start(sk, p + 1);
+  int whole = sk.sk_tiles + p;
+  for (;;) {
+    int tile, kt0, kt1;
+    if (u < u_end) {
+      tile = u / KT;
+      kt0 = u - tile * KT;
+      kt1 = kt0 + (u_end - u) < KT ? kt0 + (u_end - u) : KT;
+      u += kt1 - kt0;
+    } else if (whole < total) {
+      tile = whole;
+      kt0 = 0;
+      kt1 = KT;
+      whole += P;
+    } else {
+      break;
+    }
+    int tile_m, tile_n;
+    tile_coords(tile, tiles_m, tiles_n, &tile_m, &tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    __syncthreads();   // the previous segment's epilogue staging is done with the LDS
+    dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, kt0 * BK, kt1 - kt0, wave, lane, acc);
+    if (kt1 - kt0 != KT) {
+      // a share of the tile: which slot is ours, and how many there are
+      const int first = sk_block_of(sk, tile * KT), last = sk_block_of(sk, tile * KT + KT - 1);
+      const int parts = last - first + 1, slot = p - first;
+      // Slot layout [wave][accumulator register][lane]: one store or load instruction covers 256 consecutive bytes.
+      // The shares cross XCDs, whose L2s are not coherent with each other: they are written and read with
+      // device-scope accesses (write-through stores, loads that miss L2) instead of a release / acquire fence pair
+      // -- the fences write back and invalidate a whole L2 each and, issued by every block of an XCD at about the
+      // same time, queue up behind one another (measured: +130 us per launch).
+      float *tile_ws = sk.ws + (int64_t)tile * sk.max_parts * (BM * BN) + wave * (MT * NT * 16 * 64) + lane;
+      // Two counters per tile: `arrived` hands out tickets when a share has been computed, `stored` counts the
+      // shares that have reached memory.  The block with the last ticket keeps its share in registers and sums; the
+      // others store theirs.  Its wait is for blocks that already hold a ticket, i.e. are running and have nothing
+      // left to do but their stores, and it is bounded all the same.
+      int *arrived = sk.counters + 2 * tile, *stored = arrived + 1;
+      if (tid == 0) s_ticket = __hip_atomic_fetch_add(arrived, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (s_ticket != parts - 1) {
+        float *mine = tile_ws + (int64_t)slot * (BM * BN);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              __hip_atomic_store(mine + ((i * NT + j) * 16 + r) * 64, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share has left for memory
+        __syncthreads();
+        if (tid == 0) __hip_atomic_fetch_add(stored, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          continue;
+      }
+      if (tid == 0) {
+        for (int spin = 0; spin < (1 << 20); ++spin) {
+          if (__hip_atomic_load(stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1) break;
+          __builtin_amdgcn_s_sleep(2);
+        }
+        __hip_atomic_store(arrived, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(stored, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __syncthreads();
+      // the other slots are complete.  Sum in slot order, our registers standing in for our slot, so the result does
+      // not depend on who came last.
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          f32x16 sum = acc[i][j];
+          for (int s = 0; s < parts; ++s) {
+            if (s == slot) {
+              if (s > 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum[r] += acc[i][j][r];
+              }
+              continue;
+            }
+            const float *src = tile_ws + (int64_t)s * (BM * BN) + ((i * NT + j) * 16) * 64;
+            f32x16 v;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) v[r] = __hip_atomic_load(src + r * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (s == 0) sum = v;
+            else {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) sum[r] += v[r];
+            }
+          }
+          acc[i][j] = sum;
+        }
+    }
+    gemm_tile_epilogue<BM, BN, LDS_BYTES, WGN>(a, acc, lds, m0, n0, wave, lane, 0, nullptr);
+  }
 }
 
 // Sums the per-split partial products and applies the Linear epilogue.
@@ -730,6 +879,95 @@ static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
   RAI_TRY(launch_check("gemm_bf16_mfma_dma"));
   if (splits > 1) RAI_TRY(launch_splitk_epilogue(st, a, splits, (const float *)partial));
   return RAI_OK;
+}
+
+// Arrival counters of the stream-K kernel, one per shared tile; every launch leaves them at zero.
+static __device__ int g_streamk_counters[4 * kNumCU];
+
+// How the stream-K kernel would share out an M x N x K product: false when it does not apply (tile count a multiple
+// of the CU count, too few tiles, or a tile would be the work of more than three blocks).
+struct StreamKPlan {
+  StreamKArgs k;
+  size_t ws_bytes;
+};
+static bool streamk_plan(int M, int N, int K, StreamKPlan *plan, bool forced = false) {
+  const int P = kNumCU, KT = K / 32;
+  const int T = ((M + 255) / 256) * ((N + 255) / 256);
+  const int full = T / P, left = T % P;
+  if (left == 0 || KT < 8) return false;
+  int sk_tiles = left;
+  if (left < P / 2) {
+    if (full == 0) return false;
+    sk_tiles = left + P;   // a whole round joins the shared part: every block then works on two tiles at most
+  }
+  const long long units = (long long)sk_tiles * KT;
+  StreamKArgs k;
+  k.sk_tiles = sk_tiles;
+  k.q = (int)(units / P);
+  k.rem = (int)(units % P);
+  if (k.q < 1) return false;
+  auto block_of = [&](int u) {
+    const int big = k.rem * (k.q + 1);
+    return u < big ? u / (k.q + 1) : k.rem + (u - big) / k.q;
+  };
+  int max_parts = 1;
+  for (int t = 0; t < sk_tiles; ++t) {
+    const int parts = block_of(t * KT + KT - 1) - block_of(t * KT) + 1;
+    if (parts > max_parts) max_parts = parts;
+  }
+  if (max_parts > 3 || sk_tiles > 2 * kNumCU) return false;
+  // Worth it when the CU time saved exceeds what the exchange of the shares costs.  Measured with cold weights, bias
+  // and gelu_new: 4096 x 10240 x 2560 (two shares per tile, 40 K tiles of a round saved) 237 -> 215 us, i.e. ~18 us
+  // for the exchange; 512 x 17920 x 2560 (three shares, 36 saved) 81 -> 84 us, i.e. ~39 us: every block ends on a
+  // read of the other shares plus the epilogue, with nothing left to hide them behind.  One K tile of a 256 x 256
+  // tile takes ~1 us with all CUs busy.
+  const float saved_us = (float)(P - left) / P * KT * 1.0f;
+  const float exchange_us = max_parts <= 2 ? 18.f : 39.f;
+  if (!forced && saved_us < 1.3f * exchange_us) return false;
+  k.max_parts = max_parts;
+  k.ws = nullptr;
+  k.counters = nullptr;
+  plan->k = k;
+  plan->ws_bytes = (size_t)sk_tiles * max_parts * 256 * 256 * sizeof(float);
+  return true;
+}
+
+size_t linear_streamk_workspace_bytes(int M, int N, int K) {
+  StreamKPlan plan;
+  return streamk_plan(M, N, K, &plan) ? plan.ws_bytes : 0;
+}
+
+// True when the stream-K kernel serves this Linear (plain tile epilogue, workspace large enough, not switched off).
+static bool streamk_applies(const LinearArgs &a, StreamKPlan *plan, bool forced = false) {
+  const char *off = getenv("RAI_HIP_NO_STREAMK");   // read per call: tests compare both forms in one process
+  if (off && *off && *off != '0') return false;
+  if (!a.splitk_ws || ((uintptr_t)a.splitk_ws & 15) || a.post_ln_out) return false;
+  return streamk_plan(a.M, a.N, a.K, plan, forced) && plan->ws_bytes <= a.splitk_ws_bytes;
+}
+
+static int launch_streamk(hipStream_t st, const LinearArgs &a, StreamKPlan plan) {
+  constexpr int BM = 256, BN = 256, NS = 4, SH = 2, WGN = 4;
+  constexpr size_t lds = gemm_lds_bytes<BM, BN, 32 * NS / 2, WGN>();
+  static bool attr_set = false;
+  if (!attr_set) {
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma_streamk<BM, BN, NS, SH, WGN>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  // every GPU holds its own copy of the counter array at its own address
+  static int *counters[64];
+  int dev = 0;
+  RAI_HIP_TRY(hipGetDevice(&dev));
+  RAI_REQUIRE(dev >= 0 && dev < 64, RAI_ERR_BAD_ARG, "device %d out of range", dev);
+  if (!counters[dev]) {
+    void *p = nullptr;
+    RAI_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_streamk_counters)));
+    counters[dev] = (int *)p;
+  }
+  plan.k.ws = (float *)a.splitk_ws;
+  plan.k.counters = counters[dev];
+  hipLaunchKernelGGL((k_gemm_bf16_mfma_dma_streamk<BM, BN, NS, SH, WGN>), dim3(kNumCU), dim3(128 * WGN), lds, st, a, plan.k);
+  return launch_check("gemm_bf16_mfma_dma_streamk");
 }
 
 // ---- small M (9..64 rows): weight streaming through 16x16x32 MFMA -----------------------
@@ -1210,6 +1448,12 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
     if (!strcmp(knob, "256x256x8w")) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
+    if (!strcmp(knob, "streamk")) {
+      StreamKPlan plan;
+      RAI_REQUIRE(splits == 1 && streamk_applies(a, &plan, true), RAI_ERR_UNSUPPORTED,
+                  "linear: RAI_HIP_GEMM_TILE=streamk does not apply to %dx%dx%d", a.M, a.N, a.K);
+      return launch_streamk(st, a, plan);
+    }
   }
   const int big_tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
   const int huge_tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
@@ -1219,7 +1463,11 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   // 834, 4096 x 10240 x 2560 896 against 789, 4096 x 2560 x 10240 (160 tiles) 837 against 650, 512 x 17920 x 2560
   // (140 tiles) 689 against 621; with 128 tiles or fewer the smaller tiles win (4096 x 2048 x 2048: 618 against 760).
   // The four-wave 256x256 form is 3-9 % behind the eight-wave one everywhere.
-  if (splits == 1 && 32 * huge_tiles >= 17 * kNumCU) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
+  if (splits == 1 && 32 * huge_tiles >= 17 * kNumCU) {
+    StreamKPlan plan;
+    if (streamk_applies(a, &plan)) return launch_streamk(st, a, plan);
+    return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
+  }
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
   return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
 }

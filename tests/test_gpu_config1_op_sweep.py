@@ -218,6 +218,61 @@ def test_gemm_tile_gated_mlp(R, monkeypatch, tile, act, k_splits):
     assert_close(got, want, dt, f"{tile} splits {k_splits}: {act}(gate) * up")
 
 
+# Stream-K form of the eight-wave 256 x 256 tile: the K tiles of the last, partial round of tiles are dealt out evenly
+# over the CUs and the shares of a tile are summed by whichever block finishes last.  Shapes: 156 tiles (no whole
+# round; two or three shares per tile), 180 tiles at K = 512, 324 tiles (one whole round joins the shared part), 720
+# tiles (two whole rounds follow the shared part); all ragged in M and N.
+STREAMK_SHAPES = [(3000, 3100, 2560), (2100, 5000, 512), (4400, 4600, 320), (5000, 9000, 256)]
+
+
+@pytest.mark.parametrize("m,n,k", STREAMK_SHAPES)
+def test_gemm_streamk_plain_and_fused_epilogue(R, monkeypatch, m, n, k):
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk")   # refuses (RAI_ERR_UNSUPPORTED) where the form does not apply
+    dt = "bf16"
+    x, w, b1, _, r = packed_case(rng(120), m, n, k)
+    xd, wd = up(x, dt), up(w, dt)
+    lin = onn.linear(x, w, None, dt)
+    first = down(R.linear(xd, wd))
+    assert_close(first, lin, dt, f"stream-K linear {m}x{n}x{k}")
+    gemm_elem_check(first, lin, dt, k, f"stream-K linear {m}x{n}x{k}")
+    # the shares are summed in slot order whoever arrives last: every run gives the same bits
+    for _ in range(3):
+        assert np.array_equal(down(R.linear(xd, wd)), first)
+    want = oo.add(onn.new_gelu(onn.linear(x, w, b1, dt), dt), r, dt)
+    got = down(R.linear(xd, wd, up(b1, dt), "new_gelu", up(r, dt)))
+    assert_close(got, want, dt, f"stream-K linear + bias + new_gelu + residual {m}x{n}x{k}")
+    # against the same tile without sharing: same products, another grouping of the f32 sums
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "256x256x8w")
+    gemm_elem_check(first, down(R.linear(xd, wd)), dt, k, f"stream-K against whole tiles {m}x{n}x{k}")
+
+
+def test_gemm_streamk_packed_epilogues(R, monkeypatch):
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk")
+    dt, m, n, k, n1 = "bf16", 2100, 4936, 640, 2421      # 180 tiles; n1 odd: second output rows not 16-byte aligned
+    x, w, b1, b2, r = packed_case(rng(121), m, n, k)
+    xd, wd = up(x, dt), up(w, dt)
+    o1, o2 = R.linear_packed(xd, wd, bias=up(b1, dt), act="new_gelu", act_from=n1, n1=n1)
+    y = onn.linear(x, w, b1, dt)
+    assert_close(down(o1), y[:, :n1], dt, "stream-K: q|k|v columns")
+    assert_close(down(o2), onn.new_gelu(y[:, n1:], dt), dt, "stream-K: fc1 columns")
+    k1 = 256
+    got = down(R.linear_packed(xd, wd, bias=up(b1, dt), bias2=up(b2, dt), residual=up(r, dt)))
+    want = oo.add(oo.add(onn.linear(x[:, :k1], w[:, :k1], b1, dt), onn.linear(x[:, k1:], w[:, k1:], b2, dt), dt), r, dt)
+    assert_close(got, want, dt, "stream-K: dense + fc2 + residual")
+    wg, wu = w[0::2], w[1::2]
+    got = down(R.linear_packed(xd, wd, act="silu", glu=True))
+    want = oo.mul(onn.silu(onn.linear(x, wg, None, dt), dt), onn.linear(x, wu, None, dt), dt)
+    assert_close(got, want, dt, "stream-K: silu(gate) * up")
+
+
+def test_gemm_streamk_refuses_where_it_does_not_apply(R, monkeypatch):
+    from rai_amd._lib import RaiHipError
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk")
+    x, w = up(np.zeros((512, 64), np.float32), "bf16"), up(np.zeros((512, 64), np.float32), "bf16")
+    with pytest.raises(RaiHipError):
+        R.linear(x, w)      # four tiles
+
+
 def test_gemm_dispatcher_picks_each_tile_by_itself(R, monkeypatch):
     # no override: 3072 x 3072 gives 144 tiles of 256 x 256 (the eight-wave tile), 4096 x 2048 gives 512 of 256 x 128,
     # 600 x 520 stays on 128 x 128; K = 64 is shorter than the prefetch depth of every one of them
