@@ -353,7 +353,7 @@ def run_gemm_tiles(args):
         return HipTensor.from_storage((a.view(np.uint32) >> 16).astype(np.uint16), "bf16")
 
     shapes = [(512, 17920, 2560), (512, 10240, 2560), (512, 7680, 2560), (512, 2560, 12800), (4096, 10240, 2560)]
-    tiles = ["128x128", "256x128", "256x256", "256x256x8w", "streamk", None]
+    tiles = ["128x128", "256x128", "256x256", "256x256x8w", "256x256x8wk64", "streamk", "streamk64", None]
     rows = []
     for m, n, k in shapes:
         x, b, out = rnd((m, k)), rnd((n,)), HipTensor.empty((m, n), "bf16")
@@ -375,9 +375,9 @@ def run_gemm_tiles(args):
                 dw = dws[turn[0] % len(dws)]
                 turn[0] += 1
                 _lib.check(lib.rai_hip_linear(0, C.byref(dx), C.byref(dw), C.byref(db), UNARY["new_gelu"], None, C.byref(do)))
-            if tile == "streamk" and lib.rai_hip_linear(0, C.byref(dx), C.byref(dws[0]), C.byref(db), UNARY["new_gelu"], None,
+            if tile is not None and lib.rai_hip_linear(0, C.byref(dx), C.byref(dws[0]), C.byref(db), UNARY["new_gelu"], None,
                                                         C.byref(do)) != 0:
-                continue        # the stream-K form does not apply to this shape
+                continue        # this form does not apply to the shape (stream-K, K tiles of 64 with K split)
             t = C.c_void_p()
             _lib.call("rai_hip_timer_create", 0, C.byref(t))
             for _ in range(10):

@@ -53,6 +53,11 @@ template <int BM, int BN, int PITCH, int WGN = 2> constexpr int gemm_lds_bytes()
   return tiles > staging ? tiles : staging;
 }
 
+// LDS of the LDS-DMA tile kernels: NS stages of 32 of K, or (NS == 2) two stages of 64.
+template <int BM, int BN, int NS, int WGN> constexpr int dma_lds_bytes() {
+  return gemm_lds_bytes<BM, BN, NS == 2 ? 64 : 32 * NS / 2, WGN>();
+}
+
 // Applies activation `act` to the elements of x[8] whose column n + e is >= from.  The switch on the
 // (block-uniform) activation sits outside the element loop, so only one activation's code runs.
 // The results are rounded to bf16 (relative step 2^-8), so tanh-GELU and SiLU are evaluated through the hardware
@@ -492,6 +497,145 @@ __device__ __forceinline__ void dma_tile_mainloop(const LinearArgs &a, uint16_t 
   __syncthreads();
 }
 
+// The same K loop with K tiles of 64: a tile row is 128 bytes in LDS and one load instruction moves 8 rows x 128 bytes,
+// so every request the L1 sends to L2 is a whole 128-byte line instead of half of one (the L2s deliver 1.7x the bytes
+// per clock that way with all CUs asking, measured with the loads alone), and there is one barrier per 64 of K.  Two
+// stages (the same 128 KB for a 256 x 256 tile as four stages of 32): stage s+1 is requested when stage s-1 has been
+// left by every wave, a whole stage of multiplies before it is needed.
+//   - 16-byte chunk c (0..7) of row r lives at chunk position c ^ (r & 7): the 8 lanes that fetch one row swap places
+//     within their 128-byte line, and the fragment reads (32 rows at one chunk index) spread over all banks;
+//   - fragment sets alternate F0 / F1 over the four K steps of a stage; the reads run one set ahead of the multiplies.
+template <int BM, int BN, int WGN>
+__device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint16_t *lds, int m0, int n0, int k_begin, int KT,
+                                                      int wave, int lane, f32x16 (&acc)[BM / 64][BN / (32 * WGN)]) {
+  constexpr int BK = 64;
+  constexpr int WM = BM / 2, WN = BN / WGN;
+  constexpr int MT = WM / 32, NT = WN / 32;
+  constexpr int NW = 2 * WGN;
+  constexpr int LA = BM / (8 * NW), LB = BN / (8 * NW);   // loads per wave per stage (8 rows each)
+  constexpr int STAGE = (BM + BN) * BK;
+  static_assert(LA + LB == 8, "the wait below names the load count of one stage");
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  const uint16_t *gpa[LA], *gpb[LB];
+#pragma unroll
+  for (int j = 0; j < LA; ++j) {
+    int m = m0 + (wave * LA + j) * 8 + lrow;
+    m = m < a.M ? m : a.M - 1;
+    gpa[j] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + lchunk * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < LB; ++j) {
+    int n = n0 + (wave * LB + j) * 8 + lrow;
+    n = n < a.N ? n : a.N - 1;
+    gpb[j] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + lchunk * 8;
+  }
+  typedef __attribute__((address_space(3))) void *lds_ptr;
+  auto issue = [&](int st, int buf) {
+    uint16_t *sa = lds + buf * STAGE + wave * LA * 8 * BK;
+    uint16_t *sb = lds + buf * STAGE + BM * BK + wave * LB * 8 * BK;
+#pragma unroll
+    for (int j = 0; j < LA; ++j)
+      __builtin_amdgcn_global_load_lds((const void *)(gpa[j] + st * BK), (lds_ptr)(sa + j * 8 * BK), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < LB; ++j)
+      __builtin_amdgcn_global_load_lds((const void *)(gpb[j] + st * BK), (lds_ptr)(sb + j * 8 * BK), 16, 0, 0);
+  };
+
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  issue(0, 0);
+  if (KT > 1) {
+    issue(1, 1);
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // stage 0 has landed (this wave's part)
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  __builtin_amdgcn_s_barrier();
+
+  const int frow = (lane & 31) * BK, sw = lane & 7, hi = lane >> 5;
+  int coff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) coff[ks] = ((ks * 2 + hi) ^ sw) << 3;
+  const int a_off = wm * WM * BK + frow, b_off = BM * BK + wn * WN * BK + frow;
+  bf16x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];
+#define RAI_K64_READ(FA, FB, BUF, KS)                                                                     \
+  do {                                                                                                    \
+    const uint16_t *as_ = lds + (BUF) * STAGE + a_off + coff[KS], *bs_ = lds + (BUF) * STAGE + b_off + coff[KS]; \
+    _Pragma("unroll") for (int i = 0; i < MT; ++i) FA[i] = *reinterpret_cast<const bf16x8 *>(as_ + i * 32 * BK); \
+    _Pragma("unroll") for (int j = 0; j < NT; ++j) FB[j] = *reinterpret_cast<const bf16x8 *>(bs_ + j * 32 * BK); \
+  } while (0)
+#define RAI_K64_MUL(FA, FB)                                                                    \
+  do {                                                                                         \
+    _Pragma("unroll") for (int i = 0; i < MT; ++i)                                             \
+      _Pragma("unroll") for (int j = 0; j < NT; ++j)                                           \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[i], FB[j], acc[i][j], 0, 0, 0); \
+  } while (0)
+  // one LDS read between every MT*NT/(MT+NT) multiplies: a wave issues in order, so whatever sits between two
+  // batches of MFMAs runs with the matrix pipe idle
+#define RAI_K64_MIX_READS()                                                                                \
+  do {                                                                                                     \
+    _Pragma("unroll") for (int g = 0; g < MT + NT; ++g) {                                                  \
+      __builtin_amdgcn_sched_group_barrier(0x008, MT * NT / (MT + NT) > 0 ? MT * NT / (MT + NT) : 1, 0);   \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                   \
+    }                                                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                     \
+  } while (0)
+  RAI_K64_READ(fa0, fb0, 0, 0);
+  // Every stage but the last in one straight-line block (a branch around the multiplies would split the
+  // scheduling region and leave copies of the accumulators at the join).
+  for (int st = 0; st + 1 < KT; ++st) {
+    const int cur = st & 1;
+    RAI_K64_READ(fa1, fb1, cur, 1);
+    RAI_K64_MUL(fa0, fb0);
+    RAI_K64_MIX_READS();
+    RAI_K64_READ(fa0, fb0, cur, 2);
+    RAI_K64_MUL(fa1, fb1);
+    RAI_K64_MIX_READS();
+    RAI_K64_READ(fa1, fb1, cur, 3);
+    RAI_K64_MUL(fa0, fb0);
+    RAI_K64_MIX_READS();
+    // stage st+1 has landed (requested a stage ago) and this wave's reads of stage st are done: after the barrier
+    // stage st belongs to the loads of stage st+2 (past the end: the last stage once more, into a buffer nobody reads)
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    issue(st + 2 < KT ? st + 2 : KT - 1, cur);
+    RAI_K64_READ(fa0, fb0, cur ^ 1, 0);
+    RAI_K64_MUL(fa1, fb1);
+#pragma unroll
+    for (int g = 0; g < MT + NT; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global -> LDS load
+      __builtin_amdgcn_sched_group_barrier(0x008, MT * NT / (MT + NT) > 1 ? MT * NT / (MT + NT) - 1 : 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    const int cur = (KT - 1) & 1;
+    RAI_K64_READ(fa1, fb1, cur, 1);
+    RAI_K64_MUL(fa0, fb0);
+    RAI_K64_MIX_READS();
+    RAI_K64_READ(fa0, fb0, cur, 2);
+    RAI_K64_MUL(fa1, fb1);
+    RAI_K64_MIX_READS();
+    RAI_K64_READ(fa1, fb1, cur, 3);
+    RAI_K64_MUL(fa0, fb0);
+    RAI_K64_MIX_READS();
+    RAI_K64_MUL(fa1, fb1);
+  }
+#undef RAI_K64_READ
+#undef RAI_K64_MUL
+#undef RAI_K64_MIX_READS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+}
+
 template <int BM, int BN, int NS, int SH, int WGN = 2>
 __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
   // block = 2 x WGN waves.  WGN = 4 (eight waves, wave tile (BM/2) x (BN/4)) keeps two waves on every SIMD: one
@@ -513,9 +657,12 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, 
   const int KT = (k_end - k_begin) / BK;
 
   f32x16 acc[BM / 64][BN / (32 * WGN)];
-  dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, k_begin, KT, wave, lane, acc);
-  gemm_tile_epilogue<BM, BN, gemm_lds_bytes<BM, BN, PITCH * NS / 2, WGN>(), WGN>(a, acc, lds, m0, n0, wave, lane, split,
-                                                                                 partial);
+  if constexpr (NS == 2) {   // two stages of 64 (the launcher sends only K % 64 == 0, unsplit, here)
+    dma_tile_mainloop_k64<BM, BN, WGN>(a, lds, m0, n0, k_begin, KT / 2, wave, lane, acc);
+  } else {
+    dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, k_begin, KT, wave, lane, acc);
+  }
+  gemm_tile_epilogue<BM, BN, dma_lds_bytes<BM, BN, NS, WGN>(), WGN>(a, acc, lds, m0, n0, wave, lane, split, partial);
 }
 
 // ---- stream-K form of the eight-wave 256x256 tile kernel ---------------------------------------------------------
@@ -543,9 +690,9 @@ __device__ __forceinline__ int sk_block_of(const StreamKArgs &k, int u) {
 
 template <int BM, int BN, int NS, int SH, int WGN>
 __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma_streamk(LinearArgs a, StreamKArgs sk) {
-  constexpr int BK = 32, PITCH = BK;
+  constexpr int BK = NS == 2 ? 64 : 32;   // the unit of sharing is one K tile of the main loop
   constexpr int MT = BM / 64, NT = BN / (32 * WGN);
-  constexpr int LDS_BYTES = gemm_lds_bytes<BM, BN, PITCH * NS / 2, WGN>();
+  constexpr int LDS_BYTES = dma_lds_bytes<BM, BN, NS, WGN>();
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   __shared__ int s_ticket;
 
@@ -581,7 +728,11 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma_streamk(Linear
     tile_coords(tile, tiles_m, tiles_n, &tile_m, &tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     __syncthreads();   // the previous segment's epilogue staging is done with the LDS
-    dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, kt0 * BK, kt1 - kt0, wave, lane, acc);
+    if constexpr (NS == 2) {
+      dma_tile_mainloop_k64<BM, BN, WGN>(a, lds, m0, n0, kt0 * BK, kt1 - kt0, wave, lane, acc);
+    } else {
+      dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, kt0 * BK, kt1 - kt0, wave, lane, acc);
+    }
     if (kt1 - kt0 != KT) {
       // a share of the tile: which slot is ours, and how many there are
       const int first = sk_block_of(sk, tile * KT), last = sk_block_of(sk, tile * KT + KT - 1);
@@ -857,7 +1008,7 @@ template <int BM, int BN, int BK, int SH = 0> static int launch_cfg(hipStream_t 
 
 template <int BM, int BN, int NS, int SH, int WGN = 2>
 static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
-  constexpr size_t lds = gemm_lds_bytes<BM, BN, 32 * NS / 2, WGN>();
+  constexpr size_t lds = dma_lds_bytes<BM, BN, NS, WGN>();
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN>,
@@ -890,11 +1041,11 @@ struct StreamKPlan {
   StreamKArgs k;
   size_t ws_bytes;
 };
-static bool streamk_plan(int M, int N, int K, StreamKPlan *plan, bool forced = false) {
-  const int P = kNumCU, KT = K / 32;
+static bool streamk_plan(int M, int N, int K, int bk, StreamKPlan *plan, bool forced = false) {
+  const int P = kNumCU, KT = K / bk;
   const int T = ((M + 255) / 256) * ((N + 255) / 256);
   const int full = T / P, left = T % P;
-  if (left == 0 || KT < 8) return false;
+  if (left == 0 || K / 32 < 8) return false;
   int sk_tiles = left;
   if (left < P / 2) {
     if (full == 0) return false;
@@ -921,7 +1072,7 @@ static bool streamk_plan(int M, int N, int K, StreamKPlan *plan, bool forced = f
   // for the exchange; 512 x 17920 x 2560 (three shares, 36 saved) 81 -> 84 us, i.e. ~39 us: every block ends on a
   // read of the other shares plus the epilogue, with nothing left to hide them behind.  One K tile of a 256 x 256
   // tile takes ~1 us with all CUs busy.
-  const float saved_us = (float)(P - left) / P * KT * 1.0f;
+  const float saved_us = (float)(P - left) / P * (K / 32) * 1.0f;
   const float exchange_us = max_parts <= 2 ? 18.f : 39.f;
   if (!forced && saved_us < 1.3f * exchange_us) return false;
   k.max_parts = max_parts;
@@ -934,20 +1085,21 @@ static bool streamk_plan(int M, int N, int K, StreamKPlan *plan, bool forced = f
 
 size_t linear_streamk_workspace_bytes(int M, int N, int K) {
   StreamKPlan plan;
-  return streamk_plan(M, N, K, &plan) ? plan.ws_bytes : 0;
+  return streamk_plan(M, N, K, 32, &plan) ? plan.ws_bytes : 0;
 }
 
 // True when the stream-K kernel serves this Linear (plain tile epilogue, workspace large enough, not switched off).
-static bool streamk_applies(const LinearArgs &a, StreamKPlan *plan, bool forced = false) {
+static bool streamk_applies(const LinearArgs &a, int bk, StreamKPlan *plan, bool forced = false) {
   const char *off = getenv("RAI_HIP_NO_STREAMK");   // read per call: tests compare both forms in one process
   if (off && *off && *off != '0') return false;
   if (!a.splitk_ws || ((uintptr_t)a.splitk_ws & 15) || a.post_ln_out) return false;
-  return streamk_plan(a.M, a.N, a.K, plan, forced) && plan->ws_bytes <= a.splitk_ws_bytes;
+  return a.K % bk == 0 && streamk_plan(a.M, a.N, a.K, bk, plan, forced) && plan->ws_bytes <= a.splitk_ws_bytes;
 }
 
+template <int NS>
 static int launch_streamk(hipStream_t st, const LinearArgs &a, StreamKPlan plan) {
-  constexpr int BM = 256, BN = 256, NS = 4, SH = 2, WGN = 4;
-  constexpr size_t lds = gemm_lds_bytes<BM, BN, 32 * NS / 2, WGN>();
+  constexpr int BM = 256, BN = 256, SH = 2, WGN = 4;
+  constexpr size_t lds = dma_lds_bytes<BM, BN, NS, WGN>();
   static bool attr_set = false;
   if (!attr_set) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma_streamk<BM, BN, NS, SH, WGN>,
@@ -1448,11 +1600,17 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
     if (!strcmp(knob, "256x256x8w")) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
-    if (!strcmp(knob, "streamk")) {
+    if (!strcmp(knob, "256x256x8wk64")) {
+      RAI_REQUIRE(splits == 1 && a.K % 64 == 0, RAI_ERR_UNSUPPORTED,
+                  "linear: RAI_HIP_GEMM_TILE=256x256x8wk64 needs K %% 64 == 0 and no K split (%dx%dx%d)", a.M, a.N, a.K);
+      return launch_cfg_dma<256, 256, 2, 0, 4>(st, a, splits);
+    }
+    if (!strcmp(knob, "streamk") || !strcmp(knob, "streamk64")) {
+      const int bk = knob[7] ? 64 : 32;
       StreamKPlan plan;
-      RAI_REQUIRE(splits == 1 && streamk_applies(a, &plan, true), RAI_ERR_UNSUPPORTED,
-                  "linear: RAI_HIP_GEMM_TILE=streamk does not apply to %dx%dx%d", a.M, a.N, a.K);
-      return launch_streamk(st, a, plan);
+      RAI_REQUIRE(splits == 1 && streamk_applies(a, bk, &plan, true), RAI_ERR_UNSUPPORTED,
+                  "linear: RAI_HIP_GEMM_TILE=%s does not apply to %dx%dx%d", knob, a.M, a.N, a.K);
+      return bk == 64 ? launch_streamk<2>(st, a, plan) : launch_streamk<4>(st, a, plan);
     }
   }
   const int big_tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
@@ -1464,9 +1622,12 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   // (140 tiles) 689 against 621; with 128 tiles or fewer the smaller tiles win (4096 x 2048 x 2048: 618 against 760).
   // The four-wave 256x256 form is 3-9 % behind the eight-wave one everywhere.
   if (splits == 1 && 32 * huge_tiles >= 17 * kNumCU) {
+    // K tiles of 64 (whole 128-byte lines per request) where K allows; RAI_HIP_NO_K64 keeps the tiles of 32
+    const char *no64 = getenv("RAI_HIP_NO_K64");
+    const bool k64 = a.K % 64 == 0 && !(no64 && *no64 && *no64 != '0');
     StreamKPlan plan;
-    if (streamk_applies(a, &plan)) return launch_streamk(st, a, plan);
-    return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
+    if (streamk_applies(a, k64 ? 64 : 32, &plan)) return k64 ? launch_streamk<2>(st, a, plan) : launch_streamk<4>(st, a, plan);
+    return k64 ? launch_cfg_dma<256, 256, 2, 0, 4>(st, a, splits) : launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   }
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
   return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);

@@ -225,16 +225,18 @@ def test_gemm_tile_gated_mlp(R, monkeypatch, tile, act, k_splits):
 STREAMK_SHAPES = [(3000, 3100, 2560), (2100, 5000, 512), (4400, 4600, 320), (5000, 9000, 256)]
 
 
+# "streamk64" / "256x256x8wk64": the same with K tiles of 64 (two LDS stages, 128-byte rows), K % 64 == 0
+@pytest.mark.parametrize("form,whole_tile", [("streamk", "256x256x8w"), ("streamk64", "256x256x8wk64")])
 @pytest.mark.parametrize("m,n,k", STREAMK_SHAPES)
-def test_gemm_streamk_plain_and_fused_epilogue(R, monkeypatch, m, n, k):
-    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk")   # refuses (RAI_ERR_UNSUPPORTED) where the form does not apply
+def test_gemm_streamk_plain_and_fused_epilogue(R, monkeypatch, m, n, k, form, whole_tile):
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", form)   # refuses (RAI_ERR_UNSUPPORTED) where the form does not apply
     dt = "bf16"
     x, w, b1, _, r = packed_case(rng(120), m, n, k)
     xd, wd = up(x, dt), up(w, dt)
     lin = onn.linear(x, w, None, dt)
     first = down(R.linear(xd, wd))
-    assert_close(first, lin, dt, f"stream-K linear {m}x{n}x{k}")
-    gemm_elem_check(first, lin, dt, k, f"stream-K linear {m}x{n}x{k}")
+    assert_close(first, lin, dt, f"{form} linear {m}x{n}x{k}")
+    gemm_elem_check(first, lin, dt, k, f"{form} linear {m}x{n}x{k}")
     # the shares are summed in slot order whoever arrives last: every run gives the same bits
     for _ in range(3):
         assert np.array_equal(down(R.linear(xd, wd)), first)
@@ -242,12 +244,16 @@ def test_gemm_streamk_plain_and_fused_epilogue(R, monkeypatch, m, n, k):
     got = down(R.linear(xd, wd, up(b1, dt), "new_gelu", up(r, dt)))
     assert_close(got, want, dt, f"stream-K linear + bias + new_gelu + residual {m}x{n}x{k}")
     # against the same tile without sharing: same products, another grouping of the f32 sums
-    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "256x256x8w")
-    gemm_elem_check(first, down(R.linear(xd, wd)), dt, k, f"stream-K against whole tiles {m}x{n}x{k}")
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", whole_tile)
+    whole = down(R.linear(xd, wd))
+    assert_close(whole, lin, dt, f"{whole_tile} linear {m}x{n}x{k}")
+    gemm_elem_check(whole, lin, dt, k, f"{whole_tile} linear {m}x{n}x{k}")
+    gemm_elem_check(first, whole, dt, k, f"stream-K against whole tiles {m}x{n}x{k}")
 
 
-def test_gemm_streamk_packed_epilogues(R, monkeypatch):
-    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk")
+@pytest.mark.parametrize("form", ["streamk", "streamk64", "256x256x8wk64"])
+def test_gemm_streamk_packed_epilogues(R, monkeypatch, form):
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", form)
     dt, m, n, k, n1 = "bf16", 2100, 4936, 640, 2421      # 180 tiles; n1 odd: second output rows not 16-byte aligned
     x, w, b1, b2, r = packed_case(rng(121), m, n, k)
     xd, wd = up(x, dt), up(w, dt)
