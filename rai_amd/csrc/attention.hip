@@ -479,7 +479,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t ad_u32x4;
 template <int D, int CH>
 __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeArgs a) {
   typedef bf16_raw T;
-  constexpr int KS = D / 32, KT = CH / 64;
+  constexpr int KS = D / 32, KT = (CH + 63) / 64;  // 16-key tiles per wave (CH = 96: the last tile of waves 2, 3 is empty)
   constexpr int VP = D + 8, PP = CH + 8;           // LDS pitches (bf16 elements)
   constexpr int CPR = D / 8;                        // 16-byte chunks per K/V row
   constexpr int VL = CH * CPR / kDecodeThreads;     // V chunks per thread
@@ -521,10 +521,11 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeA
 #pragma unroll
   for (int i = 0; i < KT; ++i) {
     const int t = t0 + (wave + 4 * i) * 16 + lrow;
+    const bool tile_ok = (wave + 4 * i) * 16 < CH;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       ad_bf16x8 z = {};
-      if (t < t1c) z = *reinterpret_cast<const ad_bf16x8 *>(Kc + (int64_t)t * D + ks * 32 + lq * 8);
+      if (tile_ok && t < t1c) z = *reinterpret_cast<const ad_bf16x8 *>(Kc + (int64_t)t * D + ks * 32 + lq * 8);
       kreg[i][ks] = z;
     }
   }
@@ -608,6 +609,7 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeA
 #pragma unroll
     for (int i = 0; i < KT; ++i) {
       const int tile = wave + 4 * i;
+      if (tile * 16 >= CH) continue;
       if (has_new && new_row == tile * 16 + lrow) {   // the lanes that hold the new token's key row
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) kreg[i][ks] = *reinterpret_cast<const ad_bf16x8 *>(knew + ks * 32 + lq * 8);
@@ -729,13 +731,33 @@ template <int D, int CH> static int launch_decode_mfma_cfg(hipStream_t st, AttnD
   return launch_check("attention_decode_merge");
 }
 
-// Blocks of 64 keys (four or more per CU) while the longest context fits
-// kDecodeMaxSplits of them, else blocks of 128 keys.
+// Keys per block: 64, 96 or 128.  Every block issues all its loads up front and a CU holds as many blocks as their LDS
+// allows, so what counts is the number of rounds the blocks need on the chip: a few blocks more than one round (1056
+// blocks of 64 keys on 1024 places, Gemma-2B at batch 32 just past 2048 tokens) cost a whole block time.  Fewest
+// rounds wins, then the smaller block.
 constexpr int kMfmaDecodeKeysMax = 128;
+template <int D> static size_t decode_mfma_lds(int CH, int R) {
+  return (size_t)CH * (D + 8) * 2 + (size_t)R * CH * 4 + 16 * (CH + 8) * 2 + 2 * D * 2;
+}
 template <int D> static int launch_decode_mfma(hipStream_t st, const AttnDecodeArgs &a) {
-  const char *knob = getenv("RAI_HIP_ATTN_KEYS");  // tuning and test aid: 64 or 128 keys per block
+  const char *knob = getenv("RAI_HIP_ATTN_KEYS");  // tuning and test aid: 64, 96 or 128 keys per block
   const int forced = knob ? atoi(knob) : 0;
-  if (forced != 128 && (a.Tmax + 63) / 64 <= kDecodeMaxSplits) return launch_decode_mfma_cfg<D, 64>(st, a);
+  const int R = a.Hq / a.Hkv;
+  int best = 0, best_rounds = 0;
+  for (int ch : {64, 96, 128}) {
+    const int need = (a.Tmax + ch - 1) / ch;
+    if (need > kDecodeMaxSplits) continue;
+    int ns = decode_splits(a, a.Hkv);
+    if (ns < need) ns = need;
+    const long long blocks = (long long)ns * a.Hkv * a.B;
+    const long long per_cu = (long long)((160 * 1024) / (decode_mfma_lds<D>(ch, R) + 256));
+    const long long places = (per_cu < 1 ? 1 : per_cu) * kNumCU;
+    const int rounds = (int)((blocks + places - 1) / places);
+    if (forced == ch) { best = ch; break; }
+    if (!best || rounds < best_rounds) { best = ch; best_rounds = rounds; }
+  }
+  if (best == 64) return launch_decode_mfma_cfg<D, 64>(st, a);
+  if (best == 96) return launch_decode_mfma_cfg<D, 96>(st, a);
   return launch_decode_mfma_cfg<D, 128>(st, a);
 }
 

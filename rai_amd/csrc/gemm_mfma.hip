@@ -15,6 +15,7 @@
 //     and writes 16-byte rows with bias / activation / residual applied (or raw
 //     f32 partial sums when K is split over several blocks).
 #include <cstring>
+#include <type_traits>
 
 #include "gemm.h"
 
@@ -71,10 +72,11 @@ __device__ __forceinline__ float act_eval_bf16_out(int act, float x) {
   if (act == RAI_UN_SILU) return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
   return act_eval(act, x);
 }
-__device__ __forceinline__ void act8(int act, float (&x)[8], int n, int from) {
+template <int N>
+__device__ __forceinline__ void act_n(int act, float (&x)[N], int n, int from) {
 #define RAI_ACT_CASE(K)                                     \
   case K:                                                   \
-    _Pragma("unroll") for (int e = 0; e < 8; ++e)           \
+    _Pragma("unroll") for (int e = 0; e < N; ++e)           \
       if (n + e >= from) x[e] = act_eval_bf16_out(K, x[e]); \
     break;
   switch (act) {
@@ -87,6 +89,7 @@ __device__ __forceinline__ void act8(int act, float (&x)[8], int n, int from) {
   }
 #undef RAI_ACT_CASE
 }
+__device__ __forceinline__ void act8(int act, float (&x)[8], int n, int from) { act_n<8>(act, x, n, from); }
 __device__ __forceinline__ void unpack8(const u32x4 &p, float (&f)[8]) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) f[e] = bf16_bits_to_f32((uint16_t)(p[e >> 1] >> (16 * (e & 1))));
@@ -176,16 +179,15 @@ __device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (
       }
       if (a.glu) {  // columns n..n+7 are four (gate, up) pairs -> four outputs at column n/2
         uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
-        float gr[8], ga[8];
+        float gr[8], ga[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          gr[e] = bf16_bits_to_f32(f32_to_bf16_bits(v[e] + bv[e]));  // gate / up rounded to bf16 as the reference does
-          ga[e] = gr[e];
-        }
-        act8(a.act, ga, 0, 0);   // evaluated on all eight; only the gates (even e) are used
+        for (int e = 0; e < 8; ++e) gr[e] = bf16_bits_to_f32(f32_to_bf16_bits(v[e] + bv[e]));  // gate / up rounded to bf16 as the reference does
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ga[e] = gr[2 * e];
+        act_n<4>(a.act, ga, 0, 0);   // the four gates
         float gl[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) gl[e] = bf16_bits_to_f32(f32_to_bf16_bits(ga[2 * e])) * gr[2 * e + 1];
+        for (int e = 0; e < 4; ++e) gl[e] = bf16_bits_to_f32(f32_to_bf16_bits(ga[e])) * gr[2 * e + 1];
         if (whole && a.ld1 % 4 == 0 && (uintptr_t)a.out1 % 8 == 0) {
           typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
           u32x2 o = {pack_bf16x2(gl[0], gl[1]), pack_bf16x2(gl[2], gl[3])};
@@ -1305,7 +1307,8 @@ template <int MT, int KS, int G, bool FRAG>
 __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, int tiles, float *partial) {
   constexpr int NW = 8;
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  f32x4 *red = reinterpret_cast<f32x4 *>(lds);        // [NW][G*MT][64]
+  constexpr int PCH = 4 * G + 1;                       // row pitch of the parked accumulators, in f32x4
+  f32x4 *red = reinterpret_cast<f32x4 *>(lds);        // [NW][MT * 16 rows][PCH]
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane & 15, lq = lane >> 4;
   const int split = blockIdx.y;
@@ -1369,96 +1372,141 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
   const bf16x8 *fbase = reinterpret_cast<const bf16x8 *>(a.Wfrag) + lane;
   const int ksteps = a.K / 32;
 
-  bf16x8 wa[KS], wb[KS];
-  auto load_tile = [&](bf16x8 (&w)[KS], int tile) {
+  // A ring of tile buffers: while tile t is multiplied, the next RING-1 tiles are in flight.  Long streams (four
+  // tiles per group, i.e. at least four tiles per block) take three buffers and loads that bypass the caches
+  // (measured on a 1 GB matrix: 232 -> 193 us); short ones keep two buffers and cached loads, which a 10 MB matrix on
+  // 160 blocks prefers by 1-2 us.  The ring turns by G positions per group, so the group body exists in RING rotations.
+  constexpr int RING = G >= 4 ? 3 : 2;
+  constexpr bool NT = G >= 4;
+  bf16x8 w[RING][KS];
+  auto load_tile = [&](bf16x8 (&wt)[KS], int tile) {
     tile = tile < tiles ? tile : tiles - 1;
     if constexpr (FRAG) {   // one instruction reads 1 KB of consecutive memory
       const bf16x8 *p = fbase + (int64_t)tile * ksteps * 64;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) w[ks] = p[(koff[ks] >> 5) * 64];
+      for (int ks = 0; ks < KS; ++ks) wt[ks] = NT ? __builtin_nontemporal_load(p + (koff[ks] >> 5) * 64) : p[(koff[ks] >> 5) * 64];
     } else {
       int n = tile * 16 + lrow;
       n = n < a.N ? n : a.N - 1;
       const uint16_t *p = wbase + (int64_t)n * a.ldw;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) w[ks] = *reinterpret_cast<const bf16x8 *>(p + koff[ks]);
+      for (int ks = 0; ks < KS; ++ks)
+        wt[ks] = NT ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8 *>(p + koff[ks])) : *reinterpret_cast<const bf16x8 *>(p + koff[ks]);
     }
     // keep the whole tile's loads together and ahead of the multiplies that follow: left alone,
     // the scheduler sinks each load to just before its use and the prefetch distance collapses
     __builtin_amdgcn_sched_barrier(0);
   };
   const int stride = gridDim.x * G;
-  int g0 = blockIdx.x * G;
-  load_tile(wa, g0);
-  for (; g0 < tiles; g0 += stride) {
+  // tile at position pos (0 .. G + RING - 2) counted from the start of the group that begins at tile g0
+  auto tile_at = [&](int g0, int pos) { return g0 + (pos / G) * stride + pos % G; };
+  const uint16_t *bias = (const uint16_t *)a.bias;
+  const uint16_t *bias2 = (const uint16_t *)a.bias2;
+  const uint16_t *res = (const uint16_t *)a.residual;
+  auto group = [&](auto rot, const int g0) {
+    constexpr int R = decltype(rot)::value;
     f32x4 acc[G][MT];
 #pragma unroll
     for (int j = 0; j < G; ++j)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < G; j += 2) {
-      if (G > 1) load_tile(wb, g0 + j + 1);
-      else load_tile(wb, g0 + stride);
+    for (int j = 0; j < G; ++j) {
+      load_tile(w[(R + j + RING - 1) % RING], tile_at(g0, j + RING - 1));
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ks], xf[mt][ks], acc[j][mt], 0, 0, 0);
+          acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[(R + j) % RING][ks], xf[mt][ks], acc[j][mt], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      if (G > 1) {
-        load_tile(wa, j + 2 < G ? g0 + j + 2 : g0 + stride);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[j + 1 < G ? j + 1 : j][mt] =
-                __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[ks], xf[mt][ks], acc[j + 1 < G ? j + 1 : j][mt], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      } else {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) wa[ks] = wb[ks];
-      }
     }
-    // ---- sum the eight K slices and write G tiles of 16 columns x 16*MT rows
+    // ---- sum the eight K slices and write G tiles of 16 columns x 16*MT rows.
+    // Every wave parks its accumulators as [row m][G tiles x 4 column quads] (pitch PCH = 4 G + 1 chunks of 16 bytes,
+    // odd, so that the 16 lanes of a quad, one row each, hit distinct banks); a thread then owns four consecutive
+    // columns of one row: eight 16-byte reads, one store of four bf16, and 16 neighbouring threads cover 64 columns of
+    // a row.  (One 4-byte read per wave and element and 2-byte stores a row apart took as long as streaming the
+    // group's weights.)
     __syncthreads();   // the previous group's sums have been read
 #pragma unroll
     for (int j = 0; j < G; ++j)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) red[(wave * G * MT + j * MT + mt) * 64 + lane] = acc[j][mt];
+      for (int mt = 0; mt < MT; ++mt) red[(wave * MT * 16 + mt * 16 + lrow) * PCH + j * 4 + lq] = acc[j][mt];
     __syncthreads();
-    const float *redf = reinterpret_cast<const float *>(red);
-    const uint16_t *bias = (const uint16_t *)a.bias;
-    const uint16_t *bias2 = (const uint16_t *)a.bias2;
-    const uint16_t *res = (const uint16_t *)a.residual;
-    for (int v = tid; v < G * MT * 256; v += 512) {
-      const int slot = v >> 8, rem = v & 255, ln = rem >> 2, r = rem & 3;
-      const int j = slot / MT, mt = slot - j * MT;
-      const int tile = g0 + j;
-      const int n = tile * 16 + 4 * (ln >> 4) + r, m = mt * 16 + (ln & 15);
+    for (int v = tid; v < MT * G * 64; v += 512) {
+      const int m = v / (G * 4), c = v - m * (G * 4);
+      const int tile = g0 + (c >> 2);
+      const int n = tile * 16 + 4 * (c & 3);
       if (tile >= tiles || n >= a.N || m >= a.M) continue;
-      float x = 0.f;
+      f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < NW; ++w) x += redf[(w * G * MT + slot) * 256 + rem];
+      for (int w = 0; w < NW; ++w) {
+        const f32x4 t = red[(w * MT * 16 + m) * PCH + c];
+        s4.x += t.x; s4.y += t.y; s4.z += t.z; s4.w += t.w;
+      }
+      float x[4] = {s4.x, s4.y, s4.z, s4.w};
+      const int lim = a.N - n < 4 ? a.N - n : 4;
       if (partial) {
-        partial[((int64_t)split * a.M + m) * a.N + n] = x;
-        continue;
-      }
-      if (a.glu) {   // columns (n, n+1) are a (gate, up) pair
-        if (r & 1) continue;
-        float u = 0.f;
+        float *p = partial + ((int64_t)split * a.M + m) * a.N + n;
+        if (lim == 4 && a.N % 4 == 0) *reinterpret_cast<f32x4 *>(p) = s4;
+        else {
 #pragma unroll
-        for (int w = 0; w < NW; ++w) u += redf[(w * G * MT + slot) * 256 + rem + 1];
-        x += bias ? bf16_bits_to_f32(bias[n]) : 0.f;
-        u += bias ? bf16_bits_to_f32(bias[n + 1]) : 0.f;
-        ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + (n >> 1)] = f32_to_bf16_bits(glu_bf16(a.act, x, u));
+          for (int e = 0; e < 4; ++e)
+            if (e < lim) p[e] = x[e];
+        }
         continue;
       }
-      x += (bias ? bf16_bits_to_f32(bias[n]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[n]) : 0.f);
-      if (a.act >= 0 && n >= a.act_from) x = act_eval(a.act, x);
-      if (res) x += bf16_bits_to_f32(res[(int64_t)m * a.ldr + n]);
-      if (n < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + n] = f32_to_bf16_bits(x);
-      else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (n - a.n_split)] = f32_to_bf16_bits(x);
+      if (a.glu) {   // columns (n, n+1) and (n+2, n+3) are (gate, up) pairs (N is a multiple of 8)
+        uint16_t o[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const float gt = x[2 * e] + (bias ? bf16_bits_to_f32(bias[n + 2 * e]) : 0.f);
+          const float up = x[2 * e + 1] + (bias ? bf16_bits_to_f32(bias[n + 2 * e + 1]) : 0.f);
+          o[e] = f32_to_bf16_bits(glu_bf16(a.act, gt, up));
+        }
+        uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
+        if (((uintptr_t)dst & 3) == 0) *reinterpret_cast<uint32_t *>(dst) = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+        else { dst[0] = o[0]; dst[1] = o[1]; }
+        continue;
+      }
+      uint16_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int nn = e < lim ? n + e : n;
+        float y = x[e] + ((bias ? bf16_bits_to_f32(bias[nn]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[nn]) : 0.f));
+        if (a.act >= 0 && nn >= a.act_from) y = act_eval(a.act, y);
+        if (res) y += bf16_bits_to_f32(res[(int64_t)m * a.ldr + nn]);
+        o[e] = f32_to_bf16_bits(y);
+      }
+      // all four columns in one output and the destination 8-byte aligned: one store
+      const bool first = n + 3 < a.n_split, second = n >= a.n_split;
+      uint16_t *dst = second ? (uint16_t *)a.out2 + (int64_t)m * a.ld2 + (n - a.n_split) : (uint16_t *)a.out1 + (int64_t)m * a.ld1 + n;
+      if (lim == 4 && (first || second) && ((uintptr_t)dst & 7) == 0) {
+        typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+        const u32x2 pk = {(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+        *reinterpret_cast<u32x2 *>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (e < lim) {
+            const int nn = n + e;
+            if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = o[e];
+            else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = o[e];
+          }
+        }
+      }
+    }
+  };
+  int g0 = blockIdx.x * G;
+#pragma unroll
+  for (int pos = 0; pos + 1 < RING; ++pos) load_tile(w[pos], tile_at(g0, pos));
+  for (;;) {
+    group(std::integral_constant<int, 0>{}, g0);
+    if ((g0 += stride) >= tiles) break;
+    group(std::integral_constant<int, G % RING>{}, g0);
+    if ((g0 += stride) >= tiles) break;
+    if constexpr (RING == 3) {
+      group(std::integral_constant<int, (2 * G) % RING>{}, g0);
+      if ((g0 += stride) >= tiles) break;
     }
   }
 }
@@ -1473,7 +1521,7 @@ static int launch_mfma_stream_cfg(hipStream_t st, const LinearArgs &a, int split
   int blocks_x = kNumCU / splits;
   if (blocks_x < 1) blocks_x = 1;
   if (blocks_x > groups) blocks_x = groups;
-  const size_t lds = (size_t)8 * G * MT * 64 * sizeof(f32x4);
+  const size_t lds = (size_t)8 * MT * 16 * (4 * G + 1) * sizeof(f32x4);
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_mfma_stream<MT, KS, G, FRAG>,

@@ -121,7 +121,7 @@ GQA_CFGS = {
 }
 
 
-@pytest.mark.parametrize("splits,keys", [(None, None), ("2", None), ("2", "128"), ("5", "128")])
+@pytest.mark.parametrize("splits,keys", [(None, None), ("2", None), ("2", "128"), ("5", "128"), ("2", "96"), ("4", "96")])
 @pytest.mark.parametrize("name", list(GQA_CFGS))
 def test_grouped_query_decode_attention_long_context(hip, name, splits, keys, monkeypatch):
     # context long enough that one block holds several 16-key tiles (few splits) or a handful of keys
