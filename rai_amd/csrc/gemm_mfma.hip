@@ -504,8 +504,10 @@ __device__ __forceinline__ void dma_tile_mainloop(const LinearArgs &a, uint16_t 
 // per clock that way with all CUs asking, measured with the loads alone), and there is one barrier per 64 of K.  Two
 // stages (the same 128 KB for a 256 x 256 tile as four stages of 32): stage s+1 is requested when stage s-1 has been
 // left by every wave, a whole stage of multiplies before it is needed.
-//   - 16-byte chunk c (0..7) of row r lives at chunk position c ^ (r & 7): the 8 lanes that fetch one row swap places
-//     within their 128-byte line, and the fragment reads (32 rows at one chunk index) spread over all banks;
+//   - 16-byte chunk c (0..7) of row r lives at chunk position c ^ ((r >> 1) & 7): the 8 lanes that fetch one row swap
+//     places within their 128-byte line, and a fragment read's 16 lanes per LDS cycle (16 rows at one chunk index; two
+//     rows span the 64 banks) land on 16 different 16-byte slots.  (Swizzling by r & 7 left rows r and r + 8 on the
+//     same banks: SQ_LDS_BANK_CONFLICT at 23 % of the kernel's cycles.)
 //   - fragment sets alternate F0 / F1 over the four K steps of a stage; the reads run one set ahead of the multiplies.
 template <int BM, int BN, int WGN>
 __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint16_t *lds, int m0, int n0, int k_begin, int KT,
@@ -518,19 +520,21 @@ __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint1
   constexpr int STAGE = (BM + BN) * BK;
   static_assert(LA + LB == 8, "the wait below names the load count of one stage");
   const int wm = wave / WGN, wn = wave % WGN;
-  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  const int lrow = lane >> 3;
   const uint16_t *gpa[LA], *gpb[LB];
 #pragma unroll
   for (int j = 0; j < LA; ++j) {
-    int m = m0 + (wave * LA + j) * 8 + lrow;
+    const int r = (wave * LA + j) * 8 + lrow;     // row within the tile
+    int m = m0 + r;
     m = m < a.M ? m : a.M - 1;
-    gpa[j] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + lchunk * 8;
+    gpa[j] = (const uint16_t *)a.A + (int64_t)m * a.lda + k_begin + (((lane & 7) ^ ((r >> 1) & 7)) << 3);
   }
 #pragma unroll
   for (int j = 0; j < LB; ++j) {
-    int n = n0 + (wave * LB + j) * 8 + lrow;
+    const int r = (wave * LB + j) * 8 + lrow;
+    int n = n0 + r;
     n = n < a.N ? n : a.N - 1;
-    gpb[j] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + lchunk * 8;
+    gpb[j] = (const uint16_t *)a.W + (int64_t)n * a.ldw + k_begin + (((lane & 7) ^ ((r >> 1) & 7)) << 3);
   }
   typedef __attribute__((address_space(3))) void *lds_ptr;
   auto issue = [&](int st, int buf) {
@@ -560,7 +564,7 @@ __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint1
   }
   __builtin_amdgcn_s_barrier();
 
-  const int frow = (lane & 31) * BK, sw = lane & 7, hi = lane >> 5;
+  const int frow = (lane & 31) * BK, sw = (lane >> 1) & 7, hi = lane >> 5;   // fragment rows start at multiples of 32
   int coff[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) coff[ks] = ((ks * 2 + hi) ^ sw) << 3;
