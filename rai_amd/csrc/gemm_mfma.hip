@@ -1026,9 +1026,10 @@ static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
   int k_per_split = a.K;
   float *partial = nullptr;
   if (splits > 1) {
-    const int k_tiles = a.K / 32, per = (k_tiles + splits - 1) / splits;
+    constexpr int KU = NS == 2 ? 64 : 32;   // K tile of the main loop
+    const int k_tiles = a.K / KU, per = (k_tiles + splits - 1) / splits;
     splits = (k_tiles + per - 1) / per;
-    k_per_split = per * 32;
+    k_per_split = per * KU;
     partial = (float *)a.splitk_ws;
   }
   hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN>), dim3(grid_x, splits), dim3(128 * WGN), lds, st, a, splits,
@@ -1611,6 +1612,11 @@ bool linear_fuses_post_norm(const LinearArgs &a) {
   return a.M > 64 && post_norm_fits(a) && tile_splits(a) > 1;
 }
 
+static bool no_k64() {   // read per call: tests compare both forms in one process
+  const char *e = getenv("RAI_HIP_NO_K64");
+  return e && *e && *e != '0';
+}
+
 int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   RAI_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, RAI_ERR_BAD_SHAPE, "linear: empty problem %dx%dx%d", a.M, a.N, a.K);
   RAI_REQUIRE(a.A && a.W && a.out1, RAI_ERR_BAD_ARG, "linear: null operand");
@@ -1652,6 +1658,10 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (!strcmp(knob, "256x256")) return launch_cfg_dma<256, 256, 4, 2>(st, a, splits);
     if (!strcmp(knob, "classic")) return launch_cfg<128, 128, 32>(st, a, splits);
     if (!strcmp(knob, "256x256x8w")) return launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
+    if (!strcmp(knob, "128x128k64")) {
+      RAI_REQUIRE(a.K % 64 == 0, RAI_ERR_UNSUPPORTED, "linear: RAI_HIP_GEMM_TILE=%s needs K %% 64 == 0 (%dx%dx%d)", knob, a.M, a.N, a.K);
+      return launch_cfg_dma<128, 128, 2, 0, 2>(st, a, splits);
+    }
     if (!strcmp(knob, "256x256x8wk64")) {
       RAI_REQUIRE(splits == 1 && a.K % 64 == 0, RAI_ERR_UNSUPPORTED,
                   "linear: RAI_HIP_GEMM_TILE=256x256x8wk64 needs K %% 64 == 0 and no K split (%dx%dx%d)", a.M, a.N, a.K);
@@ -1675,13 +1685,15 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   // The four-wave 256x256 form is 3-9 % behind the eight-wave one everywhere.
   if (splits == 1 && 32 * huge_tiles >= 17 * kNumCU) {
     // K tiles of 64 (whole 128-byte lines per request) where K allows; RAI_HIP_NO_K64 keeps the tiles of 32
-    const char *no64 = getenv("RAI_HIP_NO_K64");
-    const bool k64 = a.K % 64 == 0 && !(no64 && *no64 && *no64 != '0');
+    const bool k64 = a.K % 64 == 0 && !no_k64();
     StreamKPlan plan;
     if (streamk_applies(a, k64 ? 64 : 32, &plan)) return k64 ? launch_streamk<2>(st, a, plan) : launch_streamk<4>(st, a, plan);
     return k64 ? launch_cfg_dma<256, 256, 2, 0, 4>(st, a, splits) : launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   }
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
+  // 128 x 128 with two stages of K 64 (two blocks per CU) where K allows: 12-22 % over three stages of 32 on the
+  // prefill shapes with cold weights (512 x 10240 x 2560: 66 -> 55 us, 2048^3: 33 -> 26 us)
+  if (a.K % 64 == 0 && !no_k64()) return launch_cfg_dma<128, 128, 2, 0, 2>(st, a, splits);
   return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
 }
 

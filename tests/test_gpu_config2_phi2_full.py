@@ -14,7 +14,7 @@ import pytest
 from oracle import phi2
 from oracle.dtypes import to_storage
 from tests.test_gpu_phi2 import check_tokens
-from tests.util import assert_close, progress, synthetic_params
+from tests.util import assert_logits_close, progress, synthetic_params
 
 pytestmark = pytest.mark.gpu
 
@@ -37,19 +37,25 @@ def full(hip, request):
     progress(request, "uploading")
     for n in names:
         dec.load_param(n, to_storage(params[n], "bf16"))
+    # two references over the same stored weights: rai's node-by-node evaluation with every primitive's result rounded
+    # to bf16 (`ref`, which also supplies the tokens), and the same computation in f32 arithmetic (`exact`).  Through
+    # 32 layers the first is itself ~2 % of the largest logit away from the second; the device, whose fused kernels
+    # round less often, is held to 2e-2 against `exact` and to 2e-2 plus that measured noise against `ref`.
     ref = phi2.Model(cfg, params, "bf16")
-    yield dec, ref, cfg
+    exact = phi2.Model(cfg, params, "f32")
+    yield dec, (ref, exact), cfg
     dec.close()
 
 
-def _steps(request, dec, ref, first, n, ctx0, what):
+def _steps(request, dec, refs, first, n, ctx0, what):
     """n single-token steps, the oracle's greedy token fed to both sides; returns the oracle's tokens."""
+    ref, exact = refs
     toks = []
     nxt = first
     for step in range(n):
         logits, tok = dec.forward(nxt)                    # one launch of the persistent kernel + head
         want = ref.fwd(nxt)
-        assert_close(logits, want, "bf16", f"{what}: logits of the step at context {ctx0 + step}")
+        assert_logits_close(logits, want, exact.fwd(nxt), "bf16", f"{what}: logits of the step at context {ctx0 + step}")
         check_tokens(tok, want, "bf16")
         nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
         toks.append(int(nxt[0, 0]))
@@ -60,17 +66,20 @@ def _steps(request, dec, ref, first, n, ctx0, what):
 
 def test_prefill_512_then_persistent_steps_match_oracle(full, request):
     from rai_amd import synthetic
-    dec, ref, cfg = full
+    dec, refs, cfg = full
+    ref, exact = refs
     prompt = synthetic.prompt(cfg.vocab_size, 1, 512, seed=1)       # the benchmark's prompt
     dec.clear_kv_cache()
     ref.clear_kv_cache()
+    exact.clear_kv_cache()
     logits, tok = dec.forward(prompt)                               # prefill: tile GEMMs + flash attention
-    progress(request, "oracle prefill of 512 tokens through 32 layers")
+    progress(request, "oracle prefill of 512 tokens through 32 layers, bf16 chain and f32 arithmetic")
     want = ref.fwd(prompt)
-    assert_close(logits, want, "bf16", "prefill logits")
+    errs = assert_logits_close(logits, want, exact.fwd(prompt), "bf16", "prefill logits")
+    progress(request, "prefill logits: device vs f32 arithmetic %.2e, bf16 chain vs f32 arithmetic %.2e, device vs chain %.2e" % errs)
     check_tokens(tok, want, "bf16")
     first = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
-    toks = [int(first[0, 0])] + _steps(request, dec, ref, first, 16, 512, "512-token context")
+    toks = [int(first[0, 0])] + _steps(request, dec, refs, first, 16, 512, "512-token context")
     assert dec.context_len() == 528
     # the fixture the benchmark checks its printed tokens against must be what the oracle says here
     gold = json.loads(GOLDEN.read_text())
@@ -87,15 +96,18 @@ def test_persistent_steps_past_600_cached_tokens_full_width(full, request):
     """Context 650..670: one head's cached values (from ~612) and keys (from ~665) no longer fit the registers the
     attention blocks prefetch them into and are fetched in several passes, at the benchmark's full width."""
     from rai_amd import synthetic
-    dec, ref, cfg = full
+    dec, refs, cfg = full
+    ref, exact = refs
     prompt = synthetic.prompt(cfg.vocab_size, 1, 650, seed=2)
     dec.clear_kv_cache()
     ref.clear_kv_cache()
+    exact.clear_kv_cache()
     logits, tok = dec.forward(prompt)
-    progress(request, "oracle prefill of 650 tokens through 32 layers")
+    progress(request, "oracle prefill of 650 tokens through 32 layers, bf16 chain and f32 arithmetic")
     want = ref.fwd(prompt)
-    assert_close(logits, want, "bf16", "prefill logits")
+    errs = assert_logits_close(logits, want, exact.fwd(prompt), "bf16", "prefill logits")
+    progress(request, "prefill logits: device vs f32 arithmetic %.2e, bf16 chain vs f32 arithmetic %.2e, device vs chain %.2e" % errs)
     check_tokens(tok, want, "bf16")
     first = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
-    _steps(request, dec, ref, first, 20, 650, "650-token context")
+    _steps(request, dec, refs, first, 20, 650, "650-token context")
     assert dec.context_len() == 670
