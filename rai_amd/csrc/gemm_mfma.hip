@@ -853,25 +853,37 @@ __global__ void __launch_bounds__(128) k_splitk_epilogue_ln(LinearArgs a, int sp
   const uint16_t *res = (const uint16_t *)a.residual;
   float v[ITEMS][8];
   float s = 0.f;
-  // Sum of the partial products first, for two column groups of the lane at a time: the loads of six splits of both
-  // groups (24 x 16 bytes per lane) are in flight together -- a wave has a whole row to itself and nothing else to
-  // overlap its memory round trips with -- while every element's additions stay in split order.
+  // A wave has a whole row to itself and nothing else to overlap its memory round trips with (512 rows are two waves
+  // per CU), so loads are issued as early and as many at a time as the registers allow: the bias and residual chunks
+  // of every column group first, then the partial products for three column groups of the lane at a time (six splits
+  // each, 36 x 16 bytes per lane in flight), while every element's additions stay in split order.
+  u32x4 braw[ITEMS], b2raw[ITEMS], rraw[ITEMS];
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int p = lane + it * 64;
+    const int n = (p < packs ? p : lane % packs) * 8;   // clamped groups are never used
+    braw[it] = b2raw[it] = rraw[it] = u32x4{0u, 0u, 0u, 0u};
+    if (bias) braw[it] = *reinterpret_cast<const u32x4 *>(bias + n);
+    if (bias2) b2raw[it] = *reinterpret_cast<const u32x4 *>(bias2 + n);
+    if (res) rraw[it] = *reinterpret_cast<const u32x4 *>(res + (int64_t)row * a.ldr + n);
+  }
 #pragma unroll
   for (int it = 0; it < ITEMS; ++it)
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[it][e] = 0.f;
+  constexpr int GR = 3;   // column groups in flight together
 #pragma unroll
-  for (int it0 = 0; it0 < ITEMS; it0 += 2) {
-    const float *pp[2];
+  for (int it0 = 0; it0 < ITEMS; it0 += GR) {
+    const float *pp[GR];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < GR; ++j) {
       const int p = lane + (it0 + j < ITEMS ? it0 + j : it0) * 64;
       pp[j] = partial + (int64_t)row * a.N + (p < packs ? p : lane % packs) * 8;   // clamped groups are never used
     }
     for (int s0 = 0; s0 < splits; s0 += 6) {
-      f32x4 p0[2][6], p1[2][6];
+      f32x4 p0[GR][6], p1[GR][6];
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < GR; ++j)
 #pragma unroll
         for (int u = 0; u < 6; ++u) {
           const int sp = s0 + u < splits ? s0 + u : splits - 1;
@@ -879,7 +891,7 @@ __global__ void __launch_bounds__(128) k_splitk_epilogue_ln(LinearArgs a, int sp
           p1[j][u] = *reinterpret_cast<const f32x4 *>(pp[j] + (int64_t)sp * total + 4);
         }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < GR; ++j) {
         if (it0 + j < ITEMS) {
           float *x = v[it0 + j];
 #pragma unroll
@@ -900,16 +912,14 @@ __global__ void __launch_bounds__(128) k_splitk_epilogue_ln(LinearArgs a, int sp
       const int n = p * 8;
       float (&x)[8] = v[it];
       float b1[8], b2[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) b1[e] = b2[e] = 0.f;
-      if (bias) unpack8(*reinterpret_cast<const u32x4 *>(bias + n), b1);
-      if (bias2) unpack8(*reinterpret_cast<const u32x4 *>(bias2 + n), b2);
+      unpack8(braw[it], b1);     // zero bits where there is no bias: +0.0, as before
+      unpack8(b2raw[it], b2);
 #pragma unroll
       for (int e = 0; e < 8; ++e) x[e] += b1[e] + b2[e];
       if (a.act >= 0) act8(a.act, x, n, a.act_from);
       if (res) {
         float rv[8];
-        unpack8(*reinterpret_cast<const u32x4 *>(res + (int64_t)row * a.ldr + n), rv);
+        unpack8(rraw[it], rv);
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] += rv[e];
       }
