@@ -353,7 +353,7 @@ def run_gemm_tiles(args):
         return HipTensor.from_storage((a.view(np.uint32) >> 16).astype(np.uint16), "bf16")
 
     shapes = [(512, 17920, 2560), (512, 10240, 2560), (512, 7680, 2560), (512, 2560, 12800), (4096, 10240, 2560)]
-    tiles = ["128x128", "128x128k64", "256x128", "256x256", "256x256x8w", "256x256x8wk64", "streamk", "streamk64", None]
+    tiles = ["128x128", "128x128k64", "256x128", "256x192", "256x256", "256x256x8w", "256x256x8wk64", "streamk", "streamk64", None]
     rows = []
     for m, n, k in shapes:
         x, b, out = rnd((m, k)), rnd((n,)), HipTensor.empty((m, n), "bf16")

@@ -49,14 +49,14 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
 }
 
 // LDS a tile kernel needs: two stages of A and B tiles, or the epilogue staging area if that is larger.
-template <int BM, int BN, int PITCH, int WGN = 2> constexpr int gemm_lds_bytes() {
-  constexpr int tiles = 2 * (BM + BN) * PITCH * 2, staging = 2 * WGN * 32 * (BN / WGN + 4) * 4;
+template <int BM, int BN, int PITCH, int WGN = 2, int WGM = 2> constexpr int gemm_lds_bytes() {
+  constexpr int tiles = 2 * (BM + BN) * PITCH * 2, staging = WGM * WGN * 32 * (BN / WGN + 4) * 4;
   return tiles > staging ? tiles : staging;
 }
 
 // LDS of the LDS-DMA tile kernels: NS stages of 32 of K, or (NS == 2) two stages of 64.
-template <int BM, int BN, int NS, int WGN> constexpr int dma_lds_bytes() {
-  return gemm_lds_bytes<BM, BN, NS == 2 ? 64 : 32 * NS / 2, WGN>();
+template <int BM, int BN, int NS, int WGN, int WGM = 2> constexpr int dma_lds_bytes() {
+  return gemm_lds_bytes<BM, BN, NS == 2 ? 64 : 32 * NS / 2, WGN, WGM>();
 }
 
 // Applies activation `act` to the elements of x[8] whose column n + e is >= from.  The switch on the
@@ -98,30 +98,33 @@ __device__ __forceinline__ void unpack8(const u32x4 &p, float (&f)[8]) {
 // Tile epilogue shared by the tile kernels: every wave stages 32 x WN accumulators at a time in
 // LDS (the tile buffers are free by then) and writes 16-byte rows with bias / activation /
 // residual applied, or raw f32 partial sums when K is split over several blocks.
-// (WGN = waves along N: the block is a 2 x WGN grid of waves.)
-template <int BM, int BN, int LDS_BYTES, int WGN = 2>
-__device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (&acc)[BM / 64][BN / (32 * WGN)],
+// (WGM x WGN = waves along M and N; WGM = 2 except for the 256 x 192 tile.)
+template <int BM, int BN, int LDS_BYTES, int WGN = 2, int WGM = 2>
+__device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (&acc)[BM / (32 * WGM)][BN / (32 * WGN)],
                                                    uint16_t *lds, int m0, int n0, int wave, int lane, int split,
                                                    float *partial) {
-  constexpr int WM = BM / 2, WN = BN / WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int MT = WM / 32, NT = WN / 32;
   constexpr int EP = WN + 4;                // epilogue staging pitch (floats)
   const int wm = wave / WGN, wn = wave % WGN;
   // ---- epilogue: stage 32 x WN accumulators per wave in LDS, write 8 columns per lane
   float *stage = reinterpret_cast<float *>(lds) + wave * 32 * EP;
-  static_assert(2 * WGN * 32 * EP * 4 <= LDS_BYTES, "epilogue staging does not fit the tile buffers");
+  static_assert(WGM * WGN * 32 * EP * 4 <= LDS_BYTES, "epilogue staging does not fit the tile buffers");
   constexpr int CG = WN / 8;                 // 8-column groups per staged row
-  constexpr int ITEMS = 32 * CG / 64;        // per lane
+  // rows per pass: a lane keeps its column group from pass to pass, so a pass covers a power-of-two number of whole
+  // rows (CG = 12, the 96-column wave tile, leaves 16 of the 64 lanes idle)
+  constexpr int RP = 64 / CG >= 16 ? 16 : 64 / CG >= 8 ? 8 : 64 / CG >= 4 ? 4 : 2;
+  constexpr int ITEMS = 32 / RP;             // passes
   const uint16_t *bias = (const uint16_t *)a.bias;
   const uint16_t *bias2 = (const uint16_t *)a.bias2;
   const uint16_t *res = (const uint16_t *)a.residual;
   const bool vec_out = (a.ld1 % 8 == 0) && (a.n_split % 8 == 0) && (a.n_split == a.N || a.ld2 % 8 == 0) &&
                        ((uintptr_t)a.out1 % 16 == 0) && (a.n_split == a.N || (uintptr_t)a.out2 % 16 == 0) &&
                        (!res || (a.ldr % 8 == 0 && (uintptr_t)res % 16 == 0)) && a.N % 8 == 0;
-  // A lane serves the same 8 columns in every pass (64 lanes are a multiple of the CG column groups of a staged row):
-  // their bias values are fetched once, ahead of the passes, not inside each of them, where the load's latency
-  // (about a microsecond under load) sat between the LDS read and the store of every pass.
-  static_assert(64 % CG == 0, "a lane must keep its column group from pass to pass");
+  // A lane serves the same 8 columns in every pass: their bias values are fetched once, ahead of the passes, not
+  // inside each of them, where the load's latency (about a microsecond under load) sat between the LDS read and the
+  // store of every pass.
+  static_assert(RP * CG <= 64 && 32 % RP == 0, "a pass is RP whole rows of CG column groups");
   const int n = n0 + wn * WN + (lane % CG) * 8;
   const bool whole = n + 8 <= a.N;
   float bv[8];
@@ -158,10 +161,9 @@ __device__ __forceinline__ void gemm_tile_epilogue(const LinearArgs &a, f32x16 (
     // LDS operations of one wave complete in order; no block barrier is needed for a wave-private region
 #pragma unroll 1
     for (int it = 0; it < ITEMS; ++it) {
-      const int item = lane + it * 64;
-      const int row = item / CG, cg = item % CG;
+      const int row = lane / CG + it * RP, cg = lane % CG;
       const int m = m0 + wm * WM + i * 32 + row;
-      if (m >= a.M || n >= a.N) continue;
+      if (lane >= RP * CG || m >= a.M || n >= a.N) continue;
       const f32x4 v0 = *reinterpret_cast<const f32x4 *>(stage + row * EP + cg * 8);
       const f32x4 v1 = *reinterpret_cast<const f32x4 *>(stage + row * EP + cg * 8 + 4);
       float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
@@ -509,16 +511,17 @@ __device__ __forceinline__ void dma_tile_mainloop(const LinearArgs &a, uint16_t 
 //     rows span the 64 banks) land on 16 different 16-byte slots.  (Swizzling by r & 7 left rows r and r + 8 on the
 //     same banks: SQ_LDS_BANK_CONFLICT at 23 % of the kernel's cycles.)
 //   - fragment sets alternate F0 / F1 over the four K steps of a stage; the reads run one set ahead of the multiplies.
-template <int BM, int BN, int WGN>
+template <int BM, int BN, int WGN, int WGM = 2>
 __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint16_t *lds, int m0, int n0, int k_begin, int KT,
-                                                      int wave, int lane, f32x16 (&acc)[BM / 64][BN / (32 * WGN)]) {
+                                                      int wave, int lane, f32x16 (&acc)[BM / (32 * WGM)][BN / (32 * WGN)]) {
   constexpr int BK = 64;
-  constexpr int WM = BM / 2, WN = BN / WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int MT = WM / 32, NT = WN / 32;
-  constexpr int NW = 2 * WGN;
+  constexpr int NW = WGM * WGN;
   constexpr int LA = BM / (8 * NW), LB = BN / (8 * NW);   // loads per wave per stage (8 rows each)
   constexpr int STAGE = (BM + BN) * BK;
-  static_assert(LA + LB == 8, "the wait below names the load count of one stage");
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "every wave loads whole groups of 8 rows");
+  static_assert(LA + LB == 8 || LA + LB == 7, "the wait below names the load count of one stage");
   const int wm = wave / WGN, wn = wave % WGN;
   const int lrow = lane >> 3;
   const uint16_t *gpa[LA], *gpb[LB];
@@ -558,7 +561,8 @@ __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint1
   issue(0, 0);
   if (KT > 1) {
     issue(1, 1);
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // stage 0 has landed (this wave's part)
+    if constexpr (LA + LB == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // stage 0 has landed (this wave's part)
+    else asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
@@ -642,8 +646,8 @@ __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint1
   __syncthreads();
 }
 
-template <int BM, int BN, int NS, int SH, int WGN = 2>
-__global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
+template <int BM, int BN, int NS, int SH, int WGN = 2, int WGM = 2>
+__global__ void __launch_bounds__(64 * WGM * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, int splits, int k_per_split, float *partial) {
   // block = 2 x WGN waves.  WGN = 4 (eight waves, wave tile (BM/2) x (BN/4)) keeps two waves on every SIMD: one
   // multiplies while the other sits in its wait for the next tile, and twice as many waves issue loads.
   constexpr int BK = 32, PITCH = BK;
@@ -662,13 +666,14 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma(LinearArgs a, 
   const int k_end = k_begin + k_per_split < a.K ? k_begin + k_per_split : a.K;
   const int KT = (k_end - k_begin) / BK;
 
-  f32x16 acc[BM / 64][BN / (32 * WGN)];
-  if constexpr (NS == 2) {   // two stages of 64 (the launcher sends only K % 64 == 0, unsplit, here)
-    dma_tile_mainloop_k64<BM, BN, WGN>(a, lds, m0, n0, k_begin, KT / 2, wave, lane, acc);
+  f32x16 acc[BM / (32 * WGM)][BN / (32 * WGN)];
+  if constexpr (NS == 2) {   // two stages of 64 (the launcher sends K % 64 == 0 and splits of whole stages here)
+    dma_tile_mainloop_k64<BM, BN, WGN, WGM>(a, lds, m0, n0, k_begin, KT / 2, wave, lane, acc);
   } else {
+    static_assert(WGM == 2, "the K-32 loop is written for two waves along M");
     dma_tile_mainloop<BM, BN, NS, SH, WGN>(a, lds, m0, n0, k_begin, KT, wave, lane, acc);
   }
-  gemm_tile_epilogue<BM, BN, dma_lds_bytes<BM, BN, NS, WGN>(), WGN>(a, acc, lds, m0, n0, wave, lane, split, partial);
+  gemm_tile_epilogue<BM, BN, dma_lds_bytes<BM, BN, NS, WGN, WGM>(), WGN, WGM>(a, acc, lds, m0, n0, wave, lane, split, partial);
 }
 
 // ---- stream-K form of the eight-wave 256x256 tile kernel ---------------------------------------------------------
@@ -1022,12 +1027,12 @@ template <int BM, int BN, int BK, int SH = 0> static int launch_cfg(hipStream_t 
   return RAI_OK;
 }
 
-template <int BM, int BN, int NS, int SH, int WGN = 2>
+template <int BM, int BN, int NS, int SH, int WGN = 2, int WGM = 2>
 static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
-  constexpr size_t lds = dma_lds_bytes<BM, BN, NS, WGN>();
+  constexpr size_t lds = dma_lds_bytes<BM, BN, NS, WGN, WGM>();
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
-    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN>,
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN, WGM>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
@@ -1042,8 +1047,8 @@ static int launch_cfg_dma(hipStream_t st, const LinearArgs &a, int splits) {
     k_per_split = per * KU;
     partial = (float *)a.splitk_ws;
   }
-  hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN>), dim3(grid_x, splits), dim3(128 * WGN), lds, st, a, splits,
-                     k_per_split, partial);
+  hipLaunchKernelGGL((k_gemm_bf16_mfma_dma<BM, BN, NS, SH, WGN, WGM>), dim3(grid_x, splits), dim3(64 * WGM * WGN), lds, st, a,
+                     splits, k_per_split, partial);
   RAI_TRY(launch_check("gemm_bf16_mfma_dma"));
   if (splits > 1) RAI_TRY(launch_splitk_epilogue(st, a, splits, (const float *)partial));
   return RAI_OK;
@@ -1660,7 +1665,8 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
   // Tile choice.  The LDS-DMA kernels stream K tiles straight into LDS; the 256x128 tile halves the
   // L2 -> LDS traffic per flop for one operand and is used once there are enough tiles of that size
   // to give every CU two; smaller products keep the 128x128 tile (three blocks per CU).
-  // RAI_HIP_GEMM_TILE = "128x128" | "256x128" | "256x256" | "256x256x8w" | "classic" overrides (tuning aid).
+  // RAI_HIP_GEMM_TILE = "128x128" | "128x128k64" | "256x128" | "256x192" | "256x256" | "256x256x8w" | "256x256x8wk64" |
+  // "streamk" | "streamk64" | "classic" overrides (tuning aid; a form that does not apply to the shape is an error).
   const char *knob = getenv("RAI_HIP_GEMM_TILE");
   if (knob) {
     if (!strcmp(knob, "128x128")) return launch_cfg_dma<128, 128, 3, 2>(st, a, splits);
@@ -1671,6 +1677,10 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     if (!strcmp(knob, "128x128k64")) {
       RAI_REQUIRE(a.K % 64 == 0, RAI_ERR_UNSUPPORTED, "linear: RAI_HIP_GEMM_TILE=%s needs K %% 64 == 0 (%dx%dx%d)", knob, a.M, a.N, a.K);
       return launch_cfg_dma<128, 128, 2, 0, 2>(st, a, splits);
+    }
+    if (!strcmp(knob, "256x192")) {
+      RAI_REQUIRE(a.K % 64 == 0, RAI_ERR_UNSUPPORTED, "linear: RAI_HIP_GEMM_TILE=%s needs K %% 64 == 0 (%dx%dx%d)", knob, a.M, a.N, a.K);
+      return launch_cfg_dma<256, 192, 2, 0, 2, 4>(st, a, splits);
     }
     if (!strcmp(knob, "256x256x8wk64")) {
       RAI_REQUIRE(splits == 1 && a.K % 64 == 0, RAI_ERR_UNSUPPORTED,
@@ -1698,6 +1708,12 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     const bool k64 = a.K % 64 == 0 && !no_k64();
     StreamKPlan plan;
     if (streamk_applies(a, k64 ? 64 : 32, &plan)) return k64 ? launch_streamk<2>(st, a, plan) : launch_streamk<4>(st, a, plan);
+    // 256 x 192 (eight waves as 4 x 2, 64 x 96 each) where its tiles need no more rounds over the CUs than the
+    // 256 x 256 ones: the same round then holds three quarters of the work per CU, spread over more of them
+    // (512 x 17920 x 2560 with cold weights: 188 tiles in 64.7 us against 140 tiles in 71.2 us)
+    const int tiles_192 = ((a.M + 255) / 256) * ((a.N + 191) / 192);
+    if (k64 && (tiles_192 + kNumCU - 1) / kNumCU <= (huge_tiles + kNumCU - 1) / kNumCU)
+      return launch_cfg_dma<256, 192, 2, 0, 2, 4>(st, a, splits);
     return k64 ? launch_cfg_dma<256, 256, 2, 0, 4>(st, a, splits) : launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   }
   if (splits == 1 && big_tiles >= 2 * kNumCU) return launch_cfg_dma<256, 128, 3, 2>(st, a, splits);
