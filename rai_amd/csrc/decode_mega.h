@@ -42,6 +42,7 @@ struct MegaArgs {
   float ln_eps, scale;
   int act;
   int rows_attn;            // rows of phases B/C given to each attention block
+  int stage_off;            // byte offset in LDS of the weight staging area (set by the launcher; 0 = none fits)
   unsigned long long *prof; // optional [blocks][L][16] time stamps (debugging aid), or null
   // Failure-path test hooks, honoured only by the instrumented build of the kernel (prof != null):
   unsigned spin_limit;      // polling rounds after which a wait gives up and raises DevState::fault

@@ -10,7 +10,9 @@
 //   BC  [attn | act] . Wb^T + biases + residual -> x          (whole rows of Wb = dense | fc2 columns)
 // Weights do not depend on activations: every wave keeps a ring of weight tiles
 // in flight that runs ahead across the segment boundaries, so HBM keeps streaming
-// while a block waits for its inputs.  A1 runs into A2 without a pause: each stream wave
+// while a block waits for its inputs; when the ring is full a wave has the next
+// kMegaStage tiles copied straight into LDS (global -> LDS loads need no registers) and
+// takes them from there when it streams again.  A1 runs into A2 without a pause: each stream wave
 // bumps a counter in LDS when it leaves A1, and the service wave publishes the q|k|v
 // packets when all have.
 //
@@ -48,6 +50,8 @@ constexpr int kMegaStream = kMegaWaves - 1, kMegaService = kMegaWaves - 1;
 constexpr unsigned kMegaSpinLimit = 1u << 20;
 constexpr uint32_t kMegaTagsPerLaunch = 1024;   // more than the 3 exchanges per layer of any eligible model
 constexpr int kMegaRing = 16;
+constexpr int kMegaStage = 8;              // tiles (1 KB each) per stream wave held in LDS beyond the ring
+constexpr size_t kMegaLdsMax = 160 * 1024;
 constexpr int kMegaRowsAMax = 96;
 constexpr int kMegaRowsMax = 16;
 constexpr int kMegaUK = 13, kMegaUV = 12;
@@ -184,10 +188,7 @@ __device__ __forceinline__ bool mg_seg_next(MgCursor &c, const MgSplit &sp) {
     return true;
   }
 }
-// requests the tile under the cursor and advances the cursor (past the end of the
-// stream the last tile is requested again: the ring stays full, nothing is stored)
-__device__ __forceinline__ mg_u32x4 mg_next_load(MgCursor &c, const MgSplit &sp, int lane) {
-  const mg_u32x4 v = mg_ldw(c.ptr + c.kc * 512 + lane * 8);
+__device__ __forceinline__ void mg_advance(MgCursor &c, const MgSplit &sp) {
   if (!c.done) {
     if (c.t + 1 == c.t1) {
       if (!mg_seg_next(c, sp)) c.done = true;
@@ -196,16 +197,31 @@ __device__ __forceinline__ mg_u32x4 mg_next_load(MgCursor &c, const MgSplit &sp,
       if (++c.kc == c.KT) { c.kc = 0; c.ptr += c.ld; }
     }
   }
+}
+// requests the tile under the cursor and advances the cursor (past the end of the
+// stream the last tile is requested again: the ring stays full, nothing is stored)
+__device__ __forceinline__ mg_u32x4 mg_next_load(MgCursor &c, const MgSplit &sp, int lane) {
+  const mg_u32x4 v = mg_ldw(c.ptr + c.kc * 512 + lane * 8);
+  mg_advance(c, sp);
   return v;
+}
+// the same request with LDS as its destination: lane i's 16 bytes land at slot + 16 i
+__device__ __forceinline__ void mg_next_stage(MgCursor &c, const MgSplit &sp, int lane, unsigned char *slot) {
+  typedef __attribute__((address_space(3))) void *lds_ptr;
+  __builtin_amdgcn_global_load_lds((const void *)(c.ptr + c.kc * 512 + lane * 8), (lds_ptr)slot, 16, 0, 2 /* nt */);
+  mg_advance(c, sp);
 }
 // Consumes tiles [t0, t1) of a [rows][KT] tile grid from the ring (entry 0 first), then tiles [u0, u1) of a
 // second grid with the same KT and the same activation vector, without a pause between the two; multiplies
 // them with the activation vector in LDS and leaves one partial sum per (row, wave) in `part` / `part2`.
 // When the first range is done (also when it is empty) lane 0 adds one to *done1, after its partial sums are in
 // LDS.  Returns how many entries the ring must be rotated afterwards.
+// `staged`: the kMegaStage tiles that follow the ring's sixteen are in LDS at `stage` (1 KB each, in order); the
+// first pass over the ring then refills its first kMegaStage entries from there (a wave that stages has at least
+// kMegaRing tiles in every phase that is not empty).
 __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCursor &c, const MgSplit &sp, int t0, int t1,
                                             int u0, int u1, int KT, const uint16_t *xv, float *part, float *part2,
-                                            uint32_t *done1, int lane, int wave) {
+                                            uint32_t *done1, int lane, int wave, const unsigned char *stage, bool &staged) {
   float acc = 0.f;
   const int n1 = t1 > t0 ? t1 - t0 : 0, n2 = u1 > u0 ? u1 - u0 : 0;
   const int total = n1 + n2;
@@ -219,11 +235,12 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
     t = u0; te = u1; row = u0 / KT; kc = u0 - row * KT; part = part2;                                             \
   }
   if (n1 == 0) MG_TO_SECOND
-#define MG_STEP(r)                                                                         \
+#define MG_STEP(r) MG_STEP_FROM(r, mg_next_load(c, sp, lane))
+#define MG_STEP_FROM(r, REFILL)                                                            \
   {                                                                                        \
     const mg_u32x4 x4 = *reinterpret_cast<const mg_u32x4 *>(xv + kc * 512 + lane * 8);     \
     acc = mg_dot8(r, x4, acc);                                                             \
-    r = mg_next_load(c, sp, lane);                                                         \
+    r = REFILL;                                                                            \
     ++t;                                                                                   \
     ++kc;                                                                                  \
     if (kc == KT || t == te) {                                                             \
@@ -235,6 +252,19 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
     }                                                                                      \
     --to_switch;                                                                           \
   }
+  // Everything requested before this point has landed: the ring a whole exchange ago, the staged tiles before the
+  // poll that ended the wait (loads return in order).  Saying so keeps the compiler from guarding the LDS reads of
+  // the loops below against the global -> LDS loads.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  if (staged && total > 0) {
+#pragma unroll
+    for (int p = 0; p < kMegaRing; ++p) {
+      if (p < kMegaStage) MG_STEP_FROM(ring[p], *reinterpret_cast<const mg_u32x4 *>(stage + p * 1024 + lane * 16))
+      else MG_STEP(ring[p])
+    }
+    left -= kMegaRing;
+    staged = false;
+  }
   while (left >= kMegaRing) {
 #pragma unroll
     for (int p = 0; p < kMegaRing; ++p) MG_STEP(ring[p])
@@ -244,6 +274,7 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
   for (int p = 0; p < kMegaRing; ++p)
     if (p < left) MG_STEP(ring[p])
 #undef MG_STEP
+#undef MG_STEP_FROM
 #undef MG_TO_SECOND
   return total % kMegaRing;
 }
@@ -428,9 +459,15 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   const int tA0 = streams ? ttA * wave / kMegaStream : 0, tA1 = streams ? ttA * (wave + 1) / kMegaStream : 0;
   const int tA2_0 = streams ? ttA2 * wave / kMegaStream : 0, tA2_1 = streams ? ttA2 * (wave + 1) / kMegaStream : 0;
   const int tB0 = streams ? ttB * wave / kMegaStream : 0, tB1 = streams ? ttB * (wave + 1) / kMegaStream : 0;
+  const int ttA_w = (tA1 - tA0) + (tA2_1 - tA2_0), ttB_w = tB1 - tB0;   // this wave's tiles per layer: Wa, Wb
 
   mg_u32x4 ring[kMegaRing];
   mg_u32x4 kreg[kMegaUK], vreg[kMegaUV];
+  // A stream wave whose phases all hold at least one pass over the ring (or nothing) also keeps kMegaStage tiles
+  // in LDS: requested when the wave starts to wait with a full ring, consumed first when it streams again.
+  unsigned char *const stage = mg_smem + a.stage_off + wave * (kMegaStage * 1024);
+  const bool stages = a.stage_off != 0 && streams && (ttA_w == 0 || ttA_w >= kMegaRing) && (ttB_w == 0 || ttB_w >= kMegaRing);
+  bool staged = false;
 
   MgSplit sp;
   sp.Wa0 = a.Wa0; sp.Wb0 = a.Wb0; sp.wa_stride = a.wa_stride; sp.wb_stride = a.wb_stride; sp.L = a.L; sp.H = H; sp.KB = KB; sp.QD = QD; sp.KTA = KTA; sp.KTBC = KTBC;
@@ -498,6 +535,14 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     }
   };
 
+  auto stage_ahead = [&](int lane) __attribute__((always_inline)) {
+    if (stages && !staged) {
+#pragma unroll
+      for (int j = 0; j < kMegaStage; ++j) mg_next_stage(cur, sp, lane, stage + j * 1024);
+      staged = true;
+    }
+  };
+
   for (int e = tid0; e < kMegaRowsAMax * kMegaWaves; e += kMegaThreads) partA[e] = 0.f;
   if (tid0 == 0) *a1_done = 0u;
 
@@ -522,6 +567,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     {
       const int tid = mg_opaque(tid0), lane = tid & 63;
       const bool service = wave == kMegaService;
+      stage_ahead(lane);   // the ring is full: the wait for the residual stream fetches the tiles behind it into LDS
       // An attention block requests the cached keys and values of its head first: they do not depend on this
       // layer's inputs, one CU can only keep so many cache lines in flight (the ~200 KB take several memory
       // round trips), and the block would otherwise just wait for the residual stream.
@@ -557,6 +603,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
             if (on[i]) reinterpret_cast<uint32_t *>(xa)[idx[i]] = val[i];
         }
       }
+      stamp(l, 8);   // the residual stream has arrived
       wg_sync();
       if (wave < KTA) {
 
@@ -633,7 +680,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       // are still writing, i.e. it waits for the newest of them, and by now those have had a whole exchange to land
       mg_rotate_by(ring, pending_rot);
       pending_rot = mg_run_phase(ring, cur, sp, tA0, tA1, tA2_0, tA2_1, KTA, xn, partA, partA + rowsA * kMegaWaves,
-                                 a1_done, lane, wave);
+                                 a1_done, lane, wave, stage, staged);
       if (service) {   // its own ranges are empty: it arrives here at once and waits for the seven others
         unsigned spins = 0;
         while (__hip_atomic_load(a1_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)kMegaWaves) {
@@ -644,6 +691,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           }
         }
         publish_a(nA0, rowsA, partA, bias_a, false);
+        stamp(l, 9);   // q|k|v rows of this block published
       }
       wg_sync();
       if (service && lane * 3 < rowsA2) {   // gelu(fc1) of this block's rows, three to a packet
@@ -665,8 +713,6 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       }
       stamp(l, 1);
       ++bar;   // no barrier: phase B polls the packets it needs
-      stamp(l, 8);
-      stamp(l, 9);
       wg_sync();
       stamp(l, 2);
     }
@@ -792,6 +838,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       }
       // ---- rows of Wb: [attention output | activations] . [dense columns | fc2 columns], one stream
       const bool service = wave == kMegaService;
+      stage_ahead(lane);   // (an attention block is past its head here: nothing of its own waits behind these loads)
       uint64_t res4 = 0, bd4 = 0, bf4 = 0;
       if (service && lane * 4 < nrows) {
         res4 = ld_dev64(a.x + n0 + lane * 4);
@@ -844,7 +891,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       wg_sync();
       stamp(l, 3);
       mg_rotate_by(ring, pending_rot);
-      pending_rot = mg_run_phase(ring, cur, sp, tB0, tB1, 0, 0, KTBC, xa, partB, partB, nullptr, lane, wave);
+      pending_rot = mg_run_phase(ring, cur, sp, tB0, tB1, 0, 0, KTBC, xa, partB, partB, nullptr, lane, wave, stage, staged);
       stamp(l, 4);
       wg_sync();
       stamp(l, 5);
@@ -873,6 +920,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       stamp(l, 7);
     }
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // nothing still on its way into LDS when the block ends
 }
 
 size_t mega_lds_bytes(const MegaArgs &a, int D) {
@@ -916,17 +964,26 @@ bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
 int launch_phi2_decode_step(hipStream_t st, const MegaArgs &a, int D, int num_cu) {
   const char *why = nullptr;
   RAI_REQUIRE(mega_eligible(a, D, num_cu, &why), RAI_ERR_UNSUPPORTED, "persistent decode step: %s", why ? why : "?");
-  const size_t lds = mega_lds_bytes(a, D);
+  size_t lds = mega_lds_bytes(a, D);
+  MegaArgs m = a;
+  // the weight staging area (kMegaStage KB per stream wave) goes behind everything else where the CU's LDS holds both
+  const size_t stage_bytes = (size_t)kMegaStream * kMegaStage * 1024;
+  const char *no_stage = getenv("RAI_HIP_MEGA_NO_STAGE");   // read per call: tests run both forms in one process
+  m.stage_off = 0;
+  if (lds + stage_bytes <= kMegaLdsMax && !(no_stage && *no_stage && *no_stage != '0')) {
+    m.stage_off = (int)lds;
+    lds += stage_bytes;
+  }
   static size_t attr_bytes = 0;
   if (lds > 64 * 1024 && lds > attr_bytes) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_phi2_decode_step<5, 80, false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMegaLdsMax));
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_phi2_decode_step<5, 80, true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024));
-    attr_bytes = 150 * 1024;
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMegaLdsMax));
+    attr_bytes = kMegaLdsMax;
   }
-  if (a.prof) hipLaunchKernelGGL((k_phi2_decode_step<5, 80, true>), dim3(num_cu), dim3(kMegaThreads), lds, st, a);
-  else hipLaunchKernelGGL((k_phi2_decode_step<5, 80, false>), dim3(num_cu), dim3(kMegaThreads), lds, st, a);
+  if (m.prof) hipLaunchKernelGGL((k_phi2_decode_step<5, 80, true>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
+  else hipLaunchKernelGGL((k_phi2_decode_step<5, 80, false>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
   return launch_check("phi2_decode_step");
 }
 

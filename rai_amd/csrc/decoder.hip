@@ -1110,13 +1110,14 @@ static int check_fault(rai_hip_decoder *d) {
       const int b = blocks[bi];
       for (int l = 0; l < d->L; ++l)
         for (int k = 0; k < 7; ++k) iv[k] += (at(b, l, k + 1) - at(b, l, k)) / d->L;
-      fprintf(stderr, "mega prof block %3d: A (wait x, LN, stream) %.2f | wave sync %.2f | B-pre (wait act, attention) %.2f | service %.2f | B stream %.2f | C (wait attn, stream) %.2f | wave sync %.2f us\n",
-              b, iv[0], iv[1], iv[2], iv[3], iv[4], iv[5], iv[6]);
-      double ex[6] = {0, 0, 0, 0, 0, 0};   // extra stamps 8..13, relative to stamp 1 (end of phase A)
+      double ex[6] = {0, 0, 0, 0, 0, 0};   // stamps 8, 9 relative to the layer's start, 10..13 to the end of phase A
       for (int l = 0; l < d->L; ++l)
-        for (int k = 0; k < 6; ++k) ex[k] += (at(b, l, 8 + k) - at(b, l, 1)) / d->L;
-      fprintf(stderr, "mega prof block %3d: after A: +%.2f bar | +%.2f kv issued | +%.2f qkv polled | +%.2f k partials | +%.2f softmax | +%.2f attn published\n",
-              b, ex[0], ex[1], ex[2], ex[3], ex[4], ex[5]);
+        for (int k = 0; k < 6; ++k) ex[k] += (at(b, l, 8 + k) - at(b, l, k < 2 ? 0 : 1)) / d->L;
+      fprintf(stderr, "mega prof block %3d: A %.2f (x arrived +%.2f, q|k|v published +%.2f) | sync %.2f | poll (attention) %.2f | Wb stream %.2f + sync %.2f | publish x %.2f | sync %.2f us\n",
+              b, iv[0], ex[0], ex[1], iv[1], iv[2], iv[3], iv[4], iv[5], iv[6]);
+      if (b < d->Hq)
+        fprintf(stderr, "mega prof block %3d: after A: +%.2f qkv polled | +%.2f k partials | +%.2f softmax | +%.2f attn published\n",
+                b, ex[2], ex[3], ex[4], ex[5]);
     }
   }
   if (d->mega_prof && getenv("RAI_HIP_MEGA_PROF_SKEW")) {  // how late each block reaches the end of each phase, mean over layers

@@ -521,7 +521,7 @@ __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint1
   constexpr int LA = BM / (8 * NW), LB = BN / (8 * NW);   // loads per wave per stage (8 rows each)
   constexpr int STAGE = (BM + BN) * BK;
   static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "every wave loads whole groups of 8 rows");
-  static_assert(LA + LB == 8 || LA + LB == 7, "the wait below names the load count of one stage");
+  static_assert(LA + LB <= 16, "the wait counts one stage of loads");
   const int wm = wave / WGN, wn = wave % WGN;
   const int lrow = lane >> 3;
   const uint16_t *gpa[LA], *gpb[LB];
@@ -561,8 +561,7 @@ __device__ __forceinline__ void dma_tile_mainloop_k64(const LinearArgs &a, uint1
   issue(0, 0);
   if (KT > 1) {
     issue(1, 1);
-    if constexpr (LA + LB == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // stage 0 has landed (this wave's part)
-    else asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LA + LB) : "memory");   // stage 0 has landed (this wave's part)
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }

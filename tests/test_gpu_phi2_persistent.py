@@ -114,3 +114,34 @@ def test_persistent_step_long_context_takes_several_prefetch_passes(hip):
         nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
     assert dec.context_len() == 670
     dec.close()
+
+
+def test_persistent_step_with_and_without_lds_staged_weights(hip, monkeypatch):
+    """At Phi-2's real MLP width every stream wave keeps the eight weight tiles behind its register ring in LDS
+    (fetched while it waits for its inputs).  The tiles are consumed in the same order either way, so the logits
+    are the same bits with the staging switched off, and both match the oracle."""
+    cfg = wide_cfg(intermediate_size=10240)
+    ids = np.random.Generator(np.random.PCG64(15)).integers(0, cfg.vocab_size, (1, 19)).astype(np.uint32)
+    dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
+    want = ref.fwd(ids)
+    first = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
+    runs = []
+    for off in ("0", "1"):
+        monkeypatch.setenv("RAI_HIP_MEGA_NO_STAGE", off)     # read per launch
+        dec.clear_kv_cache()
+        dec.forward(ids)
+        nxt, out = first, []
+        for step in range(6):
+            logits, tok = dec.forward(nxt)
+            out.append(logits.copy())
+            nxt = tok.reshape(1, 1).astype(np.uint32)
+        runs.append(out)
+    monkeypatch.delenv("RAI_HIP_MEGA_NO_STAGE")
+    nxt = first
+    for step in range(6):
+        assert np.array_equal(runs[0][step], runs[1][step]), f"step {step}: staged and unstaged logits differ"
+        want = ref.fwd(nxt)
+        assert_close(runs[0][step], want, "bf16", f"decode step {step}")
+        check_tokens(np.argmax(runs[0][step], -1), want, "bf16")
+        nxt = np.argmax(runs[0][step], -1).astype(np.uint32).reshape(1, 1)
+    dec.close()
