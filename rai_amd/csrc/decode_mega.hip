@@ -143,58 +143,55 @@ template <int R> __device__ __forceinline__ void mg_rotate(mg_u32x4 (&ring)[kMeg
   for (int p = 0; p < kMegaRing; ++p) ring[p] = tmp[p];
 }
 
+// A wave's weight stream: per layer up to three segments, in streaming order A1 (q|k|v rows of Wa), A2 (fc1 rows
+// of Wa), BC (whole rows of Wb: dense columns, then fc2 columns).  Everything about a segment that does not change
+// from layer to layer is worked out once, so that moving the cursor to the next segment is a few selects: no loop
+// and no division inside the streaming loops (with those in every step the compiler kept the ring in a second set
+// of registers and copied it back, after waiting for every load, once per pass).
 struct MgSplit {
   const uint16_t *Wa0, *Wb0;
   int64_t wa_stride, wb_stride;
-  int L, H, KB, QD, KTA, KTBC;
-  int nA0, nA2, n0;                  // first Wa row of segment A1 (q|k|v rows) and of A2 (fc1 rows); first Wb row
-  int tA0, tA1, tA2_0, tA2_1, tB0, tB1;
+  int L, H, KB, KTA, KTBC;
+  int64_t off0, off1, off2;   // element offset of the segment's first row from its matrix in the same layer
+  int kc0, kc1, kc2;          // column tile of its first tile
+  int cnt0, cnt1, cnt2;       // tiles
+  int nx0, nx1, nx2;          // the next segment that is not empty (cyclic; the segment itself when it is the only one)
 };
 
 struct MgCursor {
-  int layer, seg, kc, KT, t, t1;
+  int layer, seg, kc, KT, left;   // left: tiles of the segment not yet requested, the one under the cursor included
   int64_t ld;
   const uint16_t *ptr;
   bool done;
 };
 
-__device__ __forceinline__ bool mg_seg_next(MgCursor &c, const MgSplit &sp) {
-  int layer = c.layer, seg = c.seg;
-
-  // segments of a layer, in streaming order: A1 (q|k|v rows of Wa), A2 (fc1 rows of Wa), BC (whole rows of Wb:
-  // dense columns, then fc2 columns)
+__device__ __forceinline__ void mg_seg_enter(MgCursor &c, const MgSplit &sp, int layer, int seg) {
   // (the fields are copied into values first: selecting between struct members by `seg` directly makes the
   // compiler keep the struct in scratch memory and select addresses)
-  const int tA0 = sp.tA0, tA1 = sp.tA1, tA2_0 = sp.tA2_0, tA2_1 = sp.tA2_1, tB0 = sp.tB0, tB1 = sp.tB1;
-  const int KTA = sp.KTA, KTBC = sp.KTBC, nA0 = sp.nA0, nA2 = sp.nA2;
-  for (;;) {
-    if (++seg == 3) { seg = 0; ++layer; }
-    if (layer >= sp.L) return false;
-    const int t0 = seg == 0 ? tA0 : seg == 1 ? tA2_0 : tB0;
-    const int t1 = seg == 0 ? tA1 : seg == 1 ? tA2_1 : tB1;
-    if (t1 <= t0) continue;
-    const int KT = seg <= 1 ? KTA : KTBC;
-    const int row = t0 / KT;
-    c.layer = layer; c.seg = seg; c.KT = KT; c.t = t0; c.t1 = t1;
-    c.kc = t0 - row * KT;
-    if (seg <= 1) {
-      const int first = seg == 0 ? nA0 : nA2;
-      c.ld = sp.H;
-      c.ptr = sp.Wa0 + layer * sp.wa_stride + (int64_t)(first + row) * sp.H;
-    } else {
-      c.ld = sp.KB;
-      c.ptr = sp.Wb0 + layer * sp.wb_stride + (int64_t)(sp.n0 + row) * sp.KB;
-    }
-    return true;
-  }
+  const int64_t off0 = sp.off0, off1 = sp.off1, off2 = sp.off2;
+  const int kc0 = sp.kc0, kc1 = sp.kc1, kc2 = sp.kc2, cnt0 = sp.cnt0, cnt1 = sp.cnt1, cnt2 = sp.cnt2;
+  const bool wa = seg <= 1;
+  const uint16_t *base = wa ? sp.Wa0 + layer * sp.wa_stride : sp.Wb0 + layer * sp.wb_stride;
+  c.layer = layer;
+  c.seg = seg;
+  c.KT = wa ? sp.KTA : sp.KTBC;
+  c.ld = wa ? sp.H : sp.KB;
+  c.kc = seg == 0 ? kc0 : seg == 1 ? kc1 : kc2;
+  c.left = seg == 0 ? cnt0 : seg == 1 ? cnt1 : cnt2;
+  c.ptr = base + (seg == 0 ? off0 : seg == 1 ? off1 : off2);
 }
 __device__ __forceinline__ void mg_advance(MgCursor &c, const MgSplit &sp) {
   if (!c.done) {
-    if (c.t + 1 == c.t1) {
-      if (!mg_seg_next(c, sp)) c.done = true;
+    if (--c.left == 0) {
+      const int nx0 = sp.nx0, nx1 = sp.nx1, nx2 = sp.nx2;
+      const int ns = c.seg == 0 ? nx0 : c.seg == 1 ? nx1 : nx2;
+      const int nl = c.layer + (ns <= c.seg ? 1 : 0);
+      if (nl >= sp.L) c.done = true;     // the cursor stays on the last tile
+      else mg_seg_enter(c, sp, nl, ns);
     } else {
-      ++c.t;
-      if (++c.kc == c.KT) { c.kc = 0; c.ptr += c.ld; }
+      const bool wrap = c.kc + 1 == c.KT;
+      c.kc = wrap ? 0 : c.kc + 1;
+      c.ptr += wrap ? c.ld : 0;
     }
   }
 }
@@ -240,6 +237,7 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
   {                                                                                        \
     const mg_u32x4 x4 = *reinterpret_cast<const mg_u32x4 *>(xv + kc * 512 + lane * 8);     \
     acc = mg_dot8(r, x4, acc);                                                             \
+    asm volatile("" : "+v"(acc)); /* the products stay ahead of the refill, see below */   \
     r = REFILL;                                                                            \
     ++t;                                                                                   \
     ++kc;                                                                                  \
@@ -254,8 +252,11 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
   }
   // Everything requested before this point has landed: the ring a whole exchange ago, the staged tiles before the
   // poll that ended the wait (loads return in order).  Saying so keeps the compiler from guarding the LDS reads of
-  // the loops below against the global -> LDS loads.
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  // the loops below against the global -> LDS loads, and, more important, lets it count: the layer's biases are read
+  // through pointers that were themselves loaded from memory, i.e. with flat loads, and while one of those is
+  // outstanding (the service wave uses them after the stream) every wait for a ring entry becomes a wait for all
+  // loads, which empties the ring once per pass.
+  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
   if (staged && total > 0) {
 #pragma unroll
     for (int p = 0; p < kMegaRing; ++p) {
@@ -270,9 +271,17 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
     for (int p = 0; p < kMegaRing; ++p) MG_STEP(ring[p])
     left -= kMegaRing;
   }
-#pragma unroll
-  for (int p = 0; p < kMegaRing; ++p)
-    if (p < left) MG_STEP(ring[p])
+  // the rest: step p runs only if every step before it ran, and the control flow says so (an early exit, not sixteen
+  // independent conditions), so that the compiler can count the loads between a tile's request and its use; with
+  // independent conditions it has to wait for every outstanding load before each of these steps
+#define MG_REST(p)                  \
+  if (left <= p) goto rest_done;    \
+  MG_STEP(ring[p])
+  static_assert(kMegaRing == 16, "the steps below are written out");
+  MG_REST(0) MG_REST(1) MG_REST(2) MG_REST(3) MG_REST(4) MG_REST(5) MG_REST(6) MG_REST(7)
+  MG_REST(8) MG_REST(9) MG_REST(10) MG_REST(11) MG_REST(12) MG_REST(13) MG_REST(14)
+rest_done:
+#undef MG_REST
 #undef MG_STEP
 #undef MG_STEP_FROM
 #undef MG_TO_SECOND
@@ -392,7 +401,9 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
 
   // Phase A rows.  Every block takes a share of the q|k|v rows and streams them first (segment A1), so that the
   // attention blocks can start while the fc1 rows (segment A2) are still being streamed; the fc1 rows go to the
-  // blocks that run no attention head (to all blocks when every block runs one).
+  // blocks that run no attention head (to all blocks when every block runs one).  (Leaving the q|k|v rows to the
+  // blocks without a head as well, so that a head's polls do not queue behind its own weight requests, was
+  // measured: 992 against 986 us per launch.)
   const bool is_attn = wg < a.Hq;
   const int nA0 = 4 * (int)((int64_t)(a.n_qkv / 4) * wg / G), nA1 = 4 * (int)((int64_t)(a.n_qkv / 4) * (wg + 1) / G);
   const int rowsA = nA1 - nA0;
@@ -470,13 +481,27 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   bool staged = false;
 
   MgSplit sp;
-  sp.Wa0 = a.Wa0; sp.Wb0 = a.Wb0; sp.wa_stride = a.wa_stride; sp.wb_stride = a.wb_stride; sp.L = a.L; sp.H = H; sp.KB = KB; sp.QD = QD; sp.KTA = KTA; sp.KTBC = KTBC;
-  sp.nA0 = nA0; sp.nA2 = nA2; sp.n0 = n0;
-  sp.tA0 = tA0; sp.tA1 = tA1; sp.tA2_0 = tA2_0; sp.tA2_1 = tA2_1; sp.tB0 = tB0; sp.tB1 = tB1;
+  sp.Wa0 = a.Wa0; sp.Wb0 = a.Wb0; sp.wa_stride = a.wa_stride; sp.wb_stride = a.wb_stride; sp.L = a.L; sp.H = H; sp.KB = KB; sp.KTA = KTA; sp.KTBC = KTBC;
+  sp.cnt0 = tA1 - tA0; sp.cnt1 = tA2_1 - tA2_0; sp.cnt2 = tB1 - tB0;
+  sp.kc0 = tA0 % KTA; sp.kc1 = tA2_0 % KTA; sp.kc2 = tB0 % KTBC;
+  sp.off0 = (int64_t)(nA0 + tA0 / KTA) * H; sp.off1 = (int64_t)(nA2 + tA2_0 / KTA) * H; sp.off2 = (int64_t)(n0 + tB0 / KTBC) * KB;
+  {
+    const bool e0 = sp.cnt0 > 0, e1 = sp.cnt1 > 0, e2 = sp.cnt2 > 0;
+    sp.nx0 = e1 ? 1 : e2 ? 2 : 0;
+    sp.nx1 = e2 ? 2 : e0 ? 0 : 1;
+    sp.nx2 = e0 ? 0 : e1 ? 1 : 2;
+  }
   MgCursor cur;
-  cur.layer = 0; cur.seg = -1; cur.kc = 0; cur.KT = 1; cur.t = 0; cur.t1 = 0; cur.ld = 0;
+  cur.layer = 0; cur.seg = 0; cur.kc = 0; cur.KT = 1; cur.left = 0; cur.ld = 0;
   cur.ptr = a.Wa0;
-  cur.done = !mg_seg_next(cur, sp);
+  cur.done = true;
+  {
+    const int first = sp.cnt0 > 0 ? 0 : sp.cnt1 > 0 ? 1 : sp.cnt2 > 0 ? 2 : -1;
+    if (first >= 0 && a.L > 0) {
+      cur.done = false;
+      mg_seg_enter(cur, sp, 0, first);
+    }
+  }
   unsigned bar = 0;
   int pending_rot = 0;
   const uint32_t tagbase = a.state->epoch * kMegaTagsPerLaunch;   // exchange tags of this launch: tagbase + index + 1
