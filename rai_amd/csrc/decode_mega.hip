@@ -152,17 +152,19 @@ struct MgSplit {
   const uint16_t *Wa0, *Wb0;
   int64_t wa_stride, wb_stride;
   int L, H, KB, KTA, KTBC;
-  int64_t off0, off1, off2;   // element offset of the segment's first row from its matrix in the same layer
+  int64_t off0, off1, off2;   // element offset of the segment's first tile from its matrix in the same layer
   int kc0, kc1, kc2;          // column tile of its first tile
   int cnt0, cnt1, cnt2;       // tiles
   int nx0, nx1, nx2;          // the next segment that is not empty (cyclic; the segment itself when it is the only one)
 };
 
+// ptr is the tile that is requested next; the tiles of a row follow each other (512 elements), the next row
+// starts `jump` elements behind the row's last tile.  Behind the last layer the stream starts again with the
+// first (those requests are never used; they keep the loop free of an end-of-stream case).
 struct MgCursor {
   int layer, seg, kc, KT, left;   // left: tiles of the segment not yet requested, the one under the cursor included
-  int64_t ld;
+  int64_t jump;
   const uint16_t *ptr;
-  bool done;
 };
 
 __device__ __forceinline__ void mg_seg_enter(MgCursor &c, const MgSplit &sp, int layer, int seg) {
@@ -175,81 +177,75 @@ __device__ __forceinline__ void mg_seg_enter(MgCursor &c, const MgSplit &sp, int
   c.layer = layer;
   c.seg = seg;
   c.KT = wa ? sp.KTA : sp.KTBC;
-  c.ld = wa ? sp.H : sp.KB;
+  c.jump = (int64_t)(wa ? sp.H : sp.KB) - (int64_t)(c.KT - 1) * 512;
   c.kc = seg == 0 ? kc0 : seg == 1 ? kc1 : kc2;
   c.left = seg == 0 ? cnt0 : seg == 1 ? cnt1 : cnt2;
-  c.ptr = base + (seg == 0 ? off0 : seg == 1 ? off1 : off2);
+  c.ptr = base + (seg == 0 ? off0 : seg == 1 ? off1 : off2) + c.kc * 512;
 }
 __device__ __forceinline__ void mg_advance(MgCursor &c, const MgSplit &sp) {
-  if (!c.done) {
-    if (--c.left == 0) {
-      const int nx0 = sp.nx0, nx1 = sp.nx1, nx2 = sp.nx2;
-      const int ns = c.seg == 0 ? nx0 : c.seg == 1 ? nx1 : nx2;
-      const int nl = c.layer + (ns <= c.seg ? 1 : 0);
-      if (nl >= sp.L) c.done = true;     // the cursor stays on the last tile
-      else mg_seg_enter(c, sp, nl, ns);
-    } else {
-      const bool wrap = c.kc + 1 == c.KT;
-      c.kc = wrap ? 0 : c.kc + 1;
-      c.ptr += wrap ? c.ld : 0;
-    }
+  if (--c.left == 0) {
+    const int nx0 = sp.nx0, nx1 = sp.nx1, nx2 = sp.nx2;
+    const int ns = c.seg == 0 ? nx0 : c.seg == 1 ? nx1 : nx2;
+    const int nl = c.layer + (ns <= c.seg ? 1 : 0);
+    mg_seg_enter(c, sp, nl >= sp.L ? 0 : nl, ns);
+  } else {
+    const bool wrap = c.kc + 1 == c.KT;
+    c.kc = wrap ? 0 : c.kc + 1;
+    c.ptr += wrap ? c.jump : (int64_t)512;
   }
 }
-// requests the tile under the cursor and advances the cursor (past the end of the
-// stream the last tile is requested again: the ring stays full, nothing is stored)
+// requests the tile under the cursor and advances the cursor
 __device__ __forceinline__ mg_u32x4 mg_next_load(MgCursor &c, const MgSplit &sp, int lane) {
-  const mg_u32x4 v = mg_ldw(c.ptr + c.kc * 512 + lane * 8);
+  const mg_u32x4 v = mg_ldw(c.ptr + lane * 8);
   mg_advance(c, sp);
   return v;
 }
 // the same request with LDS as its destination: lane i's 16 bytes land at slot + 16 i
 __device__ __forceinline__ void mg_next_stage(MgCursor &c, const MgSplit &sp, int lane, unsigned char *slot) {
   typedef __attribute__((address_space(3))) void *lds_ptr;
-  __builtin_amdgcn_global_load_lds((const void *)(c.ptr + c.kc * 512 + lane * 8), (lds_ptr)slot, 16, 0, 2 /* nt */);
+  __builtin_amdgcn_global_load_lds((const void *)(c.ptr + lane * 8), (lds_ptr)slot, 16, 0, 2 /* nt */);
   mg_advance(c, sp);
 }
-// Consumes tiles [t0, t1) of a [rows][KT] tile grid from the ring (entry 0 first), then tiles [u0, u1) of a
-// second grid with the same KT and the same activation vector, without a pause between the two; multiplies
-// them with the activation vector in LDS and leaves one partial sum per (row, wave) in `part` / `part2`.
-// When the first range is done (also when it is empty) lane 0 adds one to *done1, after its partial sums are in
-// LDS.  Returns how many entries the ring must be rotated afterwards.
+// Two ranges of tiles of [rows][KT] tile grids that one phase of a wave consumes one after the other (the second may
+// be empty, and so may the first); the same in every layer.
+struct MgPhase {
+  int n1, kc1, row1;   // tiles, column tile and row of the first tile
+  int n2, kc2, row2;
+};
+__device__ __forceinline__ MgPhase mg_phase(int t0, int t1, int u0, int u1, int KT) {
+  MgPhase ph;
+  ph.n1 = t1 > t0 ? t1 - t0 : 0; ph.row1 = t0 / KT; ph.kc1 = t0 - ph.row1 * KT;
+  ph.n2 = u1 > u0 ? u1 - u0 : 0; ph.row2 = u0 / KT; ph.kc2 = u0 - ph.row2 * KT;
+  return ph;
+}
+// Consumes the tiles of a phase from the ring (entry 0 first), the second range behind the first without a pause;
+// multiplies them with the activation vector in LDS (the same for both ranges) and leaves one partial sum per
+// (row, wave) in `part` / `part2`.  When the first range is done (also when it is empty) lane 0 adds one to *done1,
+// after its partial sums are in LDS.  Returns how many entries the ring must be rotated afterwards.
 // `staged`: the kMegaStage tiles that follow the ring's sixteen are in LDS at `stage` (1 KB each, in order); the
 // first pass over the ring then refills its first kMegaStage entries from there (a wave that stages has at least
 // kMegaRing tiles in every phase that is not empty).
-__device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCursor &c, const MgSplit &sp, int t0, int t1,
-                                            int u0, int u1, int KT, const uint16_t *xv, float *part, float *part2,
-                                            uint32_t *done1, int lane, int wave, const unsigned char *stage, bool &staged) {
+// A wave issues one instruction every four clocks at best, and the stream is bound by that, not by the loads: a
+// step is kept to the multiply, the refill and a handful of scalar instructions.  The activation tile of the next
+// step is read from LDS a step ahead; the only counter in a step is the distance to the end of the row.
+__device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCursor &c, const MgSplit &sp, const MgPhase &ph,
+                                            int KT, const uint16_t *xv, float *part, float *part2, uint32_t *done1,
+                                            int lane, int wave, const unsigned char *stage, bool &staged) {
   float acc = 0.f;
-  const int n1 = t1 > t0 ? t1 - t0 : 0, n2 = u1 > u0 ? u1 - u0 : 0;
-  const int total = n1 + n2;
+  const int total = ph.n1 + ph.n2;
   int left = total;
-  int to_switch = n1;            // steps until the first range is exhausted (0: already in the second)
-  int t = t0, te = t1, row = t0 / KT;
-  int kc = t0 - row * KT;
-#define MG_TO_SECOND                                                                                              \
-  {                                                                                                               \
-    if (done1 && lane == 0) __hip_atomic_fetch_add(done1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);     \
-    t = u0; te = u1; row = u0 / KT; kc = u0 - row * KT; part = part2;                                             \
-  }
-  if (n1 == 0) MG_TO_SECOND
-#define MG_STEP(r) MG_STEP_FROM(r, mg_next_load(c, sp, lane))
-#define MG_STEP_FROM(r, REFILL)                                                            \
-  {                                                                                        \
-    const mg_u32x4 x4 = *reinterpret_cast<const mg_u32x4 *>(xv + kc * 512 + lane * 8);     \
-    acc = mg_dot8(r, x4, acc);                                                             \
-    asm volatile("" : "+v"(acc)); /* the products stay ahead of the refill, see below */   \
-    r = REFILL;                                                                            \
-    ++t;                                                                                   \
-    ++kc;                                                                                  \
-    if (kc == KT || t == te) {                                                             \
-      const float total_ = mg_wave_sum(acc);                                               \
-      if (lane == 0) part[row * kMegaWaves + wave] = total_;                               \
-      acc = 0.f;                                                                           \
-      if (kc == KT) { kc = 0; ++row; }                                                     \
-      if (to_switch == 1) MG_TO_SECOND                                                     \
-    }                                                                                      \
-    --to_switch;                                                                           \
-  }
+  bool second = ph.n1 == 0;
+  if (second && done1 && lane == 0) __hip_atomic_fetch_add(done1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  int rr = second ? ph.n2 : ph.n1;             // tiles left in the range, the current row included
+  int row = second ? ph.row2 : ph.row1;
+  float *prow = (second ? part2 : part) + row * kMegaWaves + wave;   // where this row's partial sum goes
+  const int kc_first = second ? ph.kc2 : ph.kc1;
+  int rem = KT - kc_first < rr ? KT - kc_first : rr;                 // steps to the end of the row (or of the range)
+  int row_len = rem;
+  const int xo2 = ph.kc2 * 1024;
+  int xo_row = (!second && ph.n2 > 0 && rr == row_len) ? xo2 : 0;    // LDS offset of the tile that follows this row's last
+  int xo = kc_first * 1024;
+  const unsigned char *xl = reinterpret_cast<const unsigned char *>(xv) + lane * 16;
   // Everything requested before this point has landed: the ring a whole exchange ago, the staged tiles before the
   // poll that ended the wait (loads return in order).  Saying so keeps the compiler from guarding the LDS reads of
   // the loops below against the global -> LDS loads, and, more important, lets it count: the layer's biases are read
@@ -257,6 +253,37 @@ __device__ __forceinline__ int mg_run_phase(mg_u32x4 (&ring)[kMegaRing], MgCurso
   // outstanding (the service wave uses them after the stream) every wait for a ring entry becomes a wait for all
   // loads, which empties the ring once per pass.
   __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+  mg_u32x4 x4n = *reinterpret_cast<const mg_u32x4 *>(xl + xo);
+#define MG_STEP(r) MG_STEP_FROM(r, mg_next_load(c, sp, lane))
+#define MG_STEP_FROM(r, REFILL)                                                                     \
+  {                                                                                                 \
+    const mg_u32x4 x4 = x4n;                                                                        \
+    const bool last = rem == 1;                                                                     \
+    xo = last ? xo_row : xo + 1024;                                                                 \
+    x4n = *reinterpret_cast<const mg_u32x4 *>(xl + xo);                                             \
+    acc = mg_dot8(r, x4, acc);                                                                      \
+    asm volatile("" : "+v"(acc)); /* the products stay ahead of the refill: were they sunk below */ \
+    r = REFILL;                   /* it, old and new tile would need two registers              */ \
+    --rem;                                                                                          \
+    if (last) {                                                                                     \
+      const float total_ = mg_wave_sum(acc);                                                        \
+      if (lane == 0) *prow = total_;                                                                \
+      acc = 0.f;                                                                                    \
+      rr -= row_len;                                                                                \
+      prow += kMegaWaves;                                                                           \
+      if (rr == 0 && !second) {                                                                     \
+        if (done1 && lane == 0) __hip_atomic_fetch_add(done1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); \
+        second = true;                                                                              \
+        rr = ph.n2;                                                                                 \
+        prow = part2 + ph.row2 * kMegaWaves + wave;                                                 \
+        row_len = KT - ph.kc2 < rr ? KT - ph.kc2 : rr;                                              \
+      } else {                                                                                      \
+        row_len = KT < rr ? KT : rr;                                                                \
+      }                                                                                             \
+      rem = row_len;                                                                                \
+      xo_row = (!second && ph.n2 > 0 && rr == row_len) ? xo2 : 0;                                   \
+    }                                                                                               \
+  }
   if (staged && total > 0) {
 #pragma unroll
     for (int p = 0; p < kMegaRing; ++p) {
@@ -284,7 +311,6 @@ rest_done:
 #undef MG_REST
 #undef MG_STEP
 #undef MG_STEP_FROM
-#undef MG_TO_SECOND
   return total % kMegaRing;
 }
 __device__ __forceinline__ void mg_rotate_by(mg_u32x4 (&ring)[kMegaRing], int r) {
@@ -401,9 +427,11 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
 
   // Phase A rows.  Every block takes a share of the q|k|v rows and streams them first (segment A1), so that the
   // attention blocks can start while the fc1 rows (segment A2) are still being streamed; the fc1 rows go to the
-  // blocks that run no attention head (to all blocks when every block runs one).  (Leaving the q|k|v rows to the
-  // blocks without a head as well, so that a head's polls do not queue behind its own weight requests, was
-  // measured: 992 against 986 us per launch.)
+  // blocks that run no attention head (to all blocks when every block runs one).  (A head's polls come back behind
+  // the weight requests of its own block, loads returning in order.  Two ways around that were measured and are not
+  // kept: no q|k|v rows for the blocks with a head, 992 against 986 us per launch; fewer rows for them, consumed from
+  // the ring while the refills go to a cached dummy tile and the real requests follow when the head is done: no
+  // change.)
   const bool is_attn = wg < a.Hq;
   const int nA0 = 4 * (int)((int64_t)(a.n_qkv / 4) * wg / G), nA1 = 4 * (int)((int64_t)(a.n_qkv / 4) * (wg + 1) / G);
   const int rowsA = nA1 - nA0;
@@ -477,7 +505,8 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   // A stream wave whose phases all hold at least one pass over the ring (or nothing) also keeps kMegaStage tiles
   // in LDS: requested when the wave starts to wait with a full ring, consumed first when it streams again.
   unsigned char *const stage = mg_smem + a.stage_off + wave * (kMegaStage * 1024);
-  const bool stages = a.stage_off != 0 && streams && (ttA_w == 0 || ttA_w >= kMegaRing) && (ttB_w == 0 || ttB_w >= kMegaRing);
+  const bool stages = a.stage_off != 0 && streams && ttA_w + ttB_w > 0 && (ttA_w == 0 || ttA_w >= kMegaRing) &&
+                      (ttB_w == 0 || ttB_w >= kMegaRing);
   bool staged = false;
 
   MgSplit sp;
@@ -492,16 +521,11 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     sp.nx2 = e0 ? 0 : e1 ? 1 : 2;
   }
   MgCursor cur;
-  cur.layer = 0; cur.seg = 0; cur.kc = 0; cur.KT = 1; cur.left = 0; cur.ld = 0;
+  cur.layer = 0; cur.seg = 0; cur.kc = 0; cur.KT = 1; cur.left = 0; cur.jump = 0;
   cur.ptr = a.Wa0;
-  cur.done = true;
-  {
-    const int first = sp.cnt0 > 0 ? 0 : sp.cnt1 > 0 ? 1 : sp.cnt2 > 0 ? 2 : -1;
-    if (first >= 0 && a.L > 0) {
-      cur.done = false;
-      mg_seg_enter(cur, sp, 0, first);
-    }
-  }
+  const bool streams_any = streams && ttA_w + ttB_w > 0;   // (a wave without tiles never requests one)
+  if (streams_any) mg_seg_enter(cur, sp, 0, sp.cnt0 > 0 ? 0 : sp.cnt1 > 0 ? 1 : 2);
+  const MgPhase phA = mg_phase(tA0, tA1, tA2_0, tA2_1, KTA), phB = mg_phase(tB0, tB1, 0, 0, KTBC);
   unsigned bar = 0;
   int pending_rot = 0;
   const uint32_t tagbase = a.state->epoch * kMegaTagsPerLaunch;   // exchange tags of this launch: tagbase + index + 1
@@ -575,7 +599,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     const int lane = tid0 & 63;
 #pragma unroll
     for (int p = 0; p < kMegaRing; ++p) {
-      ring[p] = streams ? mg_next_load(cur, sp, lane) : MG_ZERO4;
+      ring[p] = streams_any ? mg_next_load(cur, sp, lane) : MG_ZERO4;
     }
   }
 #pragma unroll
@@ -704,8 +728,8 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       // the ring is rotated only now, just before it is consumed again: a rotation moves registers that loads
       // are still writing, i.e. it waits for the newest of them, and by now those have had a whole exchange to land
       mg_rotate_by(ring, pending_rot);
-      pending_rot = mg_run_phase(ring, cur, sp, tA0, tA1, tA2_0, tA2_1, KTA, xn, partA, partA + rowsA * kMegaWaves,
-                                 a1_done, lane, wave, stage, staged);
+      pending_rot = mg_run_phase(ring, cur, sp, phA, KTA, xn, partA, partA + rowsA * kMegaWaves, a1_done, lane, wave,
+                                 stage, staged);
       if (service) {   // its own ranges are empty: it arrives here at once and waits for the seven others
         unsigned spins = 0;
         while (__hip_atomic_load(a1_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)kMegaWaves) {
@@ -916,7 +940,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
       wg_sync();
       stamp(l, 3);
       mg_rotate_by(ring, pending_rot);
-      pending_rot = mg_run_phase(ring, cur, sp, tB0, tB1, 0, 0, KTBC, xa, partB, partB, nullptr, lane, wave, stage, staged);
+      pending_rot = mg_run_phase(ring, cur, sp, phB, KTBC, xa, partB, partB, nullptr, lane, wave, stage, staged);
       stamp(l, 4);
       wg_sync();
       stamp(l, 5);
