@@ -158,12 +158,12 @@ struct MgSplit {
   int nx0, nx1, nx2;          // the next segment that is not empty (cyclic; the segment itself when it is the only one)
 };
 
-// ptr is the tile that is requested next; the tiles of a row follow each other (512 elements), the next row
-// starts `jump` elements behind the row's last tile.  Behind the last layer the stream starts again with the
-// first (those requests are never used; they keep the loop free of an end-of-stream case).
+// ptr is the tile that is requested next; the tiles of a row follow each other (`step` = 512 elements), the next
+// row starts `jump` elements behind the row's last tile.  Behind the last layer step and jump are 0: the last tile
+// is requested again and again (never used; the streaming loops need no end-of-stream case that way).
 struct MgCursor {
   int layer, seg, kc, KT, left;   // left: tiles of the segment not yet requested, the one under the cursor included
-  int64_t jump;
+  int64_t jump, step;
   const uint16_t *ptr;
 };
 
@@ -178,6 +178,7 @@ __device__ __forceinline__ void mg_seg_enter(MgCursor &c, const MgSplit &sp, int
   c.seg = seg;
   c.KT = wa ? sp.KTA : sp.KTBC;
   c.jump = (int64_t)(wa ? sp.H : sp.KB) - (int64_t)(c.KT - 1) * 512;
+  c.step = 512;
   c.kc = seg == 0 ? kc0 : seg == 1 ? kc1 : kc2;
   c.left = seg == 0 ? cnt0 : seg == 1 ? cnt1 : cnt2;
   c.ptr = base + (seg == 0 ? off0 : seg == 1 ? off1 : off2) + c.kc * 512;
@@ -187,11 +188,15 @@ __device__ __forceinline__ void mg_advance(MgCursor &c, const MgSplit &sp) {
     const int nx0 = sp.nx0, nx1 = sp.nx1, nx2 = sp.nx2;
     const int ns = c.seg == 0 ? nx0 : c.seg == 1 ? nx1 : nx2;
     const int nl = c.layer + (ns <= c.seg ? 1 : 0);
-    mg_seg_enter(c, sp, nl >= sp.L ? 0 : nl, ns);
+    if (nl >= sp.L) {   // behind the last layer: the cursor stays on the last tile (requests that hit the caches)
+      c.kc = 0; c.KT = 0x7fffffff; c.left = 0x7fffffff; c.jump = 0; c.step = 0;
+    } else {
+      mg_seg_enter(c, sp, nl, ns);
+    }
   } else {
     const bool wrap = c.kc + 1 == c.KT;
     c.kc = wrap ? 0 : c.kc + 1;
-    c.ptr += wrap ? c.jump : (int64_t)512;
+    c.ptr += wrap ? c.jump : c.step;
   }
 }
 // requests the tile under the cursor and advances the cursor
@@ -521,7 +526,7 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
     sp.nx2 = e0 ? 0 : e1 ? 1 : 2;
   }
   MgCursor cur;
-  cur.layer = 0; cur.seg = 0; cur.kc = 0; cur.KT = 1; cur.left = 0; cur.jump = 0;
+  cur.layer = 0; cur.seg = 0; cur.kc = 0; cur.KT = 1; cur.left = 0; cur.jump = 0; cur.step = 0;
   cur.ptr = a.Wa0;
   const bool streams_any = streams && ttA_w + ttB_w > 0;   // (a wave without tiles never requests one)
   if (streams_any) mg_seg_enter(cur, sp, 0, sp.cnt0 > 0 ? 0 : sp.cnt1 > 0 ? 1 : 2);
