@@ -860,18 +860,25 @@ typedef __attribute__((ext_vector_type(16))) float fa_f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t fa_u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t fa_u32x2;
 
-template <int NW, int D, bool F32S>
-__global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
+// KSP = 2: every 32-query group is worked on by two waves, one for the even and one for the odd key tiles, each with
+// its own running maximum, sum and output; the two are merged through LDS at the end.  For short sequences and few
+// heads, where the grid has about one block per CU and a wave's chain of key tiles is what the launch takes.
+template <int NW, int D, bool F32S, int KSP = 1>
+__global__ void __launch_bounds__(NW * KSP * 64) k_flash_prefill_bf16(AttnArgs a) {
   constexpr int KS = D / 16;            // K steps of the score product
   constexpr int DT = (D + 31) / 32;     // 32-row tiles of O^T
   constexpr int KP = D + 8;             // K tile pitch (elements)
   constexpr int VP = 64 + 4;            // V^T tile pitch (elements)
-  constexpr int NT = NW * 64;
+  constexpr int NT = NW * KSP * 64;
   constexpr int CPR = D / 8;            // 16-byte chunks per key row
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[64 * KP];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt[DT * 32 * VP];
+  constexpr int KTILE = 64 * KP, VTILE = DT * 32 * VP;   // elements of one K tile / one V^T tile in LDS
+  __shared__ __attribute__((aligned(16))) uint16_t fa_smem[KSP * (KTILE + VTILE)];
+  uint16_t *const Ks = fa_smem, *const Vt = fa_smem + KSP * KTILE;   // KSP tiles each, one behind the other
+  static_assert(KSP == 1 || sizeof(float) * NW * 64 * (2 + DT * 16) <= sizeof(uint16_t) * KSP * (KTILE + VTILE),
+                "the merge of the key halves reuses the tile memory");
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
+  const int wave = (tid >> 6) / KSP, kh = (tid >> 6) % KSP;   // query group of the block, key tiles kh, kh + KSP, ...
   const int h = blockIdx.y, b = blockIdx.z;
   const int hk = h / (a.Hq / a.Hkv);
   // the last query tiles see the most keys under a causal mask: they go first so that the short ones fill the tail
@@ -907,16 +914,16 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
   // K: 16-byte chunks, row-major into Ks.  V: each work item is one pair of head features (d, d+1) for 8
   // consecutive keys: eight 4-byte loads (lanes run along d, so a wave reads whole rows), repacked in
   // registers into the two 8-key rows of V^T, which are written with 8-byte stores.
-  constexpr int CH = (64 * CPR + NT - 1) / NT;   // 16-byte chunks of K per thread
-  constexpr int NP = D / 2;                      // feature pairs
-  constexpr int VI = (8 * NP + NT - 1) / NT;     // V work items per thread
+  constexpr int CH = (KSP * 64 * CPR + NT - 1) / NT;   // 16-byte chunks of K per thread (KSP tiles per round)
+  constexpr int NP = D / 2;                            // feature pairs
+  constexpr int VI = (KSP * 8 * NP + NT - 1) / NT;     // V work items per thread
   constexpr bool PF = D <= 128;
   fa_u32x4 kreg[CH];
   uint32_t vx[PF ? VI : 1][8];
   auto load_v = [&](int i, int k0, uint32_t (&x)[8]) {
     const int c = tid + i * NT;
     const int pr = c % NP, g = c / NP;
-    if (c < 8 * NP) {
+    if (c < KSP * 8 * NP) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         int t = k0 + g * 8 + j;
@@ -928,7 +935,7 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
   auto store_v = [&](int i, const uint32_t (&x)[8]) {
     const int c = tid + i * NT;
     const int pr = c % NP, g = c / NP;
-    if (c < 8 * NP) {
+    if (c < KSP * 8 * NP) {
       fa_u32x2 lo0, lo1, hi0, hi1;   // feature 2*pr: keys 0-3, 4-7; feature 2*pr+1: keys 0-3, 4-7
       lo0.x = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
       lo0.y = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
@@ -938,7 +945,7 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
       hi0.y = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
       hi1.x = __builtin_amdgcn_perm(x[5], x[4], 0x07060302u);
       hi1.y = __builtin_amdgcn_perm(x[7], x[6], 0x07060302u);
-      uint16_t *r0 = Vt + (2 * pr) * VP + g * 8, *r1 = r0 + VP;
+      uint16_t *r0 = Vt + (g / 8) * VTILE + (2 * pr) * VP + (g % 8) * 8, *r1 = r0 + VP;   // key group g: tile g / 8
       *reinterpret_cast<fa_u32x2 *>(r0) = lo0;
       *reinterpret_cast<fa_u32x2 *>(r0 + 4) = lo1;
       *reinterpret_cast<fa_u32x2 *>(r1) = hi0;
@@ -952,7 +959,7 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
       const int key = c / CPR, dc = (c % CPR) * 8;
       int t = k0 + key;
       t = t < a.T ? t : a.T - 1;
-      if (c < 64 * CPR) kreg[i] = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
+      if (c < KSP * 64 * CPR) kreg[i] = *reinterpret_cast<const fa_u32x4 *>(Kg + (int64_t)t * a.ks[2] + dc);
     }
     if constexpr (PF) {
 #pragma unroll
@@ -964,7 +971,7 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
     for (int i = 0; i < CH; ++i) {
       const int c = tid + i * NT;
       const int key = c / CPR, dc = (c % CPR) * 8;
-      if (c < 64 * CPR) *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kreg[i];
+      if (c < KSP * 64 * CPR) *reinterpret_cast<fa_u32x4 *>(Ks + key * KP + dc) = kreg[i];   // tile key / 64 follows tile 0
     }
     if constexpr (PF) {
 #pragma unroll
@@ -981,15 +988,18 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
     }
   };
   if (PF && kv_end > 0) load_tile(0);
-  for (int k0 = 0; k0 < kv_end; k0 += 64) {
+  for (int kb = 0; kb < kv_end; kb += 64 * KSP) {
     __syncthreads();
-    // ---- stage K [64][D] and V^T [D][64]
-    if (!PF) load_tile(k0);
+    // ---- stage K [64][D] and V^T [D][64], KSP tiles of each
+    if (!PF) load_tile(kb);
     store_tile();
-    if (!PF) stage_v_direct(k0);
+    if (!PF) stage_v_direct(kb);
     __syncthreads();
-    if (PF && k0 + 64 < kv_end) load_tile(k0 + 64);
-    if (k0 > wave_last_key) continue;  // every key of this tile is masked for this wave (barriers stay uniform)
+    if (PF && kb + 64 * KSP < kv_end) load_tile(kb + 64 * KSP);
+    const int k0 = kb + 64 * kh;       // this wave's tile of the round
+    // every key of this tile is masked for this wave, or the tile lies behind the block's keys (barriers stay uniform)
+    if (k0 > wave_last_key || k0 >= kv_end) continue;
+    const uint16_t *const Kt = Ks + kh * KTILE, *const Vw = Vt + kh * VTILE;
 
     // ---- S^T tile: 64 keys x 32 queries
     fa_f32x16 sc[2];
@@ -997,7 +1007,7 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
     for (int u = 0; u < 2; ++u) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) sc[u][r] = 0.f;
-      const uint16_t *kr = Ks + (u * 32 + l32) * KP + half * 8;
+      const uint16_t *kr = Kt + (u * 32 + l32) * KP + half * 8;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
         sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const fa_bf16x8 *>(kr + ks * 16), qf[ks], sc[u],
@@ -1068,7 +1078,7 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
     // ---- O^T += V^T . P^T
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const uint16_t *vr = Vt + (dt * 32 + l32) * VP + 4 * half;
+      const uint16_t *vr = Vw + (dt * 32 + l32) * VP + 4 * half;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -1081,6 +1091,31 @@ __global__ void __launch_bounds__(NW * 64) k_flash_prefill_bf16(AttnArgs a) {
     }
   }
 
+  if constexpr (KSP == 2) {
+    // the odd key tiles' wave hands its maximum, sum and output over; the even tiles' wave merges and goes on alone
+    __syncthreads();   // the tiles are no longer read
+    float *mb = reinterpret_cast<float *>(fa_smem) + (wave * 64 + lane) * (2 + DT * 16);
+    if (kh == 1) {
+      mb[0] = m_run;
+      mb[1] = l_run;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mb[2 + dt * 16 + r] = o[dt][r];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float m1 = mb[0], l1 = mb[1];
+    const float m = fmaxf(m_run, m1);
+    const float ms = m == -INFINITY ? 0.f : m;   // nothing seen by either: both weights are exp(-inf) = 0
+    const float w0 = __builtin_amdgcn_exp2f((m_run - ms) * kLog2e), w1 = __builtin_amdgcn_exp2f((m1 - ms) * kLog2e);
+    l_run = l_run * w0 + l1 * w1;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * w0 + mb[2 + dt * 16 + r] * w1;
+  }
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   if (qrow < a.S) {
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -1107,6 +1142,15 @@ template <int D> static int launch_flash(hipStream_t st, const AttnArgs &a) {
     else hipLaunchKernelGGL((k_flash_prefill_bf16<4, D, false>), dim3(tiles4, a.Hq, a.B), dim3(256), 0, st, a);
   } else {
     const dim3 grid((a.S + 63) / 64, a.Hq, a.B);
+    // about one block per CU or fewer, several key tiles per block: two waves per query group, each half of the keys
+    const char *no_split = getenv("RAI_HIP_FLASH_NO_KEY_SPLIT");   // read per call: tests compare both forms
+    if constexpr (D <= 80) {
+      if ((int64_t)grid.x * grid.y * grid.z < 2 * kNumCU && a.T > 128 && !(no_split && *no_split && *no_split != '0')) {
+        if (a.f32_scores) hipLaunchKernelGGL((k_flash_prefill_bf16<2, D, true, 2>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((k_flash_prefill_bf16<2, D, false, 2>), grid, dim3(256), 0, st, a);
+        return launch_check("flash_prefill");
+      }
+    }
     if (a.f32_scores) hipLaunchKernelGGL((k_flash_prefill_bf16<2, D, true>), grid, dim3(128), 0, st, a);
     else hipLaunchKernelGGL((k_flash_prefill_bf16<2, D, false>), grid, dim3(128), 0, st, a);
   }

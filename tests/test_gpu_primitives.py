@@ -493,6 +493,35 @@ def test_attention(R, dt, hq, hkv, s, t, d, causal, f32s):
     assert_close(got, want, dt, "attention")
 
 
+@pytest.mark.parametrize("hq,hkv,s,t,d,causal,f32s", [(4, 4, 512, 512, 80, 1, 1), (4, 2, 300, 320, 64, 1, 0),
+                                                     (3, 3, 64, 257, 80, 0, 1), (2, 2, 129, 640, 80, 1, 1)])
+def test_flash_prefill_key_split_against_single_chain(R, monkeypatch, hq, hkv, s, t, d, causal, f32s):
+    """Short sequences with few heads run the flash kernel with two waves per query group, one for the even and one
+    for the odd key tiles, merged at the end (odd tile counts, a last tile past the context and non-square causal
+    shapes included).  Both forms are held to the oracle; against each other they differ by rounding only."""
+    import math
+    dt = "bf16"
+    g = rng(29)
+    q, k, v = rand(g, (1, hq, s, d), dt), rand(g, (1, hkv, t, d), dt), rand(g, (1, hkv, t, d), dt)
+    scale = 1.0 / math.sqrt(d)
+    kr, vr = np.repeat(k, hq // hkv, 1), np.repeat(v, hq // hkv, 1)
+    mask = (np.arange(t)[None, :] > (np.arange(s)[:, None] + (t - s))) if causal else np.zeros((s, t), bool)
+    if f32s:
+        w = oo.matmul(oo.to_dtype(q, dt, "f32"), oo.mul(np.swapaxes(oo.to_dtype(kr, dt, "f32"), -1, -2),
+                                                       np.float32(scale), "f32"), "f32")
+        p = oo.to_dtype(oo.softmax(np.where(mask, np.float32(-np.inf), w), -1, "f32"), "f32", dt)
+    else:
+        w = oo.mul(oo.matmul(q, np.swapaxes(kr, -1, -2), dt), oo.full_like(np.zeros(()), scale, dt, "f64"), dt)
+        p = oo.softmax(oo.add(w, np.where(mask, np.float32(-np.inf), np.float32(0)), dt), -1, dt)
+    want = oo.matmul(p, vr, dt).transpose(0, 2, 1, 3).reshape(1, s, hq * d)
+    got = {}
+    for off in ("0", "1"):
+        monkeypatch.setenv("RAI_HIP_FLASH_NO_KEY_SPLIT", off)     # read per call
+        got[off] = down(R.attention(up(q, dt), up(k, dt), up(v, dt), scale, causal, f32s))
+        assert_close(got[off], want, dt, f"attention, key split {'off' if off == '1' else 'on'}")
+    assert_close(got["0"], got["1"], dt, "key split against single chain")
+
+
 # ------------------------------------------------------------------ error behaviour
 def test_errors_are_reported_not_silent(R):
     from rai_amd._lib import RaiHipError
