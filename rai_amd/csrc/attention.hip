@@ -863,6 +863,7 @@ typedef __attribute__((ext_vector_type(2))) uint32_t fa_u32x2;
 // KSP = 2: every 32-query group is worked on by two waves, one for the even and one for the odd key tiles, each with
 // its own running maximum, sum and output; the two are merged through LDS at the end.  For short sequences and few
 // heads, where the grid has about one block per CU and a wave's chain of key tiles is what the launch takes.
+// (Four waves per group, KSP = 4, gained another half per cent on the Phi-2 prefill: not instantiated.)
 template <int NW, int D, bool F32S, int KSP = 1>
 __global__ void __launch_bounds__(NW * KSP * 64) k_flash_prefill_bf16(AttnArgs a) {
   constexpr int KS = D / 16;            // K steps of the score product
@@ -874,7 +875,7 @@ __global__ void __launch_bounds__(NW * KSP * 64) k_flash_prefill_bf16(AttnArgs a
   constexpr int KTILE = 64 * KP, VTILE = DT * 32 * VP;   // elements of one K tile / one V^T tile in LDS
   __shared__ __attribute__((aligned(16))) uint16_t fa_smem[KSP * (KTILE + VTILE)];
   uint16_t *const Ks = fa_smem, *const Vt = fa_smem + KSP * KTILE;   // KSP tiles each, one behind the other
-  static_assert(KSP == 1 || sizeof(float) * NW * 64 * (2 + DT * 16) <= sizeof(uint16_t) * KSP * (KTILE + VTILE),
+  static_assert(KSP == 1 || sizeof(float) * NW * 64 * (KSP - 1) * (2 + DT * 16) <= sizeof(uint16_t) * KSP * (KTILE + VTILE),
                 "the merge of the key halves reuses the tile memory");
 
   const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
@@ -1091,30 +1092,43 @@ __global__ void __launch_bounds__(NW * KSP * 64) k_flash_prefill_bf16(AttnArgs a
     }
   }
 
-  if constexpr (KSP == 2) {
-    // the odd key tiles' wave hands its maximum, sum and output over; the even tiles' wave merges and goes on alone
+  if constexpr (KSP > 1) {
+    // the waves of key tiles 1 .. KSP-1 (mod KSP) hand their maximum, sum and output over; the wave of tiles 0 merges
+    // and goes on alone
     __syncthreads();   // the tiles are no longer read
-    float *mb = reinterpret_cast<float *>(fa_smem) + (wave * 64 + lane) * (2 + DT * 16);
-    if (kh == 1) {
-      mb[0] = m_run;
-      mb[1] = l_run;
+    constexpr int MS = 2 + DT * 16;
+    float *mb = reinterpret_cast<float *>(fa_smem) + (size_t)((wave * 64 + lane) * (KSP - 1)) * MS;
+    if (kh > 0) {
+      float *mine = mb + (kh - 1) * MS;
+      mine[0] = m_run;
+      mine[1] = l_run;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mb[2 + dt * 16 + r] = o[dt][r];
+        for (int r = 0; r < 16; ++r) mine[2 + dt * 16 + r] = o[dt][r];
     }
     __syncthreads();
-    if (kh == 1) return;
+    if (kh > 0) return;
     constexpr float kLog2e = 1.4426950408889634f;
-    const float m1 = mb[0], l1 = mb[1];
-    const float m = fmaxf(m_run, m1);
-    const float ms = m == -INFINITY ? 0.f : m;   // nothing seen by either: both weights are exp(-inf) = 0
-    const float w0 = __builtin_amdgcn_exp2f((m_run - ms) * kLog2e), w1 = __builtin_amdgcn_exp2f((m1 - ms) * kLog2e);
-    l_run = l_run * w0 + l1 * w1;
+    float m = m_run;
+#pragma unroll
+    for (int j = 0; j < KSP - 1; ++j) m = fmaxf(m, mb[j * MS]);
+    const float ms = m == -INFINITY ? 0.f : m;   // nothing seen by any of them: every weight is exp(-inf) = 0
+    const float w0 = __builtin_amdgcn_exp2f((m_run - ms) * kLog2e);
+    l_run *= w0;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * w0 + mb[2 + dt * 16 + r] * w1;
+      for (int r = 0; r < 16; ++r) o[dt][r] *= w0;
+#pragma unroll
+    for (int j = 0; j < KSP - 1; ++j) {
+      const float wj = __builtin_amdgcn_exp2f((mb[j * MS] - ms) * kLog2e);
+      l_run += mb[j * MS + 1] * wj;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] += mb[j * MS + 2 + dt * 16 + r] * wj;
+    }
   }
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   if (qrow < a.S) {
