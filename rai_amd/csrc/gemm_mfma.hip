@@ -842,98 +842,102 @@ __global__ void __launch_bounds__(256) k_splitk_epilogue(LinearArgs a, int split
   }
 }
 
-// The same pass for a Linear whose output rows are normalised next: a wave owns a row (N <= 512 * ITEMS columns, 8
-// per lane and item), sums the partial products, applies bias / activation / residual, stores the bf16 row, and then
-// runs LayerNorm on the stored (rounded) values with the arithmetic of the stand-alone norm kernel -- same
+// The same pass for a Linear whose output rows are normalised next.  A block of four waves owns a row (N <= 512 *
+// ITEMS columns).  The sums over the partial products, bias / activation / residual and the bf16 store are element
+// by element, so they are shared out: every wave takes a quarter of the row's 16-byte packs (512 rows are then eight
+// waves per CU with one round of loads each, instead of two waves with two rounds).  The stored (rounded) row goes
+// through LDS to the first wave, which runs LayerNorm on it with the arithmetic of the stand-alone norm kernel -- same
 // per-lane order, same wave reductions -- so fusing changes no bit (rai-nn/src/layer_norm.rs:32-42).
 template <int ITEMS>
-__global__ void __launch_bounds__(128) k_splitk_epilogue_ln(LinearArgs a, int splits, const float *partial) {
-  const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 2 + (threadIdx.x >> 6);
-  if (row >= a.M) return;
+__global__ void __launch_bounds__(256) k_splitk_epilogue_ln(LinearArgs a, int splits, const float *partial) {
+  constexpr int NWV = 4;                                 // waves per row
+  constexpr int JT = (ITEMS * 64 / NWV + 63) / 64;       // packs per lane in the summing part
+  __shared__ u32x4 rowbuf[64 * ITEMS];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = blockIdx.x;
   const int packs = a.N / 8;
+  const int quarter = (packs + NWV - 1) / NWV;
   const int64_t total = (int64_t)a.M * a.N;
   const uint16_t *bias = (const uint16_t *)a.bias, *bias2 = (const uint16_t *)a.bias2;
   const uint16_t *res = (const uint16_t *)a.residual;
-  float v[ITEMS][8];
-  float s = 0.f;
-  // A wave has a whole row to itself and nothing else to overlap its memory round trips with (512 rows are two waves
-  // per CU), so loads are issued as early and as many at a time as the registers allow: the bias and residual chunks
-  // of every column group first, then the partial products for three column groups of the lane at a time (six splits
-  // each, 36 x 16 bytes per lane in flight), while every element's additions stay in split order.
-  u32x4 braw[ITEMS], b2raw[ITEMS], rraw[ITEMS];
+  {
+    // loads are issued as early and as many at a time as the registers allow: bias and residual first, then the
+    // partial products of all the lane's packs (six splits each), while every element's additions stay in split order
+    int pk[JT];
+    bool on[JT];
+    u32x4 braw[JT], b2raw[JT], rraw[JT];
+    float x[JT][8];
 #pragma unroll
-  for (int it = 0; it < ITEMS; ++it) {
-    const int p = lane + it * 64;
-    const int n = (p < packs ? p : lane % packs) * 8;   // clamped groups are never used
-    braw[it] = b2raw[it] = rraw[it] = u32x4{0u, 0u, 0u, 0u};
-    if (bias) braw[it] = *reinterpret_cast<const u32x4 *>(bias + n);
-    if (bias2) b2raw[it] = *reinterpret_cast<const u32x4 *>(bias2 + n);
-    if (res) rraw[it] = *reinterpret_cast<const u32x4 *>(res + (int64_t)row * a.ldr + n);
-  }
+    for (int j = 0; j < JT; ++j) {
+      const int q = lane + j * 64;
+      pk[j] = wv * quarter + q;
+      on[j] = q < quarter && pk[j] < packs;
+      if (!on[j]) pk[j] = 0;   // a clamped pack is loaded and never used
+      const int n = pk[j] * 8;
+      braw[j] = b2raw[j] = rraw[j] = u32x4{0u, 0u, 0u, 0u};
+      if (bias) braw[j] = *reinterpret_cast<const u32x4 *>(bias + n);
+      if (bias2) b2raw[j] = *reinterpret_cast<const u32x4 *>(bias2 + n);
+      if (res) rraw[j] = *reinterpret_cast<const u32x4 *>(res + (int64_t)row * a.ldr + n);
 #pragma unroll
-  for (int it = 0; it < ITEMS; ++it)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[it][e] = 0.f;
-  constexpr int GR = 3;   // column groups in flight together
-#pragma unroll
-  for (int it0 = 0; it0 < ITEMS; it0 += GR) {
-    const float *pp[GR];
-#pragma unroll
-    for (int j = 0; j < GR; ++j) {
-      const int p = lane + (it0 + j < ITEMS ? it0 + j : it0) * 64;
-      pp[j] = partial + (int64_t)row * a.N + (p < packs ? p : lane % packs) * 8;   // clamped groups are never used
+      for (int e = 0; e < 8; ++e) x[j][e] = 0.f;
     }
     for (int s0 = 0; s0 < splits; s0 += 6) {
-      f32x4 p0[GR][6], p1[GR][6];
+      f32x4 p0[JT][6], p1[JT][6];
 #pragma unroll
-      for (int j = 0; j < GR; ++j)
+      for (int j = 0; j < JT; ++j)
 #pragma unroll
         for (int u = 0; u < 6; ++u) {
           const int sp = s0 + u < splits ? s0 + u : splits - 1;
-          p0[j][u] = *reinterpret_cast<const f32x4 *>(pp[j] + (int64_t)sp * total);
-          p1[j][u] = *reinterpret_cast<const f32x4 *>(pp[j] + (int64_t)sp * total + 4);
+          const float *pp = partial + (int64_t)sp * total + (int64_t)row * a.N + pk[j] * 8;
+          p0[j][u] = *reinterpret_cast<const f32x4 *>(pp);
+          p1[j][u] = *reinterpret_cast<const f32x4 *>(pp + 4);
         }
 #pragma unroll
-      for (int j = 0; j < GR; ++j) {
-        if (it0 + j < ITEMS) {
-          float *x = v[it0 + j];
+      for (int j = 0; j < JT; ++j)
 #pragma unroll
-          for (int u = 0; u < 6; ++u) {
-            if (s0 + u < splits) {
-              x[0] += p0[j][u].x; x[1] += p0[j][u].y; x[2] += p0[j][u].z; x[3] += p0[j][u].w;
-              x[4] += p1[j][u].x; x[5] += p1[j][u].y; x[6] += p1[j][u].z; x[7] += p1[j][u].w;
-            }
+        for (int u = 0; u < 6; ++u) {
+          if (s0 + u < splits) {
+            x[j][0] += p0[j][u].x; x[j][1] += p0[j][u].y; x[j][2] += p0[j][u].z; x[j][3] += p0[j][u].w;
+            x[j][4] += p1[j][u].x; x[j][5] += p1[j][u].y; x[j][6] += p1[j][u].z; x[j][7] += p1[j][u].w;
           }
         }
+    }
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+      if (on[j]) {
+        const int n = pk[j] * 8;
+        float b1[8], b2[8];
+        unpack8(braw[j], b1);     // zero bits where there is no bias: +0.0
+        unpack8(b2raw[j], b2);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[j][e] += b1[e] + b2[e];
+        if (a.act >= 0) act8(a.act, x[j], n, a.act_from);
+        if (res) {
+          float rv[8];
+          unpack8(rraw[j], rv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[j][e] += rv[e];
+        }
+        u32x4 o;
+        o.x = (uint32_t)f32_to_bf16_bits(x[j][0]) | ((uint32_t)f32_to_bf16_bits(x[j][1]) << 16);
+        o.y = (uint32_t)f32_to_bf16_bits(x[j][2]) | ((uint32_t)f32_to_bf16_bits(x[j][3]) << 16);
+        o.z = (uint32_t)f32_to_bf16_bits(x[j][4]) | ((uint32_t)f32_to_bf16_bits(x[j][5]) << 16);
+        o.w = (uint32_t)f32_to_bf16_bits(x[j][6]) | ((uint32_t)f32_to_bf16_bits(x[j][7]) << 16);
+        *reinterpret_cast<u32x4 *>((uint16_t *)a.out1 + (int64_t)row * a.ld1 + n) = o;
+        rowbuf[pk[j]] = o;
       }
     }
   }
+  __syncthreads();
+  if (wv != 0) return;
+  // ---- LayerNorm of the stored row, one wave, pack p = lane + 64 it
+  float v[ITEMS][8];
+  float s = 0.f;
 #pragma unroll
   for (int it = 0; it < ITEMS; ++it) {
     const int p = lane + it * 64;
     if (p < packs) {
-      const int n = p * 8;
-      float (&x)[8] = v[it];
-      float b1[8], b2[8];
-      unpack8(braw[it], b1);     // zero bits where there is no bias: +0.0, as before
-      unpack8(b2raw[it], b2);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] += b1[e] + b2[e];
-      if (a.act >= 0) act8(a.act, x, n, a.act_from);
-      if (res) {
-        float rv[8];
-        unpack8(rraw[it], rv);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] += rv[e];
-      }
-      u32x4 o;
-      o.x = (uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
-      o.y = (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
-      o.z = (uint32_t)f32_to_bf16_bits(x[4]) | ((uint32_t)f32_to_bf16_bits(x[5]) << 16);
-      o.w = (uint32_t)f32_to_bf16_bits(x[6]) | ((uint32_t)f32_to_bf16_bits(x[7]) << 16);
-      *reinterpret_cast<u32x4 *>((uint16_t *)a.out1 + (int64_t)row * a.ld1 + n) = o;
-      unpack8(o, v[it]);
+      unpack8(rowbuf[p], v[it]);
 #pragma unroll
       for (int e = 0; e < 8; ++e) s += v[it][e];
     }
@@ -989,7 +993,7 @@ static bool post_norm_fits(const LinearArgs &a) {
 static int launch_splitk_epilogue(hipStream_t st, const LinearArgs &a, int splits, const float *partial) {
   if (post_norm_fits(a)) {
     const int items = (a.N / 8 + 63) / 64;
-    const dim3 grid((a.M + 1) / 2), block(128);
+    const dim3 grid(a.M), block(256);
     if (items <= 2) hipLaunchKernelGGL(k_splitk_epilogue_ln<2>, grid, block, 0, st, a, splits, partial);
     else if (items <= 5) hipLaunchKernelGGL(k_splitk_epilogue_ln<5>, grid, block, 0, st, a, splits, partial);
     else hipLaunchKernelGGL(k_splitk_epilogue_ln<8>, grid, block, 0, st, a, splits, partial);
