@@ -132,3 +132,16 @@ def test_safetensors_index_files_host_only(tmp_path):
     idx.write_text("{not json")
     with pytest.raises(RaiHipError):
         safetensors_index_files(idx)
+
+
+def test_every_environment_knob_of_the_library_is_documented():
+    """The library reads a handful of RAI_HIP_* variables (tuning and test aids, most of them read per call).  Each one
+    that occurs in the sources has a row in the knob table of the integration notes."""
+    knobs = set()
+    for src in sorted((ROOT / "rai_amd" / "csrc").iterdir()):
+        if src.suffix in (".hip", ".cpp", ".h"):
+            knobs |= set(re.findall(r'getenv\("(RAI_HIP_[A-Z0-9_]+)"\)', src.read_text()))
+    assert len(knobs) >= 10, knobs
+    doc = (ROOT / "INTEGRATION.md").read_text()
+    missing = sorted(k for k in knobs if f"`{k}`" not in doc)
+    assert not missing, f"not in the knob table: {missing}"
