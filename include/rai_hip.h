@@ -400,9 +400,10 @@ int rai_hip_decoder_param_shape(rai_hip_decoder *dec, int32_t i, int64_t *rows, 
  * cached context; returns last-position logits [batch, vocab] as f32 in
  * logits_host (nullable) and greedy tokens (device argmax, first-max) in
  * tokens_host (nullable).  Synchronises only if an output pointer is given.
- * A single-token step (batch 1, seq 1) of a Phi-2-architecture model with exactly Phi-2's widths (hidden 2560 = 32
- * heads x 80, no grouped-query attention, intermediate and q|k|v widths multiples of 512, bf16) runs all layers as one
- * launch of a persistent kernel; every other model, width, batch or dtype takes one launch per primitive. */
+ * A single-token step (batch 1, seq 1) of a Phi-2-architecture model in bf16 whose hidden width is 2560 = 32 heads
+ * x 80 (Phi-2) or 2048 = 32 heads x 64 (Phi-1 / Phi-1.5), with or without grouped-query attention, intermediate and
+ * q|k|v widths multiples of 512, runs all layers as one launch of a persistent kernel; every other model, width,
+ * batch or dtype takes one launch per primitive. */
 int rai_hip_decoder_forward(rai_hip_decoder *dec, const uint32_t *ids_host, int32_t batch, int32_t seq,
                             float *logits_host, uint32_t *tokens_host);
 /* Greedy loop of examples/phi2/src/main.rs:75-95 without repeat penalty: prefill

@@ -26,13 +26,13 @@ struct MegaArgs {
   const MegaLayer *layers;  // device array [L]
   const uint16_t *Wa0, *Wb0;      // layer 0; layer l sits wa_stride / wb_stride elements further
   int64_t wa_stride, wb_stride;
-  int L, H, I, QD, NA, n_qkv, Hq, rot, Tmax;
+  int L, H, I, QD, NA, n_qkv, Hq, Hkv, rot, Tmax;   // Hkv < Hq: Hq / Hkv query heads share a key/value head
   uint16_t *x;              // [H] residual stream, updated in place
   // Vectors exchanged between blocks inside the launch, as 8-byte packets: {two bf16 values, 32-bit tag} for xp and
   // qkvp, {three bf16 values, 16-bit tag in the top bits} for actp and attnp.  A packet is valid for an exchange when
   // its tag is (the low bits of) epoch * 1024 + exchange index + 1.
   uint64_t *xp;             // [H / 2]      residual stream after a layer
-  uint64_t *qkvp;           // [3 * QD / 2]
+  uint64_t *qkvp;           // [(QD + 2 * Hkv * D) / 2]
   uint64_t *actp;           // [kMegaActPackets] gelu(fc1), three values to a packet, 16 packets per producer block
   uint64_t *attnp;          // [Hq * ceil(D / 3)] attention output, three values to a packet
   uint16_t *kcache, *vcache;

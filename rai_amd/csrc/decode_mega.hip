@@ -438,6 +438,9 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   // the ring while the refills go to a cached dummy tile and the real requests follow when the head is done: no
   // change.)
   const bool is_attn = wg < a.Hq;
+  const int kv_group = a.Hq / a.Hkv;                 // query heads per key/value head (repeat_kv, phi2.rs:190-200)
+  const int wg_kv = is_attn ? wg / kv_group : 0;     // the key/value head of this block's query head
+  const int KD = a.Hkv * D;
   const int nA0 = 4 * (int)((int64_t)(a.n_qkv / 4) * wg / G), nA1 = 4 * (int)((int64_t)(a.n_qkv / 4) * (wg + 1) / G);
   const int rowsA = nA1 - nA0;
   int fA0 = 0, fA1 = 0;
@@ -614,8 +617,9 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
 
   for (int l = 0; l < a.L; ++l) {
     const MegaLayer ly = a.layers[l];
-    uint16_t *Kc = a.kcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg * a.Tmax * D;
-    uint16_t *Vc = a.vcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg * a.Tmax * D;
+    // (a block without a head never touches the cache; wg_kv is only meaningful where is_attn)
+    uint16_t *Kc = a.kcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg_kv * a.Tmax * D;
+    uint16_t *Vc = a.vcache + ((int64_t)l * a.kv_layer_stride) + (int64_t)wg_kv * a.Tmax * D;
 
     stamp(l, 0);
     {
@@ -781,7 +785,8 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
         const int h = wg;
         {
           const int which = tid / (D / 2), pe = tid - which * (D / 2);
-          int idx[1] = {(which * QD + h * D) / 2 + pe};
+          // q of head h at h D; k and v of its key/value head behind the QD query rows and the KD key rows
+          int idx[1] = {(which == 0 ? h * D : which == 1 ? QD + wg_kv * D : QD + KD + wg_kv * D) / 2 + pe};
           bool on[1] = {tid < 3 * D / 2};
           if (!on[0]) idx[0] = 0;
           uint32_t val[1];
@@ -801,8 +806,10 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
           reinterpret_cast<uint16_t *>(qh)[tid] = f32_to_bf16_bits(qr);   // exact: qr carries bf16 precision
           knew[tid] = kr;
           vnew[tid] = vr;
-          Kc[(int64_t)pos * D + tid] = f32_to_bf16_bits(kr);
-          Vc[(int64_t)pos * D + tid] = f32_to_bf16_bits(vr);
+          if (wg % kv_group == 0) {   // one of the heads that share the key/value head appends the new row
+            Kc[(int64_t)pos * D + tid] = f32_to_bf16_bits(kr);
+            Vc[(int64_t)pos * D + tid] = f32_to_bf16_bits(vr);
+          }
         }
         wg_sync();
 
@@ -989,11 +996,12 @@ unsigned mega_default_spin_limit() { return kMegaSpinLimit; }
 
 bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why) {
   auto no = [&](const char *w) { if (why) *why = w; return false; };
-  if (a.H != 2560) return no("hidden size is not 2560");
-  if (D != 80) return no("head_dim is not 80");
+  // the widths the kernel is built for: Phi-2 (2560 = 32 heads x 80) and Phi-1 / Phi-1.5 (2048 = 32 heads x 64)
+  if (!((a.H == 2560 && D == 80) || (a.H == 2048 && D == 64))) return no("hidden size / head_dim is neither 2560 / 80 nor 2048 / 64");
   if (a.Hq * D != a.QD || a.QD % 512 || a.I % 512) return no("projection widths are not multiples of 512");
   if (a.Hq > num_cu || num_cu > 256) return no("more heads than CUs, or more than 256 CUs");
-  if (a.n_qkv != 3 * a.QD || a.NA != a.n_qkv + a.I || a.n_qkv % 4 || a.NA % 4) return no("q|k|v layout");
+  if (a.Hkv < 1 || a.Hq % a.Hkv) return no("query heads are not a multiple of the key/value heads");
+  if (a.n_qkv != a.QD + 2 * a.Hkv * D || a.NA != a.n_qkv + a.I || a.n_qkv % 4 || a.NA % 4) return no("q|k|v layout");
   if (a.rot > D || (a.rot & 1)) return no("rotary_dim");
   if (3 * a.L >= (int)kMegaTagsPerLaunch) return no("too many layers for the exchange tags of one launch");
 
@@ -1028,16 +1036,25 @@ int launch_phi2_decode_step(hipStream_t st, const MegaArgs &a, int D, int num_cu
     m.stage_off = (int)lds;
     lds += stage_bytes;
   }
-  static size_t attr_bytes = 0;
-  if (lds > 64 * 1024 && lds > attr_bytes) {
+  static bool attr_set = false;
+  if (!attr_set) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_phi2_decode_step<5, 80, false>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMegaLdsMax));
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_phi2_decode_step<5, 80, true>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMegaLdsMax));
-    attr_bytes = kMegaLdsMax;
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_phi2_decode_step<4, 64, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMegaLdsMax));
+    RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_phi2_decode_step<4, 64, true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMegaLdsMax));
+    attr_set = true;
   }
-  if (m.prof) hipLaunchKernelGGL((k_phi2_decode_step<5, 80, true>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
-  else hipLaunchKernelGGL((k_phi2_decode_step<5, 80, false>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
+  if (D == 80) {
+    if (m.prof) hipLaunchKernelGGL((k_phi2_decode_step<5, 80, true>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
+    else hipLaunchKernelGGL((k_phi2_decode_step<5, 80, false>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
+  } else {
+    if (m.prof) hipLaunchKernelGGL((k_phi2_decode_step<4, 64, true>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
+    else hipLaunchKernelGGL((k_phi2_decode_step<4, 64, false>), dim3(num_cu), dim3(kMegaThreads), lds, st, m);
+  }
   return launch_check("phi2_decode_step");
 }
 

@@ -720,7 +720,7 @@ static MegaArgs mega_args(rai_hip_decoder *d) {
   m.Wa0 = (const uint16_t *)d->layers[0].Wa; m.Wb0 = (const uint16_t *)d->layers[0].Wb;
   m.wa_stride = (int64_t)d->NA * d->H; m.wb_stride = (int64_t)d->H * d->KB;
   m.L = d->L; m.H = d->H; m.I = d->I; m.QD = d->QD; m.NA = d->NA; m.n_qkv = d->QD + 2 * d->KD;
-  m.Hq = d->Hq; m.rot = d->cfg.rotary_dim; m.Tmax = d->cfg.max_context;
+  m.Hq = d->Hq; m.Hkv = d->Hkv; m.rot = d->cfg.rotary_dim; m.Tmax = d->cfg.max_context;
   m.x = (uint16_t *)d->x;
   m.xp = d->mega_xchg;
   m.qkvp = m.xp + d->H / 2;
@@ -1254,7 +1254,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
     d->num_cu = hipGetDeviceProperties(&prop, dev) == hipSuccess ? prop.multiProcessorCount : kNumCU;
   }
   d->mega_xchg = nullptr;
-  if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && d->Hq == d->Hkv && getenv("RAI_HIP_NO_MEGA") == nullptr) {
+  if (cfg->arch == RAI_ARCH_PHI2 && cfg->dtype == RAI_BF16 && getenv("RAI_HIP_NO_MEGA") == nullptr) {
     {  // zeroed: tag 0 is never a valid exchange tag
       // x and q|k|v: two values to a packet; activations: 16 packets for each of up to 256 producers;
       // attention output: ceil(D / 3) packets per head

@@ -22,8 +22,13 @@ def wide_cfg(**kw):
     return phi2.Config(**base)
 
 
-def test_persistent_step_logits_match_oracle(hip):
-    cfg = wide_cfg()
+@pytest.mark.parametrize("width", [dict(), dict(hidden_size=2048, partial_rotary_factor=0.5),
+                                   dict(num_key_value_heads=8), dict(hidden_size=2048, partial_rotary_factor=0.5,
+                                                                     num_key_value_heads=4)])
+def test_persistent_step_logits_match_oracle(hip, width):
+    # the two widths the kernel is built for: 2560 = 32 x 80 (Phi-2) and 2048 = 32 x 64 (Phi-1 / Phi-1.5), each also
+    # with grouped-query attention (repeat_kv, rai-models/src/llm/phi2.rs:190-200)
+    cfg = wide_cfg(**width)
     dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
     ids = np.random.Generator(np.random.PCG64(11)).integers(0, cfg.vocab_size, (1, 21)).astype(np.uint32)
     logits, tok = dec.forward(ids)          # prefill: tile kernels
@@ -37,6 +42,8 @@ def test_persistent_step_logits_match_oracle(hip):
         check_tokens(tok, want, "bf16")
         nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
     assert dec.context_len() == 29
+    us, nbytes = dec.time_decode_step(2)     # refused unless the persistent kernel serves this model
+    assert us > 0 and nbytes > 0
     dec.close()
 
 
