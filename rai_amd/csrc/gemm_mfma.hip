@@ -1710,12 +1710,23 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a) {
     // K tiles of 64 (whole 128-byte lines per request) where K allows; RAI_HIP_NO_K64 keeps the tiles of 32
     const bool k64 = a.K % 64 == 0 && !no_k64();
     StreamKPlan plan;
-    if (streamk_applies(a, k64 ? 64 : 32, &plan)) return k64 ? launch_streamk<2>(st, a, plan) : launch_streamk<4>(st, a, plan);
+    const int tiles_192 = ((a.M + 255) / 256) * ((a.N + 191) / 192);
+    const int rounds_192 = (tiles_192 + kNumCU - 1) / kNumCU;
+    if (streamk_applies(a, k64 ? 64 : 32, &plan)) {
+      // Whole rounds of 256 x 192 tiles against stream-K over 256 x 256 ones, in us per tile from the two kernels'
+      // measured times (K = 1536 and 8960, all CUs busy): short K makes the exchange of the shares expensive next
+      // to the tiles themselves (16384 x 1536 x 1536: 512 tiles of 256 x 192 in 80 us, stream-K over 384 in 90 us;
+      // at K = 8960 stream-K wins, 433 against 456 us).
+      const float st64 = (float)(a.K / 64);
+      const float t256 = 5.8f + 1.69f * st64, t192 = 1.1f + 1.62f * st64;
+      const float est_sk = (float)huge_tiles / kNumCU * t256 + (plan.k.max_parts <= 2 ? 18.f : 39.f);
+      if (k64 && rounds_192 * t192 < 0.95f * est_sk) return launch_cfg_dma<256, 192, 2, 0, 2, 4>(st, a, splits);
+      return k64 ? launch_streamk<2>(st, a, plan) : launch_streamk<4>(st, a, plan);
+    }
     // 256 x 192 (eight waves as 4 x 2, 64 x 96 each) where its tiles need no more rounds over the CUs than the
     // 256 x 256 ones: the same round then holds three quarters of the work per CU, spread over more of them
     // (512 x 17920 x 2560 with cold weights: 188 tiles in 64.7 us against 140 tiles in 71.2 us)
-    const int tiles_192 = ((a.M + 255) / 256) * ((a.N + 191) / 192);
-    if (k64 && (tiles_192 + kNumCU - 1) / kNumCU <= (huge_tiles + kNumCU - 1) / kNumCU)
+    if (k64 && rounds_192 <= (huge_tiles + kNumCU - 1) / kNumCU)
       return launch_cfg_dma<256, 192, 2, 0, 2, 4>(st, a, splits);
     return k64 ? launch_cfg_dma<256, 256, 2, 0, 4>(st, a, splits) : launch_cfg_dma<256, 256, 4, 2, 4>(st, a, splits);
   }
