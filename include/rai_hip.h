@@ -217,7 +217,12 @@ int rai_hip_log_softmax(int dev, const rai_hip_tensor *in, int32_t dim, const ra
  * is never taken over a number while a NaN at element 0 is never replaced (NaN wins
  * from index 0 only; an all-NaN axis yields 0).  That NaN rule restates how candle's
  * CPU loop is believed to behave; nothing in the reference's tests pins it.
- * `out` has `dim` removed or kept as 1. */
+ * `out` has `dim` removed or kept as 1.
+ * A long axis is cut over several blocks whose partial results and per-row arrival counters live in one fixed
+ * array per GPU, shared by rai_hip_argmax, rai_hip_argmin and rai_hip_argmax_static (inputs too large for it use
+ * the grown workspace and a second launch).  Like every entry point here the call is enqueued on the library's one
+ * stream of the device, so calls are ordered and safe; kernels of these three entry points forced to overlap on
+ * one GPU by other means would race on that array. */
 int rai_hip_argmax(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
                    const rai_hip_tensor *out);
 int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
@@ -230,10 +235,11 @@ int rai_hip_argmin(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_
  * instead of the grown-on-demand workspace, and the call performs no hipMalloc /
  * hipFree: rai_hip_init(dev) must have succeeded before (otherwise RAI_ERR_HIP).
  * Limit: rows x splits <= 65536 partial results (the axis is only split while that
- * product stays below 1024, so in effect: at most 65536 rows; more returns
- * RAI_ERR_UNSUPPORTED).  All calls
- * on one GPU share that GPU's array: calls that overlap on one device (different
- * streams or threads) race; calls on the library's stream are ordered and safe. */
+ * product stays below 512, twice the CU count, so in effect: at most 65536 rows; more
+ * returns RAI_ERR_UNSUPPORTED).  All calls on one GPU, of this entry point and of
+ * rai_hip_argmax / rai_hip_argmin, share that GPU's array and its arrival counters:
+ * kernels of theirs that overlap on one device race; calls on the library's stream are
+ * ordered and safe.  The counters are left at zero by every completed launch. */
 int rai_hip_argmax_static(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep_dim,
                           const rai_hip_tensor *out);
 
@@ -406,6 +412,16 @@ int rai_hip_decoder_param_shape(rai_hip_decoder *dec, int32_t i, int64_t *rows, 
  * batch or dtype takes one launch per primitive. */
 int rai_hip_decoder_forward(rai_hip_decoder *dec, const uint32_t *ids_host, int32_t batch, int32_t seq,
                             float *logits_host, uint32_t *tokens_host);
+/* Model::fwd (phi2.rs:334-347, qwen2.rs:338-359, gemma.rs:364-386) with both ends of the layer stack open.
+ * Input: either ids_host[batch*seq] (as rai_hip_decoder_forward) or hidden_in_host, [batch*seq, hidden] rows in
+ * the model dtype's storage form that take the place of the embedding lookup (for Gemma: of the already scaled
+ * embeddings, gemma.rs:379); exactly one of the two is non-null.  hidden_out_host (nullable) receives the residual
+ * stream after the last layer, before the final norm, as f32 [batch*seq, hidden]: with a one-layer model that is
+ * what DecoderLayer::fwd returns (phi2.rs:293-299, qwen2.rs:253-266, gemma.rs:286-299).  logits_host and
+ * tokens_host as in rai_hip_decoder_forward.  Always takes the launch-per-primitive path. */
+int rai_hip_decoder_forward_hidden(rai_hip_decoder *dec, const uint32_t *ids_host, const void *hidden_in_host,
+                                   int32_t batch, int32_t seq, float *hidden_out_host, float *logits_host,
+                                   uint32_t *tokens_host);
 /* Greedy loop of examples/phi2/src/main.rs:75-95 without repeat penalty: prefill
  * prompt[batch*prompt_len], then n_new single-token steps feeding the device
  * argmax back without host round trips.  tokens_host[batch*n_new]. prefill_ms /

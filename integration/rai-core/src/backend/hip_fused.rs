@@ -147,6 +147,18 @@ impl Decoder {
         (logits, toks)
     }
 
+    /// The layer stack with both ends open: `rows` (`[batch * seq, hidden]` in the model dtype's storage form, as raw
+    /// bytes) stand in for the embedding lookup; returns the residual stream after the last layer as f32, before the
+    /// final norm.  With a one-layer model that is what `DecoderLayer::fwd` returns.
+    pub fn forward_hidden(&self, rows: &[u8], batch: usize, seq: usize, hidden: usize) -> Vec<f32> {
+        let mut out = vec![0f32; batch * seq * hidden];
+        check(unsafe {
+            rai_hip_decoder_forward_hidden(self.h, std::ptr::null(), rows.as_ptr() as *const std::ffi::c_void, batch as i32,
+                                           seq as i32, out.as_mut_ptr(), std::ptr::null_mut(), std::ptr::null_mut())
+        });
+        out
+    }
+
     /// Greedy decode on the device: `[batch, n_new]` tokens, prefill and decode milliseconds.
     pub fn generate(&self, prompt: &[u32], batch: usize, prompt_len: usize, n_new: usize) -> (Vec<u32>, f32, f32) {
         let mut toks = vec![0u32; batch * n_new];

@@ -127,6 +127,8 @@ PROTOTYPES = {
     "rai_hip_decoder_param_name": [_vp, _i32, C.c_char_p, C.c_size_t, C.POINTER(_i64)],
     "rai_hip_decoder_param_shape": [_vp, _i32, C.POINTER(_i64), C.POINTER(_i64)],
     "rai_hip_decoder_forward": [_vp, C.POINTER(C.c_uint32), _i32, _i32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)],
+    "rai_hip_decoder_forward_hidden": [_vp, C.POINTER(C.c_uint32), _vp, _i32, _i32, C.POINTER(C.c_float), C.POINTER(C.c_float),
+                                       C.POINTER(C.c_uint32)],
     "rai_hip_decoder_generate": [_vp, C.POINTER(C.c_uint32), _i32, _i32, _i32, C.POINTER(C.c_uint32),
                                  C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "rai_hip_decoder_generate_sampled": [_vp, C.POINTER(C.c_uint32), _i32, _i32, _i32, C.c_float, _i32, _i64,

@@ -43,9 +43,25 @@ DeviceCtx *ctx(int dev);
 hipStream_t stream_of(int dev);
 // The stream of an already initialised device; never creates a context (no allocation): nullptr + error otherwise.
 hipStream_t stream_if_ready(int dev);
+// Compute units of the device, asked of it once when its context is created (0 when the device cannot be set up).
+int device_cu_count(int dev);
+// Kernels that wait for other blocks bound their wait; one that gives up stores a RAI_FAULT_* code (system scope) to
+// this word, which lives in pinned host memory, and every wave still exits normally.  The host looks at the word after
+// each synchronisation of the device's stream (rai_hip_sync, rai_hip_d2h, the decoder's generate) and turns a
+// non-zero code into RAI_ERR_HIP, clears it and resets the counters those kernels share.
+int *kernel_fault_word(int dev);
+int check_kernel_fault(int dev);
+enum { RAI_FAULT_STREAMK = 1 };
+// Zeroes the stream-K tile kernel's arrival counters on `st` (gemm_mfma.hip).
+int streamk_counters_reset(int dev, hipStream_t st);
 // Looks up this device's address of the fixed scratch array of the allocation-free argmax (reduce.hip); called once
 // per device, with that device current, while its context is created.
 int arg_static_scratch_init(int dev);
+// First stage of an argmax over the last axis of contiguous [rows, n] (bf16, f16 or f32): the axis is cut into `splits`
+// shares, and share s of row r leaves its best (value, index) under rai_hip_argmax's ordering in pval / pidx
+// [r * splits + s] (a share of NaNs only leaves a NaN).  The caller merges the shares (reduce.hip).
+int launch_argmax_partials(hipStream_t st, int dtype, const void *in, int64_t rows, int64_t n, int splits, float *pval,
+                           uint32_t *pidx);
 // Workspace that lives as long as the device context (grown on demand, never
 // shrinks); used by kernels that need partial results.  Stream-ordered reuse.
 int workspace(int dev, size_t bytes, void **out);

@@ -92,6 +92,10 @@ struct rai_hip_decoder {
   int sample_last_n;
   uint32_t *token_log;        // [max_batch][token_log_cap]: every token of each sequence so far, prompt first
   int token_log_cap;
+  float *choice_val;          // [max_batch][kChoiceMaxSplits]: best value of each share of a wide logits row
+  uint32_t *choice_idx;       // and its index
+  char *hidden_copy;          // [max_rows, H]: the residual stream after the last layer, kept when a caller asks for it
+  bool want_hidden;           // the running forward copies its final residual stream to hidden_copy
   char *head_f;               // fragment-order copy of the lm_head matrix
   bool frag_ready;            // the fragment-order copies match the loaded parameters
   bool graph_sampled;         // what the cached step graphs were captured with
@@ -101,6 +105,7 @@ struct rai_hip_decoder {
 
 namespace rai {
 
+constexpr int kChoiceMaxSplits = 64;  // shares a logits row is scanned in before the token choice
 constexpr int kGraphSteps = 8;  // single-token steps recorded in the multi-step decode graph
 
 // ------------------------------------------------------------------ small kernels
@@ -281,7 +286,8 @@ __device__ __forceinline__ void publish_token(uint32_t chosen, int b, DevState *
 template <typename T>
 __global__ void __launch_bounds__(1024)
 k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, DevState *state, int B, int dpos,
-               int dstep, const T *embed, T *x_next, int H, float embed_scale) {
+               int dstep, const T *embed, T *x_next, int H, float embed_scale, const float *pval, const uint32_t *pidx,
+               int splits) {
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   __shared__ uint32_t chosen;
@@ -291,7 +297,15 @@ k_select_token(const T *logits, int64_t n, uint32_t *tokens, uint32_t *history, 
   float bv = -INFINITY;
   uint32_t bi = 0xffffffffu;
   constexpr int VEC = 16 / sizeof(T);
-  if (n % VEC == 0 && ((uintptr_t)x & 15) == 0) {
+  if (splits > 0) {
+    // wide rows: launch_argmax_partials has scanned the row in `splits` shares spread over the GPU; what is left is
+    // the choice among their (value, index) pairs (a share of NaNs only offers nothing)
+    for (int sp = threadIdx.x; sp < splits; sp += blockDim.x) {
+      const float v = pval[(int64_t)b * splits + sp];
+      const uint32_t i = pidx[(int64_t)b * splits + sp];
+      if (v == v && (bi == 0xffffffffu || v > bv || (v == bv && i < bi))) { bv = v; bi = i; }
+    }
+  } else if (n % VEC == 0 && ((uintptr_t)x & 15) == 0) {
     // 16-byte loads, four per thread in flight; every thread still visits its elements in
     // increasing index order, so the first maximum wins exactly as in the scalar scan
     struct alignas(16) Pack { T v[VEC]; };
@@ -709,7 +723,9 @@ static rai_hip_tensor desc1(void *p, int dtype, int64_t n) {
   return t;
 }
 
-static int linear(rai_hip_decoder *d, hipStream_t st, const LinearArgs &a) {
+static int linear(rai_hip_decoder *d, hipStream_t st, const LinearArgs &a0) {
+  LinearArgs a = a0;
+  a.dev = d->dev;
   return d->cfg.dtype == RAI_BF16 ? launch_linear_bf16(st, a) : launch_linear_f32(st, a);
 }
 
@@ -795,14 +811,23 @@ static int launch_token_choice(rai_hip_decoder *d, hipStream_t st, int B, int S,
                          d->H, d->embed_scale, d->token_log, d->token_log_cap, d->sample_penalty, d->sample_last_n);
     return launch_check("sample_token");
   }
+  // A wide vocabulary is scanned by many blocks first (one block per row would fetch its 100 KB - 500 KB in several
+  // dependent rounds of loads: 35 us for 32 rows of 256000); the choice kernel then merges the shares' results.
+  int splits = 0;
+  if (d->V >= 32768 && !getenv("RAI_HIP_NO_SPLIT_CHOICE")) {
+    splits = 1;
+    while (B * splits < kNumCU && splits < kChoiceMaxSplits && d->V / (splits * 2) >= 8192) splits *= 2;
+    RAI_TRY(launch_argmax_partials(st, dt, d->logits, B, d->V, splits, d->choice_val, d->choice_idx));
+  }
+  const int threads = splits > 0 ? 256 : 1024;
   if (dt == RAI_BF16)
-    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(1024), 0, st, (const bf16_raw *)d->logits,
+    hipLaunchKernelGGL((k_select_token<bf16_raw>), dim3(B), dim3(threads), 0, st, (const bf16_raw *)d->logits,
                        (int64_t)d->V, d->tokens, hist, d->state, B, S, dstep, (const bf16_raw *)d->embed,
-                       (bf16_raw *)d->x, d->H, d->embed_scale);
+                       (bf16_raw *)d->x, d->H, d->embed_scale, d->choice_val, d->choice_idx, splits);
   else
-    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(1024), 0, st, (const float *)d->logits, (int64_t)d->V,
+    hipLaunchKernelGGL((k_select_token<float>), dim3(B), dim3(threads), 0, st, (const float *)d->logits, (int64_t)d->V,
                        d->tokens, hist, d->state, B, S, dstep, (const float *)d->embed, (float *)d->x, d->H,
-                       d->embed_scale);
+                       d->embed_scale, d->choice_val, d->choice_idx, splits);
   return launch_check("select_token");
 }
 
@@ -827,7 +852,7 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   }
 
   char *x = d->x, *xn = d->x2;
-  const bool use_mega = S == 1 && B == 1 && d->mega_ok;
+  const bool use_mega = S == 1 && B == 1 && d->mega_ok && !d->want_hidden;
   if (use_mega) {
     MegaArgs m = mega_args(d);
     RAI_TRY(launch_phi2_decode_step(st, m, d->D, d->num_cu));
@@ -915,6 +940,10 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
     char *tmp = x; x = xn; xn = tmp;
   }
 
+  if (d->want_hidden) {   // the token choice below writes the next input embedding over the first rows of d->x
+    RAI_REQUIRE(!use_mega, RAI_ERR_UNSUPPORTED, "the persistent single-token kernel keeps the residual stream in its packets");
+    RAI_HIP_TRY(hipMemcpyAsync(d->hidden_copy, x, (size_t)M * H * d->es, hipMemcpyDeviceToDevice, st));
+  }
   // final LayerNorm on the last position of every sequence, then the head
   // (phi2.rs:345-346: narrow(1, S-1, 1) before lm_head).
   LinearArgs h = linear_args_default();
@@ -1065,6 +1094,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     RAI_TRY(linear(d, st, dn));
   }
 
+  if (d->want_hidden) RAI_HIP_TRY(hipMemcpyAsync(d->hidden_copy, x, (size_t)M * H * d->es, hipMemcpyDeviceToDevice, st));
   // last position -> final norm -> lm_head (qwen2.rs:355-357, gemma.rs:383-385)
   LinearArgs h = linear_args_default();
   char *last_rows = x + (size_t)(S - 1) * H * d->es;
@@ -1097,6 +1127,7 @@ static int forward_any(rai_hip_decoder *d, int B, int S, bool advance_step, bool
 // A packet poll of the persistent decode kernel that timed out leaves
 // DevState::fault set; the results of that step are not valid.
 static int check_fault(rai_hip_decoder *d) {
+  RAI_TRY(check_kernel_fault(d->dev));
   if (!d->mega_ok) return RAI_OK;
   DevState hs;
   RAI_TRY(rai_hip_d2h(d->dev, &hs, d->state, sizeof(hs)));
@@ -1197,6 +1228,8 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->token_log = nullptr; d->token_log_cap = 0;
   d->graph_sampled = false; d->graph_penalty = 0.f; d->graph_last_n = 0;
   d->head_f = nullptr; d->frag_ready = false;
+  d->hidden_copy = nullptr; d->want_hidden = false;
+  d->choice_val = nullptr; d->choice_idx = nullptr;
   const int vec = (int)(16 / d->es);
   int st = RAI_OK;
   auto bail = [&](int code) {
@@ -1243,6 +1276,10 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   if ((st = dalloc(d, attention_decode_ws_bytes(cfg->max_batch, d->Hq, d->D), &d->attn_ws))) return bail(st);
   if ((st = dalloc(d, attention_decode_counter_bytes(cfg->max_batch, d->Hq), &tmp))) return bail(st);
   d->attn_counters = (int *)tmp;
+  if ((st = dalloc(d, (size_t)cfg->max_batch * kChoiceMaxSplits * sizeof(float), &tmp))) return bail(st);
+  d->choice_val = (float *)tmp;
+  if ((st = dalloc(d, (size_t)cfg->max_batch * kChoiceMaxSplits * sizeof(uint32_t), &tmp))) return bail(st);
+  d->choice_idx = (uint32_t *)tmp;
   if (hipMemset(d->attn_counters, 0, attention_decode_counter_bytes(cfg->max_batch, d->Hq)) != hipSuccess)
     return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
 
@@ -1359,6 +1396,48 @@ int rai_hip_decoder_clear_kv_cache(rai_hip_decoder *d) {
 int rai_hip_decoder_context_len(rai_hip_decoder *d, int32_t *len) {
   RAI_REQUIRE(d && len, RAI_ERR_BAD_ARG, "null argument");
   *len = d->ctx_len;
+  return RAI_OK;
+}
+
+static int widen_to_host(rai_hip_decoder *d, hipStream_t st, const char *src, int64_t n, float *dst_host) {
+  void *ws = nullptr;
+  RAI_TRY(workspace(d->dev, (size_t)n * sizeof(float), &ws));
+  if (d->cfg.dtype == RAI_BF16)
+    hipLaunchKernelGGL((k_to_f32<bf16_raw>), dim3(grid1d(n)), dim3(256), 0, st, (float *)ws, (const bf16_raw *)src, n);
+  else
+    hipLaunchKernelGGL((k_to_f32<float>), dim3(grid1d(n)), dim3(256), 0, st, (float *)ws, (const float *)src, n);
+  RAI_TRY(launch_check("to_f32"));
+  return rai_hip_d2h(d->dev, dst_host, ws, (size_t)n * sizeof(float));
+}
+
+int rai_hip_decoder_forward_hidden(rai_hip_decoder *d, const uint32_t *ids_host, const void *hidden_in_host, int32_t batch,
+                                   int32_t seq, float *hidden_out_host, float *logits_host, uint32_t *tokens_host) {
+  RAI_REQUIRE((ids_host != nullptr) != (hidden_in_host != nullptr), RAI_ERR_BAD_ARG,
+              "forward_hidden: give either token ids or input rows");
+  RAI_TRY(check_call(d, batch, seq));
+  hipStream_t st = stream_of(d->dev);
+  const size_t rows_bytes = (size_t)batch * seq * d->H * d->es;
+  if (hidden_out_host && !d->hidden_copy) RAI_TRY(dalloc(d, (size_t)d->max_rows * d->H * d->es, &d->hidden_copy));
+  if (ids_host) {
+    RAI_HIP_TRY(hipMemcpyAsync(d->ids, ids_host, (size_t)batch * seq * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+  } else {
+    RAI_HIP_TRY(hipMemcpyAsync(d->x, hidden_in_host, rows_bytes, hipMemcpyHostToDevice, st));
+    RAI_HIP_TRY(hipStreamSynchronize(st));   // the caller's buffer is free again when this returns
+  }
+  d->want_hidden = hidden_out_host != nullptr;
+  const int rc = forward_any(d, batch, seq, false, hidden_in_host != nullptr);
+  d->want_hidden = false;
+  d->x_holds_next = false;
+  RAI_TRY(rc);
+  if (hidden_out_host) RAI_TRY(widen_to_host(d, st, d->hidden_copy, (int64_t)batch * seq * d->H, hidden_out_host));
+  if (logits_host) RAI_TRY(widen_to_host(d, st, d->logits, (int64_t)batch * d->V, logits_host));
+  if (tokens_host) RAI_TRY(rai_hip_d2h(d->dev, tokens_host, d->tokens, (size_t)batch * sizeof(uint32_t)));
+  if (hidden_out_host || logits_host || tokens_host) {
+    RAI_TRY(check_fault(d));
+    uint64_t bad = 0;
+    RAI_TRY(rai_hip_index_errors(d->dev, &bad));
+    RAI_REQUIRE(bad == 0, RAI_ERR_INDEX, "decoder: %llu token ids outside the vocabulary", (unsigned long long)bad);
+  }
   return RAI_OK;
 }
 

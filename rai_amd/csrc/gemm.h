@@ -57,6 +57,8 @@ struct LinearArgs {
   const void *post_ln_w;
   const void *post_ln_b;
   float post_ln_eps;
+  // Device the operands live on (its CU count and per-device counters are looked up by it); -1: the current device.
+  int dev;
 };
 // True when launch_linear_bf16 with these arguments will also write post_ln_out.
 bool linear_fuses_post_norm(const LinearArgs &a);
@@ -68,6 +70,7 @@ inline LinearArgs linear_args_default() {
   memset(&a, 0, sizeof(a));
   a.act = -1;
   a.ln_kind = -1;
+  a.dev = -1;
   return a;
 }
 

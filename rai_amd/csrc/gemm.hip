@@ -767,6 +767,7 @@ int rai_hip_matmul(int dev, const rai_hip_tensor *a, const rai_hip_tensor *b, co
                    (uintptr_t)base_ptr(b) % 16 == 0;
     if (b_shared && ca.rank == 1 && batch * M < (1LL << 31) && (a->dtype == RAI_F32 || aligned) && ldw >= K) {
       LinearArgs la = linear_args_default();
+  la.dev = dev;
       la.A = base_ptr(a);
       la.lda = lda;
       la.W = base_ptr(b);
@@ -861,6 +862,7 @@ int rai_hip_linear(int dev, const rai_hip_tensor *x, const rai_hip_tensor *w, co
   coalesce(1, ts, &ca);
   RAI_REQUIRE(ca.rank == 1, RAI_ERR_BAD_STRIDE, "linear: rows of x must share one stride");
   LinearArgs la = linear_args_default();
+  la.dev = dev;
   la.A = base_ptr(x);
   la.lda = M == 1 ? K : ca.stride[0][0];
   la.W = base_ptr(w);
@@ -916,6 +918,7 @@ int rai_hip_linear_packed(int dev, const rai_hip_tensor *x, const rai_hip_tensor
   RAI_REQUIRE(act_from >= 0 && act_from <= N && k_splits >= 0, RAI_ERR_BAD_ARG, "linear_packed: bad act_from / k_splits");
   const int64_t n1 = out1->shape[1];
   LinearArgs la = linear_args_default();
+  la.dev = dev;
   if (glu) {
     RAI_REQUIRE(N % 2 == 0 && n1 == N / 2 && !out2 && !residual && !bias2 && act >= 0 && act_from == 0, RAI_ERR_BAD_ARG,
                 "linear_packed: a gated product writes N/2 columns to out1 and takes an activation, no residual, "

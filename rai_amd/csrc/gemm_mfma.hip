@@ -690,6 +690,9 @@ struct StreamKArgs {
   int max_parts;  // slots per tile in the workspace
   float *ws;      // [sk_tiles][max_parts][BM * BN] f32
   int *counters;  // [sk_tiles][2] (tickets, stored shares), zero between launches
+  int *fault;     // host-visible word: RAI_FAULT_STREAMK is stored here when a wait for shares expires
+  int spin_limit; // polls of the stored-shares counter before the wait is given up
+  int drop_tile;  // test hook: the stored shares of this tile are never counted (-1: none), so its wait must expire
 };
 
 __device__ __forceinline__ int sk_start(const StreamKArgs &k, int p) { return p * k.q + (p < k.rem ? p : k.rem); }
@@ -771,18 +774,28 @@ __global__ void __launch_bounds__(128 * WGN) k_gemm_bf16_mfma_dma_streamk(Linear
               __hip_atomic_store(mine + ((i * NT + j) * 16 + r) * 64, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share has left for memory
         __syncthreads();
-        if (tid == 0) __hip_atomic_fetch_add(stored, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          continue;
+        if (tid == 0 && tile != sk.drop_tile) __hip_atomic_fetch_add(stored, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        continue;
       }
       if (tid == 0) {
-        for (int spin = 0; spin < (1 << 20); ++spin) {
-          if (__hip_atomic_load(stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1) break;
-          __builtin_amdgcn_s_sleep(2);
+        bool complete = false;
+        for (int spin = 0; spin < sk.spin_limit && !complete; ++spin) {
+          complete = __hip_atomic_load(stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1;
+          if (!complete) __builtin_amdgcn_s_sleep(2);
         }
-        __hip_atomic_store(arrived, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(stored, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (complete) {
+          __hip_atomic_store(arrived, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(stored, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          // A share is missing.  Nothing is summed and nothing written for this tile, the counters stay as they are
+          // (a late block may still count itself in; the host zeroes them all before the next launch), and the
+          // host learns of it at its next synchronisation.
+          __hip_atomic_store(sk.fault, (int)RAI_FAULT_STREAMK, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          s_ticket = -1;
+        }
       }
       __syncthreads();
+      if (s_ticket < 0) continue;
       // the other slots are complete.  Sum in slot order, our registers standing in for our slot, so the result does
       // not depend on who came last.
 #pragma unroll
@@ -1113,36 +1126,68 @@ size_t linear_streamk_workspace_bytes(int M, int N, int K) {
   return streamk_plan(M, N, K, 32, &plan) ? plan.ws_bytes : 0;
 }
 
+static int linear_device(const LinearArgs &a, int *dev) {
+  *dev = a.dev;
+  if (*dev < 0) RAI_HIP_TRY(hipGetDevice(dev));
+  RAI_REQUIRE(*dev >= 0 && *dev < 64, RAI_ERR_BAD_ARG, "device %d out of range", *dev);
+  return RAI_OK;
+}
+
 // True when the stream-K kernel serves this Linear (plain tile epilogue, workspace large enough, not switched off).
 static bool streamk_applies(const LinearArgs &a, int bk, StreamKPlan *plan, bool forced = false) {
   const char *off = getenv("RAI_HIP_NO_STREAMK");   // read per call: tests compare both forms in one process
   if (off && *off && *off != '0') return false;
   if (!a.splitk_ws || ((uintptr_t)a.splitk_ws & 15) || a.post_ln_out) return false;
+  // one block per CU of a 256-CU part: the plan, the counter array and the XCD order are laid out for that grid
+  int dev = -1;
+  if (linear_device(a, &dev) != RAI_OK || device_cu_count(dev) != kNumCU) return false;
   return a.K % bk == 0 && streamk_plan(a.M, a.N, a.K, bk, plan, forced) && plan->ws_bytes <= a.splitk_ws_bytes;
+}
+
+static int *streamk_counters_of(int dev) {   // every GPU holds its own copy of the counter array at its own address
+  static int *counters[64];
+  if (dev < 0 || dev >= 64) return nullptr;
+  if (!counters[dev]) {
+    int cur = -1;
+    void *p = nullptr;
+    if (hipGetDevice(&cur) != hipSuccess || (cur != dev && hipSetDevice(dev) != hipSuccess)) return nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_streamk_counters)) == hipSuccess) counters[dev] = (int *)p;
+    if (cur != dev) (void)hipSetDevice(cur);
+  }
+  return counters[dev];
+}
+
+int streamk_counters_reset(int dev, hipStream_t st) {
+  int *c = streamk_counters_of(dev);
+  RAI_REQUIRE(c, RAI_ERR_HIP, "stream-K counters of device %d not found", dev);
+  RAI_HIP_TRY(hipMemsetAsync(c, 0, sizeof(int) * 4 * kNumCU, st));
+  return RAI_OK;
 }
 
 template <int NS>
 static int launch_streamk(hipStream_t st, const LinearArgs &a, StreamKPlan plan) {
   constexpr int BM = 256, BN = 256, SH = 2, WGN = 4;
   constexpr size_t lds = dma_lds_bytes<BM, BN, NS, WGN>();
-  static bool attr_set = false;
-  if (!attr_set) {
+  int dev = 0;
+  RAI_TRY(linear_device(a, &dev));
+  static bool attr_set[64];
+  if (!attr_set[dev]) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_gemm_bf16_mfma_dma_streamk<BM, BN, NS, SH, WGN>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
-  // every GPU holds its own copy of the counter array at its own address
-  static int *counters[64];
-  int dev = 0;
-  RAI_HIP_TRY(hipGetDevice(&dev));
-  RAI_REQUIRE(dev >= 0 && dev < 64, RAI_ERR_BAD_ARG, "device %d out of range", dev);
-  if (!counters[dev]) {
-    void *p = nullptr;
-    RAI_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_streamk_counters)));
-    counters[dev] = (int *)p;
+    attr_set[dev] = true;
   }
   plan.k.ws = (float *)a.splitk_ws;
-  plan.k.counters = counters[dev];
+  plan.k.counters = streamk_counters_of(dev);
+  plan.k.fault = kernel_fault_word(dev);
+  RAI_REQUIRE(plan.k.counters && plan.k.fault, RAI_ERR_HIP, "stream-K: device %d has no counters / fault word", dev);
+  plan.k.spin_limit = 1 << 20;
+  plan.k.drop_tile = -1;
+  // RAI_HIP_STREAMK_TEST="<spin limit>,<tile>": a tiny wait and one tile whose shares are never counted, so that the
+  // expiry path runs with every wave still exiting normally (read per launch; the tests set it around one call)
+  if (const char *t = getenv("RAI_HIP_STREAMK_TEST")) {
+    int lim = 0, tile = -1;
+    if (sscanf(t, "%d,%d", &lim, &tile) == 2 && lim > 0) { plan.k.spin_limit = lim; plan.k.drop_tile = tile; }
+  }
   hipLaunchKernelGGL((k_gemm_bf16_mfma_dma_streamk<BM, BN, NS, SH, WGN>), dim3(kNumCU), dim3(128 * WGN), lds, st, a, plan.k);
   return launch_check("gemm_bf16_mfma_dma_streamk");
 }

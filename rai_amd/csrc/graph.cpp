@@ -600,6 +600,8 @@ struct Matcher {
     *b = n->inputs[1];
     return true;
   }
+  // which binary primitive an unevaluated node is (-1: none); records nothing
+  int bin_kind(const rai_tensor *t) const { return ok && t && !t->evaluated && t->op == RAI_OP_BINARY ? t->sub : -1; }
   rai_tensor *un(rai_tensor *t, int sub) {
     rai_tensor *n = node(t, RAI_OP_UNARY);
     if (!n || n->sub != sub) { ok = false; return nullptr; }
@@ -696,8 +698,17 @@ bool match_rms_norm(rai_tensor *t, Composite *c) {
   if (!ve || !m.bin(ve, RAI_BIN_ADD, &s, &epsc) || !m.konst(epsc, &eps)) return false;
   rai_tensor *sq = m.sum_last_keep(s);
   rai_tensor *xd = sq ? m.un(sq, RAI_UN_SQUARE) : nullptr;
-  if (!xd || !m.bin(xd, RAI_BIN_DIV, &x2, &cc) || x2 != x || !m.konst(cc, &div) || !m.ok) return false;
-  if (fabs(div * div - (double)n) > 1e-3 * (double)n) return false;
+  // the reference records (x * s).square() with s = 1 / sqrt(n) (rms_norm.rs:19-20); x / sqrt(n) is the same value
+  // recorded as a division and is taken as well
+  if (!xd) return false;
+  if (m.bin_kind(xd) == RAI_BIN_MUL) {
+    double mul = 0;
+    if (!m.bin(xd, RAI_BIN_MUL, &x2, &cc) || x2 != x || !m.konst(cc, &mul) || !m.ok) return false;
+    if (fabs(mul * mul * (double)n - 1.0) > 1e-3) return false;
+  } else {
+    if (!m.bin(xd, RAI_BIN_DIV, &x2, &cc) || x2 != x || !m.konst(cc, &div) || !m.ok) return false;
+    if (fabs(div * div - (double)n) > 1e-3 * (double)n) return false;
+  }
   c->kind = COMP_RMS_NORM;
   c->in[0] = x; c->in[1] = w;
   c->f0 = eps;

@@ -170,6 +170,62 @@ __global__ void __launch_bounds__(256) k_softmax_row(T *out, const T *in, int64_
   }
 }
 
+// The same with one row per wave (a block is four rows): every lane has all its 16-byte loads in flight at once and
+// the two reductions are wave shuffles, with no LDS and no block barrier between the row's three phases.
+template <typename T, int V, int ITEMS, bool LOG>
+__global__ void __launch_bounds__(256) k_softmax_wave(T *out, const T *in, int64_t rows, int64_t n, int64_t in_row_stride) {
+  const int lane = threadIdx.x & 63;
+  const int64_t packs = n / V;
+  for (int64_t row = blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += (int64_t)gridDim.x * 4) {
+    const T *x = in + row * in_row_stride;
+    T *y = out + row * n;
+    RowPack<T, V> pk[ITEMS];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t p = lane + it * 64;
+      if (p < packs) pk[it] = *reinterpret_cast<const RowPack<T, V> *>(x + p * V);
+    }
+    float vals[ITEMS][V];
+    float m = -INFINITY;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      if (lane + it * 64 < packs) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          vals[it][j] = (float)Scalar<T>::load(&pk[it].v[j]);
+          m = fmaxf(m, vals[it][j]);
+        }
+      }
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      if (lane + it * 64 < packs) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const float d = vals[it][j] - m;
+          const float e = expf(d);
+          sum += e;
+          vals[it][j] = LOG ? d : e;
+        }
+      }
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum, lse = logf(sum);
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t p = lane + it * 64;
+      if (p < packs) {
+        RowPack<T, V> o;
+#pragma unroll
+        for (int j = 0; j < V; ++j) Scalar<T>::store(&o.v[j], LOG ? vals[it][j] - lse : vals[it][j] * inv);
+        *reinterpret_cast<RowPack<T, V> *>(y + p * V) = o;
+      }
+    }
+  }
+}
+
 // Any stride along the softmax axis, any row length; three passes over the row.
 // One block per row when the axis is long, else one thread per row.
 template <typename T, bool LOG>
@@ -232,13 +288,15 @@ template <typename C, bool IS_MAX> __device__ __forceinline__ bool better(C bv, 
   return bv == av && bi < ai;
 }
 
+// blockDim.x = 256 or 1024: the wider block where a row's share is long enough to give every thread several 16-byte
+// loads, all of them in flight at once (one memory round trip for the share).
 template <typename T, bool IS_MAX>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int64_t axis_stride, int splits,
                   float *pval_f, double *pval_d, uint32_t *pidx, uint32_t *counters, uint32_t *out) {
   typedef typename Scalar<T>::compute C;
-  __shared__ C shv[4];
-  __shared__ uint32_t shi[4];
+  __shared__ C shv[16];
+  __shared__ uint32_t shi[16];
   int64_t row = blockIdx.x / splits;
   int split = blockIdx.x % splits;
   if (row >= rows) return;
@@ -298,7 +356,8 @@ k_arg_row_partial(const T *in, int64_t rows, int64_t n, int64_t row_stride, int6
   __syncthreads();
   if (threadIdx.x >= 64) return;   // wave 0 finishes the block
   if (threadIdx.x == 0) {
-    for (int w = 1; w < 4; ++w)
+    const int nw = (int)(blockDim.x >> 6);
+    for (int w = 1; w < nw; ++w)
       if (better<C, IS_MAX>(shv[w], shi[w], bv, bi)) { bv = shv[w]; bi = shi[w]; }
   }
   if (!out) {   // two-launch form: k_arg_row_final merges
@@ -487,6 +546,27 @@ template <bool LOG> static int softmax_impl(int dev, const rai_hip_tensor *in, i
     else if (packs <= 1024) SM_LAUNCH(T, V, 4);             \
     else SM_LAUNCH(T, V, 8);                                \
   } while (0)
+      // rows of up to 512 packs (4096 bf16 / 2048 f32 elements), several of them: one wave per row
+      if (aligned && packs <= 512 && rows >= 4) {
+        const int64_t wblocks = (rows + 3) / 4;
+        const int wgrid = (int)(wblocks < kNumCU * 32 ? wblocks : kNumCU * 32);
+#define SMW_LAUNCH(T, V, ITEMS)                                                                                 \
+  hipLaunchKernelGGL((k_softmax_wave<T, V, ITEMS, LOG>), dim3(wgrid), dim3(256), 0, st, (T *)base_ptr(out),       \
+                     (const T *)base_ptr(in), rows, n, row_stride)
+#define SMW_BY_ITEMS(T, V)                          \
+  do {                                              \
+    if (packs <= 64) SMW_LAUNCH(T, V, 1);           \
+    else if (packs <= 128) SMW_LAUNCH(T, V, 2);     \
+    else if (packs <= 256) SMW_LAUNCH(T, V, 4);     \
+    else SMW_LAUNCH(T, V, 8);                       \
+  } while (0)
+        if (in->dtype == RAI_F32) SMW_BY_ITEMS(float, 4);
+        else if (in->dtype == RAI_BF16) SMW_BY_ITEMS(bf16_raw, 8);
+        else SMW_BY_ITEMS(f16_raw, 8);
+#undef SMW_BY_ITEMS
+#undef SMW_LAUNCH
+        return launch_check("softmax_wave");
+      }
       if (packs <= 2048) {
         if (in->dtype == RAI_F32) { if (aligned) SM_BY_ITEMS(float, 4); else SM_BY_ITEMS(float, 1); }
         else if (in->dtype == RAI_BF16) { if (aligned) SM_BY_ITEMS(bf16_raw, 8); else SM_BY_ITEMS(bf16_raw, 1); }
@@ -556,8 +636,12 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
   // Row path: rows addressable by one uniform stride and a long axis.
   if (s.out_rank == 1 && n >= 1024 && in->dtype != RAI_U8 && in->dtype != RAI_U32 && in->dtype != RAI_I64) {
     int64_t rows = s.n_out, row_stride = s.out_stride[0];
+    // A row is cut over blocks only while there are fewer blocks than a quarter of the CUs, or a share would be longer
+    // than 65536 elements: a block of 1024 threads fetches a share of that size in a few rounds of loads that are all
+    // in flight together, and an uncut row needs no merge, i.e. no second memory round trip ([64, 51200]: 64 blocks).
     int splits = 1;
-    while (rows * splits < 2 * kNumCU && n / (splits * 2) >= 2048) splits *= 2;
+    while ((rows * splits < kNumCU / 4 || n / splits > 65536) && n / (splits * 2) >= 2048) splits *= 2;
+    const int threads = n / splits >= 8192 ? 1024 : 256;
     void *ws = nullptr;
     size_t nparts = (size_t)rows * splits;
     if (no_alloc)
@@ -571,7 +655,7 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
       uint32_t *pi = (uint32_t *)((char *)ws + kArgStaticParts * sizeof(double));
       uint32_t *cnt = pi + kArgStaticParts;
       RAI_DISPATCH_FLOAT(in->dtype, T,
-                         hipLaunchKernelGGL((k_arg_row_partial<T, IS_MAX>), dim3((unsigned)nparts), dim3(256), 0, st,
+                         hipLaunchKernelGGL((k_arg_row_partial<T, IS_MAX>), dim3((unsigned)nparts), dim3(threads), 0, st,
                                             (const T *)base_ptr(in), rows, n, row_stride, ax, splits, (float *)ws, pd, pi,
                                             cnt, o));
       return launch_check("arg_row");
@@ -582,7 +666,7 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
     float *pf = (float *)ws;
     uint32_t *pi = (uint32_t *)((char *)ws + nparts * sizeof(double));
     RAI_DISPATCH_FLOAT(in->dtype, T,
-                       hipLaunchKernelGGL((k_arg_row_partial<T, IS_MAX>), dim3((unsigned)nparts), dim3(256), 0, st,
+                       hipLaunchKernelGGL((k_arg_row_partial<T, IS_MAX>), dim3((unsigned)nparts), dim3(threads), 0, st,
                                           (const T *)base_ptr(in), rows, n, row_stride, ax, splits, pf, pd, pi,
                                           (uint32_t *)nullptr, (uint32_t *)nullptr));
     RAI_TRY(launch_check("arg_partial"));
@@ -602,6 +686,21 @@ static int arg_impl(int dev, const rai_hip_tensor *in, int32_t dim, int32_t keep
                    hipLaunchKernelGGL((k_arg_thread<T, IS_MAX>), dim3(grid), dim3(256), 0, st,
                                       (const T *)base_ptr(in), s, ax, o));
   return launch_check("arg_thread");
+}
+
+int launch_argmax_partials(hipStream_t st, int dtype, const void *in, int64_t rows, int64_t n, int splits, float *pval,
+                           uint32_t *pidx) {
+  RAI_REQUIRE(rows > 0 && n > 0 && splits >= 1 && in && pval && pidx, RAI_ERR_BAD_ARG, "argmax partials: bad arguments");
+  RAI_REQUIRE(dtype == RAI_BF16 || dtype == RAI_F16 || dtype == RAI_F32, RAI_ERR_BAD_DTYPE, "argmax partials: dtype %s",
+              dtype_name(dtype));
+  const int threads = n / splits >= 8192 ? 1024 : 256;
+  RAI_DISPATCH_FLOAT(dtype, T, {
+    if constexpr (sizeof(T) <= 4)
+      hipLaunchKernelGGL((k_arg_row_partial<T, true>), dim3((unsigned)(rows * splits)), dim3(threads), 0, st, (const T *)in,
+                         rows, n, n, (int64_t)1, splits, pval, (double *)nullptr, pidx, (uint32_t *)nullptr,
+                         (uint32_t *)nullptr);
+  });
+  return launch_check("argmax_partials");
 }
 
 }  // namespace rai

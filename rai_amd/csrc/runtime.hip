@@ -42,6 +42,9 @@ struct DeviceCtx {
   void *ws = nullptr;
   size_t ws_bytes = 0;
   unsigned long long *index_errors = nullptr;
+  int num_cu = 0;                      // compute units of this GPU, asked of the device once
+  int *fault_host = nullptr;           // pinned, device-visible word a kernel sets when a bounded wait of its own expires
+  int *fault_dev = nullptr;            // the same word's device address
 };
 
 static constexpr int kMaxDev = 16;
@@ -71,14 +74,32 @@ DeviceCtx *ctx(int dev) {
     set_error("no HIP device %d (count=%d, %s)", dev, n, hipGetErrorString(e));
     return nullptr;
   }
+  // a failed set-up leaves nothing behind: the next call starts from scratch instead of leaking a stream and a buffer
+  auto undo = [&]() {
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    if (c->index_errors) (void)hipFree(c->index_errors);
+    if (c->fault_host) (void)hipHostFree(c->fault_host);
+    c->stream = nullptr;
+    c->index_errors = nullptr;
+    c->fault_host = c->fault_dev = nullptr;
+  };
   if ((e = hipSetDevice(dev)) != hipSuccess || (e = hipStreamCreate(&c->stream)) != hipSuccess ||
       (e = hipMalloc((void **)&c->index_errors, sizeof(unsigned long long))) != hipSuccess ||
-      (e = hipMemset(c->index_errors, 0, sizeof(unsigned long long))) != hipSuccess) {
+      (e = hipMemset(c->index_errors, 0, sizeof(unsigned long long))) != hipSuccess ||
+      (e = hipDeviceGetAttribute(&c->num_cu, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess ||
+      (e = hipHostMalloc((void **)&c->fault_host, 64, hipHostMallocMapped)) != hipSuccess ||
+      (e = hipHostGetDevicePointer((void **)&c->fault_dev, c->fault_host, 0)) != hipSuccess) {
     set_error("device %d init failed: %s", dev, hipGetErrorString(e));
+    undo();
     return nullptr;
   }
-  // per-device addresses of the library's fixed device arrays (this device is current here)
-  if (arg_static_scratch_init(dev) != RAI_OK) return nullptr;
+  // per-device addresses of the library's fixed device arrays (this device is current here); the callee has set the
+  // error text, device number included
+  if (arg_static_scratch_init(dev) != RAI_OK) {
+    undo();
+    return nullptr;
+  }
+  *c->fault_host = 0;
   c->dev = dev;
   c->ready = true;
   return c;
@@ -95,6 +116,29 @@ hipStream_t stream_if_ready(int dev) {
 hipStream_t stream_of(int dev) {
   DeviceCtx *c = ctx(dev);
   return c ? c->stream : nullptr;
+}
+
+int device_cu_count(int dev) {
+  DeviceCtx *c = ctx(dev);
+  return c ? c->num_cu : 0;
+}
+
+int *kernel_fault_word(int dev) {
+  DeviceCtx *c = ctx(dev);
+  return c ? c->fault_dev : nullptr;
+}
+
+int check_kernel_fault(int dev) {
+  DeviceCtx *c = ctx(dev);
+  if (!c) return RAI_ERR_HIP;
+  const int code = *(volatile int *)c->fault_host;
+  if (code == 0) return RAI_OK;
+  *(volatile int *)c->fault_host = 0;
+  // whatever the kernels of that launch left behind is not to be trusted: start the next one from clean counters
+  (void)streamk_counters_reset(dev, c->stream);
+  (void)hipStreamSynchronize(c->stream);
+  return fail(RAI_ERR_HIP, "device %d: a kernel gave up a bounded wait (code %d: %s); results since the last synchronisation are invalid",
+              dev, code, code == RAI_FAULT_STREAMK ? "stream-K share never arrived" : "unknown");
 }
 
 unsigned long long *index_error_counter(int dev) {
@@ -211,7 +255,7 @@ int rai_hip_sync(int dev) {
   DeviceCtx *c = ctx(dev);
   if (!c) return RAI_ERR_HIP;
   RAI_HIP_TRY(hipStreamSynchronize(c->stream));
-  return RAI_OK;
+  return check_kernel_fault(dev);
 }
 
 int rai_hip_alloc(int dev, size_t bytes, void **out) {
@@ -325,7 +369,7 @@ int rai_hip_d2h(int dev, void *dst_host, const void *src_dev, size_t bytes) {
   RAI_REQUIRE(dst_host && src_dev, RAI_ERR_BAD_ARG, "d2h: null pointer");
   RAI_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, c->stream));
   RAI_HIP_TRY(hipStreamSynchronize(c->stream));
-  return RAI_OK;
+  return check_kernel_fault(dev);   // what was copied came from kernels that may have given up a wait
 }
 
 int rai_hip_d2d(int dev, void *dst_dev, const void *src_dev, size_t bytes) {

@@ -366,9 +366,9 @@ def layer_norm(x, weight, bias, eps):
 
 
 def rms_norm(x, weight, eps):
-    """w * x * rsqrt(sum((x / sqrt(n))^2) + eps) (rai-nn/src/rms_norm.rs:18-22)."""
+    """s = 1 / sqrt(n); weight * x * rsqrt(sum((x * s)^2) + eps) (rai-nn/src/rms_norm.rs:18-22)."""
     n = x.shape[-1]
-    s = (x / float(math.sqrt(n))).square().sum(-1, True)
+    s = (x * (1.0 / math.sqrt(n))).square().sum(-1, True)
     return weight * x * (s + eps).rsqrt()
 
 

@@ -92,6 +92,27 @@ class Decoder:
              toks.ctypes.data_as(C.POINTER(C.c_uint32)))
         return logits, toks
 
+    def forward_hidden(self, ids=None, hidden_in=None, want_logits=False):
+        """Model::fwd with the layer stack's ends open: ids [B, S] u32, or hidden_in [B, S, hidden] in the model
+        dtype's storage form in place of the embedding lookup -> (residual stream after the last layer [B, S, hidden]
+        f32, logits [B, vocab] f32 or None, greedy tokens [B] u32)."""
+        if ids is not None:
+            ids = np.ascontiguousarray(ids, dtype=np.uint32)
+            b, s = ids.shape
+            ids_p, hid_p = ids.ctypes.data_as(C.POINTER(C.c_uint32)), None
+        else:
+            hidden_in = np.ascontiguousarray(hidden_in)
+            b, s, h = hidden_in.shape
+            assert h == self.cfg.hidden_size
+            ids_p, hid_p = None, hidden_in.ctypes.data_as(C.c_void_p)
+        hidden = np.empty((b, s, self.cfg.hidden_size), np.float32)
+        logits = np.empty((b, self.cfg.vocab_size), np.float32) if want_logits else None
+        toks = np.empty((b,), np.uint32)
+        call("rai_hip_decoder_forward_hidden", self._h, ids_p, hid_p, b, s, hidden.ctypes.data_as(C.POINTER(C.c_float)),
+             logits.ctypes.data_as(C.POINTER(C.c_float)) if want_logits else None,
+             toks.ctypes.data_as(C.POINTER(C.c_uint32)))
+        return hidden, logits, toks
+
     def generate(self, prompt, n_new):
         """Greedy decode: returns (tokens [B, n_new], prefill_ms, decode_ms)."""
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)

@@ -274,6 +274,27 @@ def test_gemm_streamk_packed_epilogues(R, monkeypatch, form):
     assert_close(got, want, dt, "stream-K: silu(gate) * up")
 
 
+def test_gemm_streamk_lost_share_is_reported_and_recovers(R, monkeypatch):
+    """A share that never arrives: the block that sums a tile gives up its bounded wait, writes nothing for that tile
+    and flags the fault; the host's next synchronisation returns an error instead of wrong numbers, and the launch
+    after that works from clean counters.  Forced from the host (a tiny spin limit, one tile whose stored shares are
+    never counted): every wave exits normally."""
+    from rai_amd._lib import RaiHipError
+    from rai_amd.hip import sync
+    monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk64")
+    dt, (m, n, k) = "bf16", STREAMK_SHAPES[0]
+    x, w, _, _, _ = packed_case(rng(122), m, n, k)
+    xd, wd = up(x, dt), up(w, dt)
+    want = down(R.linear(xd, wd))
+    monkeypatch.setenv("RAI_HIP_STREAMK_TEST", "64,0")
+    with pytest.raises(RaiHipError, match="stream-K share never arrived"):
+        R.linear(xd, wd)
+        sync()
+    monkeypatch.delenv("RAI_HIP_STREAMK_TEST")
+    for _ in range(2):
+        assert np.array_equal(down(R.linear(xd, wd)), want)
+
+
 def test_gemm_streamk_refuses_where_it_does_not_apply(R, monkeypatch):
     from rai_amd._lib import RaiHipError
     monkeypatch.setenv("RAI_HIP_GEMM_TILE", "streamk")

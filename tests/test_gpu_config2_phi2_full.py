@@ -14,7 +14,7 @@ import pytest
 from oracle import phi2
 from oracle.dtypes import to_storage
 from tests.test_gpu_phi2 import check_tokens
-from tests.util import assert_logits_close, progress, synthetic_params
+from tests.util import assert_close, assert_logits_close, progress, synthetic_params
 
 pytestmark = pytest.mark.gpu
 
@@ -111,3 +111,41 @@ def test_persistent_steps_past_600_cached_tokens_full_width(full, request):
     first = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
     _steps(request, dec, refs, first, 20, 650, "650-token context")
     assert dec.context_len() == 670
+
+
+def test_single_layer_full_width_against_the_chain(hip, request):
+    """One Phi-2 layer at full width (2560 / 10240, 32 heads x 80, 512 positions, bf16) fed with rows of residual-stream
+    size, against the node-by-node bf16 chain of the same layer: no depth for rounding noise to build up over, so the
+    plain 2e-2 bound applies, both to the layer's output and to what the layer adds to its input."""
+    from oracle.dtypes import rnd
+    from rai_amd.models import Decoder
+    cfg = phi2.Config(num_hidden_layers=1, vocab_size=512)
+    params = synthetic_params(phi2.param_shapes(cfg), "bf16", seed=3)
+    g = np.random.Generator(np.random.PCG64(41))
+    for k in params:   # biases and norm parameters away from 0 / 1
+        if k.endswith(".bias"):
+            params[k] = rnd(0.05 * g.standard_normal(params[k].shape).astype(np.float32), "bf16")
+        elif k.endswith("layernorm.weight"):
+            params[k] = rnd(params[k] + 0.1 * g.standard_normal(params[k].shape).astype(np.float32), "bf16")
+    dec = Decoder("phi2", "bf16", vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
+                  intermediate_size=cfg.intermediate_size, num_hidden_layers=1, num_attention_heads=cfg.num_attention_heads,
+                  rotary_dim=cfg.rotary_dim, max_position_embeddings=cfg.max_position_embeddings, hidden_act=cfg.hidden_act,
+                  rope_theta=cfg.rope_theta, norm_eps=cfg.layer_norm_eps, max_batch=1, max_context=512)
+    for n in dec.param_names():
+        dec.load_param(n, to_storage(params[n], "bf16"))
+    x = rnd(g.standard_normal((1, 512, cfg.hidden_size)).astype(np.float32), "bf16")
+    got, _, _ = dec.forward_hidden(hidden_in=to_storage(x, "bf16"))
+    progress(request, "oracle: one layer, 512 rows, bf16 chain")
+    ref = phi2.Model(cfg, params, "bf16")
+    want = ref.layer(0, x, phi2.get_mask(512))
+    assert_close(got, want, "bf16", "Phi-2 layer output vs the bf16 chain")
+    # The layer's own contribution, attention + MLP (out - x), relative to its own largest value.  Output and input
+    # are both bf16 values of similar size, so the difference carries up to one output rounding (2^-9 of |out|) that
+    # is no error of the layer: that much is allowed on top.
+    ulp = float(np.max(np.abs(want))) * 2.0 ** -8
+    d_got, d_want = got.astype(np.float64) - x, want.astype(np.float64) - x
+    err = float(np.max(np.abs(d_got - d_want)))
+    scale = float(np.max(np.abs(d_want)))
+    progress(request, "layer contribution: max error %.3e of %.3e (%.4f), one output rounding %.3e" % (err, scale, err / scale, ulp))
+    assert err <= 2e-2 * scale + ulp, f"attention + MLP contribution off by {err:.3e} (scale {scale:.3e})"
+    dec.close()

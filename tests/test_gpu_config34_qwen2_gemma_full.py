@@ -95,3 +95,31 @@ def test_gemma_2b_widths_decode_batch32_context2048(hip, request):
         assert np.array_equal(tok, np.argmax(logits, -1).astype(np.uint32))
     assert dec.context_len() == CTX + 4
     dec.close()
+
+
+@pytest.mark.parametrize("arch", ["qwen2", "gemma"])
+def test_single_layer_full_width_against_the_chain(hip, request, arch):
+    """One layer at the full widths (Qwen2-1.5B: 1536 / 8960, 12 / 2 heads of 128, 2 x 1024 positions; Gemma-2B: 2048 /
+    16384, 8 / 1 heads of 256, 2 x 512 positions; bf16) fed with rows of residual-stream size, against the
+    node-by-node bf16 chain of the same layer.  Without depth no rounding noise builds up, so the plain 2e-2 bound
+    applies, to the layer's output and to what the layer adds to its input."""
+    if arch == "qwen2":
+        cfg = qwen2.Config("qwen2", 512, 1536, 8960, 1, 12, 2, "silu", max_position_embeddings=2048, rope_theta=1e6, head_dim=128)
+        B, S = 2, 1024
+    else:
+        cfg = qwen2.Config("gemma", 512, 2048, 16384, 1, 8, 1, "gelu", max_position_embeddings=4096, head_dim=256)
+        B, S = 2, 512
+    dec, params = build(cfg, B, S, request)
+    g = np.random.Generator(np.random.PCG64(43))
+    x = rnd(g.standard_normal((B, S, cfg.hidden_size)).astype(np.float32), "bf16")
+    got, _, _ = dec.forward_hidden(hidden_in=to_storage(x, "bf16"))
+    progress(request, "oracle: one layer, bf16 chain")
+    ref = qwen2.Model(cfg, params, "bf16")
+    want = ref.layer(0, x, qwen2.causal_mask(S, 0, "bf16"), 0)
+    assert_close(got, want, "bf16", f"{arch} layer output vs the bf16 chain")
+    ulp = float(np.max(np.abs(want))) * 2.0 ** -8     # one rounding of the output: no error of the layer
+    d_got, d_want = got.astype(np.float64) - x, want.astype(np.float64) - x
+    err, scale = float(np.max(np.abs(d_got - d_want))), float(np.max(np.abs(d_want)))
+    progress(request, "layer contribution: max error %.3e of %.3e (%.4f), one output rounding %.3e" % (err, scale, err / scale, ulp))
+    assert err <= 2e-2 * scale + ulp, f"attention + MLP contribution off by {err:.3e} (scale {scale:.3e})"
+    dec.close()

@@ -249,6 +249,11 @@ def test_compositions_are_taken_by_one_launch_each(hip, dt):
         "rms_norm": (lambda: g.rms_norm(dev(x, dt), dev(w, dt), 1e-6), onn.rms_norm(x, w, 1e-6, dt)),
         "linear": (lambda: g.linear(dev(x, dt), dev(wl, dt), dev(bl, dt)), onn.linear(x, wl, bl, dt)),
     }
+
+    def rms_norm_by_division():     # the same value recorded as x / sqrt(n): also taken
+        xt, wt = dev(x, dt), dev(w, dt)
+        return wt * xt * ((xt / float(np.sqrt(96))).square().sum(-1, True) + 1e-6).rsqrt()
+    cases["rms_norm recorded as a division"] = (rms_norm_by_division, onn.rms_norm(x, w, 1e-6, dt))
     for name, (build, want) in cases.items():
         composed, st_c, _ = run(build, True, compose=True)
         plain, st_p, _ = run(build, True, compose=False)

@@ -192,10 +192,45 @@ def test_full_width_single_layer_f32(hip):
     cfg = phi2.Config(num_hidden_layers=1, tie_word_embeddings=True, max_position_embeddings=256)
     dec, ref = make(cfg, "f32", hip, max_batch=1, max_context=160, seed=0)
     ids = np.random.Generator(np.random.PCG64(1)).integers(0, cfg.vocab_size, (1, 128)).astype(np.uint32)
-    logits, tok = dec.forward(ids)
+    # the hidden state after the layer, [1, 128, 2560] (what DecoderLayer::fwd returns, phi2.rs:293-299), then the
+    # argmax over the tied 51200-way head
+    hidden, logits, tok = dec.forward_hidden(ids=ids, want_logits=True)
+    assert hidden.shape == (1, 128, cfg.hidden_size)
+    assert_close(hidden, ref.hidden(ids), "f32", "C0 hidden state after the layer")
+    ref.clear_kv_cache()
     want = ref.fwd(ids)
     assert_close(logits, want, "f32", "C0 logits")
     assert tok[0] == np.argmax(want[0])
+    # the same through the ordinary entry point
+    dec.clear_kv_cache()
+    logits2, tok2 = dec.forward(ids)
+    np.testing.assert_array_equal(logits2, logits)
+    assert tok2[0] == tok[0]
+    dec.close()
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_forward_hidden_rows_in_place_of_the_embedding(hip, dt):
+    # rows handed in directly give what the same rows give when they come out of the embedding table
+    cfg = small_cfg()
+    dec, ref = make(cfg, dt, hip)
+    ids = np.random.Generator(np.random.PCG64(8)).integers(0, cfg.vocab_size, (2, 11)).astype(np.uint32)
+    from oracle import nn as onn
+    rows = onn.embedding(ids, ref.p["model.embed_tokens.weight"])
+    h_ids, l_ids, t_ids = dec.forward_hidden(ids=ids, want_logits=True)
+    dec.clear_kv_cache()
+    h_rows, l_rows, t_rows = dec.forward_hidden(hidden_in=to_storage(rows, dt), want_logits=True)
+    np.testing.assert_array_equal(h_ids, h_rows)
+    np.testing.assert_array_equal(l_ids, l_rows)
+    np.testing.assert_array_equal(t_ids, t_rows)
+    assert_close(h_ids, ref.hidden(ids), dt, "hidden state of the small model")
+    import ctypes as C
+    from rai_amd._lib import RaiHipError, call
+    st = to_storage(rows, dt)
+    dec.clear_kv_cache()
+    with pytest.raises(RaiHipError):      # ids and rows at once
+        call("rai_hip_decoder_forward_hidden", dec._h, ids.ctypes.data_as(C.POINTER(C.c_uint32)),
+             st.ctypes.data_as(C.c_void_p), 2, 11, None, None, None)
     dec.close()
 
 

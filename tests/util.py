@@ -111,21 +111,21 @@ def assert_logits_close(got, chain, exact, dt, what=""):
     primitive's result rounded to the storage dtype) is itself a few per cent away from the same computation without
     intermediate rounding (`exact`: the same stored weights, rotary tables and inputs, f32 arithmetic).  Measured on
     the 32-layer Phi-2 widths over a 512-token prefill and 12 steps: chain vs exact 1.5-3.0 % of the largest logit,
-    device vs exact 1.3-2.8 % (below the chain's figure in 24 of 26 cases), device vs chain 1.3-2.0 %: three bf16
-    evaluations of the same weights, each about as far from the others as the dtype tolerance.  So:
-      - against `exact` the device is held to the dtype's relative tolerance or, where the chain itself is farther
-        than that, to the chain's own distance plus a quarter;
-      - against `chain` it may not be farther than the tolerance plus the chain's measured rounding noise.
-    Errors are relative to the largest magnitude of the expected logits, as in assert_close."""
+    device vs exact 1.0-2.8 %, device vs chain 1.3-2.6 %: three bf16 evaluations of the same weights, each about as far
+    from the others as the dtype's tolerance after that many layers.  Whole-model logits are therefore held to one and
+    a half times the dtype's tolerance, against `exact` and against `chain` alike: a fixed bound that does not grow
+    with what the chain happens to measure.  Layer by layer, where no noise builds up, the chain itself is the
+    reference at the plain tolerance (the single-layer tests), and so it is for every model shallow enough
+    (assert_close).  Errors are relative to the largest magnitude of the expected logits, as in assert_close."""
     got, chain, exact = (np.asarray(a, dtype=np.float64) for a in (got, chain, exact))
     assert got.shape == chain.shape == exact.shape, f"{what}: shapes {got.shape} {chain.shape} {exact.shape}"
     assert np.isfinite(got).all(), f"{what}: non-finite logits"
     scale = float(np.max(np.abs(exact)))
     tol = RTOL[dt] * scale
     e_dev, e_chain, e_dc = (float(np.max(np.abs(a - b))) for a, b in ((got, exact), (chain, exact), (got, chain)))
-    bound = max(tol, 1.25 * e_chain)
-    assert e_dev <= bound, (f"{what}: device vs unrounded reference arithmetic {e_dev:.3e} > {bound:.3e} "
-                            f"(tolerance {tol:.3e}, chain vs the same {e_chain:.3e})")
-    assert e_dc <= tol + e_chain, (f"{what}: device vs node-by-node chain {e_dc:.3e} > {tol:.3e} + chain noise "
-                                   f"{e_chain:.3e}")
+    bound = 1.5 * tol
+    assert e_dev <= bound, (f"{what}: device vs unrounded reference arithmetic {e_dev:.3e} > 1.5 x {tol:.3e} "
+                            f"(chain vs the same {e_chain:.3e})")
+    assert e_dc <= bound, (f"{what}: device vs node-by-node chain {e_dc:.3e} > 1.5 x {tol:.3e} "
+                           f"(chain vs unrounded arithmetic {e_chain:.3e})")
     return e_dev / scale, e_chain / scale, e_dc / scale
