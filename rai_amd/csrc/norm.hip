@@ -25,28 +25,14 @@ k_norm_wave(T *out, const T *x, const T *w, const T *b, int64_t rows, int64_t n,
     const T *xr = x + row * x_row_stride;
     float v[ITEMS][V];
     float s = 0.f;
-    // the row and, right behind it, the parameters: their loads are in flight during the reductions instead of
-    // adding a memory round trip of their own before the stores
-    NPack<T, V> pk[ITEMS], wk[ITEMS], bk[ITEMS];
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
-      const int64_t p = lane + it * 64;
-      if (p < packs) pk[it] = *reinterpret_cast<const NPack<T, V> *>(xr + p * V);
-    }
-#pragma unroll
-    for (int it = 0; it < ITEMS; ++it) {
-      const int64_t p = lane + it * 64;
+      int64_t p = lane + it * 64;
       if (p < packs) {
-        if (w) wk[it] = *reinterpret_cast<const NPack<T, V> *>(w + p * V);
-        if (b) bk[it] = *reinterpret_cast<const NPack<T, V> *>(b + p * V);
-      }
-    }
-#pragma unroll
-    for (int it = 0; it < ITEMS; ++it) {
-      if (lane + it * 64 < packs) {
+        NPack<T, V> pk = *reinterpret_cast<const NPack<T, V> *>(xr + p * V);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          v[it][j] = (float)Scalar<T>::load(&pk[it].v[j]);
+          v[it][j] = (float)Scalar<T>::load(&pk.v[j]);
           s += kind == kLayerNorm ? v[it][j] : v[it][j] * v[it][j];
         }
       }
@@ -77,15 +63,17 @@ k_norm_wave(T *out, const T *x, const T *w, const T *b, int64_t rows, int64_t n,
     for (int it = 0; it < ITEMS; ++it) {
       int64_t p = lane + it * 64;
       if (p < packs) {
-        NPack<T, V> ok;
+        NPack<T, V> wk, bk, ok;
+        if (w) wk = *reinterpret_cast<const NPack<T, V> *>(w + p * V);
+        if (b) bk = *reinterpret_cast<const NPack<T, V> *>(b + p * V);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
           float y = (v[it][j] - mean) * scale;
           if (w) {
-            float wf = (float)Scalar<T>::load(&wk[it].v[j]);
+            float wf = (float)Scalar<T>::load(&wk.v[j]);
             y *= (kind == kRmsNormAddOne) ? (1.0f + wf) : wf;
           }
-          if (b) y += (float)Scalar<T>::load(&bk[it].v[j]);
+          if (b) y += (float)Scalar<T>::load(&bk.v[j]);
           Scalar<T>::store(&ok.v[j], y);
         }
         *reinterpret_cast<NPack<T, V> *>(yr + p * V) = ok;
@@ -150,7 +138,6 @@ struct RopeArgs {
   int64_t xs[4];  // input strides
   int64_t rot, half, offset;
   int64_t tab_row_stride;
-  int tab_vec;   // the tables may be read a pack (VEC entries, sizeof(TT) * VEC bytes, aligned) at a time
 };
 
 // A value rounded to storage type T and widened again: the rounding every node of the reference's rotary chain
@@ -209,20 +196,9 @@ __global__ void __launch_bounds__(256) k_rope_vec(T *out, const T *x, const TT *
       const Pack o = *reinterpret_cast<const Pack *>(xp + (d < half ? d + half : d - half));
       const int64_t trow = (a.offset + s) * a.tab_row_stride + d;
       const float sign = d < half ? -1.f : 1.f;  // rotate_half = cat(-x2, x1)
-      // the VEC table entries of this pack as one or two aligned vector loads per table where the layout allows
-      // (the launcher checks it), instead of VEC loads of one element each
-      struct alignas(sizeof(TT) * VEC) TPack { TT v[VEC]; };
-      TPack ct, st;
-      if (a.tab_vec) {
-        ct = *reinterpret_cast<const TPack *>(cos_t + trow);
-        st = *reinterpret_cast<const TPack *>(sin_t + trow);
-      } else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) { ct.v[j] = cos_t[trow + j]; st.v[j] = sin_t[trow + j]; }
-      }
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const float c = (float)Scalar<TT>::load(&ct.v[j]), sn = (float)Scalar<TT>::load(&st.v[j]);
+        const float c = (float)Scalar<TT>::load(cos_t + trow + j), sn = (float)Scalar<TT>::load(sin_t + trow + j);
         const float r = rope_round<T>((float)Scalar<T>::load(&v.v[j]) * c) +
                         rope_round<T>(sign * (float)Scalar<T>::load(&o.v[j]) * sn);
         Scalar<T>::store(&v.v[j], (typename Scalar<T>::compute)r);
@@ -368,9 +344,6 @@ int rai_hip_rope(int dev, const rai_hip_tensor *x, const rai_hip_tensor *cos_t, 
                       x->stride[0] % vec == 0 && x->stride[1] % vec == 0 && x->stride[2] % vec == 0 &&
                       (uintptr_t)base_ptr(x) % 16 == 0 && (uintptr_t)base_ptr(out) % 16 == 0 &&
                       numel(out) / vec < (int64_t)1 << 31;
-  const size_t tpack = dtype_size(cos_t->dtype) * vec;   // bytes of one pack of table entries
-  a.tab_vec = (cos_t->stride[0] * dtype_size(cos_t->dtype)) % tpack == 0 && (uintptr_t)base_ptr(cos_t) % tpack == 0 &&
-              (uintptr_t)base_ptr(sin_t) % tpack == 0;
   int64_t blocks = ((vec_ok ? numel(out) / vec : numel(out)) + 255) / 256;
   int grid = (int)(blocks < kNumCU * 32 ? blocks : kNumCU * 32);
 #define ROPE_LAUNCH(T, TT)                                                                                       \
