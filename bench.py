@@ -405,13 +405,12 @@ def run_phi2_graph(args, n_new=16):
     builds it (tests/graph_models.py, KV cache by concatenation) and evaluated by the C++ evaluator with its
     composition and elementwise passes.  Greedy decode, batch 1, 512-token prompt; the time per token includes
     recording the graph from Python (ctypes), which a Rust front end would do far faster."""
-    from oracle.phi2 import Config, param_shapes
     from rai_amd import graph as g, synthetic
     from rai_amd.graph import Tensor
-    from tests.graph_models import Phi2Graph
-    cfg = Config(num_hidden_layers=args.layers)
+    from tests.graph_models import Phi2Graph     # the stand-in for the reference's unchanged model file
+    cfg = synthetic.Phi2Shape(num_hidden_layers=args.layers)
     params = {}
-    for name, shape in param_shapes(cfg).items():
+    for name, shape in synthetic.phi2_param_shapes(cfg).items():
         a = synthetic.to_storage(synthetic.tensor(name, int(np.prod(shape)), 0, 0.02), "bf16").reshape(shape)
         params[name] = Tensor.from_array(a, "bf16")
     g.eval_all(list(params.values()))
@@ -422,7 +421,7 @@ def run_phi2_graph(args, n_new=16):
         g.set_compose(compose)
         model.clear_kv_cache()
         ids = prompt
-        toks, t_rec, t_eval, launches, nodes = [], 0.0, 0.0, 0, 0
+        toks, t_rec, t_eval, launches, nodes, t_plan, t_run = [], 0.0, 0.0, 0, 0, 0.0, 0.0
         steps = n_new if compose else min(n_new, 4)
         for step in range(steps + 1):
             g.stats(reset=True)
@@ -438,6 +437,8 @@ def run_phi2_graph(args, n_new=16):
                 t_rec += t1 - t0
                 t_eval += t2 - t1
                 launches += st["kernel_launches"]
+                t_plan += st["plan_ms"]
+                t_run += st["run_ms"]
                 nodes += st["nodes_evaluated"] + st["fused_nodes"] + st["composed_nodes"]
             toks.append(int(tok[0]))
             ids = tok.reshape(1, 1).astype(np.uint32)
@@ -445,6 +446,8 @@ def run_phi2_graph(args, n_new=16):
         out[f"{label}_record_ms_per_token"] = round(t_rec / steps * 1e3, 3)
         out[f"{label}_eval_ms_per_token"] = round(t_eval / steps * 1e3, 3)
         out[f"{label}_launches_per_token"] = round(launches / steps, 1)
+        out[f"{label}_host_plan_ms_per_token"] = round(t_plan / steps, 3)
+        out[f"{label}_host_run_ms_per_token"] = round(t_run / steps, 3)
         out[f"{label}_first_tokens"] = toks[:8]
     g.set_compose(True)
     out["recorded_nodes_per_token"] = round(nodes / steps, 1)

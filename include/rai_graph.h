@@ -144,6 +144,8 @@ typedef struct rai_graph_stats {
   uint64_t fused_nodes;       /* nodes folded into those regions */
   uint64_t composed_regions;  /* compositions evaluated by one fused launcher */
   uint64_t composed_nodes;    /* nodes folded into those compositions */
+  uint64_t plan_ns;           /* host time of rai_eval spent ordering the tape and planning the two passes */
+  uint64_t run_ns;            /* host time of rai_eval spent in the rules (allocation, launches, detach) */
 } rai_graph_stats;
 int rai_graph_get_stats(rai_graph_stats *out, int32_t reset);
 

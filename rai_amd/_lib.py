@@ -143,7 +143,8 @@ PROTOTYPES = {
 
 class GraphStats(C.Structure):
     _fields_ = [("nodes_evaluated", C.c_uint64), ("kernel_launches", C.c_uint64), ("fused_regions", C.c_uint64),
-                ("fused_nodes", C.c_uint64), ("composed_regions", C.c_uint64), ("composed_nodes", C.c_uint64)]
+                ("fused_nodes", C.c_uint64), ("composed_regions", C.c_uint64), ("composed_nodes", C.c_uint64),
+                ("plan_ns", C.c_uint64), ("run_ns", C.c_uint64)]
 
 
 _T = C.c_void_p  # rai_tensor *

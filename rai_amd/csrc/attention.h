@@ -36,7 +36,12 @@ struct AttnDecodeArgs {
   void *out;
   int64_t out_row_stride;
   const void *cos_t, *sin_t;  // [max_pos, rot] in the model dtype
-  const int *pos_dev;         // tokens already in the cache (device memory)
+  const int *pos_dev;         // tokens already in the cache (device memory); null: pos_host
+  int pos_host;
+  // The new token's key and value rows as tensors of their own ([B][Hkv*D], element strides between sequences
+  // below) instead of behind the queries in one packed row; qkv then holds the queries alone.  Null: packed.
+  const void *k_new, *v_new;
+  int64_t q_row_stride, k_row_stride, v_row_stride;
   int rot;
   int B, Hq, Hkv, D, Tmax;
   float scale;

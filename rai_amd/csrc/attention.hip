@@ -262,7 +262,7 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_split(AttnDecode
   const int n_rep = a.Hq / a.Hkv, hk = hq0 / n_rep;
   const bool writer = hq0 % n_rep == 0;     // one block per KV head appends the new token
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  int pos = *a.pos_dev;
+  int pos = a.pos_dev ? *a.pos_dev : a.pos_host;
   if (pos > a.Tmax - 1) pos = a.Tmax - 1;   // capacity is checked on the host; never write past the cache
   const int cnt = pos + 1;
   int chunk = (cnt + NS - 1) / NS;
@@ -274,7 +274,10 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_split(AttnDecode
   const int t1c = has_new ? pos : t1;       // cached keys are [t0, t1c)
 
   const int QD = a.Hq * D, KD = a.Hkv * D;
-  const T *row = (const T *)a.qkv + (int64_t)b * (QD + 2 * KD);
+  // the new token's rows: one packed [q | k | v] row per sequence, or three separate ones
+  const T *qrow = (const T *)a.qkv + (int64_t)b * (a.k_new ? a.q_row_stride : (int64_t)(QD + 2 * KD));
+  const T *krow = a.k_new ? (const T *)a.k_new + (int64_t)b * a.k_row_stride : qrow + QD;
+  const T *vrow = a.k_new ? (const T *)a.v_new + (int64_t)b * a.v_row_stride : qrow + QD + KD;
   T *Kc = (T *)a.kcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   T *Vc = (T *)a.vcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   const T *cos_t = (const T *)a.cos_t, *sin_t = (const T *)a.sin_t;
@@ -300,12 +303,12 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_split(AttnDecode
   // ---- rotary embedding of the R query rows (and of the new key where it is needed)
   for (int e = tid; e < R * D; e += NT) {
     const int r = e / D, d = e - r * D;
-    qf[e] = rope_feature<T>(row + (hq0 + r) * D, d, a.rot, cos_t, sin_t, pos);
+    qf[e] = rope_feature<T>(qrow + (hq0 + r) * D, d, a.rot, cos_t, sin_t, pos);
   }
   if (has_new) {
     for (int d = tid; d < D; d += NT) {
-      const float kr = rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos);
-      const float vr = (float)Scalar<T>::load(row + QD + KD + hk * D + d);
+      const float kr = rope_feature<T>(krow + hk * D, d, a.rot, cos_t, sin_t, pos);
+      const float vr = (float)Scalar<T>::load(vrow + hk * D + d);
       knew[d] = kr;
       vnew[d] = vr;
       if (writer) {
@@ -498,7 +501,7 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeA
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 15, lq = lane >> 4;
   const int NS = a.ns;
-  int pos = *a.pos_dev;
+  int pos = a.pos_dev ? *a.pos_dev : a.pos_host;
   if (pos > a.Tmax - 1) pos = a.Tmax - 1;   // capacity is checked on the host; never write past the cache
   const int cnt = pos + 1;
   int chunk = (cnt + NS - 1) / NS;
@@ -511,7 +514,10 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeA
   const int new_row = pos - t0;
 
   const int QD = a.Hq * D, KD = a.Hkv * D;
-  const T *row = (const T *)a.qkv + (int64_t)b * (QD + 2 * KD);
+  // the new token's rows: one packed [q | k | v] row per sequence, or three separate ones
+  const T *qrow = (const T *)a.qkv + (int64_t)b * (a.k_new ? a.q_row_stride : (int64_t)(QD + 2 * KD));
+  const T *krow = a.k_new ? (const T *)a.k_new + (int64_t)b * a.k_row_stride : qrow + QD;
+  const T *vrow = a.k_new ? (const T *)a.v_new + (int64_t)b * a.v_row_stride : qrow + QD + KD;
   T *Kc = (T *)a.kcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   T *Vc = (T *)a.vcache + ((int64_t)b * a.Hkv + hk) * a.Tmax * D;
   const T *cos_t = (const T *)a.cos_t, *sin_t = (const T *)a.sin_t;
@@ -548,7 +554,7 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeA
       const int item = tid + i * kDecodeThreads, r = item / CPR, d = (item - r * CPR) * 8;
       qx[i] = qo[i] = qc[i] = qn[i] = ad_u32x4{0u, 0u, 0u, 0u};
       if (item < 16 * CPR && r < R) {
-        const T *head = row + (hq0 + r) * D;
+        const T *head = qrow + (hq0 + r) * D;
         qx[i] = *reinterpret_cast<const ad_u32x4 *>(head + d);
         if (d < a.rot) {
           qo[i] = *reinterpret_cast<const ad_u32x4 *>(head + (d < half ? d + half : d - half));
@@ -584,15 +590,15 @@ __global__ void __launch_bounds__(kDecodeThreads) k_attn_decode_mfma(AttnDecodeA
   } else {
     for (int e = tid; e < 16 * D; e += kDecodeThreads) {
       const int r = e / D, d = e - r * D;
-      const float q = r < R ? rope_feature<T>(row + (hq0 + r) * D, d, a.rot, cos_t, sin_t, pos) : 0.f;
+      const float q = r < R ? rope_feature<T>(qrow + (hq0 + r) * D, d, a.rot, cos_t, sin_t, pos) : 0.f;
       Vs[r * VP + d] = f32_to_bf16_bits(q);
     }
   }
   for (int e = tid; e < 16 * PP; e += kDecodeThreads) ps[e] = 0;
   if (has_new) {
     for (int d = tid; d < D; d += kDecodeThreads) {
-      const uint16_t kr = f32_to_bf16_bits(rope_feature<T>(row + QD + hk * D, d, a.rot, cos_t, sin_t, pos));
-      const uint16_t vr = (row + QD + KD + hk * D + d)->bits;
+      const uint16_t kr = f32_to_bf16_bits(rope_feature<T>(krow + hk * D, d, a.rot, cos_t, sin_t, pos));
+      const uint16_t vr = (vrow + hk * D + d)->bits;
       knew[d] = kr;
       vnew[d] = vr;
       (Kc + (int64_t)pos * D + d)->bits = kr;

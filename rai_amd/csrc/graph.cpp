@@ -9,12 +9,14 @@
 // (unary, arithmetic binary, float casts, constants) whose intermediate results
 // nobody else can observe is evaluated by one launch of a small register-machine
 // kernel (fused.h) that rounds exactly where node-by-node evaluation would.
+#include <chrono>
 #include <cmath>
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
 #include <vector>
 
+#include "attention.h"
 #include "fused.h"
 #include "rai_graph.h"
 
@@ -34,14 +36,35 @@ struct rai_tensor {
   bool evaluated;
   rai_hip_tensor view;            // storage once evaluated (may alias an input's buffer)
   void *buf;                      // retained allocation the view points into
+  // A concatenation along `cap_dim` whose buffer was laid out for `cap` elements along that dim (strided view):
+  // the next concatenation that appends to this node writes its new part into the slack instead of copying both
+  // (once: `extended` says somebody already did).
+  int cap_dim;
+  int64_t cap;
+  bool extended;
+  // Scratch of the evaluation in progress, valid while mark == the evaluation's epoch: position in the tape, the
+  // edges from tape nodes that use this node (a run of the evaluation's flat user list), planning flags, the
+  // composition this node is the root of, and a stamp the matchers use to tell a composition's nodes apart.
+  uint64_t mark;
+  int tape_idx;
+  int n_users, users_at;
+  uint32_t flags;
+  int comp;
+  uint64_t stamp;
 };
 
 namespace {
 
 uint64_t g_next_id = 1;
+uint64_t g_epoch = 0;        // one per rai_eval call
+uint64_t g_stamp = 0;        // one per attempted composition
+enum : uint32_t { kInlined = 1u, kAbsorbed = 2u, kRoot = 4u, kOutput = 8u, kCoOutput = 16u };
+inline bool in_tape(const rai_tensor *t) { return t->mark == g_epoch; }
+inline bool has_flag(const rai_tensor *t, uint32_t f) { return in_tape(t) && (t->flags & f); }
+std::vector<const rai_tensor *> g_users;   // flat user lists of the evaluation in progress
 bool g_fusion = true;
 bool g_compose = true;
-rai_graph_stats g_stats = {0, 0, 0, 0, 0, 0};
+rai_graph_stats g_stats = {0, 0, 0, 0, 0, 0, 0, 0};
 
 int64_t numel_of(const std::vector<int64_t> &s) {
   int64_t n = 1;
@@ -64,6 +87,15 @@ rai_tensor *new_node(int dev, int dtype, const std::vector<int64_t> &shape, int 
   t->evaluated = false;
   memset(&t->view, 0, sizeof(t->view));
   t->buf = nullptr;
+  t->cap_dim = -1;
+  t->cap = 0;
+  t->extended = false;
+  t->mark = 0;
+  t->tape_idx = -1;
+  t->n_users = t->users_at = 0;
+  t->flags = 0;
+  t->comp = -1;
+  t->stamp = 0;
   return t;
 }
 
@@ -108,6 +140,7 @@ void drop_storage(rai_tensor *t) {
   if (t->buf) (void)rai_hip_release(t->buf);
   t->buf = nullptr;
   t->evaluated = false;
+  t->cap_dim = -1;
 }
 
 void contiguous_view(rai_tensor *t, void *data) {
@@ -271,9 +304,61 @@ int ev_to_device(rai_tensor *t) {  // ops/to_device.rs: the node lives on the ta
   ++g_stats.kernel_launches;
   return rai_hip_to_device(t->inputs[0]->dev, &t->inputs[0]->view, t->dev, &t->view);
 }
+// A key / value cache grows by concatenation along the sequence dim every step (phi2.rs:233-243): cat([cache, new], 2).
+// Copying the whole cache each time is O(T) per step and layer.  Instead such a concatenation (two inputs, the dim
+// before the last, the second input the shorter one) gets a buffer with room to grow along that dim, laid out with
+// the capacity as the stride, and the next concatenation that appends to its result writes only the new part into
+// the slack and shares the buffer.  The earlier tensor keeps its shape and its contents (its view never covered the
+// slack), so nothing observable changes; a second concatenation onto the same tensor copies as usual.
+int64_t grown_capacity(int64_t len) { return (len + len / 4 + 64 + 63) / 64 * 64; }
+
+int append_in_place(rai_tensor *t, int dim) {
+  rai_tensor *base = t->inputs[0], *add = t->inputs[1];
+  rai_hip_tensor v = base->view;
+  v.shape[dim] = t->shape[dim];
+  rai_hip_tensor dst = v;              // the slice the new part fills
+  dst.shape[dim] = add->shape[dim];
+  dst.offset += base->shape[dim] * dst.stride[dim];
+  ++g_stats.kernel_launches;
+  RAI_TRY(rai_hip_copy(t->dev, &add->view, &dst));
+  alias_storage(t, base, v);
+  t->cap_dim = dim;
+  t->cap = base->cap;
+  base->extended = true;
+  return RAI_OK;
+}
+
 int ev_concatenate(rai_tensor *t) {
-  RAI_TRY(alloc_output(t));
   const int dim = (int)t->ip[0];
+  const int rank = (int)t->shape.size();
+  const bool cache_like = t->inputs.size() == 2 && rank >= 3 && dim == rank - 2 && numel_of(t->inputs[1]->shape) > 0 &&
+                          t->inputs[1]->shape[dim] <= t->inputs[0]->shape[dim];
+  if (cache_like) {
+    rai_tensor *base = t->inputs[0];
+    if (base->cap_dim == dim && !base->extended && t->shape[dim] <= base->cap && base->buf) return append_in_place(t, dim);
+    // first growth: a buffer with slack along `dim`, viewed through strides that skip it
+    const int64_t cap = grown_capacity(t->shape[dim]);
+    std::vector<int64_t> padded = t->shape;
+    padded[dim] = cap;
+    void *p = nullptr;
+    RAI_TRY(rai_hip_alloc(t->dev, (size_t)numel_of(padded) * dtype_size(t->dtype), &p));
+    t->buf = p;
+    rai_hip_tensor &v = t->view;
+    memset(&v, 0, sizeof(v));
+    v.data = p;
+    v.dtype = t->dtype;
+    v.rank = rank;
+    int64_t st = 1;
+    for (int i = rank - 1; i >= 0; --i) {
+      v.shape[i] = t->shape[i];
+      v.stride[i] = st;
+      st *= padded[i];
+    }
+    t->cap_dim = dim;
+    t->cap = cap;
+  } else {
+    RAI_TRY(alloc_output(t));
+  }
   int64_t at = 0;
   for (rai_tensor *in : t->inputs) {
     rai_hip_tensor dst = t->view;  // the slice of the output this input fills
@@ -344,7 +429,27 @@ int ev_reshape(rai_tensor *t) {
     alias_storage(t, in, v);
     return RAI_OK;
   }
-  // a reshape of a non-contiguous view has to materialise it first
+  // inserting or dropping dims of size 1 (unsqueeze, squeeze) is a view of any layout
+  {
+    std::vector<int64_t> keep_shape, keep_stride;
+    for (int i = 0; i < in->view.rank; ++i)
+      if (in->view.shape[i] != 1) { keep_shape.push_back(in->view.shape[i]); keep_stride.push_back(in->view.stride[i]); }
+    std::vector<int64_t> want;
+    for (int64_t d : t->shape)
+      if (d != 1) want.push_back(d);
+    if (want == keep_shape && t->shape.size() <= RAI_HIP_MAX_RANK) {
+      rai_hip_tensor v = in->view;
+      v.rank = (int32_t)t->shape.size();
+      size_t k = 0;
+      for (int i = 0; i < v.rank; ++i) {
+        v.shape[i] = t->shape[i];
+        v.stride[i] = t->shape[i] == 1 ? 1 : keep_stride[k++];
+      }
+      alias_storage(t, in, v);
+      return RAI_OK;
+    }
+  }
+  // any other reshape of a non-contiguous view has to materialise it first
   RAI_TRY(alloc_output(t));
   rai_hip_tensor as_in = t->view;
   as_in.rank = in->view.rank;
@@ -381,17 +486,21 @@ const char *op_name(int op) {
 
 // ------------------------------------------------------------------ topological order (utils.rs:35-66)
 int topo_sort(rai_tensor *const *outputs, int n, std::vector<rai_tensor *> *tape) {
-  std::unordered_set<uint64_t> visited;
+  ++g_epoch;   // a node is in this tape exactly when its mark carries this epoch
   std::vector<std::pair<rai_tensor *, bool>> stack;
   for (int o = 0; o < n; ++o) {
     stack.push_back({outputs[o], outputs[o]->inputs.empty()});
     while (!stack.empty()) {
       auto [t, inputs_done] = stack.back();
       stack.pop_back();
-      if (visited.count(t->id) || t->evaluated) continue;
+      if (in_tape(t) || t->evaluated) continue;
       if (t->op == RAI_OP_ERR) return fail(RAI_ERR_BAD_SHAPE, "eval: %s", t->err.c_str());
       if (inputs_done) {
-        visited.insert(t->id);
+        t->mark = g_epoch;
+        t->tape_idx = (int)tape->size();
+        t->n_users = t->users_at = 0;
+        t->flags = 0;
+        t->comp = -1;
         tape->push_back(t);
       } else {
         stack.push_back({t, true});
@@ -416,44 +525,42 @@ bool elementwise(const rai_tensor *t) {
   }
 }
 
-struct FusionPlan {
-  std::unordered_set<uint64_t> inlined;  // nodes that never receive data: they live inside a consumer's region
-};
+// Edges of the tape: how many tape nodes use each tape node and which (rai_tensor::n_users / users_at into g_users).
+void index_users(const std::vector<rai_tensor *> &tape) {
+  size_t edges = 0;
+  for (const rai_tensor *t : tape)
+    for (rai_tensor *in : t->inputs)
+      if (in_tape(in)) { ++in->n_users; ++edges; }
+  int at = 0;
+  for (rai_tensor *t : tape) { t->users_at = at; at += t->n_users; t->n_users = 0; }
+  g_users.assign(edges, nullptr);
+  for (const rai_tensor *t : tape)
+    for (rai_tensor *in : t->inputs)
+      if (in_tape(in)) g_users[in->users_at + in->n_users++] = t;
+}
 
 // A node is folded into its consumer when it is elementwise, exactly one edge of
 // the tape uses it, that user is elementwise too, it is not a requested output,
 // and no handle outside the tape refers to it (refs == that one edge).
-void plan_fusion(const std::vector<rai_tensor *> &tape, rai_tensor *const *outputs, int n_out, FusionPlan *plan,
-                 const std::unordered_set<uint64_t> &composed) {
-  std::unordered_map<uint64_t, int> uses;
-  std::unordered_map<uint64_t, const rai_tensor *> user;
-  for (const rai_tensor *t : tape)
-    for (const rai_tensor *in : t->inputs) {
-      ++uses[in->id];
-      user[in->id] = t;
-    }
-  std::unordered_set<uint64_t> is_output;
-  for (int i = 0; i < n_out; ++i) is_output.insert(outputs[i]->id);
-  for (const rai_tensor *t : tape) {
-    if (!elementwise(t) || is_output.count(t->id) || !g_rules[t->op]) continue;  // fusion never hides a missing rule
-    if (composed.count(t->id)) continue;                                         // root or interior of a composition
-    auto u = uses.find(t->id);
-    if (u == uses.end() || u->second != 1 || t->refs != 1) continue;
-    const rai_tensor *c = user[t->id];
-    if (!elementwise(c) || composed.count(c->id) || numel_of(c->shape) != numel_of(t->shape) || c->shape != t->shape) continue;
-    plan->inlined.insert(t->id);
+void plan_fusion(const std::vector<rai_tensor *> &tape) {
+  for (rai_tensor *t : tape) {
+    if (!elementwise(t) || (t->flags & (kOutput | kAbsorbed | kRoot)) || !g_rules[t->op]) continue;  // fusion never hides a missing rule
+    if (t->n_users != 1 || t->refs != 1) continue;
+    const rai_tensor *c = g_users[t->users_at];
+    if (!elementwise(c) || (c->flags & (kAbsorbed | kRoot)) || c->shape != t->shape) continue;
+    t->flags |= kInlined;
   }
 }
 
 // Emits the instructions of `t` (post-order) into the program; returns its register or -1 when the region is too large.
-int emit(const rai_tensor *t, const FusionPlan &plan, bool root, FusedProgram *p, std::unordered_map<uint64_t, int> *leaf_reg,
+int emit(const rai_tensor *t, bool root, FusedProgram *p, std::unordered_map<uint64_t, int> *leaf_reg,
          std::vector<const rai_tensor *> *members) {
   auto push = [&](FusedInstr in) -> int {
     if (p->n_instr >= kFusedMaxInstr) return -1;
     p->instr[p->n_instr] = in;
     return p->n_instr++;
   };
-  if (!root && !plan.inlined.count(t->id)) {  // a materialised input: leaf
+  if (!root && !has_flag(t, kInlined)) {  // a materialised input: leaf
     auto it = leaf_reg->find(t->id);
     if (it != leaf_reg->end()) return it->second;
     if (p->n_leaves >= kFusedMaxLeaves) return -1;
@@ -488,7 +595,7 @@ int emit(const rai_tensor *t, const FusionPlan &plan, bool root, FusedProgram *p
       return push(in);
     }
     case RAI_OP_UNARY: {
-      const int a = emit(t->inputs[0], plan, false, p, leaf_reg, members);
+      const int a = emit(t->inputs[0], false, p, leaf_reg, members);
       if (a < 0) return -1;
       in.kind = FUSED_UNARY;
       in.op = (uint8_t)t->sub;
@@ -497,9 +604,9 @@ int emit(const rai_tensor *t, const FusionPlan &plan, bool root, FusedProgram *p
       return push(in);
     }
     case RAI_OP_BINARY: {
-      const int a = emit(t->inputs[0], plan, false, p, leaf_reg, members);
+      const int a = emit(t->inputs[0], false, p, leaf_reg, members);
       if (a < 0) return -1;
-      const int b = emit(t->inputs[1], plan, false, p, leaf_reg, members);
+      const int b = emit(t->inputs[1], false, p, leaf_reg, members);
       if (b < 0) return -1;
       in.kind = FUSED_BINARY;
       in.op = (uint8_t)t->sub;
@@ -508,7 +615,7 @@ int emit(const rai_tensor *t, const FusionPlan &plan, bool root, FusedProgram *p
       return push(in);
     }
     default: {  // RAI_OP_TO_DTYPE
-      const int a = emit(t->inputs[0], plan, false, p, leaf_reg, members);
+      const int a = emit(t->inputs[0], false, p, leaf_reg, members);
       if (a < 0) return -1;
       in.kind = FUSED_CAST;
       in.a = (uint8_t)a;
@@ -517,15 +624,15 @@ int emit(const rai_tensor *t, const FusionPlan &plan, bool root, FusedProgram *p
   }
 }
 
-bool has_inlined_input(const rai_tensor *t, const FusionPlan &plan) {
+bool has_inlined_input(const rai_tensor *t) {
   for (const rai_tensor *in : t->inputs)
-    if (plan.inlined.count(in->id)) return true;
+    if (has_flag(in, kInlined)) return true;
   return false;
 }
 
 // Evaluates the region rooted at t with one launch.  RAI_ERR_UNSUPPORTED means
 // "too large for one program": the caller falls back to node-by-node evaluation.
-int eval_region(rai_tensor *t, const FusionPlan &plan) {
+int eval_region(rai_tensor *t) {
   FusedProgram p;
   memset(&p, 0, sizeof(p));
   p.rank = (int)t->shape.size();
@@ -533,7 +640,7 @@ int eval_region(rai_tensor *t, const FusionPlan &plan) {
   for (int d = 0; d < p.rank; ++d) p.shape[d] = t->shape[d];
   std::unordered_map<uint64_t, int> leaf_reg;
   std::vector<const rai_tensor *> members;
-  if (emit(t, plan, true, &p, &leaf_reg, &members) < 0) return RAI_ERR_UNSUPPORTED;
+  if (emit(t, true, &p, &leaf_reg, &members) < 0) return RAI_ERR_UNSUPPORTED;
   RAI_TRY(alloc_output(t));
   p.out = t->view.data;
   p.out_dtype = t->dtype;
@@ -544,14 +651,14 @@ int eval_region(rai_tensor *t, const FusionPlan &plan) {
 }
 
 // Node-by-node evaluation of an inlined sub-tree (used when a region did not fit).
-int eval_plain(rai_tensor *t, const FusionPlan &plan);
-int eval_inputs_plain(rai_tensor *t, const FusionPlan &plan) {
+int eval_plain(rai_tensor *t);
+int eval_inputs_plain(rai_tensor *t) {
   for (rai_tensor *in : t->inputs)
-    if (!in->evaluated && plan.inlined.count(in->id)) RAI_TRY(eval_plain(in, plan));
+    if (!in->evaluated && has_flag(in, kInlined)) RAI_TRY(eval_plain(in));
   return RAI_OK;
 }
-int eval_plain(rai_tensor *t, const FusionPlan &plan) {
-  RAI_TRY(eval_inputs_plain(t, plan));
+int eval_plain(rai_tensor *t) {
+  RAI_TRY(eval_inputs_plain(t));
   rule_fn rule = g_rules[t->op];
   RAI_REQUIRE(rule, RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op));
   RAI_TRY(rule(t));
@@ -568,20 +675,16 @@ int eval_plain(rai_tensor *t, const FusionPlan &plan) {
 // a requested output, no handle outside the tape, every consumer inside the composition.  The fused launchers keep
 // f32 between the steps the reference rounds after, so a composed result agrees with the node-by-node one within
 // the dtype's tolerance, not bit for bit (the elementwise pass above is the bit-exact one).
-enum CompKind { COMP_LINEAR = 0, COMP_LAYER_NORM, COMP_RMS_NORM, COMP_ROPE, COMP_ATTENTION };
+enum CompKind { COMP_LINEAR = 0, COMP_LAYER_NORM, COMP_RMS_NORM, COMP_ROPE, COMP_ATTENTION, COMP_DECODE_ATTN };
 struct Composite {
   int kind;
-  rai_tensor *in[5];   // operands: evaluated before the root is reached (they precede it in the tape)
+  rai_tensor *in[7];   // operands: evaluated before the root is reached (they precede it in the tape); null: absent
   double f0;           // eps / scale
-  int64_t i0, i1;      // rotary dim and offset / causal flag
+  int64_t i0, i1, i2;  // rotary dim and offset / causal flag and f32 scores / activation / (1 + w) norm
+  // nodes that the root's launch materialises besides the root: they may be held from outside (the model keeps its
+  // key / value caches), but every use inside the tape lies within the composition
+  rai_tensor *co[2];
   std::vector<rai_tensor *> interior;
-};
-struct ComposePlan {
-  std::unordered_map<uint64_t, Composite> roots;
-  std::unordered_set<uint64_t> absorbed;
-};
-struct UseInfo {
-  std::unordered_map<uint64_t, std::vector<const rai_tensor *>> users;   // edges from nodes of the tape
 };
 
 struct Matcher {
@@ -600,8 +703,18 @@ struct Matcher {
     *b = n->inputs[1];
     return true;
   }
-  // which binary primitive an unevaluated node is (-1: none); records nothing
+  // which binary / unary primitive an unevaluated node is (-1: none); records nothing
   int bin_kind(const rai_tensor *t) const { return ok && t && !t->evaluated && t->op == RAI_OP_BINARY ? t->sub : -1; }
+  int un_kind(const rai_tensor *t) const { return ok && t && !t->evaluated && t->op == RAI_OP_UNARY ? t->sub : -1; }
+  // whether konst() would accept the node; records nothing
+  bool is_konst(const rai_tensor *t) const {
+    return t && (t->op == RAI_OP_FULL || (!t->evaluated && t->op == RAI_OP_TO_DTYPE && t->inputs[0]->op == RAI_OP_FULL));
+  }
+  // the operand behind any run of unevaluated Reshape nodes (unsqueeze is a reshape, hlops/unsqueeze.rs)
+  rai_tensor *strip_reshapes(rai_tensor *t) {
+    while (ok && t && !t->evaluated && t->op == RAI_OP_RESHAPE) { interior.push_back(t); t = t->inputs[0]; }
+    return t;
+  }
   rai_tensor *un(rai_tensor *t, int sub) {
     rai_tensor *n = node(t, RAI_OP_UNARY);
     if (!n || n->sub != sub) { ok = false; return nullptr; }
@@ -716,24 +829,146 @@ bool match_rms_norm(rai_tensor *t, Composite *c) {
   return true;
 }
 
-// rai-nn/src/linear.rs:59-69 with a bias: x @ broadcast_left(W).t() + b
-bool match_linear(rai_tensor *t, Composite *c) {
+// RmsNorm::fwd of rai-models/src/llm/gemma.rs:42-54: f32 inside for 16-bit inputs,
+// (x / sqrt(sum(x^2) / n + eps)).to_dtype(dt) * (w + 1)
+bool match_gemma_rms_norm(rai_tensor *t, Composite *c) {
   Matcher m;
-  rai_tensor *mm, *bb;
-  if ((t->dtype != RAI_BF16 && t->dtype != RAI_F32) || t->shape.size() < 2 || !m.bin(t, RAI_BIN_ADD, &mm, &bb)) return false;
-  rai_tensor *bias = m.strip_bc(bb);
+  rai_tensor *xn, *wb, *num, *den, *w, *one_c, *ms, *epsc, *sq, *nc;
+  if (!norm_dtype(t->dtype) || t->shape.empty() || m.bin_kind(t) != RAI_BIN_MUL || !m.bin(t, RAI_BIN_MUL, &xn, &wb)) return false;
+  rai_tensor *wp = m.strip_bc(wb);
+  double one = 0, eps = 0, nn = 0;
+  if (m.bin_kind(wp) != RAI_BIN_ADD || !m.bin(wp, RAI_BIN_ADD, &w, &one_c) || !m.konst(one_c, &one) || one != 1.0) return false;
+  const int64_t n = t->shape.back();
+  if (!vec_param(w, n, t->dtype)) return false;
+  xn = m.strip_cast(xn, t->dtype);
+  if (m.bin_kind(xn) != RAI_BIN_DIV || !m.bin(xn, RAI_BIN_DIV, &num, &den)) return false;
+  rai_tensor *root = m.un(m.strip_bc(den), RAI_UN_SQRT);
+  if (!root || !m.bin(root, RAI_BIN_ADD, &ms, &epsc) || !m.konst(epsc, &eps)) return false;
+  if (!m.bin(ms, RAI_BIN_DIV, &sq, &nc) || !m.konst(nc, &nn) || nn != (double)n) return false;
+  rai_tensor *sx = m.sum_last_keep(sq);
+  rai_tensor *xi = sx ? m.un(sx, RAI_UN_SQUARE) : nullptr;
+  if (!xi || xi != num || !m.ok) return false;
+  rai_tensor *x = m.strip_cast(xi, RAI_F32);
+  if (x->dtype != t->dtype || x->shape != t->shape) return false;
+  c->kind = COMP_RMS_NORM;
+  c->in[0] = x; c->in[1] = w;
+  c->f0 = eps;
+  c->i2 = 1;
+  c->interior = m.interior;
+  return true;
+}
+
+// rai-nn/src/linear.rs:59-69: x @ broadcast_left(W).t() [+ b]; fills x, w, bias (null without one)
+bool linear_core(Matcher &m, rai_tensor *t, rai_tensor **x, rai_tensor **w, rai_tensor **bias) {
+  if ((t->dtype != RAI_BF16 && t->dtype != RAI_F32) || t->shape.size() < 2) return m.ok = false;
+  rai_tensor *mm = t;
+  *bias = nullptr;
+  if (m.bin_kind(t) == RAI_BIN_ADD) {
+    rai_tensor *bb;
+    if (!m.bin(t, RAI_BIN_ADD, &mm, &bb)) return false;
+    *bias = m.strip_bc(bb);
+    if (!vec_param(*bias, t->shape.back(), t->dtype)) return m.ok = false;
+  }
   rai_tensor *mn = m.node(mm, RAI_OP_MATMUL);
-  if (!mn || !vec_param(bias, t->shape.back(), t->dtype)) return false;
-  rai_tensor *x = mn->inputs[0];
+  if (!mn) return false;
+  *x = mn->inputs[0];
   rai_tensor *wt = m.node(mn->inputs[1], RAI_OP_TRANSPOSE);
   if (!wt) return false;
   const int r = (int)wt->shape.size();
-  if (!((wt->ip[0] == r - 2 && wt->ip[1] == r - 1) || (wt->ip[0] == r - 1 && wt->ip[1] == r - 2))) return false;
-  rai_tensor *w = m.strip_bc(wt->inputs[0]);
-  if (!m.ok || w->shape.size() != 2 || w->dtype != t->dtype || x->dtype != t->dtype || x->shape.size() != t->shape.size()) return false;
-  if (w->shape[0] != t->shape.back() || w->shape[1] != x->shape.back()) return false;
+  if (!((wt->ip[0] == r - 2 && wt->ip[1] == r - 1) || (wt->ip[0] == r - 1 && wt->ip[1] == r - 2))) return m.ok = false;
+  *w = m.strip_bc(wt->inputs[0]);
+  if (!m.ok || (*w)->shape.size() != 2 || (*w)->dtype != t->dtype || (*x)->dtype != t->dtype ||
+      (*x)->shape.size() != t->shape.size())
+    return m.ok = false;
+  if ((*w)->shape[0] != t->shape.back() || (*w)->shape[1] != (*x)->shape.back()) return m.ok = false;
+  return true;
+}
+
+// The activations of rai-core/src/hlops/activations.rs:5-32 by structure: fills the argument and the RAI_UN_* code
+bool activation_of(Matcher &m, rai_tensor *t, rai_tensor **x, int *act) {
+  const int kind = m.bin_kind(t);
+  rai_tensor *a, *b;
+  double c = 0;
+  if (kind == RAI_BIN_DIV) {   // silu: x / (exp(-x) + 1)
+    rai_tensor *e, *one;
+    if (!m.bin(t, RAI_BIN_DIV, &a, &b) || !m.bin(b, RAI_BIN_ADD, &e, &one) || !m.konst(one, &c) || c != 1.0) return m.ok = false;
+    rai_tensor *ng = m.un(e, RAI_UN_EXP);
+    if (!ng || m.un(ng, RAI_UN_NEG) != a || !m.ok) return m.ok = false;
+    *x = a; *act = RAI_UN_SILU;
+    return true;
+  }
+  if (kind == RAI_BIN_MAXIMUM) {   // relu: max(x, zeros_like(x))
+    if (!m.bin(t, RAI_BIN_MAXIMUM, &a, &b) || !m.konst(b, &c) || c != 0.0) return m.ok = false;
+    *x = a; *act = RAI_UN_RELU;
+    return true;
+  }
+  if (kind != RAI_BIN_MUL) return m.ok = false;
+  rai_tensor *l, *r, *one, *inner, *p, *q;
+  if (!m.bin(t, RAI_BIN_MUL, &l, &r) || !m.bin(l, RAI_BIN_MUL, &p, &q)) return false;
+  const bool half_first = m.is_konst(p);    // new_gelu: 0.5 * x; gelu: x * 0.5
+  if (!m.konst(half_first ? p : q, &c) || c != 0.5) return m.ok = false;
+  rai_tensor *arg = half_first ? q : p;
+  if (!m.bin(r, RAI_BIN_ADD, &one, &inner) || !m.konst(one, &c) || c != 1.0) return m.ok = false;
+  if (m.un_kind(inner) == RAI_UN_TANH && half_first) {   // 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+    rai_tensor *u = m.un(inner, RAI_UN_TANH), *kc, *sum, *x1, *cub, *c4, *pw;
+    if (!u || !m.bin(u, RAI_BIN_MUL, &kc, &sum) || !m.konst(kc, &c) || fabs(c - 0.7978845608028654) > 1e-6) return m.ok = false;
+    if (!m.bin(sum, RAI_BIN_ADD, &x1, &cub) || x1 != arg || !m.bin(cub, RAI_BIN_MUL, &c4, &pw) || !m.konst(c4, &c) ||
+        fabs(c - 0.044715) > 1e-7)
+      return m.ok = false;
+    rai_tensor *pn = m.node(pw, RAI_OP_UNARY);
+    if (!pn || pn->sub != RAI_UN_POWF || pn->p0 != 3.0 || pn->inputs[0] != arg) return m.ok = false;
+    *x = arg; *act = RAI_UN_NEW_GELU;
+    return true;
+  }
+  if (m.un_kind(inner) == RAI_UN_ERF && !half_first) {   // x 0.5 (1 + erf(x / sqrt 2))
+    rai_tensor *u = m.un(inner, RAI_UN_ERF), *x1, *cs;
+    if (!u || !m.bin(u, RAI_BIN_DIV, &x1, &cs) || x1 != arg || !m.konst(cs, &c) || fabs(c - 1.4142135623730951) > 1e-6)
+      return m.ok = false;
+    *x = arg; *act = RAI_UN_GELU;
+    return true;
+  }
+  return m.ok = false;
+}
+
+// [activation of] a Linear, with or without bias
+bool act_linear(Matcher &m, rai_tensor *t, rai_tensor **x, rai_tensor **w, rai_tensor **bias, int *act) {
+  *act = -1;
+  {
+    Matcher tr = m;
+    rai_tensor *arg;
+    int a;
+    if (activation_of(tr, t, &arg, &a) && linear_core(tr, arg, x, w, bias)) {
+      // every interior use of the activation's argument is inside the activation: checked with the rest of the seal
+      *act = a;
+      m = tr;
+      return true;
+    }
+  }
+  return linear_core(m, t, x, w, bias);
+}
+
+// A Linear as the model code records it, widened by what follows it directly: the activation applied to its output
+// (MLP::fwd phi2.rs:99-101, qwen2.rs:100-104) and / or one tensor added to the result (the residual sums of
+// DecoderLayer::fwd phi2.rs:298, qwen2.rs:262-265), all of which the Linear launcher applies in its epilogue.  A plain
+// product without bias, activation or residual is left to the MatMul rule (one launch either way).
+bool match_linear(rai_tensor *t, Composite *c) {
+  rai_tensor *x = nullptr, *w = nullptr, *bias = nullptr, *res = nullptr;
+  int act = -1;
+  Matcher m;
+  bool found = act_linear(m, t, &x, &w, &bias, &act) && (bias || act >= 0);
+  if (!found && !t->evaluated && t->op == RAI_OP_BINARY && t->sub == RAI_BIN_ADD) {
+    for (int side = 0; side < 2 && !found; ++side) {   // linear + r or r + linear
+      Matcher mr;
+      mr.interior.push_back(t);
+      rai_tensor *lin = t->inputs[side], *other = t->inputs[1 - side];
+      if (other->shape != t->shape || other->dtype != t->dtype) continue;
+      if (act_linear(mr, lin, &x, &w, &bias, &act)) { m = mr; res = other; found = true; }
+    }
+  }
+  if (!found || !m.ok) return false;
   c->kind = COMP_LINEAR;
-  c->in[0] = x; c->in[1] = w; c->in[2] = bias;
+  c->in[0] = x; c->in[1] = w; c->in[2] = bias; c->in[3] = res;
+  c->i0 = act;
   c->interior = m.interior;
   return true;
 }
@@ -832,63 +1067,396 @@ bool match_attention(rai_tensor *t, Composite *c) {
   c->in[0] = q; c->in[1] = k; c->in[2] = v;
   c->f0 = scale;
   c->i0 = causal;
+  c->i1 = 1;   // scores and softmax in f32 (phi2.rs:248-251)
   c->interior = m.interior;
   return true;
 }
 
-void plan_compositions(const std::vector<rai_tensor *> &tape, const UseInfo &ui, ComposePlan *plan) {
+// RotaryEmbedding::fwd of qwen2.rs:60-71 / gemma.rs:92-103 on [B, H, S, D]: x * cos + rotate_half(x) * sin over the
+// whole head, the tables narrowed to rows [offset, offset + S) and unsqueezed twice
+bool match_rope_full(rai_tensor *t, Composite *c) {
+  Matcher m;
+  if (!norm_dtype(t->dtype) || t->shape.size() != 4 || m.bin_kind(t) != RAI_BIN_ADD) return false;
+  rai_tensor *p1, *p2, *x, *cb, *rh, *sb;
+  if (!m.bin(t, RAI_BIN_ADD, &p1, &p2) || !m.bin(p1, RAI_BIN_MUL, &x, &cb) || !m.bin(p2, RAI_BIN_MUL, &rh, &sb)) return false;
+  if (x->shape != t->shape || x->dtype != t->dtype) return false;
+  const int64_t D = t->shape[3], S = t->shape[2];
+  if (D % 2) return false;
+  int64_t off_c = 0, off_s = 0, sl = 0, st = 0, len = 0;
+  // The narrowed and unsqueezed tables are shared by the q and the k embedding (one pair per call of
+  // RotaryEmbedding::fwd): they are views that cost no launch and stay ordinary nodes; only the table behind them
+  // and the offset are read here.
+  auto table_behind = [](rai_tensor *n, int64_t *start, int64_t *rows) -> rai_tensor * {
+    while (n && !n->evaluated && n->op == RAI_OP_RESHAPE) n = n->inputs[0];
+    if (!n || n->evaluated || n->op != RAI_OP_NARROW || n->ip[0] != 0) return nullptr;
+    *start = n->ip[1];
+    *rows = n->ip[2];
+    return n->inputs[0];
+  };
+  rai_tensor *cos_t = table_behind(m.strip_bc(cb), &off_c, &sl);
+  if (!cos_t || sl != S) return false;
+  rai_tensor *sin_t = table_behind(m.strip_bc(sb), &off_s, &sl);
+  if (!sin_t || sl != S || off_s != off_c) return false;
+  rai_tensor *rhc = m.node(rh, RAI_OP_CONCATENATE);
+  if (!rhc || rhc->ip[0] != 3 || rhc->inputs.size() != 2) return false;
+  rai_tensor *x2 = m.un(rhc->inputs[0], RAI_UN_NEG);
+  if (!x2 || m.narrow(x2, 3, &st, &len) != x || st != D / 2 || len != D - D / 2) return false;
+  if (m.narrow(rhc->inputs[1], 3, &st, &len) != x || st != 0 || len != D / 2 || !m.ok) return false;
+  if (cos_t->shape.size() != 2 || cos_t->shape[1] != D || sin_t->shape != cos_t->shape || cos_t->dtype != t->dtype ||
+      sin_t->dtype != t->dtype)
+    return false;
+  c->kind = COMP_ROPE;
+  c->in[0] = x; c->in[1] = cos_t; c->in[2] = sin_t;
+  c->i0 = D;
+  c->i1 = off_c;
+  c->interior = m.interior;
+  return true;
+}
+
+// Whether `mask` is the additive causal mask of prepare_decoder_attention_mask (qwen2.rs:306-336, gemma.rs:341-362)
+// for S queries on T keys: f32 [S, S] uploaded from the host with -inf exactly above the diagonal and 0 elsewhere,
+// zeros for the T - S cached positions concatenated in front, broadcast to [B, 1, S, T] and cast to the model dtype.
+// The nodes are shared by all layers and evaluated as they are; this only reads them.
+bool is_additive_causal_mask(const rai_tensor *mask, int64_t S, int64_t T) {
+  const rai_tensor *n = mask;
+  for (int hop = 0; hop < 4 && n && !n->evaluated && (n->op == RAI_OP_BROADCAST || n->op == RAI_OP_TO_DTYPE); ++hop) n = n->inputs[0];
+  if (!n || n->evaluated) return false;
+  if (n->op == RAI_OP_CONCATENATE) {
+    if (n->inputs.size() != 2 || n->ip[0] != 1 || n->shape.size() != 2) return false;
+    const rai_tensor *z = n->inputs[0];
+    if (z->op != RAI_OP_FULL || z->p0 != 0.0 || z->shape.size() != 2 || z->shape[0] != S || z->shape[1] != T - S) return false;
+    n = n->inputs[1];
+  } else if (T != S) {
+    return false;
+  }
+  if (n->op != RAI_OP_FROM_ARRAY || n->dtype != RAI_F32 || n->shape.size() != 2 || n->shape[0] != S || n->shape[1] != S ||
+      (int64_t)n->host.size() != S * S * 4)
+    return false;
+  auto seen = g_causal_masks.find(n->id);   // one mask serves every layer: its bytes are checked once per eval
+  if (seen == g_causal_masks.end()) {
+    const float *v = reinterpret_cast<const float *>(n->host.data());
+    bool is_causal = true;
+    for (int64_t i = 0; i < S && is_causal; ++i)
+      for (int64_t j = 0; j < S; ++j) {
+        const float e = v[i * S + j];
+        if (j > i ? !(std::isinf(e) && e < 0) : e != 0.f) { is_causal = false; break; }
+      }
+    seen = g_causal_masks.emplace(n->id, is_causal).first;
+  }
+  return seen->second;
+}
+
+// Attention::fwd of qwen2.rs:205-221 / gemma.rs:238-254 in the model dtype: softmax(q k^T * scale [+ mask]) v,
+// transposed and reshaped to [B, S, H * D], with repeat_kv (gemma.rs:191-201: unsqueeze, broadcast, reshape) seen
+// through, so that the kernel reads each key / value head once instead of a materialised copy per query head.
+bool match_attention_seq(rai_tensor *t, Composite *c) {
+  Matcher m;
+  if ((t->dtype != RAI_BF16 && t->dtype != RAI_F32 && t->dtype != RAI_F16) || t->shape.size() != 3) return false;
+  rai_tensor *rs = m.node(t, RAI_OP_RESHAPE);
+  rai_tensor *tr = rs ? m.node(rs->inputs[0], RAI_OP_TRANSPOSE) : nullptr;
+  if (!tr || tr->shape.size() != 4 || !((tr->ip[0] == 1 && tr->ip[1] == 2) || (tr->ip[0] == 2 && tr->ip[1] == 1))) return false;
+  rai_tensor *pv = m.node(tr->inputs[0], RAI_OP_MATMUL);
+  if (!pv) return false;
+  rai_tensor *sm = m.node(pv->inputs[0], RAI_OP_SOFTMAX);
+  if (!sm || sm->dtype != t->dtype || sm->ip[0] != 3) return false;
+  rai_tensor *w = sm->inputs[0], *mask = nullptr, *qk_n, *sc;
+  if (m.bin_kind(w) == RAI_BIN_ADD) {
+    rai_tensor *mb;
+    if (!m.bin(w, RAI_BIN_ADD, &w, &mb)) return false;
+    mask = m.strip_bc(mb);
+  }
+  double scale = 0;
+  if (!m.bin(w, RAI_BIN_MUL, &qk_n, &sc) || !m.konst(sc, &scale)) return false;
+  rai_tensor *qk = m.node(qk_n, RAI_OP_MATMUL);
+  if (!qk) return false;
+  rai_tensor *q = qk->inputs[0];
+  rai_tensor *ktn = m.node(qk->inputs[1], RAI_OP_TRANSPOSE);
+  if (!ktn || !((ktn->ip[0] == 2 && ktn->ip[1] == 3) || (ktn->ip[0] == 3 && ktn->ip[1] == 2))) return false;
+  // repeat_kv: reshape [B, Hkv * rep, T, D] of broadcast [B, Hkv, rep, T, D] of reshape [B, Hkv, 1, T, D]
+  auto behind_repeat = [&](rai_tensor *x) -> rai_tensor * {
+    if (x->evaluated || x->op != RAI_OP_RESHAPE || x->shape.size() != 4) return x;
+    rai_tensor *bc = x->inputs[0];
+    if (bc->evaluated || bc->op != RAI_OP_BROADCAST || bc->shape.size() != 5) return x;
+    rai_tensor *us = bc->inputs[0];
+    if (us->evaluated || us->op != RAI_OP_RESHAPE || us->shape.size() != 5 || us->shape[2] != 1) return x;
+    rai_tensor *src = us->inputs[0];
+    if (src->shape.size() != 4 || src->shape[0] != bc->shape[0] || src->shape[1] != bc->shape[1] ||
+        src->shape[2] != bc->shape[3] || src->shape[3] != bc->shape[4] || x->shape[1] != bc->shape[1] * bc->shape[2])
+      return x;
+    m.interior.push_back(x); m.interior.push_back(bc); m.interior.push_back(us);
+    return src;
+  };
+  rai_tensor *k = behind_repeat(ktn->inputs[0]), *v = behind_repeat(pv->inputs[1]);
+  if (!m.ok || q->shape.size() != 4 || k->shape.size() != 4 || v->shape != k->shape) return false;
+  if (q->dtype != t->dtype || k->dtype != t->dtype || v->dtype != t->dtype) return false;
+  const int64_t B = q->shape[0], H = q->shape[1], S = q->shape[2], D = q->shape[3], T = k->shape[2], Hkv = k->shape[1];
+  if (k->shape[0] != B || Hkv < 1 || H % Hkv || k->shape[3] != D || t->shape[0] != B || t->shape[1] != S || t->shape[2] != H * D)
+    return false;
+  int causal = 0;
+  if (mask) {
+    if (S > T || !is_additive_causal_mask(mask, S, T)) return false;
+    causal = 1;
+  }
+  c->kind = COMP_ATTENTION;
+  c->in[0] = q; c->in[1] = k; c->in[2] = v;
+  c->f0 = scale;
+  c->i0 = causal;
+  c->i1 = 0;   // scores in the model dtype
+  c->interior = m.interior;
+  return true;
+}
+
+// A single-token step of Attention::fwd (phi2.rs:202-264, qwen2.rs:166-221, gemma.rs:203-259) whose key / value
+// caches have room to grow in place: rotary embedding of q and of the new k, both cache concatenations and the
+// attention block are one launch of the decode attention kernel, which appends the new rows itself.  The two
+// concatenation nodes are materialised by that launch (Composite::co): they share the old caches' buffers, one row
+// longer.  Taken from the second cached step on (the first one grows the caches, ev_concatenate).
+bool match_rope(rai_tensor *t, Composite *c);
+bool match_rope_full(rai_tensor *t, Composite *c);
+bool match_attention(rai_tensor *t, Composite *c);
+bool match_attention_seq(rai_tensor *t, Composite *c);
+bool match_decode_attention(rai_tensor *t, Composite *c) {
+  Composite at = {}, rq = {}, rk = {};
+  if (!match_attention(t, &at) && !match_attention_seq(t, &at)) return false;
+  rai_tensor *q = at.in[0], *kc = at.in[1], *vc = at.in[2];
+  if (at.i0 != 0 || q->shape[2] != 1 || (t->dtype != RAI_BF16 && t->dtype != RAI_F32)) return false;
+  auto growable = [](const rai_tensor *cat) {
+    if (cat->evaluated || cat->op != RAI_OP_CONCATENATE || cat->inputs.size() != 2 || cat->ip[0] != 2 || cat->shape.size() != 4)
+      return false;
+    const rai_tensor *base = cat->inputs[0], *add = cat->inputs[1];
+    return base->evaluated && base->buf && base->cap_dim == 2 && !base->extended && base->shape[2] + 1 <= base->cap &&
+           add->shape.size() == 4 && add->shape[2] == 1;
+  };
+  if (!growable(kc) || !growable(vc) || kc->inputs[0]->cap != vc->inputs[0]->cap) return false;
+  rai_tensor *knew = kc->inputs[1], *vx = vc->inputs[1];
+  if (!match_rope(q, &rq) && !match_rope_full(q, &rq)) return false;
+  if (!match_rope(knew, &rk) && !match_rope_full(knew, &rk)) return false;
+  const int64_t T = kc->inputs[0]->shape[2];
+  if (rq.in[1] != rk.in[1] || rq.in[2] != rk.in[2] || rq.i0 != rk.i0 || rq.i1 != rk.i1 || rq.i1 != T ||
+      vc->inputs[0]->shape[2] != T)
+    return false;
+  c->kind = COMP_DECODE_ATTN;
+  c->in[0] = rq.in[0]; c->in[1] = rk.in[0]; c->in[2] = vx;          // the new token's q, k, v before the rotary embedding
+  c->in[3] = kc->inputs[0]; c->in[4] = vc->inputs[0];               // the caches so far
+  c->in[5] = rq.in[1]; c->in[6] = rq.in[2];                         // cos / sin tables
+  c->f0 = at.f0;
+  c->i0 = rq.i0;    // rotary dim
+  c->i1 = at.i1;    // f32 scores
+  c->i2 = T;
+  c->co[0] = kc; c->co[1] = vc;
+  c->interior = at.interior;
+  c->interior.insert(c->interior.end(), rq.interior.begin(), rq.interior.end());
+  c->interior.insert(c->interior.end(), rk.interior.begin(), rk.interior.end());
+  return true;
+}
+
+// Arrival counters of the decode attention kernel's context splits: one zeroed buffer per device, grown on demand
+// (every launch leaves them at zero).
+int decode_counters(int dev, size_t bytes, int **out) {
+  static int *buf[16];
+  static size_t have[16];
+  RAI_REQUIRE(dev >= 0 && dev < 16, RAI_ERR_BAD_ARG, "device %d out of range", dev);
+  if (bytes > have[dev]) {
+    void *p = nullptr;
+    RAI_TRY(rai_hip_alloc(dev, bytes, &p));
+    RAI_HIP_TRY(hipMemsetAsync(p, 0, bytes, stream_of(dev)));
+    if (buf[dev]) (void)rai_hip_release(buf[dev]);   // stream order: earlier launches are done with it
+    buf[dev] = (int *)p;
+    have[dev] = bytes;
+  }
+  *out = buf[dev];
+  return RAI_OK;
+}
+
+int run_decode_attention(rai_tensor *t, const Composite &c) {
+  rai_tensor *qx = c.in[0], *kx = c.in[1], *vx = c.in[2], *kb = c.in[3], *vb = c.in[4];
+  const int64_t B = qx->shape[0], Hq = qx->shape[1], D = qx->shape[3], Hkv = kb->shape[1], T = c.i2, cap = kb->cap;
+  auto rows_ok = [&](const rai_tensor *x, int64_t H) {   // [B, H, 1, D] with the heads of a sequence side by side
+    const rai_hip_tensor &v = x->view;
+    return v.rank == 4 && v.shape[0] == B && v.shape[1] == H && v.shape[2] == 1 && v.shape[3] == D && v.stride[3] == 1 &&
+           (H == 1 || v.stride[1] == D) && (uintptr_t)base_ptr(&v) % 16 == 0 && (B == 1 || v.stride[0] % 8 == 0);
+  };
+  auto cache_ok = [&](const rai_tensor *x) {   // [B, Hkv, T, D] laid out for `cap` rows per head
+    const rai_hip_tensor &v = x->view;
+    return v.rank == 4 && v.shape[0] == B && v.shape[1] == Hkv && v.shape[2] == T && v.shape[3] == D && v.stride[3] == 1 &&
+           v.stride[2] == D && v.stride[1] == cap * D && (B == 1 || v.stride[0] == Hkv * cap * D) &&
+           (uintptr_t)base_ptr(&v) % 16 == 0;
+  };
+  RAI_REQUIRE(rows_ok(qx, Hq) && rows_ok(kx, Hkv) && rows_ok(vx, Hkv) && cache_ok(kb) && cache_ok(vb) && D % 8 == 0,
+              RAI_ERR_BAD_STRIDE, "decode attention: operand layout not served");
+  const rai_hip_tensor &ct = c.in[5]->view, &sn = c.in[6]->view;
+  RAI_REQUIRE(is_contiguous(&ct) && is_contiguous(&sn) && ct.rank == 2 && ct.shape[1] == c.i0 && T < ct.shape[0] &&
+                  ct.dtype == t->dtype && sn.dtype == t->dtype,
+              RAI_ERR_BAD_STRIDE, "decode attention: rotary tables not served");
+  hipStream_t st = stream_of(t->dev);
+  if (!st) return RAI_ERR_HIP;
+  void *ws = nullptr;
+  int *counters = nullptr;
+  RAI_TRY(decode_counters(t->dev, attention_decode_counter_bytes((int)B, (int)Hq), &counters));
+  RAI_TRY(rai_hip_alloc(t->dev, attention_decode_ws_bytes((int)B, (int)Hq, (int)D), &ws));
+  RAI_TRY(alloc_output(t));
+  AttnDecodeArgs a;
+  memset(&a, 0, sizeof(a));
+  a.qkv = base_ptr(&qx->view);
+  a.k_new = base_ptr(&kx->view);
+  a.v_new = base_ptr(&vx->view);
+  a.q_row_stride = qx->view.stride[0]; a.k_row_stride = kx->view.stride[0]; a.v_row_stride = vx->view.stride[0];
+  a.kcache = base_ptr(&kb->view);
+  a.vcache = base_ptr(&vb->view);
+  a.out = t->view.data;
+  a.out_row_stride = Hq * D;
+  a.cos_t = base_ptr(&ct); a.sin_t = base_ptr(&sn);
+  a.pos_dev = nullptr;
+  a.pos_host = (int)T;
+  a.rot = (int)c.i0;
+  a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.D = (int)D; a.Tmax = (int)cap;
+  a.scale = (float)c.f0;
+  a.f32_scores = (int)c.i1;
+  a.dtype = t->dtype;
+  a.ws = (float *)ws;
+  a.counters = counters;
+  const int rc = launch_attention_decode(st, a);
+  (void)rai_hip_release(ws);   // stream order keeps it intact until the launch is through
+  RAI_TRY(rc);
+  // the caches, one row longer, in the old caches' buffers
+  for (int i = 0; i < 2; ++i) {
+    rai_tensor *cat = c.co[i], *base = cat->inputs[0];
+    rai_hip_tensor v = base->view;
+    v.shape[2] = T + 1;
+    alias_storage(cat, base, v);
+    cat->cap_dim = 2;
+    cat->cap = base->cap;
+    base->extended = true;
+    cat->evaluated = true;
+    ++g_stats.nodes_evaluated;
+  }
+  return RAI_OK;
+}
+
+// Compositions found in the tape: g_comps[t->comp] for a root t (flag kRoot), interior nodes carry kAbsorbed.
+std::vector<Composite> g_comps;
+
+// Registers composition c with root t when it is sealed: every interior node is pending, claimed by nobody else, has
+// a rule (fusing never hides a missing rule), is referenced only by edges of the tape, and all of those edges come
+// from inside the composition; operands are not interior; co-outputs are read, inside the tape, by the composition
+// only.
+bool claim(rai_tensor *t, Composite &c, rai_tensor *stands_for_root = nullptr) {
+  const uint64_t stamp = ++g_stamp;
+  // a node whose recorded use of the interior the root takes over (the regrouped sum below): counts as the root
+  // where users are checked, and may be an operand
+  if (stands_for_root) stands_for_root->stamp = stamp;
+  for (int i = 0; i < 2; ++i)
+    if (c.co[i]) c.co[i]->stamp = stamp;   // inside for the purpose of "who uses this node", yet materialised
+  // interior = everything the matcher walked through except the root itself (the same node may have been reached
+  // twice): stamped so that "inside" is one comparison
+  std::vector<rai_tensor *> interior;
+  for (rai_tensor *n : c.interior)
+    if (n != t && n->stamp != stamp) { n->stamp = stamp; interior.push_back(n); }
+  auto users_inside = [&](const rai_tensor *n) {
+    for (int u = 0; u < n->n_users; ++u) {
+      const rai_tensor *usr = g_users[n->users_at + u];
+      if (usr != t && usr->stamp != stamp) return false;
+    }
+    return true;
+  };
+  for (rai_tensor *n : interior)   // evaluated constants are operands, not interior
+    if (n->evaluated || !in_tape(n) || (n->flags & (kAbsorbed | kRoot | kCoOutput)) || !g_rules[n->op] ||
+        n->refs != n->n_users || !users_inside(n))
+      return false;
+  for (int i = 0; i < 7; ++i)
+    if (c.in[i] && c.in[i] != stands_for_root && c.in[i]->stamp == stamp) return false;   // an operand must be materialised
+  for (int i = 0; i < 2; ++i) {
+    rai_tensor *n = c.co[i];
+    if (n && (n->evaluated || !in_tape(n) || (n->flags & (kAbsorbed | kRoot | kCoOutput)) || !g_rules[n->op] || !users_inside(n)))
+      return false;
+  }
+  c.interior = interior;
+  for (rai_tensor *n : interior) n->flags |= kAbsorbed;
+  for (int i = 0; i < 2; ++i)
+    if (c.co[i]) c.co[i]->flags |= kCoOutput;
+  t->flags |= kRoot;
+  t->comp = (int)g_comps.size();
+  g_comps.push_back(c);
+  return true;
+}
+
+// DecoderLayer::fwd of phi2.rs:298 sums two Linear outputs and the layer's input: (attn + mlp) + x.  One Linear
+// launch takes one added tensor, so the sums are regrouped as attn + (mlp + x): the inner sum node, which nothing
+// else can observe, receives mlp's Linear with x added, the outer one attn's Linear with that added.  Two launches
+// instead of three (and of four without any composition); the result differs from the recorded grouping by
+// rounding only, like every composed result.
+bool claim_two_linears_and_residual(rai_tensor *t) {
+  if (t->evaluated || t->op != RAI_OP_BINARY || t->sub != RAI_BIN_ADD || (t->dtype != RAI_BF16 && t->dtype != RAI_F32)) return false;
+  for (int side = 0; side < 2; ++side) {
+    rai_tensor *sum = t->inputs[side], *x = t->inputs[1 - side];
+    if (sum->evaluated || !in_tape(sum) || sum->op != RAI_OP_BINARY || sum->sub != RAI_BIN_ADD || sum->refs != 1 ||
+        sum->n_users != 1 || (sum->flags & (kAbsorbed | kRoot | kCoOutput | kOutput)) || x->shape != t->shape ||
+        x->dtype != t->dtype || sum->shape != t->shape)
+      continue;
+    if (!x->evaluated && !(in_tape(x) && x->tape_idx < sum->tape_idx)) continue;   // x must be there when `sum` runs
+    Composite outer = {}, inner = {};
+    Matcher mp, mq;
+    int act_p = -1, act_q = -1;
+    mp.interior.push_back(t);
+    mq.interior.push_back(sum);
+    if (!act_linear(mp, sum->inputs[0], &outer.in[0], &outer.in[1], &outer.in[2], &act_p) || !mp.ok) continue;
+    if (!act_linear(mq, sum->inputs[1], &inner.in[0], &inner.in[1], &inner.in[2], &act_q) || !mq.ok) continue;
+    inner.kind = outer.kind = COMP_LINEAR;
+    inner.in[3] = x;   inner.i0 = act_q; inner.interior = mq.interior;
+    outer.in[3] = sum; outer.i0 = act_p; outer.interior = mp.interior;
+    // the inner composition first: if the outer one then fails, the inner one stands by itself as "Linear + x" with
+    // `sum` as its root, which would change what `sum` means: so the outer one is checked (not registered) first
+    Composite probe = outer;
+    const size_t before = g_comps.size();
+    if (!claim(t, probe, sum)) continue;
+    if (!claim(sum, inner)) {   // undo the outer claim
+      for (rai_tensor *n : g_comps.back().interior) n->flags &= ~kAbsorbed;
+      t->flags &= ~kRoot;
+      t->comp = -1;
+      g_comps.resize(before);
+      continue;
+    }
+    return true;
+  }
+  return false;
+}
+
+void plan_compositions(const std::vector<rai_tensor *> &tape) {
   typedef bool (*match_fn)(rai_tensor *, Composite *);
-  static const match_fn kMatchers[] = {match_layer_norm, match_rms_norm, match_linear, match_rope, match_attention};
-  std::unordered_set<uint64_t> in_tape;
-  for (const rai_tensor *t : tape) in_tape.insert(t->id);
+  static const match_fn kMatchers[] = {match_layer_norm, match_rms_norm,  match_gemma_rms_norm,   match_linear,   match_rope,
+                                       match_rope_full,  match_decode_attention, match_attention, match_attention_seq};
   g_causal_masks.clear();
-  for (rai_tensor *t : tape) {
-    if (plan->absorbed.count(t->id)) continue;
+  g_comps.clear();
+  // consumers before producers: the widest composition around a node (a Linear with its activation and residual)
+  // claims it before a narrower one (the Linear alone) is tried
+  for (size_t ti = tape.size(); ti-- > 0;) {
+    rai_tensor *t = tape[ti];
+    if ((t->flags & (kAbsorbed | kRoot | kCoOutput)) || !g_rules[t->op]) continue;
+    // cheap gate: every composition's root is one of these primitives
+    if (t->op != RAI_OP_BINARY && t->op != RAI_OP_RESHAPE && t->op != RAI_OP_CONCATENATE) continue;
+    if (claim_two_linears_and_residual(t)) continue;
     for (match_fn f : kMatchers) {
       Composite c = {};
-      if (!f(t, &c)) continue;
-      // interior = everything the matcher walked through except the root itself (the same node may have been
-      // reached twice)
-      std::unordered_set<uint64_t> inside;
-      std::vector<rai_tensor *> interior;
-      for (rai_tensor *n : c.interior)
-        if (n != t && inside.insert(n->id).second) interior.push_back(n);
-      bool sealed = true;
-      for (rai_tensor *n : interior) {
-        auto u = ui.users.find(n->id);
-        const size_t n_users = u == ui.users.end() ? 0 : u->second.size();
-        // evaluated constants are operands, not interior; everything else must be pending, claimed by nobody else,
-        // have a rule (fusing never hides a missing rule), and be referenced only by edges from inside
-        if (n->evaluated || !in_tape.count(n->id) || plan->absorbed.count(n->id) || plan->roots.count(n->id) ||
-            !g_rules[n->op] || (size_t)n->refs != n_users) { sealed = false; break; }
-        for (const rai_tensor *usr : u->second)
-          if (usr != t && !inside.count(usr->id)) { sealed = false; break; }
-        if (!sealed) break;
-      }
-      for (int i = 0; i < 5 && sealed; ++i)
-        if (c.in[i] && inside.count(c.in[i]->id)) sealed = false;   // an operand must be materialised
-      if (!sealed || !g_rules[t->op]) continue;
-      c.interior = interior;
-      for (rai_tensor *n : interior) plan->absorbed.insert(n->id);
-      plan->roots[t->id] = c;
-      break;
+      if (f(t, &c) && claim(t, c)) break;
     }
   }
 }
 
 int run_composite(rai_tensor *t, const Composite &c) {
+  if (c.kind == COMP_DECODE_ATTN) return run_decode_attention(t, c);
   RAI_TRY(alloc_output(t));
   switch (c.kind) {
     case COMP_LINEAR:
-      return rai_hip_linear(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, -1, nullptr, &t->view);
+      return rai_hip_linear(t->dev, &c.in[0]->view, &c.in[1]->view, c.in[2] ? &c.in[2]->view : nullptr, (int32_t)c.i0,
+                            c.in[3] ? &c.in[3]->view : nullptr, &t->view);
     case COMP_LAYER_NORM:
       return rai_hip_layer_norm(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, c.f0, &t->view);
     case COMP_RMS_NORM:
-      return rai_hip_rms_norm(t->dev, &c.in[0]->view, &c.in[1]->view, c.f0, 0, &t->view);
+      return rai_hip_rms_norm(t->dev, &c.in[0]->view, &c.in[1]->view, c.f0, (int32_t)c.i2, &t->view);
     case COMP_ROPE:
       return rai_hip_rope(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, (int32_t)c.i0, c.i1, &t->view);
     case COMP_ATTENTION:
-      return rai_hip_attention(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, c.f0, (int32_t)c.i0, 1, &t->view);
+      return rai_hip_attention(t->dev, &c.in[0]->view, &c.in[1]->view, &c.in[2]->view, c.f0, (int32_t)c.i0, (int32_t)c.i1, &t->view);
     default:
       return fail(RAI_ERR_BAD_ARG, "unknown composition %d", c.kind);
   }
@@ -1279,44 +1847,42 @@ int rai_graph_eval_order(rai_tensor *const *outputs, int32_t n, uint64_t *ids, i
 int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
   RAI_REQUIRE(outputs && n >= 0, RAI_ERR_BAD_ARG, "null argument");
   init_rules();
+  const auto t_start = std::chrono::steady_clock::now();
   std::vector<rai_tensor *> tape;
   RAI_TRY(topo_sort(outputs, n, &tape));
-  ComposePlan comp;
-  std::unordered_set<uint64_t> composed;   // roots and interiors: the elementwise pass leaves them alone
-  if (g_compose) {
-    UseInfo ui;
-    for (const rai_tensor *t : tape)
-      for (const rai_tensor *in : t->inputs) ui.users[in->id].push_back(t);
-    plan_compositions(tape, ui, &comp);
-    composed = comp.absorbed;
-    for (const auto &r : comp.roots) composed.insert(r.first);
-  }
-  FusionPlan plan;
-  if (g_fusion) plan_fusion(tape, outputs, n, &plan, composed);
+  for (int i = 0; i < n; ++i)
+    if (in_tape(outputs[i])) outputs[i]->flags |= kOutput;
+  index_users(tape);
+  g_comps.clear();
+  if (g_compose) plan_compositions(tape);
+  if (g_fusion) plan_fusion(tape);
+  const auto t_planned = std::chrono::steady_clock::now();
+  g_stats.plan_ns += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(t_planned - t_start).count();
+  int rc = RAI_OK;
   for (rai_tensor *t : tape) {
-    if (t->evaluated || plan.inlined.count(t->id) || comp.absorbed.count(t->id)) continue;
+    if (t->evaluated || (t->flags & (kInlined | kAbsorbed | kCoOutput))) continue;   // a co-output comes with its root
     rule_fn rule = g_rules[t->op];
-    RAI_REQUIRE(rule, RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op));
+    if (!rule) { rc = fail(RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op)); break; }
     int st = RAI_ERR_UNSUPPORTED;
-    auto cr = comp.roots.find(t->id);
-    if (cr != comp.roots.end()) {
-      st = run_composite(t, cr->second);
+    if (t->flags & kRoot) {
+      const Composite &c = g_comps[t->comp];
+      st = run_composite(t, c);
       if (st == RAI_OK) {
         ++g_stats.kernel_launches;
         ++g_stats.composed_regions;
-        g_stats.composed_nodes += cr->second.interior.size() + 1;
+        g_stats.composed_nodes += c.interior.size() + 1;
       } else if (st == RAI_ERR_BAD_STRIDE || st == RAI_ERR_UNSUPPORTED || st == RAI_ERR_BAD_SHAPE || st == RAI_ERR_BAD_DTYPE) {
         // the fused launcher declines these operands: evaluate the recorded nodes one by one instead
         drop_storage(t);
         st = eval_pending_inputs(t);
         if (st == RAI_OK) st = rule(t);
       }
-    } else if (elementwise(t) && has_inlined_input(t, plan)) {
+    } else if (elementwise(t) && has_inlined_input(t)) {
       // the rules of the inlined members must exist too: fusion never hides a missing rule
-      st = eval_region(t, plan);
+      st = eval_region(t);
       if (st == RAI_ERR_UNSUPPORTED) {  // region too large for one program: evaluate its members one by one
         drop_storage(t);
-        st = eval_inputs_plain(t, plan);
+        st = eval_inputs_plain(t);
         if (st == RAI_OK) st = rule(t);
       }
     } else {
@@ -1324,15 +1890,17 @@ int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
     }
     if (st != RAI_OK) {
       drop_storage(t);
-      return st;
+      rc = st;
+      break;
     }
     t->evaluated = true;
     ++g_stats.nodes_evaluated;
   }
-  if (!retain_graph)
+  if (rc == RAI_OK && !retain_graph)
     for (rai_tensor *t : tape)
       if (t->evaluated) detach(t);
-  return RAI_OK;
+  g_stats.run_ns += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t_planned).count();
+  return rc;
 }
 
 int rai_tensor_to_host(rai_tensor *t, void *dst, size_t bytes) {

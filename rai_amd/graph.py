@@ -38,6 +38,13 @@ def _shape_arr(shape):
     return (C.c_int64 * max(len(shape), 1))(*shape), len(shape)
 
 
+class F64Scalar:
+    """An f64 scalar operand (`x * 0.5f64` in the reference): becomes Full<f64> + ToDType, not Full<f32>."""
+
+    def __init__(self, value):
+        self.value = float(value)
+
+
 class Tensor:
     """Handle of one graph node (a new reference; released with the Python object)."""
 
@@ -162,13 +169,18 @@ class Tensor:
     def powf(self, e): return self._unary("powf", e)
     def __neg__(self): return self.neg()
 
-    def full_like(self, value):
-        """Full<f32> of this shape, cast to this dtype when it differs (full.rs:85-92)."""
-        c = Tensor.full(value, self.shape, "f32")
-        return c if self.dtype == "f32" else c.to_dtype(self.dtype)
+    def full_like(self, value, scalar_dtype="f32"):
+        """Full<T> of this shape for a scalar of Rust type T (f32 or f64), cast to this dtype when it differs
+        (full.rs:85-92)."""
+        c = Tensor.full(value, self.shape, scalar_dtype)
+        return c if self.dtype == scalar_dtype else c.to_dtype(self.dtype)
 
     def _binary(self, name, other, swap=False):
-        o = other if isinstance(other, Tensor) else self.full_like(other)
+        # a bare Python float stands for an f32 scalar; F64(x) marks the f64 scalars of the reference's model code
+        if isinstance(other, F64Scalar):
+            o = self.full_like(other.value, "f64")
+        else:
+            o = other if isinstance(other, Tensor) else self.full_like(other)
         a, b = (o, self) if swap else (self, o)
         return Tensor(_lib.load().rai_binary(BINARY[name], a._h, b._h))
 
@@ -331,7 +343,8 @@ def stats(reset=False):
     check(_lib.load().rai_graph_get_stats(C.byref(s), int(reset)))
     return {"nodes_evaluated": s.nodes_evaluated, "kernel_launches": s.kernel_launches,
             "fused_regions": s.fused_regions, "fused_nodes": s.fused_nodes,
-            "composed_regions": s.composed_regions, "composed_nodes": s.composed_nodes}
+            "composed_regions": s.composed_regions, "composed_nodes": s.composed_nodes,
+            "plan_ms": s.plan_ns * 1e-6, "run_ms": s.run_ns * 1e-6}
 
 
 def dispatch_unregister(op):
