@@ -109,6 +109,13 @@ uint64_t rai_tensor_id(const rai_tensor *t);
 const char *rai_tensor_error(const rai_tensor *t);
 /* View of the evaluated storage (fails with RAI_ERR_BAD_ARG if not evaluated). */
 int rai_tensor_storage(const rai_tensor *t, rai_hip_tensor *out);
+/* The two ends of a bridge from a front end that keeps tensor objects of its own (rai-core's Tensor with HipData in
+ * its data slot, tensor.rs:28-37,151-165): rai_from_storage wraps data that already exists as an evaluated node (a
+ * view into `buf`, an allocation of rai_hip_alloc, which the node retains and releases with itself), and
+ * rai_tensor_buffer hands out the allocation an evaluated node's view points into (NULL if not evaluated; the
+ * caller retains it with rai_hip_retain if it keeps it). */
+rai_tensor *rai_from_storage(const rai_hip_tensor *view, void *buf, int32_t dev);
+void *rai_tensor_buffer(const rai_tensor *t);
 
 /* ---- evaluation (eval.rs:31-51).  Returns RAI_OK, RAI_ERR_UNSUPPORTED for a
  * (device, op) pair without a rule (Error::Unimplemented), RAI_ERR_BAD_SHAPE when

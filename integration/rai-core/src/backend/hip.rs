@@ -85,7 +85,7 @@ pub fn hip_if_available(id: usize) -> Box<dyn Device> {
 }
 
 // ------------------------------------------------------------------------------------------------ dtypes
-fn dtype_code(dt: &dyn DType) -> i32 {
+pub(crate) fn dtype_code(dt: &dyn DType) -> i32 {
     let any = dt.as_any();
     if any.is::<U8>() {
         RAI_U8
@@ -206,6 +206,19 @@ impl HipData {
             check(unsafe { rai_hip_h2d(dev, out.buf, bytes.as_ptr() as *const c_void, bytes.len()) });
         }
         out
+    }
+
+    /// Storage that the library's graph evaluator produced (backend/hip_graph.rs): `desc` is a view into `buf`, an
+    /// allocation of rai_hip_alloc, which this handle retains.
+    pub(crate) fn adopt(dev: c_int, buf: *mut c_void, desc: RaiHipTensor) -> Self {
+        check(unsafe { rai_hip_retain(buf) });
+        let shape = desc.shape[..desc.rank as usize].iter().map(|&d| d as usize).collect();
+        Self { dev, buf, desc, shape }
+    }
+
+    /// The allocation the view points into.
+    pub(crate) fn buffer(&self) -> *mut c_void {
+        self.buf
     }
 
     /// Another view of the same allocation.

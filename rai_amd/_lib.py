@@ -189,6 +189,8 @@ GRAPH_PROTOTYPES = {
     "rai_tensor_id": (C.c_uint64, [_T]),
     "rai_tensor_error": (C.c_char_p, [_T]),
     "rai_tensor_storage": (C.c_int, [_T, _TP]),
+    "rai_from_storage": (_T, [_TP, _vp, _i32]),
+    "rai_tensor_buffer": (_vp, [_T]),
     "rai_eval": (C.c_int, [C.POINTER(_T), _i32, _i32]),
     "rai_graph_eval_order": (C.c_int, [C.POINTER(_T), _i32, C.POINTER(C.c_uint64), _i32, _I32P]),
     "rai_tensor_to_host": (C.c_int, [_T, _vp, C.c_size_t]),

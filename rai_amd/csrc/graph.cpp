@@ -1835,6 +1835,19 @@ int rai_tensor_storage(const rai_tensor *t, rai_hip_tensor *out) {
 }
 
 // ------------------------------------------------------------------ evaluation
+rai_tensor *rai_from_storage(const rai_hip_tensor *view, void *buf, int32_t dev) {
+  if (!view || !buf || view->rank < 0 || view->rank > RAI_HIP_MAX_RANK || dtype_size(view->dtype) == 0) return nullptr;
+  std::vector<int64_t> shape(view->shape, view->shape + view->rank);
+  rai_tensor *t = new_node(dev, view->dtype, shape, RAI_OP_FROM_ARRAY, {});
+  if (rai_hip_retain(buf) != RAI_OK) { rai_tensor_release(t); return nullptr; }
+  t->view = *view;
+  t->buf = buf;
+  t->evaluated = true;
+  return t;
+}
+
+void *rai_tensor_buffer(const rai_tensor *t) { return t && t->evaluated ? t->buf : nullptr; }
+
 int rai_graph_eval_order(rai_tensor *const *outputs, int32_t n, uint64_t *ids, int32_t capacity, int32_t *count) {
   RAI_REQUIRE(outputs && count && n >= 0, RAI_ERR_BAD_ARG, "null argument");
   std::vector<rai_tensor *> tape;

@@ -87,6 +87,16 @@ class Tensor:
         arr, rank = _shape_arr(a.shape)
         return Tensor(_lib.load().rai_from_array(a.ctypes.data_as(C.c_void_p), dt, arr, rank, dev))
 
+    @staticmethod
+    def from_storage(desc, buf, dev=0):
+        """An already evaluated node over existing device storage: `desc` a TensorDesc view into `buf`, an allocation
+        of rai_hip_alloc (what a front end with tensor objects of its own hands over; the node retains `buf`)."""
+        return Tensor(_lib.load().rai_from_storage(C.byref(desc), buf, dev))
+
+    def buffer(self):
+        """The allocation an evaluated node's view points into (None before evaluation)."""
+        return _lib.load().rai_tensor_buffer(self._h)
+
     # ------------------------------------------------------------ metadata
     @property
     def shape(self):

@@ -476,3 +476,26 @@ def test_qwen2_and_gemma_through_the_graph(hip, arch, dt):
                 assert st["composed_regions"] == 0
             ids = np.argmax(want, -1).astype(np.uint32).reshape(2, 1)
     g.set_compose(True)
+
+
+def test_storage_crosses_the_boundary_both_ways(hip):
+    # what the Rust bridge does per tape: operands that have data come in as views of their allocations, results go
+    # back out as (view, allocation) pairs that outlive the nodes
+    rng = np.random.default_rng(24)
+    x, w = rand(rng, (4, 6), "f32"), rand(rng, (5, 6), "f32")
+    a = dev(x, "f32").eval()
+    leaf = Tensor.from_storage(a.storage(), a.buffer())
+    assert leaf.is_evaluated() and leaf.shape == (4, 6) and leaf.num_inputs() == 0
+    view = Tensor.from_storage(a.t().eval().storage(), a.buffer())        # a strided view of the same allocation
+    assert view.shape == (6, 4)
+    out = (g.linear(leaf, dev(w, "f32")) * 2.0).eval()
+    desc, buf = out.storage(), out.buffer()
+    assert buf and desc.rank == 2
+    from rai_amd import _lib
+    _lib.call("rai_hip_retain", buf)          # the front end's handle on the result
+    del out, leaf
+    again = Tensor.from_storage(desc, buf)    # still valid after the nodes are gone
+    assert_close(from_storage(again.as_storage(), "f32"), oo.mul(onn.linear(x, w, None, "f32"), np.float32(2.0), "f32"), "f32", "round trip")
+    assert np.array_equal(view.as_storage(), to_storage(x.T.copy(), "f32"))
+    del again
+    _lib.call("rai_hip_release", buf)

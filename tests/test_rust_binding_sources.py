@@ -56,3 +56,24 @@ def test_every_reference_op_is_implemented_or_named_as_unregistered():
             assert op in implemented, f"no impl Eval<Hip, ops::{op}>"
             assert op in registered, f"ops::{op} is implemented but not registered"
     assert implemented - set(REFERENCE_OPS) - {"X"} == set(), implemented - set(REFERENCE_OPS)   # "ops::X" in the prose
+
+
+def test_graph_bridge_mirrors_every_builder_and_every_registered_op():
+    """backend/hip_graph.rs hands a whole tape to the library's evaluator: every node builder of include/rai_graph.h
+    has a caller there, every primitive that hip.rs registers is mirrored (ToDevice excepted: a tape that crosses
+    devices is left to the per-node loop), and the two storage calls of the bridge are used."""
+    header = re.sub(r"/\*.*?\*/", "", (ROOT / "include" / "rai_graph.h").read_text(), flags=re.S)
+    builders = set(re.findall(r"^rai_tensor \*\s*(rai_\w+)\s*\(", header, flags=re.M))
+    assert len(builders) >= 25
+    src = (RS / "hip_graph.rs").read_text()
+    missing = sorted(b for b in builders - {"rai_to_device"} if not re.search(rf"\b{b}\b", src))
+    assert not missing, f"hip_graph.rs never calls {missing}"
+    for call in ("rai_eval", "rai_tensor_storage", "rai_tensor_buffer", "rai_from_storage", "set_data", "strong_count"):
+        assert call in src, call
+    for op in REFERENCE_OPS:
+        if op in NO_KERNEL or op == "ToDevice":
+            continue
+        assert re.search(rf"\b{op}\b", src), f"hip_graph.rs does not mirror ops::{op}"
+    sys_rs = (RS / "hip_graph_sys.rs").read_text()
+    for b in builders | {"rai_eval", "rai_tensor_buffer", "rai_from_storage"}:
+        assert f"pub fn {b}(" in sys_rs, b
