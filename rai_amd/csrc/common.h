@@ -51,7 +51,7 @@ int device_cu_count(int dev);
 // non-zero code into RAI_ERR_HIP, clears it and resets the counters those kernels share.
 int *kernel_fault_word(int dev);
 int check_kernel_fault(int dev);
-enum { RAI_FAULT_STREAMK = 1 };
+enum { RAI_FAULT_STREAMK = 1, RAI_FAULT_CHAIN = 2 };
 // Zeroes the stream-K tile kernel's arrival counters on `st` (gemm_mfma.hip).
 int streamk_counters_reset(int dev, hipStream_t st);
 // Looks up this device's address of the fixed scratch array of the allocation-free argmax (reduce.hip); called once

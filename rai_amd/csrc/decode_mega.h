@@ -14,6 +14,10 @@ struct DevState {
   int done;   // blocks of the token-selection kernel that have finished (reset by the last one)
   int fault;  // set by a packet poll that timed out; checked by the host after a generate call
   unsigned epoch;  // launches of the persistent decode kernel so far: makes its exchange tags unique
+  // Arrival flags of the decode chain kernel's barriers (decode_chain.h), one per block: a block announces barrier
+  // number n of the decoder's life by storing n, and n only grows (epoch * 4096 + launch * 8 + phase), so nothing is
+  // ever reset.
+  unsigned long long chain_flags[512];
 };
 
 struct MegaLayer {

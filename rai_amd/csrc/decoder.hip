@@ -20,6 +20,7 @@
 #include <vector>
 
 #include "attention.h"
+#include "decode_chain.h"
 #include "decode_mega.h"
 #include "gemm.h"
 
@@ -978,6 +979,12 @@ static float seq_attn_scale(const rai_hip_decoder *d) {
   return (float)(1.0 / sqrt((double)d->D));
 }
 
+// RAI_HIP_CHAIN=1 opts in to the persistent decode chain kernel (read per call: the tests switch it)
+static bool chain_wanted() {
+  const char *e = getenv("RAI_HIP_CHAIN");
+  return e && e[0] == '1';
+}
+
 // Sequential pre-norm block of Qwen2 (qwen2.rs:253-266) and Gemma (gemma.rs:286-299):
 // x1 = x + o_proj(attn(norm1(x))); x = x1 + down(act(gate(norm2(x1))) * up(norm2(x1))).
 static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool from_tokens = false) {
@@ -1004,9 +1011,28 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     return rai_hip_rms_norm(d->dev, &tx, &tw, d->cfg.norm_eps, kind == 2, &to);
   };
   char *x = d->x, *x1 = d->x2;
+  // Batched decode steps (9..32 rows): with RAI_HIP_CHAIN=1 everything between two attention calls -- o_proj,
+  // gate|up, down and the next layer's q|k|v -- runs as one persistent launch of the decode chain kernel instead of
+  // five launches (four Linears and the sum of the down projection's K splits).  Off by default: on the Gemma-2B
+  // widths at batch 32 the chain launch takes 115 us a layer against 85 us for the five launches it replaces (its
+  // four grid barriers and the reads past the L2s of what the phase before wrote cost more than the launch
+  // boundaries they stand for, and the phase dispatch inside one kernel spills registers).
+  const int down_splits = (I + 2047) / 2048;
+  bool chain = S == 1 && frag && fuse_norm && M <= 32 && chain_wanted() && decode_chain_serves((int)M, H, QD, false) &&
+               decode_chain_serves((int)M, 2 * I, H, false) && decode_chain_serves((int)M, H, I, true) &&
+               decode_chain_serves((int)M, ldq, H, false) && ldq % 8 == 0 &&
+               (size_t)down_splits * M * H * sizeof(float) <= d->splitk_ws_bytes && !d->want_hidden;
+  for (int l = 0; chain && l < d->L; ++l) {
+    const Layer &ly = d->layers[l];
+    chain = ly.Wo_f && ly.Wgu_f && ly.Wdown_f && ly.Wqkv_f;
+  }
+  chain = chain && d->num_cu == device_cu_count(d->dev) && d->num_cu <= 512 && d->L <= 512;
   for (int l = 0; l < d->L; ++l) {
     const Layer &ly = d->layers[l];
     LinearArgs a = linear_args_default();
+    if (chain && l > 0) {
+      // this layer's q|k|v was the last phase of the previous layer's chain
+    } else {
     if (fuse_norm) {
       a.A = x; a.lda = H;
       a.ln_kind = kind; a.ln_w = ly.n1_w; a.ln_eps = (float)d->cfg.norm_eps;
@@ -1020,6 +1046,7 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
     a.M = (int)M; a.N = ldq; a.K = H; a.n_split = ldq;
     a.splitk_ws = d->splitk_ws; a.splitk_ws_bytes = d->splitk_ws_bytes;
     RAI_TRY(linear(d, st, a));
+    }
 
     if (S == 1) {
       AttnDecodeArgs t;
@@ -1055,6 +1082,63 @@ static int forward_seq(rai_hip_decoder *d, int B, int S, bool advance_step, bool
       t.causal = 1; t.f32_scores = 0; t.dtype = dt;
       t.T = T_after;
       RAI_TRY(launch_attention(st, t));
+    }
+
+    if (chain) {
+      ChainArgs c;
+      memset(&c, 0, sizeof(c));
+      auto lin = [&](ChainPhase &p, const void *A, int64_t lda, bool a_fresh, const void *Wf, int N, int K, void *out, int64_t ldo) {
+        p.kind = RAI_CHAIN_LINEAR;
+        p.A = A; p.lda = lda; p.a_fresh = a_fresh;
+        p.Wfrag = Wf;
+        p.out = out; p.ldo = ldo;
+        p.M = (int)M; p.N = N; p.K = K;
+        p.splits = 1;
+        p.KS = K <= 2048 ? K / 256 : 8;
+        p.act = -1; p.ln_kind = -1;
+        const int tiles = (N + 15) / 16;
+        p.G = tiles >= 4 * d->num_cu ? 4 : 1;
+      };
+      // Every buffer a phase writes is touched with device-scope accesses only for the whole launch (x too, which
+      // phase 0 reads as its residual and phase 3 rewrites): an ordinary load would leave a line in this XCD's L2
+      // that a later phase could read stale.
+      ChainPhase &po = c.ph[0];                       // x1 = x + attn . Wo^T (+ bo)
+      lin(po, d->attn, QD, false, ly.Wo_f, H, QD, x1, H);
+      po.bias = ly.bo; po.residual = x; po.ldr = H; po.res_fresh = 1;
+      ChainPhase &pg = c.ph[1];                       // glu = act(gate(norm2(x1))) * up(norm2(x1))
+      lin(pg, x1, H, true, ly.Wgu_f, 2 * I, H, d->glu, I);
+      pg.ln_kind = kind; pg.ln_w = ly.n2_w; pg.ln_eps = (float)d->cfg.norm_eps;
+      pg.act = d->cfg.hidden_act; pg.glu = 1;
+      ChainPhase &pd = c.ph[2];                       // partial products of down over spans of 2048 of K
+      lin(pd, d->glu, I, true, ly.Wdown_f, H, I, x, H);
+      pd.splits = down_splits; pd.partial = (float *)d->splitk_ws;
+      pd.G = (H / 16) >= 4 * (d->num_cu / down_splits) ? 4 : 1;
+      ChainPhase &ps = c.ph[3];                       // x = x1 + sum of the partial products
+      ps.kind = RAI_CHAIN_SUM;
+      ps.partial = (float *)d->splitk_ws; ps.splits = down_splits;
+      ps.residual = x1; ps.ldr = H; ps.res_fresh = 1;
+      ps.out = x; ps.ldo = H;
+      ps.M = (int)M; ps.N = H; ps.act = -1;
+      c.n = 4;
+      if (l + 1 < d->L) {                             // the next layer's q|k|v behind its input norm
+        const Layer &nx = d->layers[l + 1];
+        ChainPhase &pq = c.ph[4];
+        lin(pq, x, H, true, nx.Wqkv_f, ldq, H, d->qkv, ldq);
+        pq.bias = nx.bqkv;
+        pq.ln_kind = kind; pq.ln_w = nx.n1_w; pq.ln_eps = (float)d->cfg.norm_eps;
+        c.n = 5;
+      }
+      c.flags = d->state->chain_flags;
+      c.epoch = &d->state->epoch;   // advanced by the token choice that ends every step
+      c.launch = l;
+      c.fault = kernel_fault_word(d->dev);
+      c.spin_limit = 1 << 20;
+      if (const char *e = getenv("RAI_HIP_CHAIN_SPIN_LIMIT")) {   // failure-path test hook (read per launch)
+        const int lim = atoi(e);
+        if (lim > 0) c.spin_limit = lim;
+      }
+      RAI_TRY(launch_decode_chain(st, c, d->dev));
+      continue;
     }
 
     LinearArgs o = linear_args_default();

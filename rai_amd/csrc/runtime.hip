@@ -138,7 +138,8 @@ int check_kernel_fault(int dev) {
   (void)streamk_counters_reset(dev, c->stream);
   (void)hipStreamSynchronize(c->stream);
   return fail(RAI_ERR_HIP, "device %d: a kernel gave up a bounded wait (code %d: %s); results since the last synchronisation are invalid",
-              dev, code, code == RAI_FAULT_STREAMK ? "stream-K share never arrived" : "unknown");
+              dev, code, code == RAI_FAULT_STREAMK ? "stream-K share never arrived"
+              : code == RAI_FAULT_CHAIN ? "a block never reached a barrier of the decode chain kernel" : "unknown");
 }
 
 unsigned long long *index_error_counter(int dev) {

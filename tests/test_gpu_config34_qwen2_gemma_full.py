@@ -123,3 +123,77 @@ def test_single_layer_full_width_against_the_chain(hip, request, arch):
     progress(request, "layer contribution: max error %.3e of %.3e (%.4f), one output rounding %.3e" % (err, scale, err / scale, ulp))
     assert err <= 2e-2 * scale + ulp, f"attention + MLP contribution off by {err:.3e} (scale {scale:.3e})"
     dec.close()
+
+
+@pytest.mark.parametrize("arch", ["gemma", "qwen2"])
+def test_decode_chain_against_launch_per_linear(hip, request, monkeypatch, arch):
+    """Batched decode steps through the persistent decode chain kernel (o_proj, gate|up, down, the sum of its K splits
+    and the next layer's q|k|v as phases of one launch) against the same steps with one launch per Linear: the same
+    weight-stream arithmetic, so the logits agree to within the rounding of the regrouped K-split sum and the tokens are
+    the same; and against the oracle on a few sequences."""
+    if arch == "gemma":
+        cfg = qwen2.Config("gemma", 4096, 2048, 16384, 3, 8, 1, "gelu", max_position_embeddings=256, head_dim=256)
+        B = 32
+    else:
+        cfg = qwen2.Config("qwen2", 4096, 1536, 8960, 3, 12, 2, "silu", max_position_embeddings=256, rope_theta=1e6, head_dim=128)
+        B = 16
+    CTX, STEPS = 40, 3
+    ids = np.random.Generator(np.random.PCG64(51)).integers(0, cfg.vocab_size, (B, CTX)).astype(np.uint32)
+    runs = {}
+    for label, on in (("chain", "1"), ("per linear", None)):
+        if on:
+            monkeypatch.setenv("RAI_HIP_CHAIN", on)
+        else:
+            monkeypatch.delenv("RAI_HIP_CHAIN", raising=False)
+        dec, params = build(cfg, B, CTX + STEPS + 1, request)
+        logits, tok = dec.forward(ids)
+        steps = []
+        for _ in range(STEPS):
+            logits, tok = dec.forward(tok.reshape(B, 1))
+            steps.append((logits.copy(), tok.copy()))
+        runs[label] = steps
+        dec.close()
+    for s, ((lc, tc), (lp, tp)) in enumerate(zip(runs["chain"], runs["per linear"])):
+        assert_close(lc, lp, "bf16", f"{arch} decode step {s}: chain vs launch per Linear")
+        assert np.array_equal(tc, np.argmax(lc, -1).astype(np.uint32))
+    # the chain's first step against the oracle on three sequences (the later steps were fed the device's own tokens)
+    rows = [0, B // 2, B - 1]
+    ref = qwen2.Model(cfg, params, "bf16")
+    exact = qwen2.Model(cfg, params, "f32")       # the same stored weights and rotary tables, f32 arithmetic
+    exact.sin, exact.cos = ref.sin, ref.cos
+    ref.fwd(ids[rows])
+    exact.fwd(ids[rows])
+    dec, _ = build(cfg, B, CTX + 2, request)
+    _, tok0 = dec.forward(ids)
+    logits, tok = dec.forward(tok0.reshape(B, 1))
+    nxt = tok0[rows].reshape(-1, 1)
+    want = ref.fwd(nxt)
+    assert_logits_close(logits[rows], want, exact.fwd(nxt), "bf16", f"{arch} decode step through the chain vs the oracle")
+    check_tokens(tok[rows], want, "bf16")
+    dec.close()
+
+
+def test_decode_chain_barrier_timeout_is_reported(hip, request, monkeypatch):
+    """A barrier wait of the chain kernel that expires (forced from the host with a spin limit of one poll): the kernel
+    flags the fault, later waits fall through so every wave exits, the call returns an error instead of wrong logits,
+    and after clearing the cache the decoder works again."""
+    from rai_amd._lib import RaiHipError
+    cfg = qwen2.Config("gemma", 1024, 2048, 16384, 2, 8, 1, "gelu", max_position_embeddings=128, head_dim=256)
+    B = 16
+    monkeypatch.setenv("RAI_HIP_CHAIN", "1")
+    dec, _ = build(cfg, B, 32, request)
+    ids = np.random.Generator(np.random.PCG64(52)).integers(0, cfg.vocab_size, (B, 8)).astype(np.uint32)
+    _, tok = dec.forward(ids)
+    good, good_tok = dec.forward(tok.reshape(B, 1))
+    dec.clear_kv_cache()
+    _, tok = dec.forward(ids)
+    monkeypatch.setenv("RAI_HIP_CHAIN_SPIN_LIMIT", "1")
+    with pytest.raises(RaiHipError, match="barrier of the decode chain"):
+        dec.forward(tok.reshape(B, 1))
+    monkeypatch.delenv("RAI_HIP_CHAIN_SPIN_LIMIT")
+    dec.clear_kv_cache()
+    _, tok = dec.forward(ids)
+    again, again_tok = dec.forward(tok.reshape(B, 1))
+    np.testing.assert_array_equal(again, good)
+    np.testing.assert_array_equal(again_tok, good_tok)
+    dec.close()
