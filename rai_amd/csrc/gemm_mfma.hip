@@ -1144,23 +1144,37 @@ static bool streamk_applies(const LinearArgs &a, int bk, StreamKPlan *plan, bool
   return a.K % bk == 0 && streamk_plan(a.M, a.N, a.K, bk, plan, forced) && plan->ws_bytes <= a.splitk_ws_bytes;
 }
 
-static int *streamk_counters_of(int dev) {   // every GPU holds its own copy of the counter array at its own address
-  static int *counters[64];
+// every GPU holds its own copy of a __device__ array at its own address: looked up once per device
+template <typename Sym> static int *device_ints_of(int dev, int *(&cache)[64], const Sym &symbol) {
   if (dev < 0 || dev >= 64) return nullptr;
-  if (!counters[dev]) {
+  if (!cache[dev]) {
     int cur = -1;
     void *p = nullptr;
     if (hipGetDevice(&cur) != hipSuccess || (cur != dev && hipSetDevice(dev) != hipSuccess)) return nullptr;
-    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_streamk_counters)) == hipSuccess) counters[dev] = (int *)p;
+    if (hipGetSymbolAddress(&p, symbol) == hipSuccess) cache[dev] = (int *)p;
     if (cur != dev) (void)hipSetDevice(cur);
   }
-  return counters[dev];
+  return cache[dev];
+}
+static int *streamk_counters_of(int dev) {
+  static int *counters[64];
+  return device_ints_of(dev, counters, HIP_SYMBOL(g_streamk_counters));
+}
+// Tickets of the small-M streaming Linear's K split, one per group of weight tiles; zero between launches (the block
+// that takes a group's last ticket puts it back).  Launches that overlap on one GPU would share them: the library
+// runs a device's work on one stream.
+constexpr int kSplitTickets = 16384;
+static __device__ int g_splitk_tickets[kSplitTickets];
+static int *splitk_tickets_of(int dev) {
+  static int *tickets[64];
+  return device_ints_of(dev, tickets, HIP_SYMBOL(g_splitk_tickets));
 }
 
 int streamk_counters_reset(int dev, hipStream_t st) {
-  int *c = streamk_counters_of(dev);
-  RAI_REQUIRE(c, RAI_ERR_HIP, "stream-K counters of device %d not found", dev);
+  int *c = streamk_counters_of(dev), *t = splitk_tickets_of(dev);
+  RAI_REQUIRE(c && t, RAI_ERR_HIP, "stream-K counters of device %d not found", dev);
   RAI_HIP_TRY(hipMemsetAsync(c, 0, sizeof(int) * 4 * kNumCU, st));
+  RAI_HIP_TRY(hipMemsetAsync(t, 0, sizeof(int) * kSplitTickets, st));
   return RAI_OK;
 }
 
@@ -1371,8 +1385,26 @@ int launch_linear_fragment_layout(hipStream_t st, const void *W, int64_t ldw, in
   return launch_check("linear_fragment_layout");
 }
 
+// 16 bytes to or from memory past the (per-XCD, mutually incoherent) L2s: for data that another block of the same
+// launch reads or wrote (p is 16-byte aligned)
+__device__ __forceinline__ void store_f32x4_device(float *p, f32x4 v) {
+  unsigned long long *q = reinterpret_cast<unsigned long long *>(p);
+  __hip_atomic_store(q, (unsigned long long)__float_as_uint(v.x) | ((unsigned long long)__float_as_uint(v.y) << 32), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 1, (unsigned long long)__float_as_uint(v.z) | ((unsigned long long)__float_as_uint(v.w) << 32), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 load_f32x4_device(const float *p) {
+  const unsigned long long *q = reinterpret_cast<const unsigned long long *>(p);
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return f32x4{__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
+               __uint_as_float((uint32_t)(hi >> 32))};
+}
+
 template <int MT, int KS, int G, bool FRAG>
-__global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, int tiles, float *partial) {
+__global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, int tiles, float *partial, int *tickets) {
+  __shared__ int s_ticket;
   constexpr int NW = 8;
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   constexpr int PCH = 4 * G + 1;                       // row pitch of the parked accumulators, in f32x4
@@ -1382,57 +1414,6 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
   const int split = blockIdx.y;
   const int k0 = (split * NW + wave) * KS * 32;
 
-  // activation fragments of this wave's K slice (zero beyond M and K)
-  bf16x8 xf[MT][KS];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int m = mt * 16 + lrow, k = k0 + ks * 32;
-      bf16x8 z = {};
-      if (m < a.M && k < a.K)
-        z = *reinterpret_cast<const bf16x8 *>((const uint16_t *)a.A + (int64_t)m * a.lda + k + lq * 8);
-      xf[mt][ks] = z;
-    }
-  // Optional RMSNorm of the activation rows (ln_kind 1: x * w / rms, 2: x * (1 + w) / rms), K not split
-  // over blocks: the sum of squares of a row is gathered from the four lanes and eight waves that hold
-  // its pieces, then every fragment is scaled and rounded to bf16 exactly as the stand-alone kernel does.
-  if (a.ln_kind > 0) {
-    float *rs = reinterpret_cast<float *>(lds);   // [8 waves][MT * 16 rows]; the accumulator area is not in use yet
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      float ss = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) { const float v = (float)xf[mt][ks][j]; ss = fmaf(v, v, ss); }
-      ss += __shfl_xor(ss, 16, 64);
-      ss += __shfl_xor(ss, 32, 64);
-      if (lq == 0) rs[wave * (MT * 16) + mt * 16 + lrow] = ss;
-    }
-    __syncthreads();
-    const uint16_t *lw = (const uint16_t *)a.ln_w;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      float tot = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) tot += rs[w * (MT * 16) + mt * 16 + lrow];
-      const float scale = 1.0f / sqrtf(tot / (float)a.K + a.ln_eps);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int k = k0 + ks * 32;
-        if (k < a.K) {
-          const bf16x8 wv = *reinterpret_cast<const bf16x8 *>(lw + k + lq * 8);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const float wf = (float)wv[j];
-            xf[mt][ks][j] = (__bf16)((float)xf[mt][ks][j] * scale * (a.ln_kind == 2 ? 1.0f + wf : wf));
-          }
-        }
-      }
-    }
-    __syncthreads();   // the statistics have been read before the area is reused
-  }
   int koff[KS];   // K steps beyond K read column 0 (their activation fragments are zero)
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) koff[ks] = k0 + ks * 32 < a.K ? k0 + ks * 32 : 0;
@@ -1468,9 +1449,119 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
   const int stride = gridDim.x * G;
   // tile at position pos (0 .. G + RING - 2) counted from the start of the group that begins at tile g0
   auto tile_at = [&](int g0, int pos) { return g0 + (pos / G) * stride + pos % G; };
+  // The block's first tiles are asked for behind the activation fragments (which come from the L2 and are needed
+  // first: loads return in order) and, with a fused norm, before its statistics go round the block.
+  int g0 = blockIdx.x * G;
+  auto first_tiles = [&]() {
+#pragma unroll
+    for (int pos = 0; pos + 1 < RING; ++pos) load_tile(w[pos], tile_at(g0, pos));
+  };
+  // activation fragments of this wave's K slice (zero beyond M and K)
+  bf16x8 xf[MT][KS];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int m = mt * 16 + lrow, k = k0 + ks * 32;
+      bf16x8 z = {};
+      if (m < a.M && k < a.K)
+        z = *reinterpret_cast<const bf16x8 *>((const uint16_t *)a.A + (int64_t)m * a.lda + k + lq * 8);
+      xf[mt][ks] = z;
+    }
+  // Optional RMSNorm of the activation rows (ln_kind 1: x * w / rms, 2: x * (1 + w) / rms), K not split
+  // over blocks: the sum of squares of a row is gathered from the four lanes and eight waves that hold
+  // its pieces, then every fragment is scaled and rounded to bf16 exactly as the stand-alone kernel does.
+  if (a.ln_kind > 0) {
+    float *rs = reinterpret_cast<float *>(lds);   // [8 waves][MT * 16 rows]; the accumulator area is not in use yet
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float ss = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { const float v = (float)xf[mt][ks][j]; ss = fmaf(v, v, ss); }
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      if (lq == 0) rs[wave * (MT * 16) + mt * 16 + lrow] = ss;
+    }
+    first_tiles();   // on their way while the row statistics go round the block
+    // the widened values of the statistics pass are not kept for the scaling pass (256 registers: they would spill)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[mt][ks]));
+    __syncthreads();
+    const uint16_t *lw = (const uint16_t *)a.ln_w;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) tot += rs[w * (MT * 16) + mt * 16 + lrow];
+      const float scale = 1.0f / sqrtf(tot / (float)a.K + a.ln_eps);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int k = k0 + ks * 32;
+        if (k < a.K) {
+          const bf16x8 wv = *reinterpret_cast<const bf16x8 *>(lw + k + lq * 8);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float wf = (float)wv[j];
+            xf[mt][ks][j] = (__bf16)((float)xf[mt][ks][j] * scale * (a.ln_kind == 2 ? 1.0f + wf : wf));
+          }
+        }
+      }
+    }
+    __syncthreads();   // the statistics have been read before the area is reused
+  } else {
+    first_tiles();
+  }
   const uint16_t *bias = (const uint16_t *)a.bias;
   const uint16_t *bias2 = (const uint16_t *)a.bias2;
   const uint16_t *res = (const uint16_t *)a.residual;
+  // bias, activation / gated pair, residual and the bf16 store of four consecutive columns n .. n+3 of row m
+  auto finish = [&](int m, int n, f32x4 s4) __attribute__((always_inline)) {
+    const float x[4] = {s4.x, s4.y, s4.z, s4.w};
+    const int lim = a.N - n < 4 ? a.N - n : 4;
+    if (a.glu) {   // columns (n, n+1) and (n+2, n+3) are (gate, up) pairs (N is a multiple of 8)
+      uint16_t o[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float gt = x[2 * e] + (bias ? bf16_bits_to_f32(bias[n + 2 * e]) : 0.f);
+        const float up = x[2 * e + 1] + (bias ? bf16_bits_to_f32(bias[n + 2 * e + 1]) : 0.f);
+        o[e] = f32_to_bf16_bits(glu_bf16(a.act, gt, up));
+      }
+      uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
+      if (((uintptr_t)dst & 3) == 0) *reinterpret_cast<uint32_t *>(dst) = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+      else { dst[0] = o[0]; dst[1] = o[1]; }
+      return;
+    }
+    uint16_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int nn = e < lim ? n + e : n;
+      float y = x[e] + ((bias ? bf16_bits_to_f32(bias[nn]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[nn]) : 0.f));
+      if (a.act >= 0 && nn >= a.act_from) y = act_eval(a.act, y);
+      if (res) y += bf16_bits_to_f32(res[(int64_t)m * a.ldr + nn]);
+      o[e] = f32_to_bf16_bits(y);
+    }
+    // all four columns in one output and the destination 8-byte aligned: one store
+    const bool first = n + 3 < a.n_split, second = n >= a.n_split;
+    uint16_t *dst = second ? (uint16_t *)a.out2 + (int64_t)m * a.ld2 + (n - a.n_split) : (uint16_t *)a.out1 + (int64_t)m * a.ld1 + n;
+    if (lim == 4 && (first || second) && ((uintptr_t)dst & 7) == 0) {
+      typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+      const u32x2 pk = {(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+      *reinterpret_cast<u32x2 *>(dst) = pk;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (e < lim) {
+          const int nn = n + e;
+          if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = o[e];
+          else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = o[e];
+        }
+      }
+    }
+  };
   auto group = [&](auto rot, const int g0) {
     constexpr int R = decltype(rot)::value;
     f32x4 acc[G][MT];
@@ -1511,62 +1602,48 @@ __global__ void __launch_bounds__(512) k_linear_bf16_mfma_stream(LinearArgs a, i
         const f32x4 t = red[(w * MT * 16 + m) * PCH + c];
         s4.x += t.x; s4.y += t.y; s4.z += t.z; s4.w += t.w;
       }
-      float x[4] = {s4.x, s4.y, s4.z, s4.w};
-      const int lim = a.N - n < 4 ? a.N - n : 4;
       if (partial) {
         float *p = partial + ((int64_t)split * a.M + m) * a.N + n;
-        if (lim == 4 && a.N % 4 == 0) *reinterpret_cast<f32x4 *>(p) = s4;
-        else {
+        if (tickets) {   // read by another block of this launch: past the L2 (N is a multiple of 4, checked on the host)
+          store_f32x4_device(p, s4);
+        } else if (a.N - n >= 4 && a.N % 4 == 0) {
+          *reinterpret_cast<f32x4 *>(p) = s4;
+        } else {
+          const float x[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (e < lim) p[e] = x[e];
+            if (n + e < a.N) p[e] = x[e];
         }
         continue;
       }
-      if (a.glu) {   // columns (n, n+1) and (n+2, n+3) are (gate, up) pairs (N is a multiple of 8)
-        uint16_t o[2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const float gt = x[2 * e] + (bias ? bf16_bits_to_f32(bias[n + 2 * e]) : 0.f);
-          const float up = x[2 * e + 1] + (bias ? bf16_bits_to_f32(bias[n + 2 * e + 1]) : 0.f);
-          o[e] = f32_to_bf16_bits(glu_bf16(a.act, gt, up));
-        }
-        uint16_t *dst = (uint16_t *)a.out1 + (int64_t)m * a.ld1 + (n >> 1);
-        if (((uintptr_t)dst & 3) == 0) *reinterpret_cast<uint32_t *>(dst) = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-        else { dst[0] = o[0]; dst[1] = o[1]; }
-        continue;
-      }
-      uint16_t o[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int nn = e < lim ? n + e : n;
-        float y = x[e] + ((bias ? bf16_bits_to_f32(bias[nn]) : 0.f) + (bias2 ? bf16_bits_to_f32(bias2[nn]) : 0.f));
-        if (a.act >= 0 && nn >= a.act_from) y = act_eval(a.act, y);
-        if (res) y += bf16_bits_to_f32(res[(int64_t)m * a.ldr + nn]);
-        o[e] = f32_to_bf16_bits(y);
-      }
-      // all four columns in one output and the destination 8-byte aligned: one store
-      const bool first = n + 3 < a.n_split, second = n >= a.n_split;
-      uint16_t *dst = second ? (uint16_t *)a.out2 + (int64_t)m * a.ld2 + (n - a.n_split) : (uint16_t *)a.out1 + (int64_t)m * a.ld1 + n;
-      if (lim == 4 && (first || second) && ((uintptr_t)dst & 7) == 0) {
-        typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-        const u32x2 pk = {(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
-        *reinterpret_cast<u32x2 *>(dst) = pk;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (e < lim) {
-            const int nn = n + e;
-            if (nn < a.n_split) ((uint16_t *)a.out1)[(int64_t)m * a.ld1 + nn] = o[e];
-            else ((uint16_t *)a.out2)[(int64_t)m * a.ld2 + (nn - a.n_split)] = o[e];
+      finish(m, n, s4);
+    }
+    if (partial && tickets) {
+      // K split over blocks without a second launch: a block counts itself in once its partial sums have reached
+      // memory, and the block that counts last -- whichever it is -- adds all of them in split order (the order of
+      // the separate summing pass, so the result is the same bit for bit) and runs the epilogue.  Nobody waits.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      int *ticket = tickets + g0 / G;
+      if (tid == 0) s_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (s_ticket == (int)gridDim.y - 1) {
+        if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        for (int v = tid; v < MT * G * 64; v += 512) {
+          const int m = v / (G * 4), c = v - m * (G * 4);
+          const int tile = g0 + (c >> 2);
+          const int n = tile * 16 + 4 * (c & 3);
+          if (tile >= tiles || n >= a.N || m >= a.M) continue;
+          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+          for (int sp = 0; sp < (int)gridDim.y; ++sp) {
+            const f32x4 t = load_f32x4_device(partial + ((int64_t)sp * a.M + m) * a.N + n);
+            s4.x += t.x; s4.y += t.y; s4.z += t.z; s4.w += t.w;
           }
+          finish(m, n, s4);
         }
       }
     }
   };
-  int g0 = blockIdx.x * G;
-#pragma unroll
-  for (int pos = 0; pos + 1 < RING; ++pos) load_tile(w[pos], tile_at(g0, pos));
   for (;;) {
     group(std::integral_constant<int, 0>{}, g0);
     if ((g0 += stride) >= tiles) break;
@@ -1597,10 +1674,18 @@ static int launch_mfma_stream_cfg(hipStream_t st, const LinearArgs &a, int split
     attr_set = true;
   }
   float *partial = splits > 1 ? (float *)a.splitk_ws : nullptr;
+  // K split: the block that finishes a group last sums the partial products and runs the epilogue itself (no second
+  // launch) when the tickets reach and the partial rows are 16-byte aligned; RAI_HIP_NO_FUSED_SPLITK=1 keeps the
+  // separate summing pass (the tests compare the two: same bits).
+  int *tickets = nullptr;
+  if (splits > 1 && groups <= kSplitTickets && a.N % 4 == 0 && ((uintptr_t)partial & 15) == 0 && !getenv("RAI_HIP_NO_FUSED_SPLITK")) {
+    int dev = -1;
+    if (linear_device(a, &dev) == RAI_OK) tickets = splitk_tickets_of(dev);
+  }
   hipLaunchKernelGGL((k_linear_bf16_mfma_stream<MT, KS, G, FRAG>), dim3(blocks_x, splits), dim3(512), lds, st, a, tiles,
-                     partial);
+                     partial, tickets);
   RAI_TRY(launch_check("linear_bf16_mfma_stream"));
-  if (splits > 1) {
+  if (splits > 1 && !tickets) {
     const int64_t total = (int64_t)a.M * a.N;
     const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
     hipLaunchKernelGGL(k_splitk_epilogue, dim3(blocks), dim3(256), 0, st, a, splits, (const float *)partial);

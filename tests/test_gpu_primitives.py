@@ -429,6 +429,28 @@ def test_linear_small_batch_deep_k(R, monkeypatch, m, k, n, kernel):
     assert_close(got, want, "bf16", f"linear fused {m}x{k}x{n}")
 
 
+@pytest.mark.parametrize("m,k,n", [(32, 16384, 2048), (9, 4096, 200), (64, 16384, 64), (17, 6144, 1000)])
+def test_linear_k_split_summed_by_the_last_block(R, monkeypatch, m, k, n):
+    """The weight-streaming kernel with K split over blocks: the block that finishes a group of weight tiles last sums
+    the partial products itself.  Same bits as the separate summing pass (RAI_HIP_NO_FUSED_SPLITK=1), call after call
+    (the tickets are handed back), with and without the fused epilogue."""
+    g = rng(126)
+    x, w, b = rand(g, (m, k), "bf16"), rand(g, (n, k), "bf16", 0.03), rand(g, (n,), "bf16")
+    r = rand(g, (m, n), "bf16")
+    xd, wd, bd, rd = (up(a, "bf16") for a in (x, w, b, r))
+
+    def run():
+        return down(R.linear(xd, wd, bd)), down(R.linear(xd, wd, bd, "new_gelu", rd))
+
+    fused = [run() for _ in range(3)]
+    monkeypatch.setenv("RAI_HIP_NO_FUSED_SPLITK", "1")
+    plain = run()
+    for it in fused:
+        np.testing.assert_array_equal(it[0], plain[0])
+        np.testing.assert_array_equal(it[1], plain[1])
+    assert_close(plain[0], onn.linear(x, w, b, "bf16"), "bf16", f"linear {m}x{k}x{n}")
+
+
 # ------------------------------------------------------------------ norms / rope / attention
 @pytest.mark.parametrize("dt", ["f32", "bf16", "f16", "f64"])
 @pytest.mark.parametrize("shape", [(3, 7, 2560), (5, 1536), (4, 100), (2, 9000), (6, 2048)])
