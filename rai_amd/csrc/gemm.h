@@ -59,6 +59,13 @@ struct LinearArgs {
   float post_ln_eps;
   // Device the operands live on (its CU count and per-device counters are looked up by it); -1: the current device.
   int dev;
+  // Optional second product added to the first before the epilogue (M == 1, skinny kernel only): the row A2 [K2]
+  // against W2 [N, K2], as if A and A2, W and W2 were concatenated along K.  The sum of two Linears of a decoder
+  // block (rai-models/src/llm/phi2.rs:298) in one launch; their biases go to bias and bias2.
+  const void *A2;
+  const void *W2;
+  int64_t ldw2;
+  int K2;
 };
 // True when launch_linear_bf16 with these arguments will also write post_ln_out.
 bool linear_fuses_post_norm(const LinearArgs &a);
@@ -85,6 +92,31 @@ int launch_linear_bf16_mfma(hipStream_t st, const LinearArgs &a);
 int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a);
 // Picks between the two.
 int launch_linear_bf16(hipStream_t st, const LinearArgs &a);
+
+// Up to kGemvGroupMax bf16 Linears of one activation row (M == 1, K <= 4096, a multiple of 8) in one launch: member i
+// is out[i][n] = act[i](sum_k norm(x)[k] * W[i][n, k] + bias[i][n]), n < N[i]; the optional norm (ln_kind as in
+// LinearArgs) is applied to x once per wave, as the single-Linear kernel does.  wave_base is filled by the launcher.
+constexpr int kGemvGroupMax = 4;
+struct GemvGroupArgs {
+  const void *x;
+  int K, count;
+  const void *W[kGemvGroupMax];
+  int64_t ldw[kGemvGroupMax];
+  const void *bias[kGemvGroupMax];   // null: none
+  void *out[kGemvGroupMax];
+  int N[kGemvGroupMax];
+  int act[kGemvGroupMax];            // rai_hip_unary_op or -1
+  const void *ln_w, *ln_b;
+  float ln_eps;
+  int ln_kind;
+  int wave_base[kGemvGroupMax + 1];
+};
+bool gemv_group_serves(int K, int count);
+// out[n] = x1 . W1[n] + x2 . W2[n] + bias1[n] + bias2[n] + residual[n] for one bf16 row pair (the LinearArgs::A2 form);
+// RAI_ERR_UNSUPPORTED when the widths are not served.
+int launch_linear_dual_row(hipStream_t st, int dev, const void *x1, int K1, const void *W1, int64_t ldw1, const void *bias1, const void *x2, int K2,
+                           const void *W2, int64_t ldw2, const void *bias2, const void *residual, void *out, int N);
+int launch_gemv_group(hipStream_t st, GemvGroupArgs g);
 
 // f32 tile kernel for the same NT contraction, FMA in f32.
 int launch_linear_f32(hipStream_t st, const LinearArgs &a);

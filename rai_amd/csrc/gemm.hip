@@ -50,7 +50,13 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint16_t *A = (const uint16_t *)a.A;
   const uint16_t *W = (const uint16_t *)a.W;
-  const int K = a.K;
+  // With a second product (M == 1) the K axis is the first product's K followed by the second's: position k < K1 is
+  // column k of (A, W), position k >= K1 column k - K1 of (A2, W2); a 16-byte chunk never straddles (K1 % 8 == 0).
+  const int K1 = a.K, K = a.K + a.K2;
+  const uint16_t *A2 = (const uint16_t *)a.A2 - K1;   // indexed by the position on the joint axis
+  const uint16_t *W2 = (const uint16_t *)a.W2 - K1;
+  auto x_at = [&](const uint16_t *row, int k) { return k < K1 ? row + k : A2 + k; };
+  auto w_at = [&](int n, int k) { return k < K1 ? W + (int64_t)n * a.ldw + k : W2 + (int64_t)n * a.ldw2 + k; };
 
   // Loads return in issue order: the activation rows (L2-resident) are requested
   // first, the first set of weight loads right behind them, so the staging into
@@ -62,7 +68,7 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
 #pragma unroll
   for (int i = 0; i < XCH; ++i) {
     const int k = (tid + i * NT) * 8;
-    xpre[i] = k < K ? *reinterpret_cast<const u32x4 *>(A + k) : u32x4{0u, 0u, 0u, 0u};
+    xpre[i] = k < K ? *reinterpret_cast<const u32x4 *>(x_at(A, k)) : u32x4{0u, 0u, 0u, 0u};
   }
   u32x4 wv[U][R];
 #pragma unroll
@@ -71,7 +77,7 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       int n = n_begin + r < n_end ? n_begin + r : n_end - 1;
-      if (k < K && n_begin < a.N) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(W + (int64_t)n * a.ldw + k));
+      if (k < K && n_begin < a.N) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(w_at(n, k)));
       else wv[u][r] = u32x4{0u, 0u, 0u, 0u};
     }
   }
@@ -88,7 +94,7 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
         if (k < K) *reinterpret_cast<u32x4 *>(xd + k) = xpre[i];
       }
       for (int k = (tid + XCH * NT) * 8; k < K; k += NT * 8)
-        *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(xr + k);
+        *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(x_at(xr, k));
     } else {
       for (int k = tid * 8; k < K; k += NT * 8)
         *reinterpret_cast<u32x4 *>(xd + k) = *reinterpret_cast<const u32x4 *>(xr + k);
@@ -175,7 +181,7 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           const int n = n_base + r < n_end ? n_base + r : n_end - 1;  // tail rows re-read the last row; never stored
-          if (k < K) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(W + (int64_t)n * a.ldw + k));
+          if (k < K) wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(w_at(n, k)));
         }
       }
     }
@@ -238,12 +244,10 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
 // activation vector is fetched and normalised, so the fused LayerNorm/RMSNorm
 // prologue overlaps the first HBM round trip.
 template <int KC, int R>
-__global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_per_wave) {
+__device__ __forceinline__ void gemv_reg_rows(const LinearArgs &a, int n_begin, int rows_per_wave) {
   const int lane = threadIdx.x & 63;
-  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int K = a.K;
   const uint16_t *W = (const uint16_t *)a.W;
-  const int n_begin = gw * rows_per_wave;
   if (n_begin >= a.N) return;
   const int n_end = n_begin + rows_per_wave < a.N ? n_begin + rows_per_wave : a.N;
 
@@ -366,6 +370,36 @@ __global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_pe
       }
     }
   }
+}
+
+template <int KC, int R>
+__global__ void __launch_bounds__(256) k_gemv_bf16_reg(LinearArgs a, int rows_per_wave) {
+  gemv_reg_rows<KC, R>(a, (blockIdx.x * 4 + (threadIdx.x >> 6)) * rows_per_wave, rows_per_wave);
+}
+
+// Up to four Linears of one activation vector in one launch (the q, k, v projections and the first MLP Linear of a
+// decoder block, each with its own weight, bias, activation and output): wave gw serves rows of the member whose
+// wave range [wave_base[s], wave_base[s + 1]) holds it.  The fused norm is every member's.
+template <int KC, int R>
+__global__ void __launch_bounds__(256) k_gemv_bf16_reg_group(GemvGroupArgs g, int rows_per_wave) {
+  const int gw = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
+  if (gw >= g.wave_base[g.count]) return;
+  int s = 0;
+#pragma unroll
+  for (int i = 1; i < kGemvGroupMax; ++i)
+    if (i < g.count && gw >= g.wave_base[i]) s = i;
+  LinearArgs a;
+  a.A = g.x; a.lda = g.K;
+  a.W = g.W[0]; a.ldw = g.ldw[0]; a.bias = g.bias[0]; a.out1 = g.out[0]; a.N = g.N[0]; a.act = g.act[0];
+  int base = g.wave_base[0];
+#pragma unroll
+  for (int i = 1; i < kGemvGroupMax; ++i)
+    if (s == i) { a.W = g.W[i]; a.ldw = g.ldw[i]; a.bias = g.bias[i]; a.out1 = g.out[i]; a.N = g.N[i]; a.act = g.act[i]; base = g.wave_base[i]; }
+  a.bias2 = nullptr; a.residual = nullptr; a.ldr = 0; a.ld1 = a.N; a.out2 = nullptr; a.ld2 = 0;
+  a.M = 1; a.K = g.K; a.n_split = a.N; a.act_from = 0; a.glu = 0;
+  a.ln_w = g.ln_w; a.ln_b = g.ln_b; a.ln_eps = g.ln_eps; a.ln_kind = g.ln_kind;
+  a.A2 = nullptr; a.W2 = nullptr; a.ldw2 = 0; a.K2 = 0;
+  gemv_reg_rows<KC, R>(a, (gw - base) * rows_per_wave, rows_per_wave);
 }
 
 // ============================================================ f32 NT tile kernel
@@ -535,7 +569,7 @@ static int check_linear_args(const LinearArgs &a, size_t es) {
 
 template <int MROWS, int R, int U, int NWV = 4>
 static int launch_skinny_cfg(hipStream_t st, const LinearArgs &a, int rows_per_wave) {
-  const size_t lds = (size_t)MROWS * a.K * sizeof(uint16_t);
+  const size_t lds = (size_t)MROWS * (a.K + a.K2) * sizeof(uint16_t);
   static size_t attr_bytes = 0;
   if (lds > 64 * 1024 && lds > attr_bytes) {
     RAI_HIP_TRY(hipFuncSetAttribute((const void *)k_linear_bf16_skinny<MROWS, R, U, NWV>,
@@ -563,13 +597,48 @@ static int launch_gemv_reg(hipStream_t st, const LinearArgs &a, int waves_per_cu
   return launch_check("gemv_bf16_reg");
 }
 
+bool gemv_group_serves(int K, int count) { return count >= 1 && count <= kGemvGroupMax && K % 8 == 0 && K >= 8 && K <= 4096; }
+
+int launch_gemv_group(hipStream_t st, GemvGroupArgs g) {
+  RAI_REQUIRE(gemv_group_serves(g.K, g.count) && g.x && ((uintptr_t)g.x & 15) == 0, RAI_ERR_UNSUPPORTED, "linear group: K=%d x %d members not served",
+              g.K, g.count);
+  if (g.ln_kind >= 0) RAI_REQUIRE(g.ln_w && ((uintptr_t)g.ln_w & 15) == 0 && ((uintptr_t)g.ln_b & 15) == 0, RAI_ERR_BAD_STRIDE, "linear group: norm parameters");
+  // short-lived waves, one or two groups of two rows each (what the single Linear of these widths takes);
+  // RAI_HIP_GEMV_GROUP_ROWS overrides (tuning aid, read per launch)
+  int total = 0;
+  for (int i = 0; i < g.count; ++i) total += g.N[i];
+  int rpw = total >= 8192 ? 8 : 2;
+  if (const char *e = getenv("RAI_HIP_GEMV_GROUP_ROWS")) {
+    const int v = atoi(e);
+    if (v >= 2 && v <= 64 && v % 2 == 0) rpw = v;
+  }
+  int waves = 0;
+  for (int i = 0; i < g.count; ++i) {
+    RAI_REQUIRE(g.W[i] && g.out[i] && g.N[i] >= 1 && g.ldw[i] % 8 == 0 && ((uintptr_t)g.W[i] & 15) == 0, RAI_ERR_BAD_STRIDE,
+                "linear group: member %d not served", i);
+    g.wave_base[i] = waves;
+    waves += (g.N[i] + rpw - 1) / rpw;
+  }
+  g.wave_base[g.count] = waves;
+  const dim3 grid((waves + 3) / 4), block(256);
+  if (g.K <= 2048) hipLaunchKernelGGL((k_gemv_bf16_reg_group<4, 2>), grid, block, 0, st, g, rpw);
+  else if (g.K <= 2560) hipLaunchKernelGGL((k_gemv_bf16_reg_group<5, 2>), grid, block, 0, st, g, rpw);
+  else hipLaunchKernelGGL((k_gemv_bf16_reg_group<8, 2>), grid, block, 0, st, g, rpw);
+  return launch_check("gemv_bf16_reg_group");
+}
+
 int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   RAI_TRY(check_linear_args(a, 2));
   RAI_REQUIRE(a.M <= 8, RAI_ERR_BAD_SHAPE, "linear skinny: M=%d > 8", a.M);
-  RAI_REQUIRE((size_t)a.M * a.K * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
+  RAI_REQUIRE((size_t)a.M * (a.K + a.K2) * 2 <= 150 * 1024, RAI_ERR_UNSUPPORTED, "linear skinny: activations exceed LDS");
+  const bool dual = a.K2 > 0;
+  if (dual)
+    RAI_REQUIRE(a.M == 1 && a.A2 && a.W2 && a.K2 % 8 == 0 && a.ldw2 % 8 == 0 && (uintptr_t)a.A2 % 16 == 0 && (uintptr_t)a.W2 % 16 == 0 &&
+                    a.ln_kind < 0 && !a.glu,
+                RAI_ERR_UNSUPPORTED, "linear: second product not served (one row, no norm, no gate)");
   if (a.glu) RAI_REQUIRE(a.N % 2 == 0 && !a.residual && a.n_split == a.N && a.act >= 0, RAI_ERR_BAD_ARG,
                          "linear: bad gated-MLP arguments");
-  if (a.M == 1 && a.K <= 4096 && a.N >= 1024) {
+  if (a.M == 1 && a.K <= 4096 && a.N >= 1024 && !dual) {
     // activation vector in registers (at most 8 chunks of 16 bytes per lane)
     if (a.K <= 2048) return launch_gemv_reg<4, 4>(st, a, 8);
     if (a.K <= 2560) {
@@ -611,7 +680,7 @@ int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
       }
     }
     // one row per wave with the whole row in flight when it fits the register budget
-    if (a.N <= kNumCU * 16 && a.K <= 25 * 512) return launch_skinny_cfg<1, 1, 25>(st, a, 1);
+    if (a.N <= kNumCU * 16 && a.K + a.K2 <= 25 * 512) return launch_skinny_cfg<1, 1, 25>(st, a, 1);
     if (rpw >= 4) { rpw = (rpw / 4) * 4; return launch_skinny_cfg<1, 4, 5>(st, a, rpw); }
     if (rpw >= 2) { rpw = 2; return launch_skinny_cfg<1, 2, 8>(st, a, rpw); }
     return launch_skinny_cfg<1, 1, 8>(st, a, 1);
@@ -627,6 +696,19 @@ int launch_linear_bf16_skinny(hipStream_t st, const LinearArgs &a) {
   }
   if (rpw >= 2) { rpw = (rpw / 2) * 2; return launch_skinny_cfg<8, 2, 4>(st, a, rpw); }
   return launch_skinny_cfg<8, 1, 4>(st, a, 1);
+}
+
+int launch_linear_dual_row(hipStream_t st, int dev, const void *x1, int K1, const void *W1, int64_t ldw1, const void *bias1, const void *x2, int K2,
+                           const void *W2, int64_t ldw2, const void *bias2, const void *residual, void *out, int N) {
+  LinearArgs a = linear_args_default();
+  a.dev = dev;
+  a.A = x1; a.lda = K1; a.W = W1; a.ldw = ldw1; a.K = K1;
+  a.A2 = x2; a.W2 = W2; a.ldw2 = ldw2; a.K2 = K2;
+  a.bias = bias1; a.bias2 = bias2;
+  a.residual = residual; a.ldr = N;
+  a.out1 = out; a.ld1 = N;
+  a.M = 1; a.N = N; a.n_split = N;
+  return launch_linear_bf16_skinny(st, a);
 }
 
 int launch_linear_bf16(hipStream_t st, const LinearArgs &a) {

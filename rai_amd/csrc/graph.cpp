@@ -18,6 +18,7 @@
 
 #include "attention.h"
 #include "fused.h"
+#include "gemm.h"
 #include "rai_graph.h"
 
 using namespace rai;
@@ -50,6 +51,7 @@ struct rai_tensor {
   int n_users, users_at;
   uint32_t flags;
   int comp;
+  int group;   // index of the Linear group this node leads (flag kGroupLead)
   uint64_t stamp;
 };
 
@@ -58,11 +60,12 @@ namespace {
 uint64_t g_next_id = 1;
 uint64_t g_epoch = 0;        // one per rai_eval call
 uint64_t g_stamp = 0;        // one per attempted composition
-enum : uint32_t { kInlined = 1u, kAbsorbed = 2u, kRoot = 4u, kOutput = 8u, kCoOutput = 16u };
+enum : uint32_t { kInlined = 1u, kAbsorbed = 2u, kRoot = 4u, kOutput = 8u, kCoOutput = 16u, kGroupLead = 32u, kGrouped = 64u };
 inline bool in_tape(const rai_tensor *t) { return t->mark == g_epoch; }
 inline bool has_flag(const rai_tensor *t, uint32_t f) { return in_tape(t) && (t->flags & f); }
 std::vector<const rai_tensor *> g_users;   // flat user lists of the evaluation in progress
 bool g_fusion = true;
+bool g_group_linears = true;   // RAI_HIP_GRAPH_NO_LINEAR_GROUPS=1 (read per evaluation) turns the grouping of Linears off
 bool g_compose = true;
 rai_graph_stats g_stats = {0, 0, 0, 0, 0, 0, 0, 0};
 
@@ -95,6 +98,7 @@ rai_tensor *new_node(int dev, int dtype, const std::vector<int64_t> &shape, int 
   t->n_users = t->users_at = 0;
   t->flags = 0;
   t->comp = -1;
+  t->group = -1;
   t->stamp = 0;
   return t;
 }
@@ -501,6 +505,7 @@ int topo_sort(rai_tensor *const *outputs, int n, std::vector<rai_tensor *> *tape
         t->n_users = t->users_at = 0;
         t->flags = 0;
         t->comp = -1;
+        t->group = -1;
         tape->push_back(t);
       } else {
         stack.push_back({t, true});
@@ -684,6 +689,9 @@ struct Composite {
   // nodes that the root's launch materialises besides the root: they may be held from outside (the model keeps its
   // key / value caches), but every use inside the tape lies within the composition
   rai_tensor *co[2];
+  // a Linear whose added tensor is itself "Linear + tensor" (root `dual_inner`, unobservable): at one row the two
+  // products run as one launch and dual_inner is never materialised
+  rai_tensor *dual_inner;
   std::vector<rai_tensor *> interior;
 };
 
@@ -1416,6 +1424,14 @@ bool claim_two_linears_and_residual(rai_tensor *t) {
       g_comps.resize(before);
       continue;
     }
+    // one row, no activation on either product, parameters in place: one launch for both (run_root)
+    const Composite &po = g_comps[t->comp], &pi = g_comps[sum->comp];
+    const int64_t N = t->shape.back();
+    if (g_group_linears && t->dtype == RAI_BF16 && numel_of(t->shape) == N && act_p < 0 && act_q < 0 && !(sum->flags & kOutput) &&
+        po.in[1]->evaluated && pi.in[1]->evaluated && (!po.in[2] || po.in[2]->evaluated) && (!pi.in[2] || pi.in[2]->evaluated)) {
+      g_comps[t->comp].dual_inner = sum;
+      sum->flags |= kGrouped;
+    }
     return true;
   }
   return false;
@@ -1440,6 +1456,217 @@ void plan_compositions(const std::vector<rai_tensor *> &tape) {
       if (f(t, &c) && claim(t, c)) break;
     }
   }
+}
+
+// Linears of one activation row.  The q, k and v projections and the first MLP Linear of a decoder block read the same
+// normalised row (phi2.rs:293-297; qwen2.rs:205-210 and 100-104 read theirs through RMSNorm): at one row each is a
+// matrix-vector product that cannot fill the GPU by itself, so up to kGemvGroupMax Linear compositions that share
+// their input run as one launch, at the position of the first of them in the tape (their weights and biases are
+// parameters, there before the tape starts).  When the shared input is a LayerNorm / RMSNorm composition that nothing
+// else reads, the norm goes into the same launch (the launcher applies it in its prologue) and is never materialised.
+struct LinearGroup {
+  std::vector<rai_tensor *> members;   // tape order; members[0] leads
+  rai_tensor *norm;                    // root of the absorbed norm composition, or null
+};
+std::vector<LinearGroup> g_groups;
+
+bool group_member(const rai_tensor *t) {
+  if (!(t->flags & kRoot) || (t->flags & (kGroupLead | kGrouped)) || t->dtype != RAI_BF16) return false;
+  const Composite &c = g_comps[t->comp];
+  if (c.kind != COMP_LINEAR || c.in[3]) return false;
+  const rai_tensor *x = c.in[0], *w = c.in[1], *b = c.in[2];
+  const int64_t K = x->shape.back();
+  if (numel_of(x->shape) != K || !gemv_group_serves((int)K, 1)) return false;
+  return w->evaluated && (!b || b->evaluated);
+}
+
+void plan_linear_groups(const std::vector<rai_tensor *> &tape) {
+  g_groups.clear();
+  struct Open { rai_tensor *x; int group; };
+  Open open[8];   // the groups met last: members of one group lie close together in the tape
+  int n_open = 0, next = 0;
+  for (rai_tensor *t : tape) {
+    if (t->evaluated || !group_member(t)) continue;
+    rai_tensor *x = g_comps[t->comp].in[0];
+    int gi = -1;
+    for (int i = 0; i < n_open; ++i)
+      if (open[i].x == x && (int)g_groups[open[i].group].members.size() < kGemvGroupMax) gi = open[i].group;
+    if (gi < 0) {
+      gi = (int)g_groups.size();
+      g_groups.push_back(LinearGroup{{}, nullptr});
+      open[next] = Open{x, gi};
+      next = (next + 1) % 8;
+      if (n_open < 8) ++n_open;
+    }
+    g_groups[gi].members.push_back(t);
+  }
+  for (size_t gi = 0; gi < g_groups.size(); ++gi) {
+    LinearGroup &g = g_groups[gi];
+    if (g.members.size() < 2) {
+      // a single Linear stays by itself unless the norm in front of it can go into its launch
+      rai_tensor *x1 = g_comps[g.members[0]->comp].in[0];
+      const bool norm_root = !x1->evaluated && in_tape(x1) && (x1->flags & kRoot) && x1->refs == x1->n_users &&
+                             (g_comps[x1->comp].kind == COMP_LAYER_NORM || g_comps[x1->comp].kind == COMP_RMS_NORM);
+      if (!norm_root) { g.members.clear(); continue; }
+    }
+    g.members[0]->flags |= kGroupLead;
+    g.members[0]->group = (int)gi;
+    for (size_t i = 1; i < g.members.size(); ++i) g.members[i]->flags |= kGrouped;
+    // the shared input: a norm composition read by this group only?
+    rai_tensor *x = g_comps[g.members[0]->comp].in[0];
+    if (x->evaluated || !in_tape(x) || !(x->flags & kRoot) || (x->flags & (kOutput | kCoOutput | kGroupLead | kGrouped)) || x->refs != x->n_users ||
+        x->dtype != RAI_BF16)
+      continue;
+    const Composite &nc = g_comps[x->comp];
+    if (nc.kind != COMP_LAYER_NORM && nc.kind != COMP_RMS_NORM) continue;
+    const uint64_t stamp = ++g_stamp;
+    for (rai_tensor *m : g.members) {
+      m->stamp = stamp;
+      for (rai_tensor *n : g_comps[m->comp].interior) n->stamp = stamp;
+    }
+    bool sealed = true;
+    for (int u = 0; u < x->n_users && sealed; ++u) sealed = g_users[x->users_at + u]->stamp == stamp;
+    if (!sealed) continue;
+    g.norm = x;
+    x->flags |= kAbsorbed;   // never materialised: the loop passes over it
+  }
+  for (LinearGroup &g : g_groups)   // a single Linear whose norm stayed outside: an ordinary composition again
+    if (g.members.size() == 1 && !g.norm) {
+      g.members[0]->flags &= ~kGroupLead;
+      g.members[0]->group = -1;
+      g.members.clear();
+    }
+}
+
+int run_composite(rai_tensor *t, const Composite &c);
+int eval_pending_inputs(rai_tensor *t);
+
+// One launch for the whole group; RAI_ERR_UNSUPPORTED / RAI_ERR_BAD_STRIDE when the operands' layout is not served
+// (nothing has been written then).
+int launch_linear_group(const LinearGroup &g) {
+  const rai_tensor *lead = g.members[0];
+  const Composite *nc = g.norm ? &g_comps[g.norm->comp] : nullptr;
+  const rai_tensor *x = nc ? nc->in[0] : g_comps[lead->comp].in[0];
+  const int64_t K = x->shape.back();
+  RAI_REQUIRE(x->dtype == RAI_BF16 && is_contiguous(&x->view), RAI_ERR_BAD_STRIDE, "linear group: input row not dense");
+  GemvGroupArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = base_ptr(&x->view);
+  a.K = (int)K;
+  a.count = (int)g.members.size();
+  a.ln_kind = -1;
+  if (nc) {
+    const rai_tensor *w = nc->in[1], *b = nc->kind == COMP_LAYER_NORM ? nc->in[2] : nullptr;
+    RAI_REQUIRE(is_contiguous(&w->view) && (!b || is_contiguous(&b->view)), RAI_ERR_BAD_STRIDE, "linear group: norm parameters not dense");
+    a.ln_w = base_ptr(&w->view);
+    a.ln_b = b ? base_ptr(&b->view) : nullptr;
+    a.ln_eps = (float)nc->f0;
+    a.ln_kind = nc->kind == COMP_LAYER_NORM ? 0 : (nc->i2 ? 2 : 1);
+  }
+  for (int i = 0; i < a.count; ++i) {
+    const Composite &c = g_comps[g.members[i]->comp];
+    const rai_hip_tensor &w = c.in[1]->view;
+    RAI_REQUIRE(w.rank == 2 && w.stride[1] == 1 && w.shape[1] == K && (!c.in[2] || is_contiguous(&c.in[2]->view)), RAI_ERR_BAD_STRIDE,
+                "linear group: weight layout not served");
+    a.W[i] = base_ptr(&w);
+    a.ldw[i] = w.stride[0];
+    a.bias[i] = c.in[2] ? base_ptr(&c.in[2]->view) : nullptr;
+    a.N[i] = (int)w.shape[0];
+    a.act[i] = (int)c.i0;
+  }
+  hipStream_t st = stream_of(lead->dev);
+  if (!st) return RAI_ERR_HIP;
+  for (int i = 0; i < a.count; ++i) {
+    RAI_TRY(alloc_output(g.members[i]));
+    a.out[i] = g.members[i]->view.data;
+  }
+  return launch_gemv_group(st, a);
+}
+
+// A composition's root through its fused launcher, or -- when that declines the operands' layout -- the recorded
+// nodes one by one.
+int run_dual_linear(rai_tensor *t, const Composite &outer, const Composite &inner) {
+  const rai_tensor *x1 = outer.in[0], *w1 = outer.in[1], *b1 = outer.in[2], *x2 = inner.in[0], *w2 = inner.in[1], *b2 = inner.in[2],
+                   *res = inner.in[3];
+  const int64_t N = t->shape.back(), K1 = x1->shape.back(), K2 = x2->shape.back();
+  auto row = [](const rai_tensor *v, int64_t n) { return v->dtype == RAI_BF16 && numel_of(v->shape) == n && is_contiguous(&v->view); };
+  auto weight = [&](const rai_tensor *w, int64_t K) {
+    return w->dtype == RAI_BF16 && w->view.rank == 2 && w->view.shape[0] == N && w->view.shape[1] == K && w->view.stride[1] == 1;
+  };
+  RAI_REQUIRE(row(x1, K1) && row(x2, K2) && row(res, N) && weight(w1, K1) && weight(w2, K2) && (!b1 || row(b1, N)) && (!b2 || row(b2, N)),
+              RAI_ERR_BAD_STRIDE, "two Linears of one row: operand layout not served");
+  hipStream_t st = stream_of(t->dev);
+  if (!st) return RAI_ERR_HIP;
+  RAI_TRY(alloc_output(t));
+  return launch_linear_dual_row(st, t->dev, base_ptr(&x1->view), (int)K1, base_ptr(&w1->view), w1->view.stride[0], b1 ? base_ptr(&b1->view) : nullptr,
+                                base_ptr(&x2->view), (int)K2, base_ptr(&w2->view), w2->view.stride[0], b2 ? base_ptr(&b2->view) : nullptr,
+                                base_ptr(&res->view), t->view.data, (int)N);
+}
+
+int run_root(rai_tensor *t) {
+  const Composite &c = g_comps[t->comp];
+  if (c.dual_inner) {
+    rai_tensor *sum = c.dual_inner;
+    const Composite &inner = g_comps[sum->comp];
+    int st = run_dual_linear(t, c, inner);
+    if (st == RAI_OK) {
+      ++g_stats.kernel_launches;
+      g_stats.composed_regions += 2;
+      g_stats.composed_nodes += c.interior.size() + inner.interior.size() + 2;
+      return RAI_OK;
+    }
+    if (st != RAI_ERR_BAD_STRIDE && st != RAI_ERR_UNSUPPORTED && st != RAI_ERR_BAD_SHAPE && st != RAI_ERR_BAD_DTYPE) return st;
+    drop_storage(t);
+    // not served: the inner sum by itself first, then this root as an ordinary Linear with it added
+    sum->flags &= ~kGrouped;
+    g_comps[t->comp].dual_inner = nullptr;
+    st = run_root(sum);
+    if (st != RAI_OK) { drop_storage(sum); return st; }
+    sum->evaluated = true;
+    ++g_stats.nodes_evaluated;
+  }
+  int st = run_composite(t, c);
+  if (st == RAI_OK) {
+    ++g_stats.kernel_launches;
+    ++g_stats.composed_regions;
+    g_stats.composed_nodes += c.interior.size() + 1;
+  } else if (st == RAI_ERR_BAD_STRIDE || st == RAI_ERR_UNSUPPORTED || st == RAI_ERR_BAD_SHAPE || st == RAI_ERR_BAD_DTYPE) {
+    drop_storage(t);
+    st = eval_pending_inputs(t);
+    if (st == RAI_OK) st = g_rules[t->op](t);
+  }
+  return st;
+}
+
+int run_linear_group(const LinearGroup &g) {
+  int st = launch_linear_group(g);
+  if (st == RAI_OK) {
+    ++g_stats.kernel_launches;
+    if (g.norm) {
+      ++g_stats.composed_regions;
+      g_stats.composed_nodes += g_comps[g.norm->comp].interior.size() + 1;
+    }
+    for (rai_tensor *m : g.members) {
+      ++g_stats.composed_regions;
+      g_stats.composed_nodes += g_comps[m->comp].interior.size() + 1;
+      if (m != g.members[0]) { m->evaluated = true; ++g_stats.nodes_evaluated; }   // the loop does the leader's
+    }
+    return RAI_OK;
+  }
+  if (st != RAI_ERR_BAD_STRIDE && st != RAI_ERR_UNSUPPORTED && st != RAI_ERR_BAD_SHAPE && st != RAI_ERR_BAD_DTYPE) return st;
+  // not served as a group: the norm and every member by themselves
+  for (rai_tensor *m : g.members) drop_storage(m);
+  if (g.norm) {
+    RAI_TRY(run_root(g.norm));
+    g.norm->evaluated = true;
+    ++g_stats.nodes_evaluated;
+  }
+  for (rai_tensor *m : g.members) {
+    st = run_root(m);
+    if (st != RAI_OK) { drop_storage(m); return st; }
+    if (m != g.members[0]) { m->evaluated = true; ++g_stats.nodes_evaluated; }
+  }
+  return RAI_OK;
 }
 
 int run_composite(rai_tensor *t, const Composite &c) {
@@ -1860,6 +2087,7 @@ int rai_graph_eval_order(rai_tensor *const *outputs, int32_t n, uint64_t *ids, i
 int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
   RAI_REQUIRE(outputs && n >= 0, RAI_ERR_BAD_ARG, "null argument");
   init_rules();
+  g_group_linears = getenv("RAI_HIP_GRAPH_NO_LINEAR_GROUPS") == nullptr;
   const auto t_start = std::chrono::steady_clock::now();
   std::vector<rai_tensor *> tape;
   RAI_TRY(topo_sort(outputs, n, &tape));
@@ -1867,29 +2095,24 @@ int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
     if (in_tape(outputs[i])) outputs[i]->flags |= kOutput;
   index_users(tape);
   g_comps.clear();
-  if (g_compose) plan_compositions(tape);
+  g_groups.clear();
+  if (g_compose) {
+    plan_compositions(tape);
+    if (g_group_linears) plan_linear_groups(tape);
+  }
   if (g_fusion) plan_fusion(tape);
   const auto t_planned = std::chrono::steady_clock::now();
   g_stats.plan_ns += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(t_planned - t_start).count();
   int rc = RAI_OK;
   for (rai_tensor *t : tape) {
-    if (t->evaluated || (t->flags & (kInlined | kAbsorbed | kCoOutput))) continue;   // a co-output comes with its root
+    if (t->evaluated || (t->flags & (kInlined | kAbsorbed | kCoOutput | kGrouped))) continue;   // a co-output comes with its root
     rule_fn rule = g_rules[t->op];
     if (!rule) { rc = fail(RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op)); break; }
     int st = RAI_ERR_UNSUPPORTED;
-    if (t->flags & kRoot) {
-      const Composite &c = g_comps[t->comp];
-      st = run_composite(t, c);
-      if (st == RAI_OK) {
-        ++g_stats.kernel_launches;
-        ++g_stats.composed_regions;
-        g_stats.composed_nodes += c.interior.size() + 1;
-      } else if (st == RAI_ERR_BAD_STRIDE || st == RAI_ERR_UNSUPPORTED || st == RAI_ERR_BAD_SHAPE || st == RAI_ERR_BAD_DTYPE) {
-        // the fused launcher declines these operands: evaluate the recorded nodes one by one instead
-        drop_storage(t);
-        st = eval_pending_inputs(t);
-        if (st == RAI_OK) st = rule(t);
-      }
+    if (t->flags & kGroupLead) {
+      st = run_linear_group(g_groups[t->group]);
+    } else if (t->flags & kRoot) {
+      st = run_root(t);
     } else if (elementwise(t) && has_inlined_input(t)) {
       // the rules of the inlined members must exist too: fusion never hides a missing rule
       st = eval_region(t);

@@ -401,6 +401,87 @@ def test_linear_takes_its_activation_and_one_residual(hip, dt):
     assert_close(from_storage(composed, dt), oo.add(onn.silu(y, dt), y, dt), dt, "silu(y) + y")
 
 
+def test_linears_of_one_row_share_a_launch(hip, monkeypatch):
+    """A decode step's q, k, v projections and first MLP Linear (phi2.rs:293-297) read one normalised row: at one row
+    they run as one launch, the LayerNorm in its prologue when nothing else reads it.  Against the oracle, against the
+    same graph with the grouping off (RAI_HIP_GRAPH_NO_LINEAR_GROUPS=1; same bits when no norm is folded in), and with a
+    fifth Linear on the same row (a second launch; the norm is then materialised)."""
+    dt, K = "bf16", 256
+    rng = np.random.default_rng(31)
+    x = rand(rng, (1, 1, K), dt)
+    lw, lb = rnd(1.0 + 0.1 * rng.standard_normal(K).astype(np.float32), dt), rand(rng, (K,), dt, 0.1)
+    shapes = [64, 32, 48, 512, 40]
+    ws = [rand(rng, (n, K), dt, 0.1) for n in shapes]
+    bs = [rand(rng, (n,), dt) for n in shapes]
+    params = [dev(a, dt) for a in ws + bs + [lw, lb]]
+    g.eval_all(params)
+    wd, bd, lwd, lbd = params[:5], params[5:10], params[10], params[11]
+
+    def build(norm, count):
+        xt = dev(x, dt)
+        h = g.layer_norm(xt, lwd, lbd, 1e-5) if norm else xt
+        outs = [g.linear(h, wd[i], bd[i]) for i in range(count)]
+        if count > 3:
+            outs[3] = outs[3].new_gelu()
+        return outs
+
+    def want(norm, count):
+        h = onn.layer_norm(x, lw, lb, 1e-5, dt) if norm else x
+        outs = [onn.linear(h, ws[i], bs[i], dt) for i in range(count)]
+        if count > 3:
+            outs[3] = onn.new_gelu(outs[3], dt)
+        return outs
+
+    def evaluate(norm, count):
+        g.stats(reset=True)
+        outs = build(norm, count)
+        g.eval_all(outs)
+        return [o.as_storage() for o in outs], g.stats()
+
+    for norm, count, launches in ((True, 4, 1), (False, 4, 1), (True, 5, 3), (False, 2, 1)):
+        got, st = evaluate(norm, count)
+        assert st["kernel_launches"] == launches, (norm, count, st)
+        for i, (a, b) in enumerate(zip(got, want(norm, count))):
+            assert_close(from_storage(a, dt), b, dt, f"grouped linear {i} norm={norm} count={count}")
+        monkeypatch.setenv("RAI_HIP_GRAPH_NO_LINEAR_GROUPS", "1")
+        plain, st_p = evaluate(norm, count)
+        monkeypatch.delenv("RAI_HIP_GRAPH_NO_LINEAR_GROUPS")
+        assert st_p["kernel_launches"] == count + (1 if norm else 0), st_p
+        for i, (a, b) in enumerate(zip(got, plain)):
+            if norm and count <= 4:
+                assert_close(from_storage(a, dt), from_storage(b, dt), dt, f"grouped vs single linear {i}")
+            else:
+                np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.parametrize("k1,k2,n", [(64, 1024, 96), (2560, 10240, 2560), (512, 256, 40)])
+def test_two_linears_and_the_layer_input_of_one_row_share_a_launch(hip, monkeypatch, k1, k2, n):
+    """(dense(attn) + fc2(act)) + x of DecoderLayer::fwd (phi2.rs:298) at one row: one launch that streams both weight
+    matrices; two launches with the grouping off; both against the oracle's node-by-node sums."""
+    dt = "bf16"
+    rng = np.random.default_rng(37)
+    x1, x2, r = rand(rng, (1, 1, k1), dt), rand(rng, (1, 1, k2), dt), rand(rng, (1, 1, n), dt)
+    w1, w2 = rand(rng, (n, k1), dt, 0.05), rand(rng, (n, k2), dt, 0.02)
+    b1, b2 = rand(rng, (n,), dt), rand(rng, (n,), dt)
+    params = [dev(a, dt) for a in (w1, w2, b1, b2)]
+    g.eval_all(params)
+    want = oo.add(oo.add(onn.linear(x1, w1, b1, dt), onn.linear(x2, w2, b2, dt), dt), r, dt)
+
+    def evaluate():
+        g.stats(reset=True)
+        out = (g.linear(dev(x1, dt), params[0], params[2]) + g.linear(dev(x2, dt), params[1], params[3])) + dev(r, dt)
+        got = from_storage(out.as_storage(), dt)
+        return got, g.stats()
+
+    got, st = evaluate()
+    assert st["kernel_launches"] == 1 and st["composed_regions"] == 2, st
+    assert_close(got, want, dt, "two linears + x, one launch")
+    monkeypatch.setenv("RAI_HIP_GRAPH_NO_LINEAR_GROUPS", "1")
+    plain, st_p = evaluate()
+    assert st_p["kernel_launches"] == 2 and st_p["composed_regions"] == 2, st_p
+    assert_close(plain, want, dt, "two linears + x, two launches")
+
+
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 def test_cache_concatenation_appends_in_place(hip, dt):
     # cat([cache, new], 2) step after step, as the models' key / value caches grow: after the first growth only the
