@@ -400,6 +400,39 @@ def run_gemm_tiles(args):
           {"weights": "cold (rotating copies)" if args.cold else "warm (one copy)", "tiles": rows})
 
 
+def run_peaks(args):
+    """What this GPU sustains with no workload around the loop (rai_hip_measure_peak, include/rai_hip_peaks.h): matrix
+    pipes alone and with LDS fragment reads beside them, LDS reads alone, a plain 1 GiB read and copy, and 64 KB tile
+    staging global -> LDS by every CU at once, both ways.  The roofline fractions elsewhere are against the published
+    peaks; these are the ceilings the kernels actually meet."""
+    from rai_amd import _lib
+    from rai_amd.hip import measure_peak
+    _lib.call("rai_hip_init", 0)
+    launches = max(10, args.steps)
+    out = {}
+    gib = 1 << 30
+    for label, kind, nbytes in (("mfma_bf16", "mfma_bf16", 0), ("mfma_bf16_lds", "mfma_bf16_lds", 0), ("lds_read", "lds_read", 0),
+                                ("hbm_read", "hbm_read", gib), ("hbm_copy", "hbm_copy", gib),
+                                ("stage_dma_2MiB", "stage_dma", 2 << 20), ("stage_vgpr_2MiB", "stage_vgpr", 2 << 20),
+                                ("stage_dma_32MiB", "stage_dma", 32 << 20), ("stage_vgpr_32MiB", "stage_vgpr", 32 << 20)):
+        for _ in range(max(0, args.warmup)):
+            measure_peak(kind, nbytes, 1)
+        sec, work = measure_peak(kind, nbytes, launches)
+        rate = work / sec
+        if kind.startswith("mfma"):
+            out[label] = {"TFLOP/s": round(rate / 1e12, 1), "frac_of_2.5_PFLOP/s": round(rate / 2.5e15, 3), "us_per_launch": round(sec * 1e6, 1)}
+        elif kind == "hbm_copy":
+            out[label] = {"GB/s_read_plus_written": round(2 * rate / 1e9, 1), "frac_of_8_TB/s": round(2 * rate / 8e12, 3),
+                         "us_per_launch": round(sec * 1e6, 1)}
+        elif kind == "hbm_read":
+            out[label] = {"GB/s": round(rate / 1e9, 1), "frac_of_8_TB/s": round(rate / 8e12, 3), "us_per_launch": round(sec * 1e6, 1)}
+        else:
+            out[label] = {"GB/s_per_CU": round(rate / 1e9 / 256, 1), "GB/s": round(rate / 1e9, 1), "us_per_launch": round(sec * 1e6, 1)}
+    mf = out["mfma_bf16"]
+    _line("bf16 MFMA ceiling measured on 1 MI355X (matrix pipes alone)", mf["TFLOP/s"], "TFLOP/s", launches, args.warmup,
+          mf["us_per_launch"] / 1e3, "ceiling loops of rai_hip_measure_peak: no model, no tensors", {"peaks": out})
+
+
 def run_phi2_graph(args, n_new=16):
     """The drop-in path: Phi-2 recorded node for node through the lazy-graph API the way rai-models/src/llm/phi2.rs
     builds it (tests/graph_models.py, KV cache by concatenation) and evaluated by the C++ evaluator with its
@@ -469,7 +502,7 @@ def main():
                     help="tokens decoded through the lazy-graph path for the graph_decode_* fields (0: skip)")
     ap.add_argument("--cold", action="store_true",
                     help="gemm-tiles: rotate over weight copies so every launch reads its weight from HBM, as in a model")
-    ap.add_argument("--workload", default="phi2-decode", choices=["phi2-decode", "qwen2-prefill", "gemma-decode", "ops", "gemm-tiles"],
+    ap.add_argument("--workload", default="phi2-decode", choices=["phi2-decode", "qwen2-prefill", "gemma-decode", "ops", "gemm-tiles", "peaks"],
                     help="phi2-decode is the headline line; the others are the remaining configurations of the path")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -482,6 +515,8 @@ def main():
         return run_ops(args)
     if args.workload == "gemm-tiles":
         return run_gemm_tiles(args)
+    if args.workload == "peaks":
+        return run_peaks(args)
 
     from rai_amd import synthetic
     from rai_amd.hip import sync

@@ -151,6 +151,12 @@ _T = C.c_void_p  # rai_tensor *
 _I64P = C.POINTER(_i64)
 _I32P = C.POINTER(_i32)
 # include/rai_graph.h: name -> (restype, argtypes)
+# include/rai_hip_peaks.h (measurement aid)
+PEAK_PROTOTYPES = {
+    "rai_hip_measure_peak": [C.c_int, C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)],
+}
+PEAK_KINDS = {"mfma_bf16": 0, "mfma_bf16_lds": 1, "lds_read": 2, "hbm_read": 3, "hbm_copy": 4, "stage_dma": 5, "stage_vgpr": 6}
+
 GRAPH_PROTOTYPES = {
     "rai_full": (_T, [_dbl, _i32, _I64P, _i32, _i32]),
     "rai_arange": (_T, [_dbl, _dbl, _dbl, _i32, _i32]),
@@ -215,7 +221,7 @@ def load():
     lib = C.CDLL(str(LIB_PATH))
     lib.rai_hip_last_error.restype = C.c_char_p
     lib.rai_hip_last_error.argtypes = []
-    for name, args in PROTOTYPES.items():
+    for name, args in list(PROTOTYPES.items()) + list(PEAK_PROTOTYPES.items()):
         fn = getattr(lib, name)  # AttributeError if the symbol is missing
         fn.restype = C.c_int
         fn.argtypes = args

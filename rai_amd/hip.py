@@ -181,3 +181,11 @@ def device_count():
     n = C.c_int(0)
     st = _lib.load().rai_hip_device_count(C.byref(n))
     return n.value if st == 0 else 0
+
+
+def measure_peak(kind, nbytes=0, launches=10, dev=0):
+    """One of the library's ceiling loops (include/rai_hip_peaks.h; kind: a key of _lib.PEAK_KINDS): returns
+    (seconds per launch, work per launch in flops or bytes)."""
+    sec, work = C.c_double(0.0), C.c_double(0.0)
+    call("rai_hip_measure_peak", dev, _lib.PEAK_KINDS[kind], int(nbytes), int(launches), C.byref(sec), C.byref(work))
+    return sec.value, work.value

@@ -12,8 +12,8 @@ import pytest
 ROOT = Path(__file__).resolve().parents[1]
 
 
-def header_functions():
-    text = (ROOT / "include" / "rai_hip.h").read_text()
+def header_functions(header="rai_hip.h"):
+    text = (ROOT / "include" / header).read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(rai_hip_\w+)\s*\(", text)))
 
@@ -29,6 +29,16 @@ def test_library_exports_every_declared_symbol():
     declared = set(names)
     bound = set(_lib.PROTOTYPES) | {"rai_hip_last_error"}
     assert bound == declared, (sorted(bound - declared), sorted(declared - bound))
+    # the measurement aid of include/rai_hip_peaks.h
+    peaks = header_functions("rai_hip_peaks.h")
+    assert peaks == sorted(_lib.PEAK_PROTOTYPES), peaks
+    for n in peaks:
+        assert hasattr(so, n), f"{n} declared in rai_hip_peaks.h but not exported"
+    text = (ROOT / "include" / "rai_hip_peaks.h").read_text()
+    for name, val in re.findall(r"RAI_PEAK_(\w+)\s*=\s*(\d+)", text):
+        assert _lib.PEAK_KINDS[name.lower()] == int(val)
+    # every header of include/ is covered by one of the checks of this file or of test_graph_host.py
+    assert sorted(p.name for p in (ROOT / "include").glob("*.h")) == ["rai_graph.h", "rai_hip.h", "rai_hip_peaks.h"]
 
 
 def test_ctypes_structs_match_header_layout():
