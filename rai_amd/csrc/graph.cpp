@@ -958,12 +958,15 @@ bool act_linear(Matcher &m, rai_tensor *t, rai_tensor **x, rai_tensor **w, rai_t
 // A Linear as the model code records it, widened by what follows it directly: the activation applied to its output
 // (MLP::fwd phi2.rs:99-101, qwen2.rs:100-104) and / or one tensor added to the result (the residual sums of
 // DecoderLayer::fwd phi2.rs:298, qwen2.rs:262-265), all of which the Linear launcher applies in its epilogue.  A plain
-// product without bias, activation or residual is left to the MatMul rule (one launch either way).
+// product without bias, activation or residual is left to the MatMul rule (one launch either way) unless it has a
+// single row: then it is taken, so that it can share a launch with the other Linears of that row (the bias-free
+// q / k / v and gate / up projections of gemma.rs and qwen2.rs in a decode step).
 bool match_linear(rai_tensor *t, Composite *c) {
   rai_tensor *x = nullptr, *w = nullptr, *bias = nullptr, *res = nullptr;
   int act = -1;
   Matcher m;
-  bool found = act_linear(m, t, &x, &w, &bias, &act) && (bias || act >= 0);
+  const bool one_row = g_group_linears && !t->shape.empty() && numel_of(t->shape) == t->shape.back();
+  bool found = act_linear(m, t, &x, &w, &bias, &act) && (bias || act >= 0 || one_row);
   if (!found && !t->evaluated && t->op == RAI_OP_BINARY && t->sub == RAI_BIN_ADD) {
     for (int side = 0; side < 2 && !found; ++side) {   // linear + r or r + linear
       Matcher mr;
@@ -1449,7 +1452,8 @@ void plan_compositions(const std::vector<rai_tensor *> &tape) {
     rai_tensor *t = tape[ti];
     if ((t->flags & (kAbsorbed | kRoot | kCoOutput)) || !g_rules[t->op]) continue;
     // cheap gate: every composition's root is one of these primitives
-    if (t->op != RAI_OP_BINARY && t->op != RAI_OP_RESHAPE && t->op != RAI_OP_CONCATENATE) continue;
+    const bool row_product = t->op == RAI_OP_MATMUL && g_group_linears && numel_of(t->shape) == t->shape.back();
+    if (t->op != RAI_OP_BINARY && t->op != RAI_OP_RESHAPE && t->op != RAI_OP_CONCATENATE && !row_product) continue;
     if (claim_two_linears_and_residual(t)) continue;
     for (match_fn f : kMatchers) {
       Composite c = {};

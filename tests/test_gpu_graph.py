@@ -454,6 +454,43 @@ def test_linears_of_one_row_share_a_launch(hip, monkeypatch):
                 np.testing.assert_array_equal(a, b)
 
 
+@pytest.mark.parametrize("arch", ["qwen2", "gemma"])
+def test_bias_free_linears_of_one_row_are_grouped_too(hip, monkeypatch, arch):
+    """A decode step of gemma.rs / qwen2.rs at batch 1: q, k, v (no bias in Gemma) behind one RMSNorm, gate and up behind
+    the other.  Each norm and its Linears are one launch; the whole model agrees with the oracle step for step, with
+    the grouping on and off."""
+    from oracle import qwen2
+    from tests.graph_models import SeqGraph
+    dt = "bf16"
+    if arch == "qwen2":
+        cfg = qwen2.Config("qwen2", 300, 128, 256, 2, 4, 2, "silu", max_position_embeddings=64, rope_theta=1e6, head_dim=32)
+    else:
+        cfg = qwen2.Config("gemma", 300, 128, 256, 2, 4, 1, "gelu", max_position_embeddings=64, head_dim=32)
+    params = qwen2.random_params(cfg, dt, seed=0)
+    rng = np.random.default_rng(29)
+    for k in params:
+        if k.endswith("norm.weight") or k.endswith(".bias"):
+            params[k] = rnd(params[k] + 0.1 * rng.standard_normal(params[k].shape).astype(np.float32), dt)
+    launches = {}
+    for grouped in (True, False):
+        if not grouped:
+            monkeypatch.setenv("RAI_HIP_GRAPH_NO_LINEAR_GROUPS", "1")
+        ref = qwen2.Model(cfg, params, dt)
+        model = SeqGraph(cfg, {k: dev(v, dt) for k, v in params.items()}, dt)
+        ids = np.random.Generator(np.random.PCG64(3)).integers(0, cfg.vocab_size, (1, 9)).astype(np.uint32)
+        for step in range(4):
+            g.stats(reset=True)
+            got = from_storage(model.fwd(Tensor.from_array(ids, "u32")).as_storage(), dt)[:, 0, :]
+            want = ref.fwd(ids)
+            assert_close(got, want, dt, f"{arch} one-row graph step {step} grouped={grouped}")
+            launches[grouped] = g.stats()["kernel_launches"]
+            ids = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
+    monkeypatch.delenv("RAI_HIP_GRAPH_NO_LINEAR_GROUPS", raising=False)
+    # per layer: norm + q|k|v, rotary + append + attention, o + x, norm + gate|up, act(gate) * up, down + x1
+    assert launches[True] <= 2 * 6 + 5, launches
+    assert launches[False] >= launches[True] + 2 * 5, launches
+
+
 @pytest.mark.parametrize("k1,k2,n", [(64, 1024, 96), (2560, 10240, 2560), (512, 256, 40)])
 def test_two_linears_and_the_layer_input_of_one_row_share_a_launch(hip, monkeypatch, k1, k2, n):
     """(dense(attn) + fc2(act)) + x of DecoderLayer::fwd (phi2.rs:298) at one row: one launch that streams both weight
