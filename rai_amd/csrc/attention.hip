@@ -448,6 +448,11 @@ static int decode_splits(const AttnDecodeArgs &a, int head_groups) {
   const char *knob = getenv("RAI_HIP_ATTN_SPLITS");  // tuning and test aid, read at every launch
   const int forced = knob ? atoi(knob) : 0;
   int ns = forced > 0 ? forced : (2 * kNumCU + head_groups * a.B - 1) / (head_groups * a.B);
+  // not more blocks than there are runs of 64 keys: below that a block's share no longer pays for its part of the
+  // merge (a 530-key context of 32 heads: 8 splits 1.89 ms per Phi-2 token through the graph path, 16 splits 1.96,
+  // 32 splits 2.34).  The length is the host's when it knows it, the cache's capacity otherwise.
+  const int len = a.pos_dev ? a.Tmax : a.pos_host + 1;
+  if (forced <= 0 && ns > (len + 63) / 64) ns = (len + 63) / 64;
   const int need = (a.Tmax + 1023) / 1024;
   if (ns < need) ns = need;
   if (ns > kDecodeMaxSplits) ns = kDecodeMaxSplits;

@@ -1471,8 +1471,18 @@ void plan_compositions(const std::vector<rai_tensor *> &tape) {
 struct LinearGroup {
   std::vector<rai_tensor *> members;   // tape order; members[0] leads
   rai_tensor *norm;                    // root of the absorbed norm composition, or null
+  // a view between the norm and the Linears that changes nothing at one row (the last-position `narrow` in front of
+  // the head, phi2.rs:343-345), absorbed with the norm; or null
+  rai_tensor *view;
 };
 std::vector<LinearGroup> g_groups;
+
+// An unevaluated Narrow or Reshape that keeps every element (and so, at one row, the layout), seen by the tape only
+bool identity_view(const rai_tensor *v) {
+  return !v->evaluated && in_tape(v) && (v->op == RAI_OP_NARROW || v->op == RAI_OP_RESHAPE) && v->inputs.size() == 1 &&
+         numel_of(v->shape) == numel_of(v->inputs[0]->shape) && v->refs == v->n_users &&
+         !(v->flags & (kOutput | kAbsorbed | kRoot | kCoOutput | kGroupLead | kGrouped | kInlined)) && g_rules[v->op];
+}
 
 bool group_member(const rai_tensor *t) {
   if (!(t->flags & kRoot) || (t->flags & (kGroupLead | kGrouped)) || t->dtype != RAI_BF16) return false;
@@ -1497,7 +1507,7 @@ void plan_linear_groups(const std::vector<rai_tensor *> &tape) {
       if (open[i].x == x && (int)g_groups[open[i].group].members.size() < kGemvGroupMax) gi = open[i].group;
     if (gi < 0) {
       gi = (int)g_groups.size();
-      g_groups.push_back(LinearGroup{{}, nullptr});
+      g_groups.push_back(LinearGroup{{}, nullptr, nullptr});
       open[next] = Open{x, gi};
       next = (next + 1) % 8;
       if (n_open < 8) ++n_open;
@@ -1509,6 +1519,7 @@ void plan_linear_groups(const std::vector<rai_tensor *> &tape) {
     if (g.members.size() < 2) {
       // a single Linear stays by itself unless the norm in front of it can go into its launch
       rai_tensor *x1 = g_comps[g.members[0]->comp].in[0];
+      if (identity_view(x1)) x1 = x1->inputs[0];
       const bool norm_root = !x1->evaluated && in_tape(x1) && (x1->flags & kRoot) && x1->refs == x1->n_users &&
                              (g_comps[x1->comp].kind == COMP_LAYER_NORM || g_comps[x1->comp].kind == COMP_RMS_NORM);
       if (!norm_root) { g.members.clear(); continue; }
@@ -1517,7 +1528,8 @@ void plan_linear_groups(const std::vector<rai_tensor *> &tape) {
     g.members[0]->group = (int)gi;
     for (size_t i = 1; i < g.members.size(); ++i) g.members[i]->flags |= kGrouped;
     // the shared input: a norm composition read by this group only?
-    rai_tensor *x = g_comps[g.members[0]->comp].in[0];
+    rai_tensor *x = g_comps[g.members[0]->comp].in[0], *view = nullptr;
+    if (identity_view(x)) { view = x; x = x->inputs[0]; }
     if (x->evaluated || !in_tape(x) || !(x->flags & kRoot) || (x->flags & (kOutput | kCoOutput | kGroupLead | kGrouped)) || x->refs != x->n_users ||
         x->dtype != RAI_BF16)
       continue;
@@ -1529,10 +1541,16 @@ void plan_linear_groups(const std::vector<rai_tensor *> &tape) {
       for (rai_tensor *n : g_comps[m->comp].interior) n->stamp = stamp;
     }
     bool sealed = true;
+    if (view) {
+      for (int u = 0; u < view->n_users && sealed; ++u) sealed = g_users[view->users_at + u]->stamp == stamp;
+      view->stamp = stamp;
+    }
     for (int u = 0; u < x->n_users && sealed; ++u) sealed = g_users[x->users_at + u]->stamp == stamp;
     if (!sealed) continue;
     g.norm = x;
+    g.view = view;
     x->flags |= kAbsorbed;   // never materialised: the loop passes over it
+    if (view) view->flags |= kAbsorbed;
   }
   for (LinearGroup &g : g_groups)   // a single Linear whose norm stayed outside: an ordinary composition again
     if (g.members.size() == 1 && !g.norm) {
@@ -1664,6 +1682,11 @@ int run_linear_group(const LinearGroup &g) {
     RAI_TRY(run_root(g.norm));
     g.norm->evaluated = true;
     ++g_stats.nodes_evaluated;
+    if (g.view) {
+      RAI_TRY(g_rules[g.view->op](g.view));
+      g.view->evaluated = true;
+      ++g_stats.nodes_evaluated;
+    }
   }
   for (rai_tensor *m : g.members) {
     st = run_root(m);

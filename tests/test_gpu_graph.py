@@ -454,6 +454,28 @@ def test_linears_of_one_row_share_a_launch(hip, monkeypatch):
                 np.testing.assert_array_equal(a, b)
 
 
+def test_head_takes_the_final_norm_through_the_last_position_view(hip, monkeypatch):
+    """Model::fwd of phi2.rs ends with final_layernorm, narrow to the last position, lm_head.  At one row the narrow
+    keeps every element, and norm + view + Linear are one launch; with more rows the norm stays a launch of its own."""
+    dt, K, N = "bf16", 256, 1000
+    rng = np.random.default_rng(41)
+    lw, lb = rnd(1.0 + 0.1 * rng.standard_normal(K).astype(np.float32), dt), rand(rng, (K,), dt, 0.1)
+    w, b = rand(rng, (N, K), dt, 0.1), rand(rng, (N,), dt)
+    params = [dev(a, dt) for a in (lw, lb, w, b)]
+    g.eval_all(params)
+    for rows, launches in ((1, 1), (5, 2)):
+        x = rand(rng, (1, rows, K), dt)
+        g.stats(reset=True)
+        def head():   # the handles of the norm and of the view end with the function, as in Model::fwd
+            h = g.layer_norm(dev(x, dt), params[0], params[1], 1e-5).narrow(1, rows - 1, 1)
+            return g.linear(h, params[2], params[3])
+        got = from_storage(head().as_storage(), dt)
+        st = g.stats()
+        want = onn.linear(onn.layer_norm(x, lw, lb, 1e-5, dt)[:, rows - 1:, :], w, b, dt)
+        assert_close(got, want, dt, f"head behind the final norm, {rows} rows")
+        assert st["kernel_launches"] == launches, (rows, st)
+
+
 @pytest.mark.parametrize("arch", ["qwen2", "gemma"])
 def test_bias_free_linears_of_one_row_are_grouped_too(hip, monkeypatch, arch):
     """A decode step of gemma.rs / qwen2.rs at batch 1: q, k, v (no bias in Gemma) behind one RMSNorm, gate and up behind
