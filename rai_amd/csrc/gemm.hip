@@ -53,8 +53,8 @@ __global__ void __launch_bounds__(NWV * 64) k_linear_bf16_skinny(LinearArgs a, i
   // With a second product (M == 1) the K axis is the first product's K followed by the second's: position k < K1 is
   // column k of (A, W), position k >= K1 column k - K1 of (A2, W2); a 16-byte chunk never straddles (K1 % 8 == 0).
   const int K1 = a.K, K = a.K + a.K2;
-  const uint16_t *A2 = (const uint16_t *)a.A2 - K1;   // indexed by the position on the joint axis
-  const uint16_t *W2 = (const uint16_t *)a.W2 - K1;
+  const uint16_t *A2 = a.K2 ? (const uint16_t *)a.A2 - K1 : nullptr;   // indexed by the position on the joint axis
+  const uint16_t *W2 = a.K2 ? (const uint16_t *)a.W2 - K1 : nullptr;
   auto x_at = [&](const uint16_t *row, int k) { return k < K1 ? row + k : A2 + k; };
   auto w_at = [&](int n, int k) { return k < K1 ? W + (int64_t)n * a.ldw + k : W2 + (int64_t)n * a.ldw2 + k; };
 
