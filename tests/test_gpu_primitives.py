@@ -409,7 +409,7 @@ def test_fused_linear_bias_act_residual(R, dt, m):
 
 @pytest.mark.parametrize("kernel", ["stream", "skinny", "tile"])
 @pytest.mark.parametrize("m", [9, 16, 31, 64])
-@pytest.mark.parametrize("k,n", [(4096, 200), (1056, 2048), (16384, 64), (96, 50)])
+@pytest.mark.parametrize("k,n", [(4096, 200), (1056, 2048), (16384, 64), (96, 50), (2048, 16384)])
 def test_linear_small_batch_deep_k(R, monkeypatch, m, k, n, kernel):
     # 9..64 rows: the weight-streaming MFMA kernel by default; its two fallbacks (activations in LDS with K split over
     # blocks, and the tile kernel) are forced through the switches the library reads at every call
