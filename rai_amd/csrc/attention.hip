@@ -1060,7 +1060,13 @@ __global__ void __launch_bounds__(NW * KSP * 64) k_flash_prefill_bf16(AttnArgs a
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[u][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
+    // m_run is the exponent every p, the running sum and the output are relative to; it need not be the maximum.
+    // It is moved (and sum and output rescaled) only when some query of the wave has met a score more than kLazy
+    // above its own: after the first tiles that is rare, and the rescaling multiplies -- a third of this loop's
+    // vector instructions at D = 128 -- are skipped.  A p may then reach e^kLazy instead of 1: nothing to bf16 or f32.
+    constexpr float kLazy = 6.0f;
+    const bool move = __builtin_amdgcn_ballot_w64(mx > m_run + kLazy) != 0;   // (-inf + kLazy = -inf: the first tile moves)
+    const float m_new = move ? fmaxf(m_run, mx) : m_run;
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // fully masked so far: every p is exp(-inf) = 0
     constexpr float kLog2e = 1.4426950408889634f;
     const float ml2 = m_safe * kLog2e;
@@ -1081,12 +1087,15 @@ __global__ void __launch_bounds__(NW * KSP * 64) k_flash_prefill_bf16(AttnArgs a
         }
         pf[u][s2] = __builtin_bit_cast(fa_bf16x8, w);
       }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
+    if (move) {
+      l_run *= alpha;
+      m_run = m_new;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    }
+    l_run += psum;
     // ---- O^T += V^T . P^T
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
