@@ -414,12 +414,14 @@ def run_peaks(args):
     for label, kind, nbytes in (("mfma_bf16", "mfma_bf16", 0), ("mfma_bf16_lds", "mfma_bf16_lds", 0), ("lds_read", "lds_read", 0),
                                 ("hbm_read", "hbm_read", gib), ("hbm_copy", "hbm_copy", gib),
                                 ("stage_dma_2MiB", "stage_dma", 2 << 20), ("stage_vgpr_2MiB", "stage_vgpr", 2 << 20),
-                                ("stage_dma_32MiB", "stage_dma", 32 << 20), ("stage_vgpr_32MiB", "stage_vgpr", 32 << 20)):
+                                ("stage_dma_32MiB", "stage_dma", 32 << 20), ("stage_vgpr_32MiB", "stage_vgpr", 32 << 20),
+                                ("gemm_loop_2MiB", "gemm_loop", 2 << 20), ("gemm_loop_32MiB", "gemm_loop", 32 << 20),
+                                ("gemm_loop_1GiB", "gemm_loop", 1 << 30)):
         for _ in range(max(0, args.warmup)):
             measure_peak(kind, nbytes, 1)
         sec, work = measure_peak(kind, nbytes, launches)
         rate = work / sec
-        if kind.startswith("mfma"):
+        if kind.startswith("mfma") or kind == "gemm_loop":
             out[label] = {"TFLOP/s": round(rate / 1e12, 1), "frac_of_2.5_PFLOP/s": round(rate / 2.5e15, 3), "us_per_launch": round(sec * 1e6, 1)}
         elif kind == "hbm_copy":
             out[label] = {"GB/s_read_plus_written": round(2 * rate / 1e9, 1), "frac_of_8_TB/s": round(2 * rate / 8e12, 3),

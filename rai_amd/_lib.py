@@ -155,7 +155,7 @@ _I32P = C.POINTER(_i32)
 PEAK_PROTOTYPES = {
     "rai_hip_measure_peak": [C.c_int, C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)],
 }
-PEAK_KINDS = {"mfma_bf16": 0, "mfma_bf16_lds": 1, "lds_read": 2, "hbm_read": 3, "hbm_copy": 4, "stage_dma": 5, "stage_vgpr": 6}
+PEAK_KINDS = {"mfma_bf16": 0, "mfma_bf16_lds": 1, "lds_read": 2, "hbm_read": 3, "hbm_copy": 4, "stage_dma": 5, "stage_vgpr": 6, "gemm_loop": 7}
 
 GRAPH_PROTOTYPES = {
     "rai_full": (_T, [_dbl, _i32, _I64P, _i32, _i32]),

@@ -153,6 +153,52 @@ __global__ void __launch_bounds__(kPeakThreads) k_peak_stage(const pk_u32x4 *src
   if ((v0.x ^ v0.y ^ v0.z ^ v0.w) == 0x9e3779b9u && stage[1][tid].x == 0x7f4a7c15u) *sink = 1u;
 }
 
+// The tile GEMM's main loop without the GEMM: per iteration (one K tile of 64 of a 256 x 256 block) every wave
+// issues its eight global_load_lds of the next 64 KB stage, reads 24 fragments of 1 KB from the current stage, issues
+// 32 v_mfma_f32_32x32x16_bf16, waits for its loads and meets the block at a barrier.  The stages come out of a buffer
+// of `tiles` tiles as in k_peak_stage, so the same loop can be fed from the L2, from the memory-side cache or from HBM.
+__global__ void __launch_bounds__(kPeakThreads) k_peak_gemm_loop(const pk_u32x4 *src, int64_t tiles, int iters, float *out) {
+  extern __shared__ __attribute__((aligned(16))) pk_u32x4 stage_lds[];   // two stages of 64 KB
+  pk_u32x4(*stage)[4096] = reinterpret_cast<pk_u32x4(*)[4096]>(stage_lds);
+  typedef __attribute__((address_space(3))) void *lds_ptr;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  auto issue = [&](int it) {
+    const pk_u32x4 *t = src + ((int64_t)(blockIdx.x * 7 + it) % tiles) * 4096 + wave * 512 + lane;
+    pk_u32x4 *dst = stage[it & 1] + wave * 512;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) __builtin_amdgcn_global_load_lds((const void *)(t + j * 64), (lds_ptr)(dst + j * 64), 16, 0, 0);
+  };
+  pk_f32x16 acc[8];
+  for (int j = 0; j < 8; ++j)
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+  issue(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int it = 0; it < iters; ++it) {
+    issue(it + 1);
+    const pk_u32x4 *cur = stage[it & 1];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      pk_u32x4 f[12];
+#pragma unroll
+      for (int r = 0; r < 12; ++r) f[r] = cur[((half * 12 + r) * 64 + lane + wave * 37) & 4095];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        pk_bf16x8 a, b;
+        __builtin_memcpy(&a, &f[j % 12], 16);
+        __builtin_memcpy(&b, &f[(j + 5) % 12], 16);
+        acc[j % 8] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j % 8], 0, 0, 0);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the next stage has landed
+    __builtin_amdgcn_s_barrier();                       // ... for every wave, and this stage is free again
+  }
+  float sum = 0.f;
+  for (int j = 0; j < 8; ++j)
+    for (int r = 0; r < 16; ++r) sum += acc[j][r];
+  out[blockIdx.x * kPeakThreads + tid] = sum;
+}
+
 struct Timed {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   ~Timed() {
@@ -172,10 +218,10 @@ extern "C" int rai_hip_measure_peak(int dev, int32_t kind, int64_t bytes, int32_
   if (!st) return RAI_ERR_HIP;
   const int cus = device_cu_count(dev);
   RAI_REQUIRE(cus > 0, RAI_ERR_HIP, "measure_peak: device %d reports no CUs", dev);
-  RAI_REQUIRE(kind >= RAI_PEAK_MFMA_BF16 && kind <= RAI_PEAK_STAGE_VGPR, RAI_ERR_BAD_ARG, "measure_peak: unknown kind %d", kind);
+  RAI_REQUIRE(kind >= RAI_PEAK_MFMA_BF16 && kind <= RAI_PEAK_GEMM_LOOP, RAI_ERR_BAD_ARG, "measure_peak: unknown kind %d", kind);
   if (kind == RAI_PEAK_HBM_READ || kind == RAI_PEAK_HBM_COPY)
     RAI_REQUIRE(bytes >= (1 << 20) && bytes <= ((int64_t)8 << 30) && bytes % 16 == 0, RAI_ERR_BAD_ARG, "measure_peak: 1 MiB .. 8 GiB, a multiple of 16");
-  if (kind == RAI_PEAK_STAGE_DMA || kind == RAI_PEAK_STAGE_VGPR)
+  if (kind == RAI_PEAK_STAGE_DMA || kind == RAI_PEAK_STAGE_VGPR || kind == RAI_PEAK_GEMM_LOOP)
     RAI_REQUIRE(bytes >= 65536 && bytes <= ((int64_t)1 << 30) && bytes % 65536 == 0, RAI_ERR_BAD_ARG, "measure_peak: 64 KiB .. 1 GiB of 64 KiB tiles");
   void *buf = nullptr, *out = nullptr;
   uint32_t *sink = nullptr;
@@ -185,7 +231,7 @@ extern "C" int rai_hip_measure_peak(int dev, int32_t kind, int64_t bytes, int32_
   double work = 0.0;
   int64_t words = 0;
   const bool streams = kind == RAI_PEAK_HBM_READ || kind == RAI_PEAK_HBM_COPY;
-  const bool stages = kind == RAI_PEAK_STAGE_DMA || kind == RAI_PEAK_STAGE_VGPR;
+  const bool stages = kind == RAI_PEAK_STAGE_DMA || kind == RAI_PEAK_STAGE_VGPR || kind == RAI_PEAK_GEMM_LOOP;
   if (streams) {
     words = bytes / 16;
     const size_t total = (size_t)bytes * (kind == RAI_PEAK_HBM_COPY ? 2 : 1);
@@ -198,7 +244,8 @@ extern "C" int rai_hip_measure_peak(int dev, int32_t kind, int64_t bytes, int32_
     int rc = rai_hip_alloc(dev, total, &buf);
     if (rc != RAI_OK) { (void)rai_hip_release(out); return rc; }
     (void)hipMemsetAsync(buf, 0x11, total, st);
-    work = (double)cus * iters * 65536.0;
+    work = kind == RAI_PEAK_GEMM_LOOP ? (double)cus * (kPeakThreads / 64) * (double)iters * 32.0 * (2.0 * 32 * 32 * 16)   // flops
+                                      : (double)cus * iters * 65536.0;
   } else if (kind == RAI_PEAK_LDS_READ) {
     work = (double)cus * (kPeakThreads / 64) * (double)iters * 16.0 * 1024.0;
   } else {
@@ -206,9 +253,9 @@ extern "C" int rai_hip_measure_peak(int dev, int32_t kind, int64_t bytes, int32_
   }
   constexpr size_t kStageLds = 2 * 65536;
   if (stages) {
-    hipError_t e = kind == RAI_PEAK_STAGE_DMA
-                       ? hipFuncSetAttribute((const void *)k_peak_stage<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStageLds)
-                       : hipFuncSetAttribute((const void *)k_peak_stage<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStageLds);
+    const void *fn = kind == RAI_PEAK_STAGE_DMA ? (const void *)k_peak_stage<true>
+                     : kind == RAI_PEAK_STAGE_VGPR ? (const void *)k_peak_stage<false> : (const void *)k_peak_gemm_loop;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStageLds);
     if (e != hipSuccess) {
       (void)rai_hip_release(buf);
       (void)rai_hip_release(out);
@@ -227,6 +274,9 @@ extern "C" int rai_hip_measure_peak(int dev, int32_t kind, int64_t bytes, int32_
         hipLaunchKernelGGL(k_peak_stream<true>, dim3(cus * 8), dim3(256), 0, st, (const pk_u32x4 *)buf, (pk_u32x4 *)buf + words, words, sink);
         break;
       case RAI_PEAK_STAGE_DMA: hipLaunchKernelGGL(k_peak_stage<true>, dim3(cus), dim3(kPeakThreads), kStageLds, st, (const pk_u32x4 *)buf, (int64_t)(bytes / 65536), iters, sink); break;
+      case RAI_PEAK_GEMM_LOOP:
+        hipLaunchKernelGGL(k_peak_gemm_loop, dim3(cus), dim3(kPeakThreads), kStageLds, st, (const pk_u32x4 *)buf, (int64_t)(bytes / 65536), iters, (float *)out);
+        break;
       default: hipLaunchKernelGGL(k_peak_stage<false>, dim3(cus), dim3(kPeakThreads), kStageLds, st, (const pk_u32x4 *)buf, (int64_t)(bytes / 65536), iters, sink); break;
     }
   };

@@ -17,6 +17,7 @@ pytestmark = pytest.mark.gpu
     ("hbm_copy", 1 << 28, 1.0e12, 4.05e12),     # bytes read per second (as many written)
     ("stage_dma", 2 << 20, 2.0e12, 256 * 64 * 2.5e9),
     ("stage_vgpr", 32 << 20, 2.0e12, 256 * 64 * 2.5e9),
+    ("gemm_loop", 2 << 20, 0.5e15, 2.52e15),    # flop/s of the GEMM main loop fed from the L2
 ])
 def test_ceiling_loops_report_plausible_rates(hip, kind, nbytes, low, high):
     measure_peak(kind, nbytes, 1)
