@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
     ("lds_read", 0, 20e12, 256 * 256 * 2.5e9),  # bytes/s over the chip: below 256 B/clk/CU at 2.5 GHz
     ("hbm_read", 1 << 30, 3.0e12, 8.05e12),
     ("hbm_copy", 1 << 28, 1.0e12, 4.05e12),     # bytes read per second (as many written)
-    ("stage_dma", 2 << 20, 2.0e12, 256 * 64 * 2.5e9),
-    ("stage_vgpr", 32 << 20, 2.0e12, 256 * 64 * 2.5e9),
+    ("stage_dma", 2 << 20, 2.0e12, 256 * 128 * 2.5e9),
+    ("stage_vgpr", 32 << 20, 2.0e12, 256 * 128 * 2.5e9),
     ("gemm_loop", 2 << 20, 0.5e15, 2.52e15),    # flop/s of the GEMM main loop fed from the L2
 ])
 def test_ceiling_loops_report_plausible_rates(hip, kind, nbytes, low, high):
