@@ -1235,10 +1235,11 @@ bool match_decode_attention(rai_tensor *t, Composite *c) {
     if (cat->evaluated || cat->op != RAI_OP_CONCATENATE || cat->inputs.size() != 2 || cat->ip[0] != 2 || cat->shape.size() != 4)
       return false;
     const rai_tensor *base = cat->inputs[0], *add = cat->inputs[1];
-    return base->evaluated && base->buf && base->cap_dim == 2 && !base->extended && base->shape[2] + 1 <= base->cap &&
-           add->shape.size() == 4 && add->shape[2] == 1;
+    // a cache without room to grow (the prefill's, or one somebody already appended to) is moved into a buffer with
+    // room by the launch itself (run_decode_attention)
+    return base->evaluated && base->buf && base->shape.size() == 4 && add->shape.size() == 4 && add->shape[2] == 1;
   };
-  if (!growable(kc) || !growable(vc) || kc->inputs[0]->cap != vc->inputs[0]->cap) return false;
+  if (!growable(kc) || !growable(vc)) return false;
   rai_tensor *knew = kc->inputs[1], *vx = vc->inputs[1];
   if (!match_rope(q, &rq) && !match_rope_full(q, &rq)) return false;
   if (!match_rope(knew, &rk) && !match_rope_full(knew, &rk)) return false;
@@ -1281,19 +1282,22 @@ int decode_counters(int dev, size_t bytes, int **out) {
 
 int run_decode_attention(rai_tensor *t, const Composite &c) {
   rai_tensor *qx = c.in[0], *kx = c.in[1], *vx = c.in[2], *kb = c.in[3], *vb = c.in[4];
-  const int64_t B = qx->shape[0], Hq = qx->shape[1], D = qx->shape[3], Hkv = kb->shape[1], T = c.i2, cap = kb->cap;
+  const int64_t B = qx->shape[0], Hq = qx->shape[1], D = qx->shape[3], Hkv = kb->shape[1], T = c.i2;
+  auto has_room = [&](const rai_tensor *b) { return b->cap_dim == 2 && !b->extended && T + 1 <= b->cap; };
+  const bool in_place = has_room(kb) && has_room(vb) && kb->cap == vb->cap;
+  const int64_t cap = in_place ? kb->cap : grown_capacity(T + 1);
   auto rows_ok = [&](const rai_tensor *x, int64_t H) {   // [B, H, 1, D] with the heads of a sequence side by side
     const rai_hip_tensor &v = x->view;
     return v.rank == 4 && v.shape[0] == B && v.shape[1] == H && v.shape[2] == 1 && v.shape[3] == D && v.stride[3] == 1 &&
            (H == 1 || v.stride[1] == D) && (uintptr_t)base_ptr(&v) % 16 == 0 && (B == 1 || v.stride[0] % 8 == 0);
   };
-  auto cache_ok = [&](const rai_tensor *x) {   // [B, Hkv, T, D] laid out for `cap` rows per head
-    const rai_hip_tensor &v = x->view;
+  auto cache_ok = [&](const rai_hip_tensor &v) {   // [B, Hkv, T, D] laid out for `cap` rows per head
     return v.rank == 4 && v.shape[0] == B && v.shape[1] == Hkv && v.shape[2] == T && v.shape[3] == D && v.stride[3] == 1 &&
            v.stride[2] == D && v.stride[1] == cap * D && (B == 1 || v.stride[0] == Hkv * cap * D) &&
            (uintptr_t)base_ptr(&v) % 16 == 0;
   };
-  RAI_REQUIRE(rows_ok(qx, Hq) && rows_ok(kx, Hkv) && rows_ok(vx, Hkv) && cache_ok(kb) && cache_ok(vb) && D % 8 == 0,
+  RAI_REQUIRE(rows_ok(qx, Hq) && rows_ok(kx, Hkv) && rows_ok(vx, Hkv) && D % 8 == 0 && kb->view.rank == 4 && vb->view.rank == 4 &&
+                  kb->view.shape[2] == T && vb->view.shape[2] == T && (!in_place || (cache_ok(kb->view) && cache_ok(vb->view))),
               RAI_ERR_BAD_STRIDE, "decode attention: operand layout not served");
   const rai_hip_tensor &ct = c.in[5]->view, &sn = c.in[6]->view;
   RAI_REQUIRE(is_contiguous(&ct) && is_contiguous(&sn) && ct.rank == 2 && ct.shape[1] == c.i0 && T < ct.shape[0] &&
@@ -1304,16 +1308,48 @@ int run_decode_attention(rai_tensor *t, const Composite &c) {
   void *ws = nullptr;
   int *counters = nullptr;
   RAI_TRY(decode_counters(t->dev, attention_decode_counter_bytes((int)B, (int)Hq), &counters));
-  RAI_TRY(rai_hip_alloc(t->dev, attention_decode_ws_bytes((int)B, (int)Hq, (int)D), &ws));
-  RAI_TRY(alloc_output(t));
+  // caches without room: both move, once, into buffers laid out for `cap` rows per head (two copies; from then on
+  // every step appends in place)
+  rai_hip_tensor cache_view[2] = {kb->view, vb->view};
+  void *grown[2] = {nullptr, nullptr};
+  if (!in_place) {
+    for (int i = 0; i < 2; ++i) {
+      const rai_tensor *base = i ? vb : kb;
+      int rc = rai_hip_alloc(t->dev, (size_t)(B * Hkv * cap * D) * dtype_size(t->dtype), &grown[i]);
+      rai_hip_tensor &v = cache_view[i];
+      if (rc == RAI_OK) {
+        memset(&v, 0, sizeof(v));
+        v.data = grown[i];
+        v.dtype = t->dtype;
+        v.rank = 4;
+        v.shape[0] = B; v.shape[1] = Hkv; v.shape[2] = T; v.shape[3] = D;
+        v.stride[0] = Hkv * cap * D; v.stride[1] = cap * D; v.stride[2] = D; v.stride[3] = 1;
+        ++g_stats.kernel_launches;
+        rc = rai_hip_copy(t->dev, &base->view, &v);
+      }
+      if (rc != RAI_OK) {
+        for (int j = 0; j <= i; ++j)
+          if (grown[j]) (void)rai_hip_release(grown[j]);
+        return rc;
+      }
+    }
+  }
+  auto drop_grown = [&]() {
+    for (int j = 0; j < 2; ++j)
+      if (grown[j]) (void)rai_hip_release(grown[j]);
+  };
+  if (!cache_ok(cache_view[0]) || !cache_ok(cache_view[1])) { drop_grown(); return fail(RAI_ERR_BAD_STRIDE, "decode attention: cache layout not served"); }
+  int arc = rai_hip_alloc(t->dev, attention_decode_ws_bytes((int)B, (int)Hq, (int)D), &ws);
+  if (arc == RAI_OK) arc = alloc_output(t);
+  if (arc != RAI_OK) { if (ws) (void)rai_hip_release(ws); drop_grown(); return arc; }
   AttnDecodeArgs a;
   memset(&a, 0, sizeof(a));
   a.qkv = base_ptr(&qx->view);
   a.k_new = base_ptr(&kx->view);
   a.v_new = base_ptr(&vx->view);
   a.q_row_stride = qx->view.stride[0]; a.k_row_stride = kx->view.stride[0]; a.v_row_stride = vx->view.stride[0];
-  a.kcache = base_ptr(&kb->view);
-  a.vcache = base_ptr(&vb->view);
+  a.kcache = base_ptr(&cache_view[0]);
+  a.vcache = base_ptr(&cache_view[1]);
   a.out = t->view.data;
   a.out_row_stride = Hq * D;
   a.cos_t = base_ptr(&ct); a.sin_t = base_ptr(&sn);
@@ -1328,16 +1364,21 @@ int run_decode_attention(rai_tensor *t, const Composite &c) {
   a.counters = counters;
   const int rc = launch_attention_decode(st, a);
   (void)rai_hip_release(ws);   // stream order keeps it intact until the launch is through
-  RAI_TRY(rc);
-  // the caches, one row longer, in the old caches' buffers
+  if (rc != RAI_OK) { drop_grown(); return rc; }
+  // the caches, one row longer: in the old caches' buffers, or in the grown ones, which the new nodes then own
   for (int i = 0; i < 2; ++i) {
     rai_tensor *cat = c.co[i], *base = cat->inputs[0];
-    rai_hip_tensor v = base->view;
+    rai_hip_tensor v = cache_view[i];
     v.shape[2] = T + 1;
-    alias_storage(cat, base, v);
+    if (in_place) {
+      alias_storage(cat, base, v);
+      base->extended = true;
+    } else {
+      cat->view = v;
+      cat->buf = grown[i];
+    }
     cat->cap_dim = 2;
-    cat->cap = base->cap;
-    base->extended = true;
+    cat->cap = cap;
     cat->evaluated = true;
     ++g_stats.nodes_evaluated;
   }
