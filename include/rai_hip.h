@@ -131,14 +131,17 @@ int rai_hip_init(int dev);
 int rai_hip_sync(int dev);
 
 /* Ref-counted device allocation (refcount starts at 1).  Freed blocks go back to
- * a per-device size-class pool, so steady-state evaluation calls no hipMalloc.
+ * a per-device size-class pool, so steady-state evaluation calls no hipMalloc;
+ * blocks of up to 32 MiB are cut from 256 MiB slabs, so the first use of a size
+ * costs no hipMalloc of its own either.
  * Replaces candle's Arc<Storage> behind rai-core/src/tensor.rs:151-165 set_data. */
 int rai_hip_alloc(int dev, size_t bytes, void **out);
 int rai_hip_retain(void *ptr);
 int rai_hip_release(void *ptr);
 /* bytes currently handed out / bytes held in the pool / number of real hipMalloc calls */
 int rai_hip_mem_stats(int dev, uint64_t *in_use, uint64_t *pooled, uint64_t *n_device_mallocs);
-/* Return pooled blocks to the driver. */
+/* Return pooled blocks to the driver (blocks cut from a slab stay pooled: a slab is
+ * never handed back piecemeal). */
 int rai_hip_trim(int dev);
 
 /* Host<->device copies of raw bytes.  h2d is stream-ordered and returns after the

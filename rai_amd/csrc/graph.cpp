@@ -2172,8 +2172,38 @@ int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
   const auto t_planned = std::chrono::steady_clock::now();
   g_stats.plan_ns += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(t_planned - t_start).count();
   int rc = RAI_OK;
-  for (rai_tensor *t : tape) {
-    if (t->evaluated || (t->flags & (kInlined | kAbsorbed | kCoOutput | kGrouped))) continue;   // a co-output comes with its root
+  // The walk owns one reference to every tape node and hands it back as it passes the node, after dropping the
+  // node's inputs (eval.rs:45-49 detaches inside the loop): an intermediate result is freed as soon as its last
+  // consumer has run, so a long tape reuses the buffers of its early nodes instead of holding every activation of
+  // every layer until the end.  (Taken after planning, which compares reference counts with in-tape uses.)
+  for (rai_tensor *t : tape) ++t->refs;
+  // A composition's operands are kept by pointer; most are held by the root's own inputs, but one reached behind a
+  // shared view (the rotary tables) is not once that view has been passed: the plan holds a reference of its own to
+  // every operand until the composition's root has run (or, for roots that never run themselves, until the end).
+  std::vector<char> operands_held(g_comps.size(), 1);
+  auto release_operands = [&](int ci) {
+    if (ci < 0 || !operands_held[ci]) return;
+    operands_held[ci] = 0;
+    for (rai_tensor *o : g_comps[ci].in)
+      if (o) rai_tensor_release(o);
+  };
+  for (const Composite &c : g_comps)
+    for (rai_tensor *o : c.in)
+      if (o) ++o->refs;
+  std::vector<rai_tensor *> late;   // co-outputs: materialised by a root further on, handed back after the walk
+  size_t at = 0;
+  for (; at < tape.size(); ++at) {
+    rai_tensor *t = tape[at];
+    auto hand_back = [&]() {
+      if (t->flags & kCoOutput) { late.push_back(t); return; }
+      if ((t->flags & kRoot) && t->evaluated) release_operands(t->comp);
+      if (t->evaluated && !retain_graph) detach(t);
+      rai_tensor_release(t);
+    };
+    if (t->evaluated || (t->flags & (kInlined | kAbsorbed | kCoOutput | kGrouped))) {   // a co-output comes with its root
+      hand_back();
+      continue;
+    }
     rule_fn rule = g_rules[t->op];
     if (!rule) { rc = fail(RAI_ERR_UNSUPPORTED, "Unimplemented { op: %s, device: Hip }", op_name(t->op)); break; }
     int st = RAI_ERR_UNSUPPORTED;
@@ -2199,10 +2229,14 @@ int rai_eval(rai_tensor *const *outputs, int32_t n, int32_t retain_graph) {
     }
     t->evaluated = true;
     ++g_stats.nodes_evaluated;
+    hand_back();
   }
-  if (rc == RAI_OK && !retain_graph)
-    for (rai_tensor *t : tape)
-      if (t->evaluated) detach(t);
+  for (rai_tensor *t : late) {
+    if (rc == RAI_OK && t->evaluated && !retain_graph) detach(t);
+    rai_tensor_release(t);
+  }
+  for (; at < tape.size(); ++at) rai_tensor_release(tape[at]);   // after a failure: the nodes the walk never passed
+  for (size_t ci = 0; ci < g_comps.size(); ++ci) release_operands((int)ci);
   g_stats.run_ns += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t_planned).count();
   return rc;
 }

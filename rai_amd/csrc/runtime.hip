@@ -4,6 +4,7 @@
 #include <map>
 #include <mutex>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "common.h"
@@ -39,6 +40,13 @@ struct DeviceCtx {
   std::mutex mu;
   std::map<size_t, std::vector<void *>> pool;  // size class -> free blocks
   uint64_t in_use = 0, pooled = 0, n_mallocs = 0;
+  // Blocks of up to kCarveMax bytes are cut from slabs of kSlabBytes (one hipMalloc per slab instead of one per first
+  // use of a size: a 32-layer prefill through the graph evaluator asks for ~80 sizes it has not seen, at ~0.2 ms per
+  // hipMalloc).  A cut block lives in the pool like any other once released; only whole hipMalloc blocks go back to
+  // the driver in rai_hip_trim.
+  char *slab = nullptr;
+  size_t slab_left = 0;
+  std::unordered_set<void *> carved;
   void *ws = nullptr;
   size_t ws_bytes = 0;
   unsigned long long *index_errors = nullptr;
@@ -51,6 +59,8 @@ static constexpr int kMaxDev = 16;
 static DeviceCtx g_ctx[kMaxDev];
 static std::mutex g_mu;
 static std::unordered_map<void *, Block> g_blocks;  // live (handed out) blocks
+
+static constexpr size_t kSlabBytes = size_t(256) << 20, kCarveMax = size_t(32) << 20;
 
 static size_t size_class(size_t bytes) {
   if (bytes == 0) bytes = 1;
@@ -274,6 +284,25 @@ int rai_hip_alloc(int dev, size_t bytes, void **out) {
       c->pooled -= cls;
     }
   }
+  if (!p && cls <= kCarveMax) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (c->slab_left < cls) {   // the rest of the old slab stays unused (at most one block's worth)
+      void *fresh = nullptr;
+      if (hipSetDevice(dev) == hipSuccess && hipMalloc(&fresh, kSlabBytes) == hipSuccess) {
+        c->slab = (char *)fresh;
+        c->slab_left = kSlabBytes;
+        c->n_mallocs++;
+      } else {
+        (void)hipGetLastError();   // no room for a slab: a block of its own below
+      }
+    }
+    if (c->slab_left >= cls) {
+      p = c->slab;
+      c->slab += cls;
+      c->slab_left -= cls;
+      c->carved.insert(p);
+    }
+  }
   if (!p) {
     RAI_HIP_TRY(hipSetDevice(dev));
     hipError_t e = hipMalloc(&p, cls);
@@ -344,10 +373,15 @@ int rai_hip_trim(int dev) {
   RAI_HIP_TRY(hipSetDevice(dev));
   RAI_HIP_TRY(hipStreamSynchronize(c->stream));
   std::lock_guard<std::mutex> lk(c->mu);
-  for (auto &kv : c->pool)
-    for (void *p : kv.second) (void)hipFree(p);
-  c->pool.clear();
-  c->pooled = 0;
+  for (auto &kv : c->pool) {
+    std::vector<void *> kept;
+    for (void *p : kv.second) {
+      if (c->carved.count(p)) { kept.push_back(p); continue; }   // part of a slab: stays pooled
+      (void)hipFree(p);
+      c->pooled -= kv.first;
+    }
+    kv.second.swap(kept);
+  }
   return RAI_OK;
 }
 
