@@ -173,6 +173,54 @@ def test_decode_chain_against_launch_per_linear(hip, request, monkeypatch, arch)
     dec.close()
 
 
+@pytest.mark.parametrize("arch", ["qwen2", "gemma"])
+def test_every_sequence_through_a_second_device_path(hip, request, monkeypatch, arch):
+    """The oracle follows three sequences of these batches (a size it covers in minutes); the other 13 / 29 are held
+    here to a second, independent device path: the same prefill and two decode steps once through the default kernels
+    (DMA tile GEMMs with stream-K, streaming MFMA Linears over fragment-order weights with fused norms, MFMA decode
+    attention, captured graph) and once through the register-staged 128 x 128 tile kernel on whole tiles, the
+    LDS-staged small-M Linears over row-major weights, stand-alone norms, the context-split VALU decode attention and
+    plain launches.  Every sequence's logits agree within the dtype's tolerance; tokens are each path's own argmax."""
+    if arch == "qwen2":
+        cfg = qwen2.Config("qwen2", 151936, 1536, 8960, 2, 12, 2, "silu", max_position_embeddings=2048, rope_theta=1e6,
+                           head_dim=128)
+        B, CTX = 16, 1024
+    else:
+        cfg = qwen2.Config("gemma", 256000, 2048, 16384, 2, 8, 1, "gelu", max_position_embeddings=4096, head_dim=256)
+        B, CTX = 32, 2048
+    ids = np.random.Generator(np.random.PCG64(61)).integers(0, cfg.vocab_size, (B, CTX)).astype(np.uint32)
+    second = {"RAI_HIP_GEMM_TILE": "classic", "RAI_HIP_NO_STREAMK": "1", "RAI_HIP_NO_MFMA_STREAM": "1", "RAI_HIP_NO_MFMA_DECODE": "1",
+              "RAI_HIP_NO_FRAG": "1", "RAI_HIP_NO_FUSED_NORM": "1", "RAI_HIP_NO_POST_NORM": "1", "RAI_HIP_NO_GRAPH": "1",
+              "RAI_HIP_NO_SPLIT_CHOICE": "1", "RAI_HIP_NO_FUSED_SPLITK": "1"}
+    runs = {}
+    for label in ("default", "second"):
+        for k, v in second.items():
+            if label == "second":
+                monkeypatch.setenv(k, v)
+            else:
+                monkeypatch.delenv(k, raising=False)
+        dec, _ = build(cfg, B, CTX + 8, request)
+        progress(request, f"{label} path: prefill {B} x {CTX} and two decode steps")
+        logits, tok = dec.forward(ids)
+        steps = [(logits.copy(), tok.copy())]
+        feed = tok if label == "default" else runs["default"][0][1]     # both paths decode the same tokens
+        for s in range(2):
+            logits, tok = dec.forward(feed.reshape(B, 1))
+            steps.append((logits.copy(), tok.copy()))
+            feed = tok if label == "default" else runs["default"][s + 1][1]
+        runs[label] = steps
+        dec.close()
+    for k in second:
+        monkeypatch.delenv(k, raising=False)
+    for s, ((la, ta), (lb, tb)) in enumerate(zip(runs["default"], runs["second"])):
+        assert la.shape == (B, cfg.vocab_size)
+        for b in range(B):
+            assert_close(la[b], lb[b], "bf16", f"{arch} sequence {b}, step {s}: default vs second device path")
+        assert np.array_equal(ta, np.argmax(la, -1).astype(np.uint32))
+        assert np.array_equal(tb, np.argmax(lb, -1).astype(np.uint32))
+
+
+
 def test_decode_chain_barrier_timeout_is_reported(hip, request, monkeypatch):
     """A barrier wait of the chain kernel that expires (forced from the host with a spin limit of one poll): the kernel
     flags the fault, later waits fall through so every wave exits, the call returns an error instead of wrong logits,
