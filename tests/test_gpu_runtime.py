@@ -27,7 +27,7 @@ def test_small_blocks_are_cut_from_slabs_and_pooled(hip):
     # twenty sizes the pool has not seen: at most one slab's worth of hipMalloc
     sizes = [3_000_017 + 700_001 * i for i in range(20)]
     blocks = [alloc(s) for s in sizes]
-    in_use1, _, n1 = stats()
+    in_use1, pooled1, n1 = stats()
     assert n1 - n0 <= 2, (n0, n1)
     assert in_use1 - in_use0 >= sum(sizes)
     addrs = sorted(b.value for b in blocks)
@@ -35,7 +35,8 @@ def test_small_blocks_are_cut_from_slabs_and_pooled(hip):
     for b in blocks:
         _lib.call("rai_hip_release", b)
     in_use2, pooled2, _ = stats()
-    assert in_use2 == in_use0 and pooled2 - pooled0 >= sum(sizes)
+    # everything taken is back in the pool (a warm pool may have served some of the requests itself)
+    assert in_use2 == in_use0 and pooled2 - pooled1 >= sum(sizes) and pooled2 >= pooled0
     # the same sizes again come out of the pool: no hipMalloc, the same addresses
     again = [alloc(s) for s in sizes]
     assert stats()[2] == n1
@@ -54,6 +55,6 @@ def test_small_blocks_are_cut_from_slabs_and_pooled(hip):
     _, pooled3, _ = stats()
     _lib.call("rai_hip_trim", 0)
     _, pooled4, _ = stats()
-    assert pooled3 - pooled4 >= (96 << 20) and pooled4 >= pooled2 - pooled0
+    assert pooled3 - pooled4 >= (96 << 20) and pooled4 >= pooled2 - pooled1
     with pytest.raises(_lib.RaiHipError):
         _lib.call("rai_hip_release", C.c_void_p(12345))
