@@ -152,3 +152,44 @@ def test_persistent_step_with_and_without_lds_staged_weights(hip, monkeypatch):
         check_tokens(np.argmax(runs[0][step], -1), want, "bf16")
         nxt = np.argmax(runs[0][step], -1).astype(np.uint32).reshape(1, 1)
     dec.close()
+
+
+@pytest.mark.parametrize("vocab", [16384, 32768])
+def test_greedy_choice_takes_the_first_maximum_and_passes_over_nans(hip, vocab):
+    # The token choice behind the head product (rai-models/examples/phi2/src/main.rs:76-87 takes the argmax of the
+    # last logits row), at both of its forms: one block scanning the row, and, from 32768 logits on, shares of the row
+    # scanned by many blocks and merged.  Ties and NaNs are planted through the head's bias: rows 100 and 200 (different
+    # shares) and 301, 302 (neighbours) share the largest logit; a NaN at row 7 is passed over; a NaN at row 0 wins
+    # (a scan that starts from element 0 and replaces on a strict comparison never leaves it).
+    from tests.test_gpu_phi2 import to_storage
+    cfg = wide_cfg(vocab_size=vocab, intermediate_size=512)
+    prompt = np.random.Generator(np.random.PCG64(31)).integers(0, cfg.vocab_size, (1, 19)).astype(np.uint32)
+    dec, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
+    logits, tok = dec.forward(prompt)
+    assert tok[0] == int(np.argmax(logits[0]))
+    for _ in range(3):   # single-token steps: the persistent kernel, then the same head and choice
+        logits, tok = dec.forward(np.array([[tok[0]]], np.uint32))
+        assert tok[0] == int(np.argmax(logits[0]))
+    params = phi2.random_params(cfg, "bf16", seed=0)
+    w, b = params["lm_head.weight"].copy(), params["lm_head.bias"].copy()
+    for r in (100, 200, 301, 302):
+        w[r] = 0
+        b[r] = 64.0
+    b[7] = np.nan
+    dec.load_param("lm_head.weight", to_storage(w, "bf16"))
+    dec.load_param("lm_head.bias", to_storage(b, "bf16"))
+    dec.clear_kv_cache()
+    logits, tok = dec.forward(prompt)
+    assert np.isnan(logits[0, 7]) and logits[0, 100] == logits[0, 200] == logits[0, 301] == 64.0
+    assert np.nanmax(logits[0]) == 64.0
+    assert tok[0] == 100
+    b[100] = 0.0
+    b[200] = 0.0
+    dec.load_param("lm_head.bias", to_storage(b, "bf16"))
+    dec.clear_kv_cache()
+    assert dec.forward(prompt)[1][0] == 301
+    b[0] = np.nan
+    dec.load_param("lm_head.bias", to_storage(b, "bf16"))
+    dec.clear_kv_cache()
+    assert dec.forward(prompt)[1][0] == 0
+    dec.close()
