@@ -53,6 +53,26 @@ struct MegaArgs {
   int mute_block;           // this block sends no phase-A packets, so its consumers time out; -1 = none
 };
 
+// The head of the same decoder behind the persistent step: final LayerNorm, the vocabulary product and the greedy
+// choice in one launch (k_phi2_head_choice, one block per CU, the weight stream of the step kernel).
+struct HeadArgs {
+  const uint16_t *W, *bias;       // [V, H] and [V] (bias may be null)
+  const uint16_t *x;              // [H] residual stream after the last layer
+  const uint16_t *ln_w, *ln_b;
+  float ln_eps;
+  int V, H;
+  uint16_t *logits;               // [V], written as the product is rounded
+  unsigned long long *best;       // one (value bits << 32 | row) per block, exchanged inside the launch
+  uint32_t *token, *history;      // history may be null; history[state->step] otherwise
+  DevState *state;                // done is the arrival counter (zero between launches); pos, step, epoch are advanced
+  int dpos, dstep;
+  const uint16_t *embed;          // [V, H]: row `token` times embed_scale becomes x_next (the next step's input)
+  uint16_t *x_next;
+  float embed_scale;
+};
+bool head_choice_eligible(const HeadArgs &a, int num_cu);
+int launch_phi2_head_choice(hipStream_t st, const HeadArgs &a, int num_cu);
+
 unsigned mega_default_spin_limit();
 bool mega_eligible(const MegaArgs &a, int D, int num_cu, const char **why);
 int launch_phi2_decode_step(hipStream_t st, const MegaArgs &a, int D, int num_cu);

@@ -984,6 +984,208 @@ __global__ void __launch_bounds__(kMegaThreads) k_phi2_decode_step(MegaArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0F70);   // nothing still on its way into LDS when the block ends
 }
 
+// ---- the head behind the step -------------------------------------------------------------------------------------
+// logits = LayerNorm(x) . W^T + bias for one row, and the greedy choice on them, in one launch of one block per CU.
+// Every block normalises x once (as the step kernel does at the start of a layer), streams its share of the rows of W
+// through the same register ring (seven stream waves as there: with all eight streaming the launch took 48 us
+// instead of 43; the first sixteen tiles are requested before x is even read),
+// rounds its logits to bf16, stores them and keeps the best of them: the first maximum, NaNs passed over, except
+// that a NaN in row 0 takes the choice (what a scan from element 0 that replaces on a strict comparison gives).  The
+// blocks' bests travel as 8-byte (value, row) words written past the L2; a block counts itself in when its word has
+// reached memory, and the block that counts last, whichever it is, picks among the words, writes the token, copies
+// its embedding row to the next step's input and advances the device-side counters.  Nobody waits for anybody.
+constexpr int kHeadRowsMax = 256;
+
+// whether candidate (v, i) replaces (bv, bi): a NaN value only ever comes with row 0 and is final; row 0xffffffff
+// means nothing seen yet
+__device__ __forceinline__ bool head_replaces(float v, uint32_t i, float bv, uint32_t bi) {
+  if (bv != bv) return false;
+  if (v != v) return true;
+  if (i == 0xffffffffu) return false;
+  return bi == 0xffffffffu || v > bv || (v == bv && i < bi);
+}
+
+template <int KTA>
+__global__ void __launch_bounds__(kMegaThreads) k_phi2_head_choice(HeadArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char hd_smem[];
+  constexpr int H = KTA * 512;
+  uint16_t *xr = reinterpret_cast<uint16_t *>(hd_smem);   // x as it is
+  uint16_t *xn = xr + H;                                   // LayerNorm(x), bf16
+  float *part = reinterpret_cast<float *>(xn + H);         // [rows][kMegaWaves]
+  __shared__ float s_v[kMegaWaves];
+  __shared__ uint32_t s_i[kMegaWaves];
+  __shared__ int s_ticket;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wg = blockIdx.x, G = gridDim.x;
+  const int r0 = (int)((int64_t)a.V * wg / G), r1 = (int)((int64_t)a.V * (wg + 1) / G);
+  const int nrows = r1 - r0;
+
+  const bool streams = wave < kMegaStream;
+  const int tt = nrows * KTA;
+  const int t0 = streams ? tt * wave / kMegaStream : 0, t1 = streams ? tt * (wave + 1) / kMegaStream : 0;
+  MgSplit sp;
+  sp.Wa0 = a.W; sp.Wb0 = a.W; sp.wa_stride = 0; sp.wb_stride = 0; sp.L = 1; sp.H = H; sp.KB = H; sp.KTA = KTA; sp.KTBC = 1;
+  sp.cnt0 = t1 - t0; sp.cnt1 = 0; sp.cnt2 = 0;
+  sp.kc0 = t0 % KTA; sp.kc1 = 0; sp.kc2 = 0;
+  sp.off0 = (int64_t)(r0 + t0 / KTA) * H; sp.off1 = 0; sp.off2 = 0;
+  sp.nx0 = 0; sp.nx1 = 0; sp.nx2 = 0;
+  MgCursor cur;
+  cur.layer = 0; cur.seg = 0; cur.kc = 0; cur.KT = 1; cur.left = 0; cur.jump = 0; cur.step = 0;
+  cur.ptr = a.W;
+  const bool streams_any = sp.cnt0 > 0;
+  if (streams_any) mg_seg_enter(cur, sp, 0, 0);
+  const MgPhase ph = mg_phase(t0, t1, 0, 0, KTA);
+  mg_u32x4 ring[kMegaRing];
+#pragma unroll
+  for (int p = 0; p < kMegaRing; ++p) ring[p] = streams_any ? mg_next_load(cur, sp, lane) : MG_ZERO4;
+
+  // x into LDS, the partial sums to zero (a wave leaves one per row it touches)
+  for (int i = tid; i < H / 2; i += kMegaThreads) reinterpret_cast<uint32_t *>(xr)[i] = reinterpret_cast<const uint32_t *>(a.x)[i];
+  for (int e = tid; e < nrows * kMegaWaves; e += kMegaThreads) part[e] = 0.f;
+  wg_sync();
+  if (wave < KTA) {   // wave u normalises features [512 u, 512 u + 512); every one of them computes the statistics
+    mg_u32x4 xv[KTA];
+#pragma unroll
+    for (int u = 0; u < KTA; ++u) xv[u] = *reinterpret_cast<const mg_u32x4 *>(xr + u * 512 + lane * 8);
+    const mg_u32x4 lw = *reinterpret_cast<const mg_u32x4 *>(a.ln_w + wave * 512 + lane * 8);
+    const mg_u32x4 lb = *reinterpret_cast<const mg_u32x4 *>(a.ln_b + wave * 512 + lane * 8);
+    const uint32_t ones = 0x3f803f80u;
+    float s1 = 0.f, s2 = 0.f;
+    mg_u32x4 mine = MG_ZERO4;
+#pragma unroll
+    for (int u = 0; u < KTA; ++u) {
+      const uint32_t w4[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s1 = mg_dot2(w4[j], ones, s1);
+        s2 = mg_dot2(w4[j], w4[j], s2);
+      }
+      if (wave == u) mine = xv[u];
+    }
+    s1 = mg_wave_sum(s1);
+    s2 = mg_wave_sum(s2);
+    const float mean = s1 / (float)H;
+    float var = s2 / (float)H - mean * mean;
+    var = var > 0.f ? var : 0.f;
+    const float scale = 1.0f / sqrtf(var + a.ln_eps), shift = -mean * scale;
+    const uint32_t xx[4] = {mine.x, mine.y, mine.z, mine.w};
+    const uint32_t ww[4] = {lw.x, lw.y, lw.z, lw.w};
+    const uint32_t bb[4] = {lb.x, lb.y, lb.z, lb.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float y0 = fmaf(fmaf(__uint_as_float(xx[j] << 16), scale, shift), __uint_as_float(ww[j] << 16), __uint_as_float(bb[j] << 16));
+      const float y1 = fmaf(fmaf(__uint_as_float(xx[j] & 0xffff0000u), scale, shift), __uint_as_float(ww[j] & 0xffff0000u),
+                            __uint_as_float(bb[j] & 0xffff0000u));
+      o[j] = pack_bf16x2(y0, y1);
+    }
+    *reinterpret_cast<mg_u32x4 *>(xn + wave * 512 + lane * 8) = mg_u32x4{o[0], o[1], o[2], o[3]};
+  }
+  wg_sync();
+
+  bool staged = false;
+  (void)mg_run_phase(ring, cur, sp, ph, KTA, xn, part, part, nullptr, lane, wave, nullptr, staged);
+  wg_sync();
+
+  // this block's logits and the best of them
+  float bv = -INFINITY;
+  uint32_t bi = 0xffffffffu;
+  for (int e = tid; e < nrows; e += kMegaThreads) {
+    float sacc = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMegaStream; ++w) sacc += part[e * kMegaWaves + w];
+    if (a.bias) sacc += bf16_bits_to_f32(a.bias[r0 + e]);
+    const uint16_t vb = f32_to_bf16_bits(sacc);
+    a.logits[r0 + e] = vb;
+    const float r = bf16_bits_to_f32(vb);
+    const uint32_t n = (uint32_t)(r0 + e);
+    if (r != r) {
+      if (n == 0u) { bv = r; bi = 0u; }
+    } else if (head_replaces(r, n, bv, bi)) {
+      bv = r;
+      bi = n;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const uint32_t oi = (uint32_t)__shfl_xor((int)bi, o, 64);
+    if (head_replaces(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+  }
+  if (lane == 0) { s_v[wave] = bv; s_i[wave] = bi; }
+  wg_sync();
+  if (tid == 0) {
+#pragma unroll
+    for (int w = 1; w < kMegaWaves; ++w)
+      if (head_replaces(s_v[w], s_i[w], bv, bi)) { bv = s_v[w]; bi = s_i[w]; }
+    st_dev64(a.best + wg, ((uint64_t)__float_as_uint(bv) << 32) | bi);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the word has reached memory before this block counts itself in
+    s_ticket = __hip_atomic_fetch_add(&a.state->done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  wg_sync();
+  if (s_ticket != G - 1) return;
+
+  // the last block: every word is in memory
+  if (tid == 0) __hip_atomic_store(&a.state->done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+  bv = -INFINITY;
+  bi = 0xffffffffu;
+  for (int p = tid; p < G; p += kMegaThreads) {
+    const uint64_t pk = ld_dev64(a.best + p);
+    const float v = __uint_as_float((uint32_t)(pk >> 32));
+    const uint32_t i = (uint32_t)pk;
+    if (head_replaces(v, i, bv, bi)) { bv = v; bi = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const uint32_t oi = (uint32_t)__shfl_xor((int)bi, o, 64);
+    if (head_replaces(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+  }
+  if (lane == 0) { s_v[wave] = bv; s_i[wave] = bi; }
+  wg_sync();
+  bv = s_v[0];
+  bi = s_i[0];
+#pragma unroll
+  for (int w = 1; w < kMegaWaves; ++w)
+    if (head_replaces(s_v[w], s_i[w], bv, bi)) { bv = s_v[w]; bi = s_i[w]; }
+  const uint32_t chosen = bi == 0xffffffffu ? 0u : bi;   // (every logit NaN)
+  if (a.x_next) {
+    const uint16_t *row = a.embed + (int64_t)chosen * H;
+    for (int k = tid; k < H; k += kMegaThreads)
+      a.x_next[k] = a.embed_scale != 1.0f ? f32_to_bf16_bits(bf16_bits_to_f32(row[k]) * a.embed_scale) : row[k];
+  }
+  if (tid == 0) {
+    *a.token = chosen;
+    if (a.history) a.history[a.state->step] = chosen;
+    a.state->epoch += 1u;   // the next launch of the step kernel tags its packets differently
+    a.state->pos += a.dpos;
+    a.state->step += a.dstep;
+  }
+}
+
+static size_t head_lds_bytes(const HeadArgs &a, int num_cu) {
+  const int rows = (a.V + num_cu - 1) / num_cu + 1;
+  return (size_t)a.H * 4 + (size_t)rows * kMegaWaves * sizeof(float);
+}
+
+bool head_choice_eligible(const HeadArgs &a, int num_cu) {
+  if (!(a.H == 2560 || a.H == 2048) || num_cu < 1 || num_cu > 256) return false;
+  if (a.V < num_cu * 16 || (a.V + num_cu - 1) / num_cu + 1 > kHeadRowsMax) return false;   // at least a pass over the ring per wave
+  auto al16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+  return a.W && a.x && a.ln_w && a.ln_b && a.logits && a.best && a.token && a.state && al16(a.W) && al16(a.x) && al16(a.ln_w) &&
+         al16(a.ln_b) && (!a.x_next || a.embed);
+}
+
+int launch_phi2_head_choice(hipStream_t st, const HeadArgs &a, int num_cu) {
+  RAI_REQUIRE(head_choice_eligible(a, num_cu), RAI_ERR_UNSUPPORTED, "head with choice: H=%d V=%d on %d CUs not served", a.H, a.V, num_cu);
+  const size_t lds = head_lds_bytes(a, num_cu);
+  if (a.H == 2560) hipLaunchKernelGGL((k_phi2_head_choice<5>), dim3(num_cu), dim3(kMegaThreads), lds, st, a);
+  else hipLaunchKernelGGL((k_phi2_head_choice<4>), dim3(num_cu), dim3(kMegaThreads), lds, st, a);
+  return launch_check("phi2_head_choice");
+}
+
 size_t mega_lds_bytes(const MegaArgs &a, int D) {
   const int NG_V = kMegaThreads / (D / 8);
   size_t n = (size_t)(a.I + a.QD + a.H) * 2;

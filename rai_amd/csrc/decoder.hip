@@ -95,6 +95,7 @@ struct rai_hip_decoder {
   int token_log_cap;
   float *choice_val;          // [max_batch][kChoiceMaxSplits]: best value of each share of a wide logits row
   uint32_t *choice_idx;       // and its index
+  unsigned long long *head_best;   // one (value, row) word per block of the head kernel that also chooses the token
   char *hidden_copy;          // [max_rows, H]: the residual stream after the last layer, kept when a caller asks for it
   bool want_hidden;           // the running forward copies its final residual stream to hidden_copy
   char *head_f;               // fragment-order copy of the lm_head matrix
@@ -965,6 +966,27 @@ static int forward_phi2(rai_hip_decoder *d, int B, int S, bool advance_step, boo
   }
   h.out1 = d->logits; h.ld1 = d->V;
   h.M = B; h.N = d->V; h.K = H; h.n_split = d->V;
+  // One sequence, greedy: final norm, head and token choice as one launch of the step kernel's weight stream
+  // (RAI_HIP_NO_HEAD_KERNEL=1 keeps the three launches; read per call: tests compare both forms in one process).
+  const char *no_head = getenv("RAI_HIP_NO_HEAD_KERNEL");
+  if (B == 1 && dt == RAI_BF16 && !d->sample_on && d->mega_ok && !(no_head && *no_head && *no_head != '0')) {
+    HeadArgs ha;
+    memset(&ha, 0, sizeof(ha));
+    ha.W = (const uint16_t *)d->head_w; ha.bias = (const uint16_t *)d->head_b;
+    ha.x = (const uint16_t *)last_rows;
+    ha.ln_w = (const uint16_t *)d->lnf_w; ha.ln_b = (const uint16_t *)d->lnf_b; ha.ln_eps = (float)d->cfg.norm_eps;
+    ha.V = d->V; ha.H = H;
+    ha.logits = (uint16_t *)d->logits;
+    ha.best = d->head_best;
+    ha.token = d->tokens; ha.history = advance_step ? d->history : nullptr;
+    ha.state = d->state; ha.dpos = S; ha.dstep = advance_step ? 1 : 0;
+    ha.embed = (const uint16_t *)d->embed; ha.x_next = (uint16_t *)d->x; ha.embed_scale = d->embed_scale;
+    if (head_choice_eligible(ha, d->num_cu)) {
+      RAI_TRY(launch_phi2_head_choice(st, ha, d->num_cu));
+      d->ctx_len = T_after;
+      return RAI_OK;
+    }
+  }
   RAI_TRY(linear(d, st, h));
 
   RAI_TRY(launch_token_choice(d, st, B, S, advance_step));
@@ -1313,7 +1335,7 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->graph_sampled = false; d->graph_penalty = 0.f; d->graph_last_n = 0;
   d->head_f = nullptr; d->frag_ready = false;
   d->hidden_copy = nullptr; d->want_hidden = false;
-  d->choice_val = nullptr; d->choice_idx = nullptr;
+  d->choice_val = nullptr; d->choice_idx = nullptr; d->head_best = nullptr;
   const int vec = (int)(16 / d->es);
   int st = RAI_OK;
   auto bail = [&](int code) {
@@ -1364,6 +1386,8 @@ int rai_hip_decoder_create(int dev, const rai_hip_decoder_config *cfg, rai_hip_d
   d->choice_val = (float *)tmp;
   if ((st = dalloc(d, (size_t)cfg->max_batch * kChoiceMaxSplits * sizeof(uint32_t), &tmp))) return bail(st);
   d->choice_idx = (uint32_t *)tmp;
+  if ((st = dalloc(d, 256 * sizeof(unsigned long long), &tmp))) return bail(st);
+  d->head_best = (unsigned long long *)tmp;
   if (hipMemset(d->attn_counters, 0, attention_decode_counter_bytes(cfg->max_batch, d->Hq)) != hipSuccess)
     return bail(fail(RAI_ERR_HIP, "decoder_create: memset failed"));
 

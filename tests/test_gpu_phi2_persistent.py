@@ -193,3 +193,44 @@ def test_greedy_choice_takes_the_first_maximum_and_passes_over_nans(hip, vocab):
     dec.clear_kv_cache()
     assert dec.forward(prompt)[1][0] == 0
     dec.close()
+
+
+def test_head_kernel_against_norm_head_and_choice_as_three_launches(hip, monkeypatch):
+    # One sequence, greedy: the final LayerNorm, the head product and the token choice run as one launch (every block
+    # normalises once, streams its rows of the head like the step kernel does, and the block that finishes last picks
+    # among the blocks' best rows).  Against the three launches it replaces: logits to the bf16 bar (the rows are summed
+    # in a different order), the same tokens up to a near tie, the same device-side counters; graph replays repeat.
+    cfg = wide_cfg(vocab_size=16384, intermediate_size=512, num_hidden_layers=3)
+    prompt = np.random.Generator(np.random.PCG64(41)).integers(0, cfg.vocab_size, (1, 23)).astype(np.uint32)
+    monkeypatch.setenv("RAI_HIP_NO_HEAD_KERNEL", "1")
+    apart, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
+    la, ta = apart.forward(prompt)
+    ctx_forward = apart.context_len()
+    ga, _, _ = apart.generate(prompt, 20)
+    ctx_generate = apart.context_len()
+    monkeypatch.delenv("RAI_HIP_NO_HEAD_KERNEL")
+    one, _ = make(cfg, "bf16", hip, max_batch=1, max_context=96)
+    lo, to = one.forward(prompt)          # prefill, then the head kernel on the last row
+    want = ref.fwd(prompt)
+    assert_close(lo, want, "bf16", "prefill logits through the head kernel")
+    assert_close(lo, la, "bf16", "head kernel vs three launches")
+    assert to[0] == int(np.argmax(lo[0]))
+    assert one.context_len() == ctx_forward
+    nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
+    for step in range(4):                 # single-token steps: step kernel + head kernel
+        lo, to = one.forward(nxt)
+        want = ref.fwd(nxt)
+        assert_close(lo, want, "bf16", f"decode step {step}")
+        assert to[0] == int(np.argmax(lo[0]))
+        check_tokens(to, want, "bf16")
+        nxt = np.argmax(want, -1).astype(np.uint32).reshape(1, 1)
+    go, _, _ = one.generate(prompt, 20)
+    assert one.context_len() == ctx_generate
+    assert np.array_equal(go, one.generate(prompt, 20)[0])   # graph replays
+    wanted, logits_all = phi2.greedy_decode(ref, prompt, 20)
+    for s in range(20):
+        if go[0, s] != ga[0, s] or go[0, s] != wanted[0, s]:
+            check_tokens(go[:, s], logits_all[s], "bf16")   # a near tie in the oracle's own logits
+            break
+    apart.close()
+    one.close()
