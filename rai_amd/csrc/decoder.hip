@@ -14,6 +14,7 @@
 // residual).  A decode step fuses the LayerNorm into the weight-streaming
 // kernel: 3 launches per layer.  Context length and the current tokens live in
 // device memory, so consecutive greedy steps need no host round trip.
+#include <algorithm>
 #include <cstdlib>
 #include <map>
 #include <string>
@@ -1256,6 +1257,27 @@ static int check_fault(rai_hip_decoder *d) {
         fprintf(stderr, "mega prof block %3d: after A: +%.2f qkv polled | +%.2f k partials | +%.2f softmax | +%.2f attn published\n",
                 b, ex[2], ex[3], ex[4], ex[5]);
     }
+  }
+  if (d->mega_prof) {   // the exchange of the residual stream: from the last block's publication to a block's arrival
+    std::vector<unsigned long long> t((size_t)d->num_cu * d->L * 16);
+    RAI_HIP_TRY(hipMemcpy(t.data(), d->mega_prof, t.size() * 8, hipMemcpyDeviceToHost));
+    auto at = [&](int b, int l, int k) { return (double)t[((size_t)b * d->L + l) * 16 + k] * 0.01; };
+    double lat_min = 0, lat_mean = 0, lat_max = 0, spread = 0, behind_median = 0;
+    for (int l = 1; l < d->L; ++l) {
+      std::vector<double> pub(d->num_cu), arr(d->num_cu);
+      for (int b = 0; b < d->num_cu; ++b) { pub[b] = at(b, l - 1, 6); arr[b] = at(b, l, 8); }
+      const double last = *std::max_element(pub.begin(), pub.end());
+      std::vector<double> sorted = pub;
+      std::sort(sorted.begin(), sorted.end());
+      spread += (last - sorted.front()) / (d->L - 1);
+      behind_median += (last - sorted[sorted.size() / 2]) / (d->L - 1);
+      double mn = 1e30, mx = -1e30, sum = 0;
+      for (int b = 0; b < d->num_cu; ++b) { const double v = arr[b] - last; mn = v < mn ? v : mn; mx = v > mx ? v : mx; sum += v; }
+      lat_min += mn / (d->L - 1); lat_max += mx / (d->L - 1); lat_mean += sum / d->num_cu / (d->L - 1);
+    }
+    fprintf(stderr, "mega prof x exchange: the last block publishes %.2f us after the first and %.2f us after the median one; "
+                    "from that publication to the arrival at a block: min %.2f, mean %.2f, max %.2f us\n",
+            spread, behind_median, lat_min, lat_mean, lat_max);
   }
   if (d->mega_prof && getenv("RAI_HIP_MEGA_PROF_SKEW")) {  // how late each block reaches the end of each phase, mean over layers
     std::vector<unsigned long long> t((size_t)d->num_cu * d->L * 16);
