@@ -195,12 +195,15 @@ def test_greedy_choice_takes_the_first_maximum_and_passes_over_nans(hip, vocab):
     dec.close()
 
 
-def test_head_kernel_against_norm_head_and_choice_as_three_launches(hip, monkeypatch):
+@pytest.mark.parametrize("width", [dict(), dict(hidden_size=2048, partial_rotary_factor=0.5, vocab_size=8192),
+                                   dict(tie_word_embeddings=True, vocab_size=4096)])
+def test_head_kernel_against_norm_head_and_choice_as_three_launches(hip, monkeypatch, width):
     # One sequence, greedy: the final LayerNorm, the head product and the token choice run as one launch (every block
     # normalises once, streams its rows of the head like the step kernel does, and the block that finishes last picks
     # among the blocks' best rows).  Against the three launches it replaces: logits to the bf16 bar (the rows are summed
     # in a different order), the same tokens up to a near tie, the same device-side counters; graph replays repeat.
-    cfg = wide_cfg(vocab_size=16384, intermediate_size=512, num_hidden_layers=3)
+    # (both widths the kernel is built for; a head tied to the embedding matrix has no bias)
+    cfg = wide_cfg(**{**dict(vocab_size=16384, intermediate_size=512, num_hidden_layers=3), **width})
     prompt = np.random.Generator(np.random.PCG64(41)).integers(0, cfg.vocab_size, (1, 23)).astype(np.uint32)
     monkeypatch.setenv("RAI_HIP_NO_HEAD_KERNEL", "1")
     apart, ref = make(cfg, "bf16", hip, max_batch=1, max_context=96)
